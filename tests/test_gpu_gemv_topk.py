@@ -1,0 +1,132 @@
+"""Fused GEMV + top-k: fp32 scores bit-identical to the oracle's canonical order (and within 1e-5 of the
+fp64 dot), selected indices bit-identical, for the flat, chunked, grouped, centre-only and two-level forms."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.util import announce, randn_bits, to_dev
+
+pytestmark = pytest.mark.gpu
+
+SCALE = float(np.float32(1.0 / np.sqrt(128.0)))
+
+
+def _run_flat(dtype, B, H, G, N, k, seed, shared_kv=False, num_chunks=1, scale=SCALE, levels=False):
+    from topk_attn_amd import ops
+    rng = np.random.default_rng(seed)
+    q = randn_bits(rng, (B, H * G, 128), dtype)
+    kshape = (N, H, 128) if shared_kv else (B, N, H, 128)
+    if levels:
+        lv = np.linspace(-2, 2, 16)
+        K = oracle.to_bits(lv[rng.integers(0, 16, kshape)], dtype)
+    else:
+        K = randn_bits(rng, kshape, dtype)
+    idx, val, scores = ops.gemv_topk(to_dev(q, dtype), to_dev(K, dtype), k, group=G, scale=scale,
+                                     num_chunks=num_chunks, return_scores=True)
+    torch.cuda.synchronize()
+    idx, val, scores = idx.cpu().numpy(), val.cpu().numpy(), scores.cpu().numpy()
+    chunk = N // num_chunks
+    for b in range(B):
+        for h in range(H):
+            Kh = K[:, h, :] if shared_kv else K[b, :, h, :]
+            qf = oracle.group_query(q[b, h * G:(h + 1) * G], dtype, G)
+            ref = oracle.scores_canonical(Kh, dtype, qf, scale)
+            assert np.array_equal(scores[b, h].view(np.uint32), ref.view(np.uint32)), "scores differ (b=%d h=%d)" % (b, h)
+            truth = oracle.scores_f64(Kh, dtype, q[b, h * G:(h + 1) * G], scale)
+            assert np.abs(ref.astype(np.float64) - truth).max() < 1e-5 * max(1.0, np.abs(truth).max() / 4)
+            for c in range(num_chunks):
+                ei, ev = oracle.topk_stable(ref[c * chunk:(c + 1) * chunk], k)
+                got = idx[b, h, c * k:(c + 1) * k]
+                assert np.array_equal(got, ei + c * chunk), "indices differ (b=%d h=%d c=%d)" % (b, h, c)
+                assert np.array_equal(val[b, h, c * k:(c + 1) * k].view(np.uint32), ev.view(np.uint32))
+
+
+def test_config1_single_head():
+    """q fp16 [128], K fp16 [32768,128] N(0,1), scores K.q/sqrt(128), top-2048."""
+    announce("gemv_topk config 1: N=32768 k=2048 fp16")
+    _run_flat(oracle.F16, 1, 1, 1, 32768, 2048, seed=1)
+
+
+@pytest.mark.parametrize("dtype", [oracle.F16, oracle.BF16])
+def test_small_shapes(dtype):
+    announce("gemv_topk small shapes dtype=%d" % dtype)
+    _run_flat(dtype, 2, 3, 1, 1000, 100, seed=2)
+    _run_flat(dtype, 1, 2, 4, 4099, 257, seed=3)
+    _run_flat(dtype, 1, 1, 8, 130, 130, seed=4)
+
+
+def test_grouped_batched():
+    announce("gemv_topk B=2 Hkv=8 G=4 N=16384 k=2048 fp16")
+    _run_flat(oracle.F16, 2, 8, 4, 16384, 2048, seed=5)
+
+
+def test_shared_kv_chunked():
+    """The reference op's stage 1: 4 chunks of 2048 keys, top-K per chunk, no scale, KV shared by the batch."""
+    announce("gemv_topk chunked N=8192 chunks=4 k=128 shared KV")
+    _run_flat(oracle.F16, 2, 4, 1, 8192, 128, seed=6, shared_kv=True, num_chunks=4, scale=1.0)
+
+
+def test_tie_stress_bf16_levels():
+    """K quantised to 16 levels: many exact score ties; indices must still match bit for bit."""
+    announce("gemv_topk tie stress bf16 N=65536 G=8 k=4096")
+    _run_flat(oracle.BF16, 1, 2, 8, 65536, 4096, seed=7, levels=True)
+
+
+def test_unit_query_reproduces_column():
+    """q = e_i makes the score K[:, i] * scale exactly — a check that does not go through the oracle."""
+    from topk_attn_amd import ops
+    announce("gemv_scores unit query")
+    rng = np.random.default_rng(8)
+    K = randn_bits(rng, (3000, 2, 128), oracle.F16)
+    for i in (0, 7, 64, 127):
+        qv = np.zeros((1, 2, 128))
+        qv[0, :, i] = 1.0
+        s = ops.gemv_scores(to_dev(oracle.to_bits(qv, oracle.F16), oracle.F16), to_dev(K, oracle.F16), scale=0.5)
+        torch.cuda.synchronize()
+        want = oracle.from_bits(K[:, :, i], oracle.F16).T * np.float32(0.5)
+        assert np.array_equal(s[0].cpu().numpy(), want)
+
+
+def test_center_only_config2_shape():
+    """32 heads x 4096 centroids with a per-head mean shift, top-64, expand x64 -> 4096 token ids per head."""
+    from topk_attn_amd import ops
+    announce("center_topk_expand config 2")
+    rng = np.random.default_rng(2)
+    H, Cn, top_c, clen = 32, 4096, 64, 64
+    cen = rng.standard_normal((H, Cn, 128)) + 0.5 * rng.standard_normal((H, 1, 128))
+    cen_b = oracle.to_bits(cen, oracle.F16)
+    q_b = randn_bits(rng, (H, 128), oracle.F16)
+    out, cids, cval = ops.center_topk_expand(to_dev(q_b, oracle.F16), to_dev(cen_b, oracle.F16), top_c, clen, SCALE)
+    torch.cuda.synchronize()
+    out, cids, cval = out.cpu().numpy(), cids.cpu().numpy(), cval.cpu().numpy()
+    for h in range(H):
+        eo, ec, ev = oracle.center_topk_expand(q_b[h], cen_b[h], oracle.F16, top_c, clen, SCALE)
+        assert np.array_equal(cids[h], ec) and np.array_equal(out[h], eo)
+        assert np.array_equal(cval[h].view(np.uint32), ev.view(np.uint32))
+        # closed form of the expansion, independent of the oracle
+        assert np.array_equal(out[h].reshape(top_c, clen), cids[h][:, None] * clen + np.arange(clen)[None])
+
+
+def test_two_level_cluster_reference_shape():
+    """Reference constants of gemv_topk.cu:21-28 scaled down in heads: 32 centroids, clusters of 1280 tokens,
+    top-5 clusters, top-512 inside each."""
+    from topk_attn_amd import ops
+    announce("cluster_gemv_topk CSZ=32 CLEN=1280 TOPC=5 k=512")
+    rng = np.random.default_rng(12345)
+    H, CSZ, CLEN, TOPC, K = 4, 32, 1280, 5, 512
+    cen = rng.uniform(-0.5, 0.5, (H, CSZ, 128))
+    keys = cen.transpose(1, 0, 2)[:, None, :, :] + 0.05 * rng.standard_normal((CSZ, CLEN, H, 128))
+    keys = keys.reshape(CSZ * CLEN, H, 128)
+    cen_b, keys_b = oracle.to_bits(cen, oracle.F16), oracle.to_bits(keys, oracle.F16)
+    q_b = oracle.to_bits(rng.uniform(-0.5, 0.5, (H, 128)), oracle.F16)
+    out = ops.cluster_gemv_topk(to_dev(q_b, oracle.F16), to_dev(cen_b, oracle.F16), to_dev(keys_b, oracle.F16),
+                                TOPC, CLEN, K, 1.0)
+    torch.cuda.synchronize()
+    out = out.cpu().numpy()
+    for h in range(H):
+        want = oracle.cluster_topk(q_b[h], cen_b[h], keys_b[:, h, :], oracle.F16, TOPC, CLEN, K, 1.0)
+        assert np.array_equal(out[h], want)
+        # the reference's own check (gemv_topk.cu:138-170): set equality per (head, rank) slice
+        for r in range(TOPC):
+            assert set(out[h, r * K:(r + 1) * K]) == set(want[r * K:(r + 1) * K])

@@ -1,0 +1,94 @@
+"""Selection phase on caller-supplied fp32 scores: indices must equal the oracle's stable order bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.util import announce
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(scores_np, k):
+    from topk_attn_amd import ops
+    scores_np = np.ascontiguousarray(scores_np, np.float32)
+    if scores_np.ndim == 1:
+        scores_np = scores_np[None]
+    s = torch.from_numpy(scores_np).cuda()
+    idx, val = ops.topk(s, k)
+    torch.cuda.synchronize()
+    idx, val = idx.cpu().numpy(), val.cpu().numpy()
+    for r in range(scores_np.shape[0]):
+        ei, ev = oracle.topk_stable(scores_np[r], k)
+        assert np.array_equal(idx[r], ei), "row %d: first mismatch at rank %d" % (r, int(np.argmax(idx[r] != ei)))
+        assert np.array_equal(val[r].view(np.uint32), ev.view(np.uint32))
+
+
+CASES = [(1, 1), (1000, 1), (1000, 1000), (1024, 64), (2048, 1024), (4096, 64), (5000, 777), (32768, 2048),
+         (131072, 2048), (100000, 4096), (20000, 8192)]
+
+
+@pytest.mark.parametrize("n,k", CASES)
+def test_random_scores(n, k):
+    announce("topk random n=%d k=%d" % (n, k))
+    rng = np.random.default_rng(n * 31 + k)
+    _check(rng.standard_normal(n).astype(np.float32), k)
+
+
+@pytest.mark.parametrize("n,k", [(4096, 64), (32768, 2048), (70000, 4096)])
+def test_all_equal(n, k):
+    announce("topk all-equal n=%d k=%d" % (n, k))
+    _check(np.full(n, 1.5, np.float32), k)
+
+
+@pytest.mark.parametrize("n,k", [(8192, 100), (32768, 2048), (262144, 4096)])
+def test_few_levels(n, k):
+    """Scores drawn from 16 values: every rank boundary falls inside a large tie bucket."""
+    announce("topk 16-level n=%d k=%d" % (n, k))
+    rng = np.random.default_rng(7)
+    levels = np.linspace(-2, 2, 16).astype(np.float32)
+    _check(levels[rng.integers(0, 16, n)], k)
+
+
+def test_signed_zero_inf_nan():
+    announce("topk special values")
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(6000).astype(np.float32)
+    x[::7] = 0.0
+    x[3::7] = -0.0
+    x[5::97] = np.inf
+    x[11::89] = -np.inf
+    x[13::101] = np.nan
+    for k in (1, 50, 900, 3000, 6000):
+        _check(x, k)
+
+
+def test_ramps_and_segments():
+    announce("topk ramps, several segments")
+    n = 10000
+    up = np.arange(n, dtype=np.float32)
+    down = up[::-1].copy()
+    two = np.where(np.arange(n) % 2 == 0, 1.0, -1.0).astype(np.float32)
+    _check(np.stack([up, down, two, -up]), 1500)
+
+
+def test_strided_segments():
+    announce("topk strided rows")
+    from topk_attn_amd import ops
+    rng = np.random.default_rng(11)
+    full = rng.standard_normal((5, 9000)).astype(np.float32)
+    s = torch.from_numpy(full).cuda()
+    idx, _ = ops.topk(s[:, :7000], 300)
+    torch.cuda.synchronize()
+    for r in range(5):
+        ei, _ = oracle.topk_stable(full[r, :7000], 300)
+        assert np.array_equal(idx[r].cpu().numpy(), ei)
+
+
+def test_rejects_bad_k():
+    from topk_attn_amd import ops, TkaError
+    s = torch.zeros(2, 100, device="cuda")
+    with pytest.raises(TkaError):
+        ops.topk(s, 101)
+    with pytest.raises(TkaError):
+        ops.topk(s, 0)

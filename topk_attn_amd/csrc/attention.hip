@@ -1,0 +1,231 @@
+// Stages 2 and 3: split-K decode attention over a token list (dense range, gathered index list, or an
+// index list with caller-supplied logits) and the log-sum-exp combine.
+//
+// attn_partial_kernel — one workgroup per (split, KV head, batch entry), 4 waves.  A 16-lane row group
+// owns one token at a time: 16 B of the K row and 16 B of the V row per lane, scores for the G query
+// heads of the group by fma chain + DPP row reduce, online softmax in the exp2 domain
+// (baseline_1.cu:406-468 of the reference), fp32 accumulators of 8 output dims per lane and head.
+// The 16 row-group states of the workgroup are merged through LDS and written as one fp32
+// (m, l, acc[128]) partial per query head; nothing is atomically added and nothing needs pre-zeroing.
+//
+// lse_combine_kernel — out = sum_s acc_s 2^(m_s-M) / sum_s l_s 2^(m_s-M), written once
+// (replaces the DSM ring reduce + half atomicAdd of flash_decoding.cu:325-387).
+#include "kernels.hpp"
+
+namespace tka {
+
+namespace {
+
+constexpr int kAttnThreads = 256;
+constexpr int kAttnRowGroups = kAttnThreads / 16;  // 16 tokens in flight per step and load slot
+constexpr int kAttnUnroll = 4;                     // tokens per row group per step
+constexpr int kAttnStep = kAttnRowGroups * kAttnUnroll;  // 64 positions per workgroup step
+
+enum { MODE_DENSE = 0, MODE_INDEXED = 1, MODE_LOGIT = 2 };
+
+template <int DT, int G, int MODE>
+__global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p) {
+  __shared__ float sh_acc[kAttnRowGroups][kHeadDim];
+  __shared__ float sh_m[kAttnRowGroups];
+  __shared__ float sh_l[kAttnRowGroups];
+
+  const int tid = threadIdx.x;
+  const int j = tid & 15;
+  const int rg = tid >> 4;
+  const int split = blockIdx.x;
+  const int h = blockIdx.y;
+  const int b = blockIdx.z;
+  const int64_t seg = (int64_t)b * p.num_kv_heads + h;
+
+  int64_t count = p.seq_len;
+  if (MODE != MODE_DENSE) {
+    count = p.kv_count ? p.kv_count[seg] : p.idx_len;
+    if (count > p.idx_len) count = p.idx_len;
+    if (count < 0) count = 0;
+  }
+  const int64_t begin = (int64_t)split * p.tokens_per_split;
+  int64_t end = begin + p.tokens_per_split;
+  if (end > count) end = count;
+
+  const int32_t* idx = MODE != MODE_DENSE ? p.kv_idx + seg * p.idx_len : nullptr;
+  const float* logit = MODE == MODE_LOGIT ? p.kv_logit + seg * p.idx_len : nullptr;
+
+  float qf[G][8];
+  if (MODE != MODE_LOGIT) {
+    const uint16_t* qb = (const uint16_t*)p.q + (int64_t)b * p.q_stride_b + (int64_t)h * G * kHeadDim + 8 * j;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      u32x4 v = *(const u32x4*)(qb + g * kHeadDim);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[g][i] = Elem<DT>::get(v, i);
+    }
+  }
+
+  const int64_t head_off = (int64_t)b * p.kv_stride_b + (int64_t)h * p.kv_stride_h + 8 * j;
+  const uint16_t* kbase = (const uint16_t*)p.keys + head_off;
+  const uint16_t* vbase = (const uint16_t*)p.values + head_off;
+
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
+  }
+
+  for (int64_t base = begin; base < end; base += kAttnStep) {
+    int64_t tok[kAttnUnroll];
+    bool valid[kAttnUnroll];
+    float lg[kAttnUnroll];
+#pragma unroll
+    for (int u = 0; u < kAttnUnroll; ++u) {
+      int64_t pos = base + rg * kAttnUnroll + u;
+      valid[u] = pos < end;
+      int64_t pc = valid[u] ? pos : end - 1;
+      tok[u] = MODE == MODE_DENSE ? pc : (int64_t)idx[pc];
+      lg[u] = MODE == MODE_LOGIT ? logit[pc] : 0.0f;
+      if (MODE != MODE_DENSE && (tok[u] < 0 || tok[u] >= p.seq_len)) {  // skip ids outside the cache
+        valid[u] = false;                                                // (retrieval_attention.cu:1325)
+        tok[u] = 0;
+      }
+    }
+    u32x4 kv[kAttnUnroll], vv[kAttnUnroll];
+#pragma unroll
+    for (int u = 0; u < kAttnUnroll; ++u) {
+      if (MODE != MODE_LOGIT) kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + tok[u] * p.kv_stride_n));
+      vv[u] = __builtin_nontemporal_load((const u32x4*)(vbase + tok[u] * p.kv_stride_n));
+    }
+    float x[G][kAttnUnroll];
+#pragma unroll
+    for (int u = 0; u < kAttnUnroll; ++u) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float s;
+        if (MODE == MODE_LOGIT) {
+          s = lg[u] * p.scale_log2e;
+        } else {
+          float a = 0.0f;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) a = __builtin_fmaf(qf[g][i], Elem<DT>::get(kv[u], i), a);
+          s = row16_sum(a) * p.scale_log2e;
+        }
+        x[g][u] = valid[u] ? s : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float mx = m[g];
+#pragma unroll
+      for (int u = 0; u < kAttnUnroll; ++u) mx = fmaxf(mx, x[g][u]);
+      if (mx == -INFINITY) continue;  // nothing valid so far
+      const float alpha = __builtin_amdgcn_exp2f(m[g] - mx);  // m = -inf -> 0
+      m[g] = mx;
+      l[g] *= alpha;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+#pragma unroll
+      for (int u = 0; u < kAttnUnroll; ++u) {
+        const float pu = __builtin_amdgcn_exp2f(x[g][u] - mx);  // invalid -> 0
+        l[g] += pu;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = __builtin_fmaf(pu, Elem<DT>::get(vv[u], i), acc[g][i]);
+      }
+    }
+  }
+
+  // merge the 16 row-group states, one query head at a time
+  const int64_t row0 = ((int64_t)b * p.num_kv_heads + h) * G;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sh_acc[rg][8 * j + i] = acc[g][i];
+    if (j == 0) { sh_m[rg] = m[g]; sh_l[rg] = l[g]; }
+    __syncthreads();
+    if (tid < kHeadDim) {
+      float M = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < kAttnRowGroups; ++r) M = fmaxf(M, sh_m[r]);
+      float L = 0.0f, o = 0.0f;
+      if (M != -INFINITY) {
+#pragma unroll
+        for (int r = 0; r < kAttnRowGroups; ++r) {
+          const float w = __builtin_amdgcn_exp2f(sh_m[r] - M);
+          L += sh_l[r] * w;
+          o += sh_acc[r][tid] * w;
+        }
+      }
+      const int64_t slot = (row0 + g) * p.num_splits + split;
+      p.part_acc[slot * kHeadDim + tid] = o;
+      if (tid == 0) { p.part_m[slot] = M; p.part_l[slot] = L; }
+    }
+  }
+}
+
+template <int ODT>
+__global__ __launch_bounds__(kHeadDim) void lse_combine_kernel(CombineParams p) {
+  const int row = blockIdx.x;
+  const int d = threadIdx.x;
+  const float* pm = p.part_m + (int64_t)row * p.num_splits;
+  const float* pl = p.part_l + (int64_t)row * p.num_splits;
+  const float* pa = p.part_acc + (int64_t)row * p.num_splits * kHeadDim;
+  float M = -INFINITY;
+  for (int s = 0; s < p.num_splits; ++s)
+    if (pl[s] > 0.0f) M = fmaxf(M, pm[s]);
+  float L = 0.0f, o = 0.0f;
+  for (int s = 0; s < p.num_splits; ++s) {
+    const float ls = pl[s];
+    if (!(ls > 0.0f)) continue;
+    const float w = __builtin_amdgcn_exp2f(pm[s] - M);
+    L += ls * w;
+    o += pa[(int64_t)s * kHeadDim + d] * w;
+  }
+  const float r = L > 0.0f ? o / L : 0.0f;
+  const int bb = row / p.rows_per_batch, hh = row % p.rows_per_batch;
+  uint16_t* out = (uint16_t*)p.out + (int64_t)bb * p.out_stride_b + (int64_t)hh * kHeadDim;
+  out[d] = Elem<ODT>::narrow(r);
+  if (p.out_lse && d == 0) p.out_lse[row] = L > 0.0f ? (M + __builtin_log2f(L)) * 0.69314718055994531f : -INFINITY;
+}
+
+template <int DT, int MODE>
+int launch_partial_g(const AttnParams& p, dim3 grid, hipStream_t stream) {
+  switch (p.group) {
+    case 1: attn_partial_kernel<DT, 1, MODE><<<grid, kAttnThreads, 0, stream>>>(p); break;
+    case 2: attn_partial_kernel<DT, 2, MODE><<<grid, kAttnThreads, 0, stream>>>(p); break;
+    case 4: attn_partial_kernel<DT, 4, MODE><<<grid, kAttnThreads, 0, stream>>>(p); break;
+    case 8: attn_partial_kernel<DT, 8, MODE><<<grid, kAttnThreads, 0, stream>>>(p); break;
+    default: return TKA_EUNSUPPORTED;
+  }
+  return hip_status(hipGetLastError());
+}
+
+template <int DT>
+int launch_partial_dt(const AttnParams& p, dim3 grid, hipStream_t stream) {
+  if (p.kv_logit) {
+    if (p.group != 1) return TKA_EUNSUPPORTED;
+    attn_partial_kernel<DT, 1, MODE_LOGIT><<<grid, kAttnThreads, 0, stream>>>(p);
+    return hip_status(hipGetLastError());
+  }
+  if (p.kv_idx) return launch_partial_g<DT, MODE_INDEXED>(p, grid, stream);
+  return launch_partial_g<DT, MODE_DENSE>(p, grid, stream);
+}
+
+}  // namespace
+
+int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream) {
+  dim3 grid((unsigned)p.num_splits, (unsigned)p.num_kv_heads, (unsigned)p.batch);
+  LaunchTimer timer(p.kv_logit ? "attn_partial_logit" : (p.kv_idx ? "attn_partial_indexed" : "attn_partial_dense"), stream);
+  return dtype == TKA_F16 ? launch_partial_dt<TKA_F16>(p, grid, stream) : launch_partial_dt<TKA_BF16>(p, grid, stream);
+}
+
+int launch_lse_combine(const CombineParams& p, hipStream_t stream) {
+  LaunchTimer timer("lse_combine", stream);
+  if (p.out_dtype == TKA_F16)
+    lse_combine_kernel<TKA_F16><<<(unsigned)p.rows, kHeadDim, 0, stream>>>(p);
+  else
+    lse_combine_kernel<TKA_BF16><<<(unsigned)p.rows, kHeadDim, 0, stream>>>(p);
+  return hip_status(hipGetLastError());
+}
+
+}  // namespace tka

@@ -1,0 +1,138 @@
+// Shared device helpers for the gfx950 kernels: 16-bit element widening, DPP / ds_swizzle lane
+// exchanges for wave64, the order-preserving score key, and host-side launch bookkeeping.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/topk_attn.h"
+
+namespace tka {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kHeadDim = TKA_HEAD_DIM;
+constexpr int kWave = 64;
+constexpr int kHistBits = 11;
+constexpr int kHistBins = 1 << kHistBits;  // first-level selection histogram: top 11 bits of the key
+
+// ---- lane exchanges ---------------------------------------------------------------------------
+
+// DPP move: returns the value of the lane selected by CTRL inside the 16-lane row.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, false);
+}
+
+// Sum over the 16 lanes of a DPP row; every lane ends with the same value.  row_ror by 8, 4, 2, 1
+// pairs each lane with its xor-8, xor-4, xor-2, xor-1 partner's partial (the partials have period 8,
+// 4, 2 after each step), so the tree is the butterfly of gemv_topk.cu:325-328 bit for bit.
+__device__ __forceinline__ float row16_sum(float p) {
+  p = p + dpp_f32<0x128>(p);
+  p = p + dpp_f32<0x124>(p);
+  p = p + dpp_f32<0x122>(p);
+  p = p + dpp_f32<0x121>(p);
+  return p;
+}
+
+// Value held by lane (lane ^ M) of the wave, M a power of two.
+//   M = 1, 2  : DPP quad_perm          M = 8 : DPP row_ror:8
+//   M = 4, 16 : ds_swizzle bit mode    M = 32: ds_bpermute
+template <int M>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t v) {
+  if constexpr (M == 1) {
+    return dpp_u32<0xB1>(v);  // quad_perm [1,0,3,2]
+  } else if constexpr (M == 2) {
+    return dpp_u32<0x4E>(v);  // quad_perm [2,3,0,1]
+  } else if constexpr (M == 8) {
+    return dpp_u32<0x128>(v);  // row_ror:8
+  } else if constexpr (M == 4 || M == 16) {
+    return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (M << 10) | 0x1f);
+  } else {
+    static_assert(M == 32, "lane_xor: unsupported distance");
+    int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    return (uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, (int)v);
+  }
+}
+
+template <int M>
+__device__ __forceinline__ uint64_t lane_xor64(uint64_t v) {
+  uint32_t lo = lane_xor<M>((uint32_t)v);
+  uint32_t hi = lane_xor<M>((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
+__device__ __forceinline__ int lane_id() {
+  return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+// ---- 16-bit elements --------------------------------------------------------------------------
+
+template <int DT>
+struct Elem;
+
+template <>
+struct Elem<TKA_F16> {
+  // widen element `i` (0..7) of a 16-byte packet
+  static __device__ __forceinline__ float get(const u32x4& v, int i) {
+    uint32_t w = v[i >> 1];
+    uint16_t h = (i & 1) ? (uint16_t)(w >> 16) : (uint16_t)w;
+    return (float)__builtin_bit_cast(_Float16, h);
+  }
+  static __device__ __forceinline__ float widen(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+  static __device__ __forceinline__ uint16_t narrow(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+};
+
+template <>
+struct Elem<TKA_BF16> {
+  static __device__ __forceinline__ float get(const u32x4& v, int i) {
+    uint32_t w = v[i >> 1];
+    return __builtin_bit_cast(float, (i & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+  static __device__ __forceinline__ float widen(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
+  static __device__ __forceinline__ uint16_t narrow(float f) {  // round to nearest even
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+  }
+};
+
+// ---- score key --------------------------------------------------------------------------------
+
+// Order-preserving fp32 -> uint32 (bigger score, bigger key); -0.0 == +0.0; NaN is the lowest key.
+__device__ __forceinline__ uint32_t score_key(float x) {
+  if (x != x) return 0u;
+  uint32_t u = __builtin_bit_cast(uint32_t, x + 0.0f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_score(uint32_t key) {
+  uint32_t u = (key & 0x80000000u) ? (key & 0x7fffffffu) : ~key;
+  return __builtin_bit_cast(float, u);
+}
+// 64-bit composite: all elements distinct, larger = earlier in (score desc, index asc) order.
+__device__ __forceinline__ uint64_t composite(uint32_t key, uint32_t idx) { return ((uint64_t)key << 32) | (uint32_t)~idx; }
+
+// ---- host-side launch bookkeeping -------------------------------------------------------------
+
+// Records an event pair around a launch when profiling is on (see tka_profile_enable).
+struct LaunchTimer {
+  LaunchTimer(const char* name, hipStream_t stream);
+  ~LaunchTimer();
+  const char* name_;
+  hipStream_t stream_;
+  void* slot_;
+};
+
+inline int hip_status(hipError_t e) { return e == hipSuccess ? TKA_OK : TKA_EHIP; }
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace tka

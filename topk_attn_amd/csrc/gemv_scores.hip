@@ -1,0 +1,122 @@
+// Stage 1, GEMV phase: stream the key rows of one KV head once, produce fp32 scores in the canonical
+// 16-lane order (gemv_topk.cu:303-332 of the reference) and the first-level selection histogram.
+//
+// Mapping (wave64): 16 lanes x 16 B cover one 256-byte head row, so one global_load_dwordx4 brings
+// four rows per wave; each lane keeps its 8 query dims in registers for the whole
+// kernel; the 16-lane reduce is four DPP row rotations (no LDS).  Eight loads are in flight per lane.
+// HBM-bound: 256 B read + 4 B written per row.
+#include "kernels.hpp"
+
+namespace tka {
+
+namespace {
+
+constexpr int kGemvThreads = 256;
+constexpr int kGemvUnroll = 8;                                         // loads in flight per lane
+constexpr int kGemvRowsPerIter = (kGemvThreads / 16) * kGemvUnroll;    // 128 tokens per WG iteration
+
+template <int DT>
+__global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p) {
+  __shared__ uint32_t sh_hist[kHistBins];
+
+  const int tid = threadIdx.x;
+  const int j = tid & 15;            // lane inside the row: dims 8j..8j+7
+  const int rg = tid >> 4;           // row group 0..15 inside the workgroup
+  const int h = blockIdx.y;
+  const int b = blockIdx.z;
+  const int chunk = blockIdx.x / p.wgs_per_chunk;
+  const int wg_in_chunk = blockIdx.x % p.wgs_per_chunk;
+  const int64_t seg = ((int64_t)b * p.num_kv_heads + h) * p.num_chunks + chunk;
+  // tokens are counted inside the chunk; the chunk starts at chunk*chunk_len, or at the start of the
+  // cluster chosen for this (head, rank) in two-level selection
+  const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
+  const int64_t t_begin = (int64_t)wg_in_chunk * p.tokens_per_wg;
+  int64_t t_end = t_begin + p.tokens_per_wg;
+  if (t_end > p.chunk_len) t_end = p.chunk_len;
+
+  const bool do_hist = p.hist != nullptr;
+  if (do_hist) {
+    for (int i = tid; i < kHistBins; i += kGemvThreads) sh_hist[i] = 0;
+    __syncthreads();
+  }
+
+  // Group query in fp32: ((q0 + q1) + q2) + ... in ascending head order.
+  float qf[8];
+  {
+    const uint16_t* qb = (const uint16_t*)p.q + (int64_t)b * p.q_stride_b + (int64_t)h * p.group * kHeadDim + 8 * j;
+    u32x4 v = *(const u32x4*)qb;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] = Elem<DT>::get(v, i);
+    for (int g = 1; g < p.group; ++g) {
+      u32x4 w = *(const u32x4*)(qb + (int64_t)g * kHeadDim);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[i] = qf[i] + Elem<DT>::get(w, i);
+    }
+  }
+
+  const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
+                          chunk_base * p.key_stride_n + 8 * j;
+  float* sc_out = p.scores + seg * p.chunk_len;
+
+  for (int64_t base = t_begin; base < t_end; base += kGemvRowsPerIter) {
+    // row group rg owns 8 consecutive tokens per iteration: load u brings token base + rg*8 + u
+    u32x4 kv[kGemvUnroll];
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      int64_t t = base + rg * kGemvUnroll + u;
+      int64_t tc = t < t_end ? t : t_end - 1;
+      kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + tc * p.key_stride_n));
+    }
+    float mine = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc = __builtin_fmaf(qf[i], Elem<DT>::get(kv[u], i), acc);
+      float s = row16_sum(acc) * p.scale;
+      if (j == u) mine = s;
+    }
+    // lane j < 8 of row group rg now holds the score of token base + rg*8 + j: a wave writes 32
+    // consecutive floats
+    if (j < kGemvUnroll) {
+      int64_t t = base + rg * kGemvUnroll + j;
+      if (t < t_end) {
+        sc_out[t] = mine;
+        if (do_hist) atomicAdd(&sh_hist[score_key(mine) >> (32 - kHistBits)], 1u);
+      }
+    }
+  }
+
+  if (do_hist) {
+    __syncthreads();
+    uint32_t* gh = p.hist + seg * kHistBins;
+    for (int i = tid; i < kHistBins; i += kGemvThreads) {
+      uint32_t c = sh_hist[i];
+      if (c) atomicAdd(&gh[i], c);
+    }
+  }
+}
+
+}  // namespace
+
+int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
+  dim3 grid((unsigned)(p.num_chunks * p.wgs_per_chunk), (unsigned)p.num_kv_heads, (unsigned)p.batch);
+  LaunchTimer timer("gemv_scores", stream);
+  if (dtype == TKA_F16)
+    gemv_scores_kernel<TKA_F16><<<grid, kGemvThreads, 0, stream>>>(p);
+  else
+    gemv_scores_kernel<TKA_BF16><<<grid, kGemvThreads, 0, stream>>>(p);
+  return hip_status(hipGetLastError());
+}
+
+// Tokens per workgroup: enough workgroups to fill 256 CUs several times over, but long enough runs
+// that the per-workgroup histogram flush stays small.
+int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len) {
+  int64_t t = total_rows / 4096;
+  int64_t tpw = 128;
+  while (tpw * 2 <= t && tpw < 2048) tpw *= 2;
+  while (tpw > 128 && tpw > chunk_len) tpw /= 2;
+  return (int)tpw;
+}
+
+}  // namespace tka

@@ -1,0 +1,93 @@
+// Parameter blocks and launch functions of the device kernels (internal to the library).
+#pragma once
+#include "common.hpp"
+
+namespace tka {
+
+// ---- stage 1: GEMV ----------------------------------------------------------------------------
+struct GemvParams {
+  const void* q;        // [batch][num_kv_heads*group][128]
+  const void* keys;
+  float* scores;        // [batch][num_kv_heads][num_chunks][chunk_len]
+  const int32_t* cluster_ids;  // [batch*num_kv_heads*num_chunks] or nullptr: chunk c covers the tokens of that cluster
+  uint32_t* hist;       // [batch*num_kv_heads*num_chunks][kHistBins] or nullptr; must be zero on entry
+  int64_t chunk_len;    // tokens per chunk
+  int64_t q_stride_b, key_stride_b, key_stride_n, key_stride_h;
+  int batch, num_kv_heads, group, num_chunks;
+  int wgs_per_chunk, tokens_per_wg;
+  float scale;
+};
+int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream);
+int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);
+
+// ---- stage 1: selection -----------------------------------------------------------------------
+struct SelectParams {
+  const float* scores;    // segment s starts at scores + s*seg_stride
+  int64_t seg_len;
+  int64_t seg_stride;
+  uint32_t* hist;         // [num_segments][kHistBins]
+  uint32_t* counters;     // [num_segments][4]: sure count, maybe count, parts done, unused; zero on entry
+  uint64_t* sure;         // [num_segments][k]       composites known to be selected
+  uint64_t* maybe;        // [num_segments][seg_len] composites of the threshold bin
+  int32_t* out_idx;       // [num_segments][out_stride]
+  float* out_val;         // same shape or nullptr
+  int32_t* out_expand;    // [num_segments][k*expand] or nullptr (centre-only expansion)
+  int64_t out_stride;
+  int num_segments;
+  int k;
+  int parts;              // workgroups per segment
+  int part_len;           // scores per workgroup (multiple of 1024)
+  const int32_t* seg_base_ids;  // nullptr, or per segment a cluster id: index base = id * seg_len
+  int segs_per_row;       // chunks per (batch, head): index base = (s % segs_per_row) * seg_len
+  int expand;             // cluster_len of the expansion, 0 = none
+};
+size_t select_workspace_bytes(int num_segments, int64_t seg_len, int k);
+// Carves the workspace: hist, counters, sure, maybe (in that order, 256-byte aligned).
+void select_carve(void* ws, int num_segments, int64_t seg_len, int k, SelectParams* p);
+void select_plan(int64_t seg_len, int num_segments, SelectParams* p);
+int launch_zero_u32(uint32_t* ptr, size_t count, hipStream_t stream);
+int launch_select_hist(const SelectParams& p, hipStream_t stream);
+int launch_select(const SelectParams& p, hipStream_t stream);   // filter + finalize
+
+struct UnionParams {
+  const int32_t* idx;     // [num_segments][k]
+  int32_t* out_idx;       // [num_segments][k+sink+local]
+  int32_t* out_count;     // [num_segments]
+  int64_t seq_len;
+  int num_segments, k, sink, local;
+};
+int launch_index_union(const UnionParams& p, hipStream_t stream);
+
+// ---- stages 2/3: attention --------------------------------------------------------------------
+struct AttnParams {
+  const void* q;
+  const void* keys;
+  const void* values;
+  const int32_t* kv_idx;    // [batch][num_kv_heads][idx_len] or nullptr (dense)
+  const int32_t* kv_count;  // [batch][num_kv_heads] or nullptr
+  const float* kv_logit;    // [batch][num_kv_heads][idx_len] or nullptr
+  float* part_m;            // [rows][num_splits]
+  float* part_l;            // [rows][num_splits]
+  float* part_acc;          // [rows][num_splits][128]
+  int64_t seq_len;
+  int64_t q_stride_b, kv_stride_b, kv_stride_n, kv_stride_h;
+  int batch, num_kv_heads, group, num_splits;
+  int idx_len;
+  int tokens_per_split;     // positions per workgroup
+  float scale_log2e;        // scale * log2(e)
+};
+int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream);
+
+struct CombineParams {
+  const float* part_m;
+  const float* part_l;
+  const float* part_acc;
+  void* out;
+  float* out_lse;
+  int64_t out_stride_b;     // elements between batch entries of out
+  int rows_per_batch;       // query heads
+  int rows, num_splits, out_dtype;
+};
+int launch_lse_combine(const CombineParams& p, hipStream_t stream);
+
+}  // namespace tka
