@@ -163,29 +163,56 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
   }
 }
 
+constexpr int kCombineGroups = 8;  // split subsets reduced in parallel, then merged through LDS
+
 template <int ODT>
-__global__ __launch_bounds__(kHeadDim) void lse_combine_kernel(CombineParams p) {
+__global__ __launch_bounds__(kHeadDim * kCombineGroups) void lse_combine_kernel(CombineParams p) {
+  __shared__ float sh_m[kCombineGroups], sh_l[kCombineGroups][kHeadDim], sh_o[kCombineGroups][kHeadDim];
   const int row = blockIdx.x;
-  const int d = threadIdx.x;
+  const int d = threadIdx.x & (kHeadDim - 1);
+  const int g = threadIdx.x / kHeadDim;
   const float* pm = p.part_m + (int64_t)row * p.num_splits;
   const float* pl = p.part_l + (int64_t)row * p.num_splits;
   const float* pa = p.part_acc + (int64_t)row * p.num_splits * kHeadDim;
   float M = -INFINITY;
-  for (int s = 0; s < p.num_splits; ++s)
-    if (pl[s] > 0.0f) M = fmaxf(M, pm[s]);
-  float L = 0.0f, o = 0.0f;
-  for (int s = 0; s < p.num_splits; ++s) {
-    const float ls = pl[s];
-    if (!(ls > 0.0f)) continue;
-    const float w = __builtin_amdgcn_exp2f(pm[s] - M);
-    L += ls * w;
-    o += pa[(int64_t)s * kHeadDim + d] * w;
+  for (int s = g; s < p.num_splits; s += kCombineGroups) {
+    const float ls = pl[s], ms = pm[s];
+    if (ls > 0.0f) M = fmaxf(M, ms);
   }
-  const float r = L > 0.0f ? o / L : 0.0f;
+  float L = 0.0f, o = 0.0f;
+  for (int s = g; s < p.num_splits; s += kCombineGroups) {
+    const float ls = pl[s], ms = pm[s], as = pa[(int64_t)s * kHeadDim + d];
+    if (ls > 0.0f) {
+      const float w = __builtin_amdgcn_exp2f(ms - M);
+      L += ls * w;
+      o += as * w;
+    }
+  }
+  if (d == 0) sh_m[g] = M;
+  sh_l[g][d] = L;
+  sh_o[g][d] = o;
+  __syncthreads();
+  if (g != 0) return;
+  float Mt = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kCombineGroups; ++i) Mt = fmaxf(Mt, sh_m[i]);
+  float Lt = 0.0f, ot = 0.0f;
+  if (Mt != -INFINITY) {
+#pragma unroll
+    for (int i = 0; i < kCombineGroups; ++i) {
+      const float mi = sh_m[i];
+      if (mi != -INFINITY) {
+        const float w = __builtin_amdgcn_exp2f(mi - Mt);
+        Lt += sh_l[i][d] * w;
+        ot += sh_o[i][d] * w;
+      }
+    }
+  }
+  const float r = Lt > 0.0f ? ot / Lt : 0.0f;
   const int bb = row / p.rows_per_batch, hh = row % p.rows_per_batch;
   uint16_t* out = (uint16_t*)p.out + (int64_t)bb * p.out_stride_b + (int64_t)hh * kHeadDim;
   out[d] = Elem<ODT>::narrow(r);
-  if (p.out_lse && d == 0) p.out_lse[row] = L > 0.0f ? (M + __builtin_log2f(L)) * 0.69314718055994531f : -INFINITY;
+  if (p.out_lse && d == 0) p.out_lse[row] = Lt > 0.0f ? (Mt + __builtin_log2f(Lt)) * 0.69314718055994531f : -INFINITY;
 }
 
 template <int DT, int MODE>
@@ -222,9 +249,9 @@ int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream) {
 int launch_lse_combine(const CombineParams& p, hipStream_t stream) {
   LaunchTimer timer("lse_combine", stream);
   if (p.out_dtype == TKA_F16)
-    lse_combine_kernel<TKA_F16><<<(unsigned)p.rows, kHeadDim, 0, stream>>>(p);
+    lse_combine_kernel<TKA_F16><<<(unsigned)p.rows, kHeadDim * kCombineGroups, 0, stream>>>(p);
   else
-    lse_combine_kernel<TKA_BF16><<<(unsigned)p.rows, kHeadDim, 0, stream>>>(p);
+    lse_combine_kernel<TKA_BF16><<<(unsigned)p.rows, kHeadDim * kCombineGroups, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 

@@ -5,6 +5,7 @@
 // four rows per wave; each lane keeps its 8 query dims in registers for the whole
 // kernel; the 16-lane reduce is four DPP row rotations (no LDS).  Eight loads are in flight per lane.
 // HBM-bound: 256 B read + 4 B written per row.
+#include <stdlib.h>
 #include "kernels.hpp"
 
 namespace tka {
@@ -112,6 +113,7 @@ int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
 // Tokens per workgroup: enough workgroups to fill 256 CUs several times over, but long enough runs
 // that the per-workgroup histogram flush stays small.
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len) {
+  if (const char* e = getenv("TKA_TPW")) return atoi(e);  // TEMP sweep knob
   int64_t t = total_rows / 4096;
   int64_t tpw = 128;
   while (tpw * 2 <= t && tpw < 2048) tpw *= 2;

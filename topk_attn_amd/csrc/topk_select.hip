@@ -9,12 +9,13 @@
 //   2. filter: each workgroup finds the threshold bin b1 from the histogram, keeps its slice of the
 //      scores in registers, and appends composites with bin > b1 to the "sure" list and bin == b1 to
 //      the "maybe" list (one global reservation per workgroup and list);
-//   3. the last workgroup of a segment to finish refines the threshold inside the maybe list with
-//      further 11-bit radix passes (stops as soon as a bucket is taken whole), gathers the k
-//      survivors in LDS, sorts them with a bitonic network (registers, DPP / ds_swizzle across lanes,
-//      LDS across waves) and writes indices and values.
+//   3. finalize (next kernel, one workgroup per segment): refines the threshold inside the maybe
+//      list with further 11-bit radix passes (stops as soon as a bucket is taken whole), gathers
+//      the k survivors in LDS, sorts them with a bitonic network (registers, DPP / ds_swizzle across
+//      lanes, LDS across waves) and writes indices and values.
 //
-// No workgroup ever waits for another: the hand-off is "last one to arrive does the rest".
+// No workgroup ever waits for another: the hand-off between 2 and 3 is the kernel boundary (a
+// device-scope fence per workgroup would write back the whole L2 of its XCD each time).
 // Traffic: 4 B read per score plus 8 B written and read per sure/maybe element; scores come from L2 /
 // Infinity Cache when the GEMV has just written them.
 #include "kernels.hpp"
@@ -167,18 +168,12 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(SelectParams p
   }
 }
 
-// Dynamic LDS layout of select_kernel: [0, 8 KB) histogram; then kpad composites (sort buffer);
-// then kpad composites (cross-wave exchange buffer).
-__global__ __launch_bounds__(kSelThreads) void select_kernel(SelectParams p, int kpad) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint32_t* sh_hist = (uint32_t*)smem;
-  uint64_t* sh_sort = (uint64_t*)(smem + kHistBins * sizeof(uint32_t));
-  uint64_t* sh_xchg = sh_sort + kpad;
+__global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams p) {
+  __shared__ uint32_t sh_hist[kHistBins];
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
   __shared__ uint32_t sh_cnt[2];    // workgroup totals: sure, maybe
   __shared__ uint32_t sh_base[2];   // global reservation bases
-  __shared__ uint32_t sh_last;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -256,16 +251,35 @@ __global__ __launch_bounds__(kSelThreads) void select_kernel(SelectParams p, int
     }
   }
 
-  // ---- 3. the last workgroup of the segment finishes the job
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) sh_last = (atomicAdd(&ctr[2], 1u) == (uint32_t)(p.parts - 1));
-  __syncthreads();
-  if (!sh_last) return;
-  __threadfence();
+}
 
-  const uint32_t n_sure = __hip_atomic_load(&ctr[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const uint32_t n_maybe = __hip_atomic_load(&ctr[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Dynamic LDS layout of select_finalize_kernel: [0, 8 KB) histogram; then kpad composites (sort
+// buffer); then kpad composites (cross-wave exchange buffer).
+__global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectParams p, int kpad) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint32_t* sh_hist = (uint32_t*)smem;
+  uint64_t* sh_sort = (uint64_t*)(smem + kHistBins * sizeof(uint32_t));
+  uint64_t* sh_xchg = sh_sort + kpad;
+  __shared__ uint32_t sh_wtot[kSelWaves];
+  __shared__ uint32_t sh_res[4];
+  __shared__ uint32_t sh_cnt[2];
+
+  const int tid = threadIdx.x;
+  const int seg = blockIdx.x;
+  const uint32_t k = (uint32_t)p.k;
+  const uint32_t* ctr = p.counters + (int64_t)seg * 4;
+  const uint32_t n_sure = ctr[0];
+  const uint32_t n_maybe = ctr[1];
+
+  // threshold bin again (cheap) — the maybe list holds exactly the elements of bin b1
+  {
+    const uint32_t* gh = p.hist + (int64_t)seg * kHistBins;
+    sh_hist[2 * tid] = gh[2 * tid];
+    sh_hist[2 * tid + 1] = gh[2 * tid + 1];
+    __syncthreads();
+    find_threshold_bin(sh_hist, k, sh_wtot, sh_res);
+  }
+  const uint32_t b1 = sh_res[0];
   const uint64_t* sure = p.sure + (int64_t)seg * p.k;
   const uint64_t* maybe = p.maybe + (int64_t)seg * p.seg_len;
 
@@ -467,12 +481,17 @@ int launch_select(const SelectParams& p, hipStream_t stream) {
   const size_t lds = kHistBins * sizeof(uint32_t) + 2 * (size_t)kpad * sizeof(uint64_t);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)select_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);
+    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);
     if (e != hipSuccess) return TKA_EHIP;
     attr_set = true;
   }
-  LaunchTimer timer("topk_select", stream);
-  select_kernel<<<dim3((unsigned)p.parts, (unsigned)p.num_segments), kSelThreads, lds, stream>>>(p, kpad);
+  {
+    LaunchTimer timer("select_filter", stream);
+    select_filter_kernel<<<dim3((unsigned)p.parts, (unsigned)p.num_segments), kSelThreads, 0, stream>>>(p);
+    if (hipGetLastError() != hipSuccess) return TKA_EHIP;
+  }
+  LaunchTimer timer("select_finalize", stream);
+  select_finalize_kernel<<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(p, kpad);
   return hip_status(hipGetLastError());
 }
 
