@@ -74,8 +74,10 @@ def main():
     w = WORKLOADS[args.workload]
     scale = float(torch.tensor(1.0 / 128.0 ** 0.5, dtype=torch.float32).item())
     q, K, V = make_inputs(torch, w, dev)
+    # production configuration: the attention consumes the union list; the optional rank-ordered top-k
+    # output (a sort per KV head) is not requested
     plan = ops.SparseDecodePlan(q, K, V, w["k"], w["sink"], w["local"], scale, w["group"],
-                                out_dtype=getattr(torch, w["out_dtype"]))
+                                out_dtype=getattr(torch, w["out_dtype"]), want_topk=False)
 
     for _ in range(args.warmup):
         plan.step()
@@ -139,14 +141,19 @@ def main():
         times.sort()
         cpu_s = times[len(times) // 2] * B
         # sanity (not the parity oracle): same selected sets, outputs close
-        same_sets = all(set(ref_top[h].tolist()) == set(plan.topk_idx[0, h].tolist()) for h in range(H))
+        lo, hi = min(w["sink"], N), max(N - w["local"], min(w["sink"], N))
+        same_sets = True
+        for h in range(H):
+            want = set(range(lo)) | set(range(hi, N)) | set(ref_top[h].tolist())
+            got = plan.union_idx[0, h, :int(plan.union_count[0, h])].tolist()
+            same_sets = same_sets and got == sorted(want)
         max_err = (plan.out[0].float().cpu() - ref_out).abs().max().item()
         out["cpu_baseline"] = {
             "value": round(step_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "us_per_step": round(cpu_s * 1e6, 1),
             "cores": torch.get_num_threads(), "host_cpus": os.cpu_count(), "kind": "port",
             "sample": "batch entry 0 of %d (all %d KV heads, full N=%d), median of %d runs, scaled x%d" % (
                 B, H, N, args.cpu_runs, B),
-            "topk_sets_equal_gpu": bool(same_sets), "out_max_abs_diff_vs_gpu": round(max_err, 5)}
+            "union_sets_equal_gpu": bool(same_sets), "out_max_abs_diff_vs_gpu": round(max_err, 5)}
     print(json.dumps(out))
     return 0
 

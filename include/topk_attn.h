@@ -321,8 +321,8 @@ typedef struct tka_sparse_decode_args {
   int64_t kv_stride_h;
   float scale;
   int32_t reserved0;
-  int32_t* out_topk_idx;  /* device [batch][num_kv_heads][k] rank order; may be NULL          */
-  float* out_topk_val;    /* device, same shape; may be NULL                                  */
+  int32_t* out_topk_idx;  /* device [batch][num_kv_heads][k] rank order; may be NULL (saves a sort) */
+  float* out_topk_val;    /* device, same shape; may be NULL; needs out_topk_idx              */
   int32_t* out_union_idx; /* device [batch][num_kv_heads][k+sink+local]; may be NULL          */
   int32_t* out_union_count;/* device [batch][num_kv_heads]; may be NULL                       */
   void* workspace;

@@ -129,8 +129,16 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
 }
 
-// Runs zero + GEMV(+histogram) + select.  `ws` holds [scores][select workspace].
-int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, const int32_t* cluster_ids = nullptr) {
+struct UnionOut {
+  int32_t* idx;
+  int32_t* count;
+  int sink, local;
+};
+
+// Runs clear + GEMV (+histogram) + select.  `ws` holds [scores][select workspace].
+// a->out_idx == nullptr skips the rank-order sort (then `u` must ask for the union list).
+int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, const int32_t* cluster_ids = nullptr,
+                  const UnionOut* u = nullptr) {
   hipStream_t stream = (hipStream_t)a->stream;
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
@@ -140,7 +148,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
 
   SelectParams sp;
   memset(&sp, 0, sizeof sp);
-  select_carve(ws, segs, chunk_len, a->k, &sp);
+  const size_t zero_words = select_carve(ws, segs, chunk_len, &sp);
   select_plan(chunk_len, segs, &sp);
   sp.scores = scores;
   sp.seg_len = chunk_len;
@@ -154,9 +162,13 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   sp.segs_per_row = a->num_chunks;
   sp.expand = expand;
   sp.seg_base_ids = cluster_ids;
+  if (u) {
+    sp.union_idx = u->idx;
+    sp.union_count = u->count;
+    sp.sink = u->sink;
+    sp.local = u->local;
+  }
 
-  // histogram and counters are adjacent: one clear
-  const size_t zero_words = ((unsigned char*)sp.sure - (unsigned char*)sp.hist) / sizeof(uint32_t);
   int rc = launch_zero_u32(sp.hist, zero_words, stream);
   if (rc != TKA_OK) return rc;
   GemvParams gp;
@@ -291,7 +303,7 @@ int tka_version(void) { return 100; }
 size_t tka_gemv_topk_workspace_bytes(const tka_gemv_topk_args* a) {
   if (check_gemv(a, true) != TKA_OK) return 0;
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
-  return gemv_scores_bytes(a) + select_workspace_bytes(segs, a->seq_len / a->num_chunks, a->k);
+  return gemv_scores_bytes(a) + select_workspace_bytes(segs, a->seq_len / a->num_chunks);
 }
 
 int tka_gemv_topk(const tka_gemv_topk_args* a) {
@@ -319,7 +331,7 @@ static int check_topk(const tka_topk_args* a) {
 
 size_t tka_topk_workspace_bytes(const tka_topk_args* a) {
   if (check_topk(a) != TKA_OK) return 0;
-  return select_workspace_bytes(a->num_segments, a->seg_len, a->k);
+  return select_workspace_bytes(a->num_segments, a->seg_len);
 }
 
 int tka_topk_f32(const tka_topk_args* a) {
@@ -329,7 +341,7 @@ int tka_topk_f32(const tka_topk_args* a) {
   hipStream_t stream = (hipStream_t)a->stream;
   SelectParams sp;
   memset(&sp, 0, sizeof sp);
-  select_carve(a->workspace, a->num_segments, a->seg_len, a->k, &sp);
+  const size_t zero_words = select_carve(a->workspace, a->num_segments, a->seg_len, &sp);
   select_plan(a->seg_len, a->num_segments, &sp);
   sp.scores = a->scores;
   sp.seg_len = a->seg_len;
@@ -340,7 +352,6 @@ int tka_topk_f32(const tka_topk_args* a) {
   sp.num_segments = a->num_segments;
   sp.k = a->k;
   sp.segs_per_row = 1;
-  const size_t zero_words = ((unsigned char*)sp.sure - (unsigned char*)sp.hist) / sizeof(uint32_t);
   rc = launch_zero_u32(sp.hist, zero_words, stream);
   if (rc != TKA_OK) return rc;
   rc = launch_select_hist(sp, stream);
@@ -757,22 +768,13 @@ int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
   if (a->out_union_idx) uidx = a->out_union_idx;
   if (a->out_union_count) ucnt = a->out_union_count;
   const size_t gemv_ws = tka_gemv_topk_workspace_bytes(&g);
-  g.out_idx = tidx;
-  g.out_val = tval;
+  // rank-ordered top-k only if the caller asked for it; the attention needs the union list alone
+  g.out_idx = a->out_topk_idx ? tidx : nullptr;
+  g.out_val = a->out_topk_idx ? tval : nullptr;
   g.workspace = ws;
   g.workspace_bytes = gemv_ws;
-  rc = run_gemv_topk(&g, nullptr, 0);
-  if (rc != TKA_OK) return rc;
-  UnionParams up;
-  up.idx = tidx;
-  up.out_idx = uidx;
-  up.out_count = ucnt;
-  up.seq_len = a->seq_len;
-  up.num_segments = (int)segs;
-  up.k = a->k;
-  up.sink = a->sink;
-  up.local = a->local;
-  rc = launch_index_union(up, (hipStream_t)a->stream);
+  UnionOut uo = {uidx, ucnt, a->sink, a->local};
+  rc = run_gemv_topk(&g, nullptr, 0, nullptr, &uo);
   if (rc != TKA_OK) return rc;
   f.kv_idx = uidx;
   f.kv_count = ucnt;

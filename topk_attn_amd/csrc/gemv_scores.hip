@@ -5,7 +5,6 @@
 // four rows per wave; each lane keeps its 8 query dims in registers for the whole
 // kernel; the 16-lane reduce is four DPP row rotations (no LDS).  Eight loads are in flight per lane.
 // HBM-bound: 256 B read + 4 B written per row.
-#include <stdlib.h>
 #include "kernels.hpp"
 
 namespace tka {
@@ -110,15 +109,12 @@ int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
   return hip_status(hipGetLastError());
 }
 
-// Tokens per workgroup: enough workgroups to fill 256 CUs several times over, but long enough runs
-// that the per-workgroup histogram flush stays small.
+// Tokens per workgroup.  Short runs win: with 256 tokens (64 KB of keys) per workgroup the streaming rate
+// measured on MI355X is about 5% above that of 2048-token runs, and the histogram flush still costs
+// little.  Tiny problems take 128 so that every CU gets a workgroup.
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len) {
-  if (const char* e = getenv("TKA_TPW")) return atoi(e);  // TEMP sweep knob
-  int64_t t = total_rows / 4096;
-  int64_t tpw = 128;
-  while (tpw * 2 <= t && tpw < 2048) tpw *= 2;
-  while (tpw > 128 && tpw > chunk_len) tpw /= 2;
-  return (int)tpw;
+  (void)chunk_len;
+  return total_rows <= 65536 ? 128 : 256;
 }
 
 }  // namespace tka

@@ -26,24 +26,27 @@ struct SelectParams {
   int64_t seg_len;
   int64_t seg_stride;
   uint32_t* hist;         // [num_segments][kHistBins]
-  uint32_t* counters;     // [num_segments][4]: sure count, maybe count, parts done, unused; zero on entry
-  uint64_t* sure;         // [num_segments][k]       composites known to be selected
-  uint64_t* maybe;        // [num_segments][seg_len] composites of the threshold bin
-  int32_t* out_idx;       // [num_segments][out_stride]
+  uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)
+  uint64_t* list;         // [num_segments][list_stride] composites with bin >= threshold bin, slice p at p*part_len
+  int64_t list_stride;
+  int32_t* out_idx;       // [num_segments][out_stride] rank order, or nullptr (no sort)
   float* out_val;         // same shape or nullptr
   int32_t* out_expand;    // [num_segments][k*expand] or nullptr (centre-only expansion)
+  int32_t* union_idx;     // [num_segments][k+sink+local] ascending union with sink/local ranges, or nullptr
+  int32_t* union_count;   // [num_segments]
+  const int32_t* seg_base_ids;  // nullptr, or per segment a cluster id: index base = id * seg_len
   int64_t out_stride;
   int num_segments;
   int k;
-  int parts;              // workgroups per segment
-  int part_len;           // scores per workgroup (multiple of 1024)
-  const int32_t* seg_base_ids;  // nullptr, or per segment a cluster id: index base = id * seg_len
+  int parts;              // workgroups (slices) per segment
+  int part_len;           // scores per slice: 4096 or 16384
   int segs_per_row;       // chunks per (batch, head): index base = (s % segs_per_row) * seg_len
   int expand;             // cluster_len of the expansion, 0 = none
+  int sink, local;        // union mode
 };
-size_t select_workspace_bytes(int num_segments, int64_t seg_len, int k);
-// Carves the workspace: hist, counters, sure, maybe (in that order, 256-byte aligned).
-void select_carve(void* ws, int num_segments, int64_t seg_len, int k, SelectParams* p);
+size_t select_workspace_bytes(int num_segments, int64_t seg_len);
+// Carves the workspace; returns how many leading 32-bit words (the histograms) need clearing.
+size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p);
 void select_plan(int64_t seg_len, int num_segments, SelectParams* p);
 int launch_zero_u32(uint32_t* ptr, size_t count, hipStream_t stream);
 int launch_select_hist(const SelectParams& p, hipStream_t stream);

@@ -1,23 +1,28 @@
-// Stage 1, selection phase: exact top-k of fp32 scores per segment, ties to the lower index, output in
-// rank order.  Replaces the full cub::BlockRadixSort of the reference (gemv_topk.cu:353-378) with a
-// radix SELECT followed by a sort of the k survivors only.
+// Stage 1, selection phase: exact top-k of fp32 scores per segment, ties to the lower index.
+// Replaces the full cub::BlockRadixSort of the reference (gemv_topk.cu:353-378) with a radix SELECT;
+// only a caller that wants rank order pays for a sort, and then of the k survivors only.
 //
 // Every element is ranked by the 64-bit composite (score key << 32) | ~index, so all elements are
 // distinct and "top k" is unique: score descending, index ascending.
 //
 //   1. first-level histogram of the top 11 key bits (by the GEMV kernel, or select_hist_kernel);
-//   2. filter: each workgroup finds the threshold bin b1 from the histogram, keeps its slice of the
-//      scores in registers, and appends composites with bin > b1 to the "sure" list and bin == b1 to
-//      the "maybe" list (one global reservation per workgroup and list);
-//   3. finalize (next kernel, one workgroup per segment): refines the threshold inside the maybe
-//      list with further 11-bit radix passes (stops as soon as a bucket is taken whole), gathers
-//      the k survivors in LDS, sorts them with a bitonic network (registers, DPP / ds_swizzle across
-//      lanes, LDS across waves) and writes indices and values.
+//   2. filter (workgroups = slices x segments): find the threshold bin b1 from the histogram; every
+//      thread reads a contiguous run of its slice with 16-byte loads and the workgroup writes the
+//      composites with bin >= b1, in index order, to the slice's own list.  No atomics: the layout is
+//      deterministic and each list is ascending in token index;
+//   3. finalize (one workgroup per segment): turns the slice counts into offsets, refines the threshold
+//      inside bin b1 with further 11-bit radix passes over the listed entries (stops as soon as a
+//      bucket is taken whole), then walks the lists in order and
+//        - writes the ascending union with the sink / local-window ranges by ordered compaction
+//          (no sort), and / or
+//        - gathers the k survivors in LDS, sorts them with a bitonic network (registers, DPP /
+//          ds_swizzle across lanes, LDS across waves) and writes rank-ordered indices and values.
 //
-// No workgroup ever waits for another: the hand-off between 2 and 3 is the kernel boundary (a
-// device-scope fence per workgroup would write back the whole L2 of its XCD each time).
-// Traffic: 4 B read per score plus 8 B written and read per sure/maybe element; scores come from L2 /
-// Infinity Cache when the GEMV has just written them.
+// No workgroup waits for another: the hand-off between 2 and 3 is the kernel boundary (a device-scope
+// fence per workgroup would write back the whole L2 of its XCD each time).
+// Traffic: 4 B read per score, 8 B written and read per listed element (about k + one bin per segment).
+#include <stdlib.h>
+
 #include "kernels.hpp"
 
 namespace tka {
@@ -26,7 +31,6 @@ namespace {
 
 constexpr int kSelThreads = 1024;
 constexpr int kSelWaves = kSelThreads / kWave;
-constexpr int kSelMaxPerThread = 16;  // scores per thread held in registers by the filter
 
 // ---- block-wide helpers (1024 threads, 2048 bins) ---------------------------------------------
 
@@ -148,7 +152,57 @@ __global__ __launch_bounds__(256) void zero_u32_kernel(uint32_t* p, size_t n) {
   if (i < n) p[i] = 0u;
 }
 
+// Exclusive prefix of v over the 1024 threads of the block; *total = block sum.  Two barriers.
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* sh_wtot, uint32_t* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t inc = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    uint32_t t = __shfl_up(inc, d, 64);
+    if (lane >= d) inc += t;
+  }
+  __syncthreads();  // sh_wtot may still be read by the previous call
+  if (lane == 63) sh_wtot[wave] = inc;
+  __syncthreads();
+  uint32_t before = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < kSelWaves; ++w) {
+    const uint32_t t = sh_wtot[w];
+    before += w < wave ? t : 0u;
+    all += t;
+  }
+  *total = all;
+  return before + inc - v;
+}
+
+// Loads the `per_thread` (4 or 16) consecutive scores of this thread as keys; positions at or beyond
+// seg_len get key 0 and valid = false.
+template <int PT>
+__device__ __forceinline__ void load_keys(const float* sc, int64_t first, int64_t seg_len, bool vec_ok, uint32_t (&keys)[PT],
+                                          uint32_t* valid_mask) {
+  uint32_t vm = 0;
+#pragma unroll
+  for (int v = 0; v < PT / 4; ++v) {
+    const int64_t i = first + 4 * v;
+    if (vec_ok && i + 3 < seg_len) {
+      const f32x4 x = *(const f32x4*)(sc + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) keys[4 * v + e] = score_key(x[e]);
+      vm |= 0xfu << (4 * v);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool ok = i + e < seg_len;
+        keys[4 * v + e] = ok ? score_key(sc[ok ? i + e : 0]) : 0u;
+        vm |= (ok ? 1u : 0u) << (4 * v + e);
+      }
+    }
+  }
+  *valid_mask = vm;
+}
+
 // First-level histogram when the scores do not come from the GEMV kernel.
+template <int PT>
 __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(SelectParams p) {
   __shared__ uint32_t sh_hist[kHistBins];
   const int tid = threadIdx.x;
@@ -156,10 +210,12 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(SelectParams p
   for (int i = tid; i < kHistBins; i += kSelThreads) sh_hist[i] = 0;
   __syncthreads();
   const float* sc = p.scores + (int64_t)seg * p.seg_stride;
-  const int64_t begin = (int64_t)blockIdx.x * p.part_len;
-  int64_t end = begin + p.part_len;
-  if (end > p.seg_len) end = p.seg_len;
-  for (int64_t i = begin + tid; i < end; i += kSelThreads) atomicAdd(&sh_hist[score_key(sc[i]) >> (32 - kHistBits)], 1u);
+  const bool vec_ok = (((uintptr_t)sc) & 15u) == 0;
+  uint32_t keys[PT], vm;
+  load_keys<PT>(sc, (int64_t)blockIdx.x * p.part_len + (int64_t)tid * PT, p.seg_len, vec_ok, keys, &vm);
+#pragma unroll
+  for (int e = 0; e < PT; ++e)
+    if (vm >> e & 1u) atomicAdd(&sh_hist[keys[e] >> (32 - kHistBits)], 1u);
   __syncthreads();
   uint32_t* gh = p.hist + (int64_t)seg * kHistBins;
   for (int i = tid; i < kHistBins; i += kSelThreads) {
@@ -168,110 +224,56 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(SelectParams p
   }
 }
 
+template <int PT>
 __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams p) {
   __shared__ uint32_t sh_hist[kHistBins];
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
-  __shared__ uint32_t sh_cnt[2];    // workgroup totals: sure, maybe
-  __shared__ uint32_t sh_base[2];   // global reservation bases
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63;
   const int seg = blockIdx.y;
-  const uint32_t k = (uint32_t)p.k;
+  const int part = blockIdx.x;
 
-  // ---- 1. threshold bin from the first-level histogram
+  // threshold bin from the first-level histogram
   const uint32_t* gh = p.hist + (int64_t)seg * kHistBins;
   sh_hist[2 * tid] = gh[2 * tid];
   sh_hist[2 * tid + 1] = gh[2 * tid + 1];
-  if (tid < 2) sh_cnt[tid] = 0;
   __syncthreads();
-  find_threshold_bin(sh_hist, k, sh_wtot, sh_res);
+  find_threshold_bin(sh_hist, (uint32_t)p.k, sh_wtot, sh_res);
   const uint32_t b1 = sh_res[0];
 
-  // ---- 2. filter this workgroup's slice (kept in registers between count and write)
   const float* sc = p.scores + (int64_t)seg * p.seg_stride;
-  const int64_t begin = (int64_t)blockIdx.x * p.part_len;
-  uint32_t keys[kSelMaxPerThread];
-  uint32_t my_sure = 0, my_maybe = 0;
-  const int iters = p.part_len / kSelThreads;
+  const bool vec_ok = (((uintptr_t)sc) & 15u) == 0;
+  const int64_t first = (int64_t)part * p.part_len + (int64_t)tid * PT;
+  uint32_t keys[PT], vm;
+  load_keys<PT>(sc, first, p.seg_len, vec_ok, keys, &vm);
+  uint32_t mine = 0;
 #pragma unroll
-  for (int it = 0; it < kSelMaxPerThread; ++it) {
-    keys[it] = 0;
-    if (it < iters) {
-      int64_t i = begin + (int64_t)it * kSelThreads + tid;
-      if (i < p.seg_len) {
-        uint32_t key = score_key(sc[i]);
-        uint32_t bin = key >> (32 - kHistBits);
-        keys[it] = key;
-        my_sure += bin > b1;
-        my_maybe += bin == b1;
-      } else {
-        keys[it] = 0;  // bin 0 <= b1; excluded below by the bounds test
-      }
-    }
-  }
-  // wave-level exclusive prefix of the per-thread counts, wave totals reserved in LDS
-  uint32_t ps = my_sure, pm = my_maybe;
+  for (int e = 0; e < PT; ++e) mine += ((vm >> e) & 1u) && (keys[e] >> (32 - kHistBits)) >= b1;
+  uint32_t total;
+  uint32_t slot = block_exclusive_scan(mine, sh_wtot, &total);
+  uint64_t* list = p.list + (int64_t)seg * p.list_stride + (int64_t)part * p.part_len;
 #pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    uint32_t ts = __shfl_up(ps, d, 64), tm = __shfl_up(pm, d, 64);
-    if (lane >= d) { ps += ts; pm += tm; }
-  }
-  uint32_t wbase_s = 0, wbase_m = 0;
-  if (lane == 63) {
-    wbase_s = atomicAdd(&sh_cnt[0], ps);
-    wbase_m = atomicAdd(&sh_cnt[1], pm);
-  }
-  wbase_s = __shfl(wbase_s, 63, 64);
-  wbase_m = __shfl(wbase_m, 63, 64);
-  __syncthreads();
-  uint32_t* ctr = p.counters + (int64_t)seg * 4;
-  if (tid == 0) {
-    sh_base[0] = sh_cnt[0] ? atomicAdd(&ctr[0], sh_cnt[0]) : 0u;
-    sh_base[1] = sh_cnt[1] ? atomicAdd(&ctr[1], sh_cnt[1]) : 0u;
-  }
-  __syncthreads();
-  {
-    uint64_t* sure = p.sure + (int64_t)seg * p.k;
-    uint64_t* maybe = p.maybe + (int64_t)seg * p.seg_len;
-    uint32_t slot_s = sh_base[0] + wbase_s + (ps - my_sure);
-    uint32_t slot_m = sh_base[1] + wbase_m + (pm - my_maybe);
-#pragma unroll
-    for (int it = 0; it < kSelMaxPerThread; ++it) {
-      if (it < iters) {
-        int64_t i = begin + (int64_t)it * kSelThreads + tid;
-        if (i < p.seg_len) {
-          uint32_t bin = keys[it] >> (32 - kHistBits);
-          uint64_t c = composite(keys[it], (uint32_t)i);
-          if (bin > b1) sure[slot_s++] = c;
-          else if (bin == b1) maybe[slot_m++] = c;
-        }
-      }
-    }
-  }
-
+  for (int e = 0; e < PT; ++e)
+    if (((vm >> e) & 1u) && (keys[e] >> (32 - kHistBits)) >= b1) list[slot++] = composite(keys[e], (uint32_t)(first + e));
+  if (tid == 0) p.list_cnt[(int64_t)seg * p.parts + part] = total;
 }
 
-// Dynamic LDS layout of select_finalize_kernel: [0, 8 KB) histogram; then kpad composites (sort
-// buffer); then kpad composites (cross-wave exchange buffer).
+// Dynamic LDS of select_finalize_kernel (rank mode only): kpad composites (sort buffer), then kpad
+// composites (cross-wave exchange buffer).
 __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectParams p, int kpad) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint32_t* sh_hist = (uint32_t*)smem;
-  uint64_t* sh_sort = (uint64_t*)(smem + kHistBins * sizeof(uint32_t));
+  uint64_t* sh_sort = (uint64_t*)smem;
   uint64_t* sh_xchg = sh_sort + kpad;
+  __shared__ uint32_t sh_hist[kHistBins];
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
-  __shared__ uint32_t sh_cnt[2];
 
   const int tid = threadIdx.x;
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
-  const uint32_t* ctr = p.counters + (int64_t)seg * 4;
-  const uint32_t n_sure = ctr[0];
-  const uint32_t n_maybe = ctr[1];
 
-  // threshold bin again (cheap) — the maybe list holds exactly the elements of bin b1
+  // threshold bin, count above it, count inside it
   {
     const uint32_t* gh = p.hist + (int64_t)seg * kHistBins;
     sh_hist[2 * tid] = gh[2 * tid];
@@ -279,16 +281,41 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
     __syncthreads();
     find_threshold_bin(sh_hist, k, sh_wtot, sh_res);
   }
-  const uint32_t b1 = sh_res[0];
-  const uint64_t* sure = p.sure + (int64_t)seg * p.k;
-  const uint64_t* maybe = p.maybe + (int64_t)seg * p.seg_len;
+  const uint32_t b1 = sh_res[0], n_above = sh_res[1], n_bin = sh_res[2];
 
-  // Refine: composites of the maybe list share their top 11 bits (= b1).  Take `need` of them.
-  uint32_t need = k - n_sure;           // >= 1 by construction of b1
+  // slice counts -> inclusive offsets, in place (entries of the segment get one running index)
+  uint32_t* ends = p.list_cnt + (int64_t)seg * p.parts;
+  {
+    uint32_t running = 0;
+    for (int base = 0; base < p.parts; base += kSelThreads) {
+      const int i = base + tid;
+      const uint32_t c = i < p.parts ? ends[i] : 0u;
+      uint32_t total;
+      const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
+      if (i < p.parts) ends[i] = running + ex + c;
+      running += total;
+    }
+    __syncthreads();
+  }
+  const uint32_t n_entries = n_above + n_bin;  // == ends[parts-1]
+  const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
+  // entry v of the segment: slice s with ends[s-1] <= v < ends[s], position v - ends[s-1] in that slice
+  auto entry = [&](uint32_t v) -> uint64_t {
+    int lo = 0, hi = p.parts - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (ends[mid] > v) hi = mid; else lo = mid + 1;
+    }
+    const uint32_t start = lo ? ends[lo - 1] : 0u;
+    return lists[(int64_t)lo * p.part_len + (v - start)];
+  };
+
+  // Refine inside bin b1: the listed entries of that bin share their top 11 bits.  Take `need` of them.
+  uint32_t need = k - n_above;          // >= 1 by construction of b1
   uint64_t prefix = b1;                 // value of the bits fixed so far
   int fixed = kHistBits;                // number of top bits fixed
-  uint64_t threshold = 0;               // selected maybe elements: composite >= threshold
-  bool done = (need == n_maybe);        // whole bin taken
+  uint64_t threshold = 0;               // selected: composite >= threshold
+  bool done = (need == n_bin);          // whole bin taken
   if (done) threshold = (uint64_t)b1 << (64 - kHistBits);
   while (!done) {
     const int bits = (64 - fixed) >= kHistBits ? kHistBits : (64 - fixed);
@@ -297,8 +324,8 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
     sh_hist[2 * tid] = 0;
     sh_hist[2 * tid + 1] = 0;
     __syncthreads();
-    for (uint32_t i = tid; i < n_maybe; i += kSelThreads) {
-      uint64_t c = maybe[i];
+    for (uint32_t v = tid; v < n_entries; v += kSelThreads) {
+      const uint64_t c = entry(v);
       if ((c >> (64 - fixed)) == prefix) atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
     }
     __syncthreads();
@@ -313,19 +340,47 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
     }
   }
 
-  // Gather the k survivors (order irrelevant), pad with 0 (below every real composite).
-  __syncthreads();
-  for (int i = tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;
-  if (tid < 2) sh_cnt[tid] = 0;
-  __syncthreads();
-  for (uint32_t i = tid; i < n_sure; i += kSelThreads) sh_sort[i] = sure[i];
-  for (uint32_t i = tid; i < n_maybe; i += kSelThreads) {
-    uint64_t c = maybe[i];
-    if (c >= threshold) {
-      uint32_t slot = atomicAdd(&sh_cnt[0], 1u);
-      if (n_sure + slot < k) sh_sort[n_sure + slot] = c;
+  // Walk the entries in index order.  Union mode: ordered compaction of the selected ids that lie
+  // between the sink range and the local window.  Rank mode: selected composites into the sort buffer.
+  const bool want_rank = p.out_idx != nullptr;
+  const bool want_union = p.union_idx != nullptr;
+  const int64_t n = p.seg_len;
+  const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
+  const uint32_t hi = (uint32_t)(n - p.local > lo ? n - p.local : lo);
+  int32_t* uo = want_union ? p.union_idx + (int64_t)seg * (p.k + p.sink + p.local) : nullptr;
+  if (want_rank) {
+    __syncthreads();
+    for (int i = tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite
+  }
+  uint32_t run_sel = 0, run_mid = 0;
+  for (uint32_t base = 0; base < n_entries; base += kSelThreads) {
+    const uint32_t v = base + tid;
+    const uint64_t c = v < n_entries ? entry(v) : 0ull;
+    const bool sel = v < n_entries && c >= threshold;
+    const uint32_t idx = ~(uint32_t)c;
+    uint32_t total;
+    if (want_rank) {
+      const uint32_t ex = block_exclusive_scan(sel ? 1u : 0u, sh_wtot, &total);
+      if (sel && run_sel + ex < k) sh_sort[run_sel + ex] = c;
+      run_sel += total;
+    }
+    if (want_union) {
+      const bool mid = sel && idx >= lo && idx < hi;
+      const uint32_t ex = block_exclusive_scan(mid ? 1u : 0u, sh_wtot, &total);
+      if (mid) uo[lo + run_mid + ex] = (int32_t)idx;
+      run_mid += total;
     }
   }
+  if (want_union) {
+    const int cap = p.k + p.sink + p.local;
+    for (uint32_t t = tid; t < lo; t += kSelThreads) uo[t] = (int32_t)t;
+    const uint32_t mid_end = lo + run_mid;
+    for (int64_t t = (int64_t)hi + tid; t < n; t += kSelThreads) uo[mid_end + (t - hi)] = (int32_t)t;
+    const uint32_t count = mid_end + (uint32_t)(n - hi);
+    for (int i = (int)count + tid; i < cap; i += kSelThreads) uo[i] = -1;
+    if (tid == 0) p.union_count[seg] = (int32_t)count;
+  }
+  if (!want_rank) return;
   __syncthreads();
 
   switch (kpad / kSelThreads) {
@@ -430,36 +485,46 @@ int kpad_for(int k) {
 
 }  // namespace
 
-size_t select_workspace_bytes(int num_segments, int64_t seg_len, int k) {
-  size_t b = 0;
-  b += align_up((size_t)num_segments * kHistBins * sizeof(uint32_t), 256);
-  b += align_up((size_t)num_segments * 4 * sizeof(uint32_t), 256);
-  b += align_up((size_t)num_segments * (size_t)k * sizeof(uint64_t), 256);
-  b += align_up((size_t)num_segments * (size_t)seg_len * sizeof(uint64_t), 256);
-  return b;
+// Workspace layout (each part 256-byte aligned):
+//   hist [S][2048] u32 (cleared per call) | list_cnt [S][parts] u32 | list [S][parts*part_len] u64
+namespace {
+struct SelectLayout {
+  size_t hist, list_cnt, list, total;
+  int64_t list_stride;
+};
+SelectLayout select_layout(int num_segments, int64_t seg_len) {
+  SelectLayout l;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t at = off; off += align_up(bytes, 256); return at; };
+  const int64_t min_part = 4 * kSelThreads;
+  const int64_t max_parts = (seg_len + min_part - 1) / min_part;
+  l.list_stride = (seg_len + 16 * kSelThreads - 1) / (16 * kSelThreads) * (16 * kSelThreads);  // whole slices
+  l.hist = take((size_t)num_segments * kHistBins * sizeof(uint32_t));
+  l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
+  l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
+  l.total = off;
+  return l;
 }
+}  // namespace
 
-void select_carve(void* ws, int num_segments, int64_t seg_len, int k, SelectParams* p) {
+size_t select_workspace_bytes(int num_segments, int64_t seg_len) { return select_layout(num_segments, seg_len).total; }
+
+// Carves the workspace; returns how many leading 32-bit words (the histograms) need clearing.
+size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p) {
+  const SelectLayout l = select_layout(num_segments, seg_len);
   unsigned char* c = (unsigned char*)ws;
-  p->hist = (uint32_t*)c;
-  c += align_up((size_t)num_segments * kHistBins * sizeof(uint32_t), 256);
-  p->counters = (uint32_t*)c;
-  c += align_up((size_t)num_segments * 4 * sizeof(uint32_t), 256);
-  p->sure = (uint64_t*)c;
-  c += align_up((size_t)num_segments * (size_t)k * sizeof(uint64_t), 256);
-  p->maybe = (uint64_t*)c;
+  p->hist = (uint32_t*)(c + l.hist);
+  p->list_cnt = (uint32_t*)(c + l.list_cnt);
+  p->list = (uint64_t*)(c + l.list);
+  p->list_stride = l.list_stride;
+  return (size_t)num_segments * kHistBins;
 }
 
-// Slice size per workgroup: a multiple of 1024 up to 16384, small enough that a segment is spread
-// over several CUs when there are few segments.
+// Slice per workgroup: 16384 scores (16 per thread) when that still gives every CU work, else 4096.
 void select_plan(int64_t seg_len, int num_segments, SelectParams* p) {
-  int per_thread = kSelMaxPerThread;
-  while (per_thread > 1) {
-    int64_t parts = (seg_len + (int64_t)per_thread * kSelThreads - 1) / ((int64_t)per_thread * kSelThreads);
-    if (parts * num_segments >= 256) break;
-    per_thread >>= 1;
-  }
-  p->part_len = per_thread * kSelThreads;
+  const int64_t big = 16 * kSelThreads;
+  const int64_t parts_big = (seg_len + big - 1) / big;
+  p->part_len = parts_big * num_segments >= 256 ? (int)big : 4 * kSelThreads;
   p->parts = (int)((seg_len + p->part_len - 1) / p->part_len);
 }
 
@@ -472,22 +537,31 @@ int launch_zero_u32(uint32_t* ptr, size_t count, hipStream_t stream) {
 
 int launch_select_hist(const SelectParams& p, hipStream_t stream) {
   LaunchTimer timer("select_hist", stream);
-  select_hist_kernel<<<dim3((unsigned)p.parts, (unsigned)p.num_segments), kSelThreads, 0, stream>>>(p);
+  const dim3 grid((unsigned)p.parts, (unsigned)p.num_segments);
+  if (p.part_len == 16 * kSelThreads)
+    select_hist_kernel<16><<<grid, kSelThreads, 0, stream>>>(p);
+  else
+    select_hist_kernel<4><<<grid, kSelThreads, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 
 int launch_select(const SelectParams& p, hipStream_t stream) {
+  const bool want_rank = p.out_idx != nullptr;
   const int kpad = kpad_for(p.k);
-  const size_t lds = kHistBins * sizeof(uint32_t) + 2 * (size_t)kpad * sizeof(uint64_t);
+  const size_t lds = want_rank ? 2 * (size_t)kpad * sizeof(uint64_t) : 0;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);
+    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
     if (e != hipSuccess) return TKA_EHIP;
     attr_set = true;
   }
   {
     LaunchTimer timer("select_filter", stream);
-    select_filter_kernel<<<dim3((unsigned)p.parts, (unsigned)p.num_segments), kSelThreads, 0, stream>>>(p);
+    const dim3 grid((unsigned)p.parts, (unsigned)p.num_segments);
+    if (p.part_len == 16 * kSelThreads)
+      select_filter_kernel<16><<<grid, kSelThreads, 0, stream>>>(p);
+    else
+      select_filter_kernel<4><<<grid, kSelThreads, 0, stream>>>(p);
     if (hipGetLastError() != hipSuccess) return TKA_EHIP;
   }
   LaunchTimer timer("select_finalize", stream);
@@ -500,7 +574,7 @@ int launch_index_union(const UnionParams& p, hipStream_t stream) {
   const size_t lds = 2 * (size_t)kpad * sizeof(uint64_t);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)index_union_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);
+    hipError_t e = hipFuncSetAttribute((const void*)index_union_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
     if (e != hipSuccess) return TKA_EHIP;
     attr_set = true;
   }

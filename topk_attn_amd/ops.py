@@ -261,7 +261,7 @@ class SparseDecodePlan:
     a step is a single C call (used by the benchmark and by callers that decode repeatedly)."""
 
     def __init__(self, q, keys, values, k, sink, local, scale, group, out_dtype=None, num_splits=0,
-                 keep_selection=True):
+                 want_topk=True, want_union=True):
         _need_cuda(q, keys, values)
         q = _q3(q)
         B = q.shape[0]
@@ -279,12 +279,14 @@ class SparseDecodePlan:
         a.seq_len, a.q_stride_b, a.out_stride_b = N, q.stride(0), self.out.stride(0)
         a.kv_stride_b, a.kv_stride_n, a.kv_stride_h = sb, sn, sh
         a.scale = scale
-        if keep_selection:
+        self.topk_idx = self.topk_val = self.union_idx = self.union_count = None
+        if want_topk:  # rank-ordered selection: costs a sort per KV head, not needed by the attention
             self.topk_idx = torch.empty((B, H, k), dtype=torch.int32, device=q.device)
             self.topk_val = torch.empty((B, H, k), dtype=torch.float32, device=q.device)
+            a.out_topk_idx, a.out_topk_val = self.topk_idx.data_ptr(), self.topk_val.data_ptr()
+        if want_union:
             self.union_idx = torch.empty((B, H, k + sink + local), dtype=torch.int32, device=q.device)
             self.union_count = torch.empty((B, H), dtype=torch.int32, device=q.device)
-            a.out_topk_idx, a.out_topk_val = self.topk_idx.data_ptr(), self.topk_val.data_ptr()
             a.out_union_idx, a.out_union_count = self.union_idx.data_ptr(), self.union_count.data_ptr()
         need = L.lib().tka_sparse_decode_workspace_bytes(C.byref(a))
         if need == 0:
