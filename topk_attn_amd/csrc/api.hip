@@ -202,7 +202,7 @@ int check_flash(const tka_flash_decode_args* a) {
   return TKA_OK;
 }
 
-// Positions per workgroup (multiple of 64) and the split count that follows from it.
+// Positions per workgroup (multiple of 128, one or more kernel steps) and the split count that follows.
 void flash_plan(const tka_flash_decode_args* a, int* splits, int* tokens_per_split) {
   const int64_t len = a->kv_idx ? a->idx_len : a->seq_len;
   int64_t want = a->num_splits;
@@ -211,12 +211,12 @@ void flash_plan(const tka_flash_decode_args* a, int* splits, int* tokens_per_spl
     if (want < 1) want = 1;
   }
   int64_t tps = (len + want - 1) / want;
-  tps = (tps + 63) / 64 * 64;
-  if (tps < 64) tps = 64;
+  tps = (tps + 127) / 128 * 128;
+  if (tps < 128) tps = 128;
   int64_t s = (len + tps - 1) / tps;
   if (s > TKA_MAX_SPLITS) {
     s = TKA_MAX_SPLITS;
-    tps = ((len + s - 1) / s + 63) / 64 * 64;
+    tps = ((len + s - 1) / s + 127) / 128 * 128;
     s = (len + tps - 1) / tps;
   }
   *splits = (int)s;

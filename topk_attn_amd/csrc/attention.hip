@@ -2,7 +2,7 @@
 // index list with caller-supplied logits) and the log-sum-exp combine.
 //
 // attn_partial_kernel — one workgroup per (split, KV head, batch entry), 4 waves.  A 16-lane row group
-// owns one token at a time: 16 B of the K row and 16 B of the V row per lane, scores for the G query
+// owns one token at a time (4 or 8 tokens in flight): 16 B of the K row and 16 B of the V row per lane, scores for the G query
 // heads of the group by fma chain + DPP row reduce, online softmax in the exp2 domain
 // (baseline_1.cu:406-468 of the reference), fp32 accumulators of 8 output dims per lane and head.
 // The 16 row-group states of the workgroup are merged through LDS and written as one fp32
@@ -17,14 +17,21 @@ namespace tka {
 namespace {
 
 constexpr int kAttnThreads = 256;
-constexpr int kAttnRowGroups = kAttnThreads / 16;  // 16 tokens in flight per step and load slot
-constexpr int kAttnUnroll = 4;                     // tokens per row group per step
-constexpr int kAttnStep = kAttnRowGroups * kAttnUnroll;  // 64 positions per workgroup step
+constexpr int kAttnRowGroups = kAttnThreads / 16;  // 16 tokens per load slot of the workgroup
 
 enum { MODE_DENSE = 0, MODE_INDEXED = 1, MODE_LOGIT = 2 };
 
+// Tokens per row group per step: K and V rows of U tokens are in flight together (2*U 16-byte loads per
+// lane).  Large groups keep fewer in flight to stay inside the register file.
+template <int G>
+struct AttnUnroll {
+  static constexpr int value = G <= 4 ? 8 : 4;
+};
+
 template <int DT, int G, int MODE>
 __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p) {
+  constexpr int U = AttnUnroll<G>::value;
+  constexpr int kStep = kAttnRowGroups * U;  // positions per workgroup step
   __shared__ float sh_acc[kAttnRowGroups][kHeadDim];
   __shared__ float sh_m[kAttnRowGroups];
   __shared__ float sh_l[kAttnRowGroups];
@@ -74,31 +81,46 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
     for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
   }
 
-  for (int64_t base = begin; base < end; base += kAttnStep) {
-    int64_t tok[kAttnUnroll];
-    bool valid[kAttnUnroll];
-    float lg[kAttnUnroll];
+  // token ids (and supplied logits) of one step; fetched one step ahead so that the row loads of a step
+  // do not wait for an index load
+  int32_t nid[U];
+  float nlg[U];
+  auto fetch_ids = [&](int64_t base) {
 #pragma unroll
-    for (int u = 0; u < kAttnUnroll; ++u) {
-      int64_t pos = base + rg * kAttnUnroll + u;
+    for (int u = 0; u < U; ++u) {
+      const int64_t pos = base + rg * U + u;
+      const int64_t pc = pos < end ? pos : (end > 0 ? end - 1 : 0);
+      nid[u] = MODE == MODE_DENSE ? 0 : (base < end ? idx[pc] : 0);
+      nlg[u] = MODE == MODE_LOGIT ? (base < end ? logit[pc] : 0.0f) : 0.0f;
+    }
+  };
+  fetch_ids(begin);
+
+  for (int64_t base = begin; base < end; base += kStep) {
+    int64_t tok[U];
+    bool valid[U];
+    float lg[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t pos = base + rg * U + u;
       valid[u] = pos < end;
-      int64_t pc = valid[u] ? pos : end - 1;
-      tok[u] = MODE == MODE_DENSE ? pc : (int64_t)idx[pc];
-      lg[u] = MODE == MODE_LOGIT ? logit[pc] : 0.0f;
+      tok[u] = MODE == MODE_DENSE ? (valid[u] ? pos : end - 1) : (int64_t)nid[u];
+      lg[u] = nlg[u];
       if (MODE != MODE_DENSE && (tok[u] < 0 || tok[u] >= p.seq_len)) {  // skip ids outside the cache
         valid[u] = false;                                                // (retrieval_attention.cu:1325)
         tok[u] = 0;
       }
     }
-    u32x4 kv[kAttnUnroll], vv[kAttnUnroll];
+    u32x4 kv[U], vv[U];
 #pragma unroll
-    for (int u = 0; u < kAttnUnroll; ++u) {
+    for (int u = 0; u < U; ++u) {
       if (MODE != MODE_LOGIT) kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + tok[u] * p.kv_stride_n));
       vv[u] = __builtin_nontemporal_load((const u32x4*)(vbase + tok[u] * p.kv_stride_n));
     }
-    float x[G][kAttnUnroll];
+    if (MODE != MODE_DENSE) fetch_ids(base + kStep);
+    float x[G][U];
 #pragma unroll
-    for (int u = 0; u < kAttnUnroll; ++u) {
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         float s;
@@ -117,7 +139,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
     for (int g = 0; g < G; ++g) {
       float mx = m[g];
 #pragma unroll
-      for (int u = 0; u < kAttnUnroll; ++u) mx = fmaxf(mx, x[g][u]);
+      for (int u = 0; u < U; ++u) mx = fmaxf(mx, x[g][u]);
       if (mx == -INFINITY) continue;  // nothing valid so far
       const float alpha = __builtin_amdgcn_exp2f(m[g] - mx);  // m = -inf -> 0
       m[g] = mx;
@@ -125,7 +147,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
 #pragma unroll
-      for (int u = 0; u < kAttnUnroll; ++u) {
+      for (int u = 0; u < U; ++u) {
         const float pu = __builtin_amdgcn_exp2f(x[g][u] - mx);  // invalid -> 0
         l[g] += pu;
 #pragma unroll

@@ -31,6 +31,8 @@ namespace {
 
 constexpr int kSelThreads = 1024;
 constexpr int kSelWaves = kSelThreads / kWave;
+constexpr int kEndsInLds = 1024;   // slice offsets of one segment kept in LDS by the finalize kernel
+constexpr int kEntryCache = 8;     // listed entries per thread kept in registers by the finalize kernel
 
 // ---- block-wide helpers (1024 threads, 2048 bins) ---------------------------------------------
 
@@ -234,6 +236,13 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams
   const int seg = blockIdx.y;
   const int part = blockIdx.x;
 
+  // this thread's run of scores first: the loads do not depend on the threshold
+  const float* sc = p.scores + (int64_t)seg * p.seg_stride;
+  const bool vec_ok = (((uintptr_t)sc) & 15u) == 0;
+  const int64_t first = (int64_t)part * p.part_len + (int64_t)tid * PT;
+  uint32_t keys[PT], vm;
+  load_keys<PT>(sc, first, p.seg_len, vec_ok, keys, &vm);
+
   // threshold bin from the first-level histogram
   const uint32_t* gh = p.hist + (int64_t)seg * kHistBins;
   sh_hist[2 * tid] = gh[2 * tid];
@@ -242,11 +251,6 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams
   find_threshold_bin(sh_hist, (uint32_t)p.k, sh_wtot, sh_res);
   const uint32_t b1 = sh_res[0];
 
-  const float* sc = p.scores + (int64_t)seg * p.seg_stride;
-  const bool vec_ok = (((uintptr_t)sc) & 15u) == 0;
-  const int64_t first = (int64_t)part * p.part_len + (int64_t)tid * PT;
-  uint32_t keys[PT], vm;
-  load_keys<PT>(sc, first, p.seg_len, vec_ok, keys, &vm);
   uint32_t mine = 0;
 #pragma unroll
   for (int e = 0; e < PT; ++e) mine += ((vm >> e) & 1u) && (keys[e] >> (32 - kHistBits)) >= b1;
@@ -283,24 +287,30 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   }
   const uint32_t b1 = sh_res[0], n_above = sh_res[1], n_bin = sh_res[2];
 
-  // slice counts -> inclusive offsets, in place (entries of the segment get one running index)
-  uint32_t* ends = p.list_cnt + (int64_t)seg * p.parts;
+  // slice counts -> inclusive offsets (entries of the segment get one running index); kept in LDS when
+  // they fit, in place in global memory otherwise
+  __shared__ uint32_t sh_ends[kEndsInLds];
+  uint32_t* g_ends = p.list_cnt + (int64_t)seg * p.parts;
+  const bool ends_in_lds = p.parts <= kEndsInLds;
   {
     uint32_t running = 0;
     for (int base = 0; base < p.parts; base += kSelThreads) {
       const int i = base + tid;
-      const uint32_t c = i < p.parts ? ends[i] : 0u;
+      const uint32_t c = i < p.parts ? g_ends[i] : 0u;
       uint32_t total;
       const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
-      if (i < p.parts) ends[i] = running + ex + c;
+      if (i < p.parts) {
+        if (ends_in_lds) sh_ends[i] = running + ex + c; else g_ends[i] = running + ex + c;
+      }
       running += total;
     }
     __syncthreads();
   }
+  const uint32_t* ends = ends_in_lds ? sh_ends : g_ends;
   const uint32_t n_entries = n_above + n_bin;  // == ends[parts-1]
   const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
   // entry v of the segment: slice s with ends[s-1] <= v < ends[s], position v - ends[s-1] in that slice
-  auto entry = [&](uint32_t v) -> uint64_t {
+  auto fetch = [&](uint32_t v) -> uint64_t {
     int lo = 0, hi = p.parts - 1;
     while (lo < hi) {
       const int mid = (lo + hi) >> 1;
@@ -309,6 +319,14 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
     const uint32_t start = lo ? ends[lo - 1] : 0u;
     return lists[(int64_t)lo * p.part_len + (v - start)];
   };
+  // the first kEntryCache*1024 entries live in registers (typical segments fit entirely)
+  uint64_t cache[kEntryCache];
+#pragma unroll
+  for (int i = 0; i < kEntryCache; ++i) {
+    const uint32_t v = (uint32_t)i * kSelThreads + tid;
+    cache[i] = v < n_entries ? fetch(v) : 0ull;
+  }
+  auto entry = [&](uint32_t v) -> uint64_t { return fetch(v); };
 
   // Refine inside bin b1: the listed entries of that bin share their top 11 bits.  Take `need` of them.
   uint32_t need = k - n_above;          // >= 1 by construction of b1
@@ -324,7 +342,13 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
     sh_hist[2 * tid] = 0;
     sh_hist[2 * tid + 1] = 0;
     __syncthreads();
-    for (uint32_t v = tid; v < n_entries; v += kSelThreads) {
+#pragma unroll
+    for (int i = 0; i < kEntryCache; ++i) {
+      const uint64_t c = cache[i];
+      if ((uint32_t)i * kSelThreads + tid < n_entries && (c >> (64 - fixed)) == prefix)
+        atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
+    }
+    for (uint32_t v = kEntryCache * kSelThreads + tid; v < n_entries; v += kSelThreads) {
       const uint64_t c = entry(v);
       if ((c >> (64 - fixed)) == prefix) atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
     }
@@ -353,9 +377,16 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
     for (int i = tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite
   }
   uint32_t run_sel = 0, run_mid = 0;
-  for (uint32_t base = 0; base < n_entries; base += kSelThreads) {
+  for (uint32_t base = 0, step = 0; base < n_entries; base += kSelThreads, ++step) {
     const uint32_t v = base + tid;
-    const uint64_t c = v < n_entries ? entry(v) : 0ull;
+    uint64_t c = 0;
+    if (step < kEntryCache) {
+#pragma unroll
+      for (int i = 0; i < kEntryCache; ++i)
+        if ((uint32_t)i == step) c = cache[i];
+    } else if (v < n_entries) {
+      c = entry(v);
+    }
     const bool sel = v < n_entries && c >= threshold;
     const uint32_t idx = ~(uint32_t)c;
     uint32_t total;
