@@ -261,7 +261,9 @@ int run_flash(const tka_flash_decode_args* a, void* workspace) {
   ap.idx_len = a->idx_len;
   ap.tokens_per_split = tps;
   ap.scale_log2e = a->scale * 1.44269504088896340736f;
-  int rc = launch_attn_partial(ap, a->dtype, stream);
+  // grouped queries go to the matrix cores; one query head per KV head (and supplied logits) stay on VALU
+  int rc = (a->group >= 2 && !a->kv_logit) ? launch_attn_partial_mfma(ap, a->dtype, stream)
+                                           : launch_attn_partial(ap, a->dtype, stream);
   if (rc != TKA_OK) return rc;
   CombineParams cp;
   memset(&cp, 0, sizeof cp);

@@ -79,7 +79,8 @@ struct AttnParams {
   int tokens_per_split;     // positions per workgroup
   float scale_log2e;        // scale * log2(e)
 };
-int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream);
+int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream);       // VALU path (any group, logits)
+int launch_attn_partial_mfma(const AttnParams& p, int dtype, hipStream_t stream);  // matrix-core path, group >= 2
 
 struct CombineParams {
   const float* part_m;
