@@ -1,14 +1,19 @@
 #!/usr/bin/env python3
-"""Benchmark of the sparse-decode step on one MI355X.
+"""Benchmark of the sparse-decode path on one MI355X.
 
-A step = one pass of the hot path over one batch of seeded synthetic input, inputs resident in HBM:
-fused GEMV + top-k per KV head -> union with sink/local -> gathered attention -> LSE combine.
-Workload "c4": batch 8, 32 query / 8 KV heads, head_dim 128, KV length 131072 fp16 N(0,1) with 1% of the keys
-per head scaled x4, k=2048, 64 sink + 512 local tokens, bf16 output.
+A step = one pass of the hot path over one batch of seeded synthetic input, inputs resident in HBM.
+The default workload is the one the headline metric is quoted on:
+
+  c4  end-to-end decode at 128k: batch 8, 32 query / 8 KV heads, head_dim 128, KV length 131072 fp16 N(0,1)
+      with 1% of the keys per head scaled x4; fused GEMV + top-2048 per KV head -> union with 64 sink + 512
+      local tokens -> gathered attention -> LSE combine; bf16 output.
+
+The other workloads time one stage each at the sizes of the remaining configurations (c1 single-head
+GEMV + top-k, c2 centre-only top-k, c3 dense flash-decoding, c5 one-million-token tie stress).
 
 Prints ONE JSON line.  `value` is algorithmic bytes per step / step time (GB/s); `roofline` is the dominant
-kernel (gemv_scores) timed with HIP events on its launch stream; `cpu_baseline` is the torch-CPU restatement
-of the same step timed on this machine's host cores on a bounded sample.
+kernel timed with HIP events on its launch stream; `cpu_baseline` is the torch-CPU restatement of the same
+step timed on this machine's host cores on a bounded sample (c4 only).
 """
 import argparse
 import json
@@ -21,32 +26,181 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-
-WORKLOADS = {
-    # name: batch, kv heads, group, seq_len, k, sink, local, in dtype, out dtype, heavy-hitter fraction, seed
-    "c4": dict(batch=8, hkv=8, group=4, seq_len=131072, k=2048, sink=64, local=512, dtype="float16",
-               out_dtype="bfloat16", heavy=0.01, seed=4),
-    "c4-small": dict(batch=2, hkv=8, group=4, seq_len=16384, k=2048, sink=64, local=512, dtype="float16",
-                     out_dtype="bfloat16", heavy=0.01, seed=4),
-}
+SCALE = 0.08838834764831845  # fl32(1/sqrt(128)) as Python float
 
 
-def make_inputs(torch, w, device):
-    g = torch.Generator(device=device)
-    g.manual_seed(w["seed"])
-    dt = getattr(torch, w["dtype"])
-    B, H, G, N = w["batch"], w["hkv"], w["group"], w["seq_len"]
-    q = torch.randn((B, H * G, 128), generator=g, device=device, dtype=torch.float32).to(dt)
-    K = torch.empty((B, N, H, 128), device=device, dtype=dt)
-    V = torch.empty((B, N, H, 128), device=device, dtype=dt)
-    for b in range(B):  # per batch entry to bound the fp32 temporaries
-        K[b] = torch.randn((N, H, 128), generator=g, device=device, dtype=torch.float32).to(dt)
-        V[b] = torch.randn((N, H, 128), generator=g, device=device, dtype=torch.float32).to(dt)
-        n_heavy = int(N * w["heavy"])
+def randn16(torch, shape, dt, g, dev, chunk_dim0=True):
+    """N(0,1) tensor of a 16-bit type, generated slice by slice to bound the fp32 temporaries."""
+    out = torch.empty(shape, device=dev, dtype=dt)
+    if len(shape) >= 3 and shape[0] > 1 and chunk_dim0:
+        for i in range(shape[0]):
+            out[i] = torch.randn(shape[1:], generator=g, device=dev, dtype=torch.float32).to(dt)
+    else:
+        step = max(1, (1 << 26) // max(1, int(out[0].numel()))) if out.dim() > 1 else out.numel()
+        if out.dim() == 1:
+            out.copy_(torch.randn(shape, generator=g, device=dev, dtype=torch.float32).to(dt))
+        else:
+            for i in range(0, shape[0], step):
+                j = min(shape[0], i + step)
+                out[i:j] = torch.randn((j - i,) + tuple(shape[1:]), generator=g, device=dev, dtype=torch.float32).to(dt)
+    return out
+
+
+class SparseDecode:
+    """c4 (and a small variant): the end-to-end step."""
+
+    def __init__(self, torch, ops, dev, batch=8, hkv=8, group=4, seq_len=131072, k=2048, sink=64, local=512,
+                 dtype="float16", out_dtype="bfloat16", heavy=0.01, seed=4, name="c4"):
+        self.torch, self.name = torch, name
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        dt = getattr(torch, dtype)
+        B, H, G, N = batch, hkv, group, seq_len
+        self.B, self.H, self.G, self.N, self.k, self.sink, self.local = B, H, G, N, k, sink, local
+        self.q = randn16(torch, (B, H * G, 128), dt, g, dev, chunk_dim0=False)
+        self.K = randn16(torch, (B, N, H, 128), dt, g, dev)
+        self.V = randn16(torch, (B, N, H, 128), dt, g, dev)
+        n_heavy = int(N * heavy)
+        for b in range(B):
+            for h in range(H):
+                hh = torch.randperm(N, generator=g, device=dev)[:n_heavy]
+                self.K[b, hh, h] = (self.K[b, hh, h].float() * 4.0).to(dt)
+        # production configuration: the attention consumes the union list; the optional rank-ordered top-k
+        # output (a sort per KV head) is not requested
+        self.plan = ops.SparseDecodePlan(self.q, self.K, self.V, k, sink, local, SCALE, G,
+                                         out_dtype=getattr(torch, out_dtype), want_topk=False)
+        self.desc = "%s: B=%d Hq=%d Hkv=%d D=128 N=%d %s k=%d sink=%d local=%d out=%s" % (
+            name, B, H * G, H, N, dtype, k, sink, local, out_dtype)
+        self.dominant = "gemv_scores"
+
+    def step(self):
+        self.plan.step()
+
+    def bytes(self):
+        sel = int(self.plan.union_count.sum().item())
+        gemv = self.B * self.N * self.H * 128 * 2
+        sparse = sel * 128 * 2 * 2 + sel * 4 * 2          # gathered K and V rows, index lists written + read
+        qo = self.B * self.H * self.G * 128 * 4           # q read, out written (2 bytes each)
+        return gemv + sparse + qo, gemv, {"selected_tokens": sel}
+
+    def cpu_baseline(self, runs):
+        torch = self.torch
+        from oracle.cpu_baseline import sparse_decode_cpu
+        # bounded sample: batch entry 0 (1/B of the step); the step is B independent copies of it
+        qc, Kc, Vc = self.q[0].cpu(), self.K[0].cpu(), self.V[0].cpu()
+        times = []
+        for r in range(runs + 1):
+            c0 = time.perf_counter()
+            ref_out, ref_top = sparse_decode_cpu(qc, Kc, Vc, self.k, self.sink, self.local, SCALE, self.G)
+            c1 = time.perf_counter()
+            if r > 0:
+                times.append(c1 - c0)
+        times.sort()
+        cpu_s = times[len(times) // 2] * self.B
+        # sanity (not the parity oracle): same selected sets, outputs close
+        N, H = self.N, self.H
+        lo, hi = min(self.sink, N), max(N - self.local, min(self.sink, N))
+        same_sets = True
         for h in range(H):
-            hh = torch.randperm(N, generator=g, device=device)[:n_heavy]
-            K[b, hh, h] = (K[b, hh, h].float() * 4.0).to(dt)
-    return q, K, V
+            want = set(range(lo)) | set(range(hi, N)) | set(ref_top[h].tolist())
+            got = self.plan.union_idx[0, h, :int(self.plan.union_count[0, h])].tolist()
+            same_sets = same_sets and got == sorted(want)
+        max_err = (self.plan.out[0].float().cpu() - ref_out).abs().max().item()
+        return cpu_s, {"cores": torch.get_num_threads(), "host_cpus": os.cpu_count(), "kind": "port",
+                       "sample": "batch entry 0 of %d (all %d KV heads, full N=%d), median of %d runs, scaled x%d" % (
+                           self.B, H, N, runs, self.B),
+                       "union_sets_equal_gpu": bool(same_sets), "out_max_abs_diff_vs_gpu": round(max_err, 5)}
+
+
+class GemvTopk:
+    """c1 / c5: fused GEMV + top-k alone."""
+
+    def __init__(self, torch, ops, dev, batch, hkv, group, seq_len, k, dtype, seed, name, levels=False):
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        dt = getattr(torch, dtype)
+        self.B, self.H, self.G, self.N, self.k = batch, hkv, group, seq_len, k
+        self.q = randn16(torch, (batch, hkv * group, 128), dt, g, dev, chunk_dim0=False)
+        if levels:  # 16 uniform levels in [-2, 2]: many exact score ties
+            self.K = torch.empty((batch, seq_len, hkv, 128), device=dev, dtype=dt)
+            lv = torch.linspace(-2.0, 2.0, 16, device=dev)
+            for b in range(batch):
+                for t0 in range(0, seq_len, 131072):
+                    t1 = min(seq_len, t0 + 131072)
+                    ids = torch.randint(0, 16, (t1 - t0, hkv, 128), generator=g, device=dev)
+                    self.K[b, t0:t1] = lv[ids].to(dt)
+        else:
+            self.K = randn16(torch, (batch, seq_len, hkv, 128), dt, g, dev)
+        self.plan = ops.GemvTopkPlan(self.q, self.K, k, group=group, scale=SCALE)
+        self.desc = "%s: B=%d Hkv=%d G=%d D=128 N=%d %s k=%d (GEMV + top-k only)" % (name, batch, hkv, group, seq_len, dtype, k)
+        self.dominant = "gemv_scores"
+
+    def step(self):
+        self.plan.run()
+
+    def bytes(self):
+        gemv = self.B * self.N * self.H * 128 * 2
+        return gemv + self.B * self.H * self.G * 128 * 2 + self.B * self.H * self.k * 8, gemv, {}
+
+
+class CenterTopk:
+    """c2: centre-only top-k with expansion."""
+
+    def __init__(self, torch, ops, dev):
+        g = torch.Generator(device=dev)
+        g.manual_seed(2)
+        H, Cn = 32, 4096
+        self.ops, self.H, self.Cn, self.top_c, self.clen = ops, H, Cn, 64, 64
+        cen = torch.randn((H, Cn, 128), generator=g, device=dev) + 0.5 * torch.randn((H, 1, 128), generator=g, device=dev)
+        self.cen = cen.half()
+        self.q = torch.randn((H, 128), generator=g, device=dev).half()
+        self.desc = "c2: 32 heads x 4096 centroids fp16, top-64, expand x64"
+        self.dominant = "gemv_scores"
+
+    def step(self):
+        self.out = self.ops.center_topk_expand(self.q, self.cen, self.top_c, self.clen, SCALE)
+
+    def bytes(self):
+        gemv = self.H * self.Cn * 128 * 2
+        return gemv + self.H * 128 * 2 + self.H * self.top_c * self.clen * 4, gemv, {}
+
+
+class FlashDecode:
+    """c3: dense split-K flash-decoding."""
+
+    def __init__(self, torch, ops, dev, num_splits=0):
+        g = torch.Generator(device=dev)
+        g.manual_seed(3)
+        self.H, self.G, self.N = 8, 4, 131072
+        self.q = randn16(torch, (1, 32, 128), torch.float16, g, dev, chunk_dim0=False)
+        self.K = randn16(torch, (self.N, 8, 128), torch.float16, g, dev, chunk_dim0=False)
+        self.V = randn16(torch, (self.N, 8, 128), torch.float16, g, dev, chunk_dim0=False)
+        self.plan = ops.FlashDecodePlan(self.q, self.K, self.V, SCALE, group=4, num_splits=num_splits)
+        self.desc = "c3: dense flash-decoding B=1 Hq=32 Hkv=8 D=128 N=131072 fp16, splits=%s" % (num_splits or "auto")
+        self.dominant = "attn_mfma_dense"
+
+    def step(self):
+        self.plan.run()
+
+    def bytes(self):
+        kv = 2 * self.N * self.H * 128 * 2
+        return kv + 2 * 32 * 128 * 2, kv, {}
+
+
+def build_workload(name, torch, ops, dev, args):
+    if name == "c4":
+        return SparseDecode(torch, ops, dev)
+    if name == "c4-small":
+        return SparseDecode(torch, ops, dev, batch=2, seq_len=16384, name="c4-small")
+    if name == "c1":
+        return GemvTopk(torch, ops, dev, 1, 1, 1, 32768, 2048, "float16", 1, "c1")
+    if name == "c2":
+        return CenterTopk(torch, ops, dev)
+    if name == "c3":
+        return FlashDecode(torch, ops, dev, args.splits)
+    if name == "c5":
+        return GemvTopk(torch, ops, dev, 1, 8, 8, 1048576, 4096, "bfloat16", 5, "c5", levels=True)
+    raise ValueError(name)
 
 
 def main():
@@ -54,7 +208,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c4-small", "c5"])
+    ap.add_argument("--splits", type=int, default=0, help="c3: split count (0 = library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-runs", type=int, default=3)
     args = ap.parse_args()
@@ -71,45 +226,33 @@ def main():
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = WORKLOADS[args.workload]
-    scale = float(torch.tensor(1.0 / 128.0 ** 0.5, dtype=torch.float32).item())
-    q, K, V = make_inputs(torch, w, dev)
-    # production configuration: the attention consumes the union list; the optional rank-ordered top-k
-    # output (a sort per KV head) is not requested
-    plan = ops.SparseDecodePlan(q, K, V, w["k"], w["sink"], w["local"], scale, w["group"],
-                                out_dtype=getattr(torch, w["out_dtype"]), want_topk=False)
+    w = build_workload(args.workload, torch, ops, dev, args)
 
     for _ in range(args.warmup):
-        plan.step()
+        w.step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        plan.step()
+        w.step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
 
-    # algorithmic bytes of one step: every key row once, the selected K and V rows once, q/out, index lists
-    B, H, G, N = w["batch"], w["hkv"], w["group"], w["seq_len"]
-    esz = 2
-    sel = int(plan.union_count.sum().item())
-    gemv_bytes = B * N * H * 128 * esz
-    sparse_bytes = sel * 128 * esz * 2 + sel * 4 * 2
-    qo_bytes = B * H * G * 128 * (esz + 2)
-    step_bytes = gemv_bytes + sparse_bytes + qo_bytes
+    step_bytes, dom_bytes, extra = w.bytes()
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # dominant kernel, timed with HIP events recorded by the library on the launch stream
+    # per-kernel times from HIP events recorded by the library on the launch stream (second timed loop: the
+    # event pairs add a few microseconds per kernel, so they stay out of the loop that `value` comes from)
     ops.profile_reset()
     ops.profile_enable(True)
     for _ in range(args.steps):
-        plan.step()
+        w.step()
     torch.cuda.synchronize()
     prof = ops.profile_read()
     ops.profile_enable(False)
     kern = {name: ms / max(n, 1) * 1e3 for name, (ms, n) in prof.items()}  # us per launch
-    gemv_us = kern.get("gemv_scores", float("nan"))
-    achieved = gemv_bytes / (gemv_us * 1e-6) / 1e9
+    dom_us = kern.get(w.dominant, float("nan"))
+    achieved = dom_bytes / (dom_us * 1e-6) / 1e9
 
     out = {
         "metric": "us/decode-step + achieved HBM GB/s (% of peak), GEMV+top-k+sparse attn @128k",
@@ -117,43 +260,17 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "us_per_step": round(ms_per_step * 1e3, 2),
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic (seeded torch.randn on the GPU; 1% heavy-hitter keys x4)",
-        "config": {"workload": "%s: B=%d Hq=%d Hkv=%d D=128 N=%d %s k=%d sink=%d local=%d out=%s" % (
-            args.workload, B, H * G, H, N, w["dtype"], w["k"], w["sink"], w["local"], w["out_dtype"]),
-            "algorithmic_bytes_per_step": step_bytes, "selected_tokens": sel},
-        "roofline": {"bound": "hbm", "kernel": "gemv_scores", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "data": "synthetic (seeded torch generator on the GPU)",
+        "config": dict({"workload": w.desc, "algorithmic_bytes_per_step": step_bytes}, **extra),
+        "roofline": {"bound": "hbm", "kernel": w.dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "algorithmic_bytes_per_launch": gemv_bytes, "avg_launch_us": round(gemv_us, 2)},
+                     "algorithmic_bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 2)},
         "kernels_us": {k_: round(v, 2) for k_, v in sorted(kern.items())},
     }
-
-    if not args.no_cpu:
-        from oracle.cpu_baseline import sparse_decode_cpu
-        # bounded sample: batch entry 0 (1/B of the step); the step is B independent copies of it
-        qc, Kc, Vc = q[0].cpu(), K[0].cpu(), V[0].cpu()
-        times = []
-        for r in range(args.cpu_runs + 1):
-            c0 = time.perf_counter()
-            ref_out, ref_top = sparse_decode_cpu(qc, Kc, Vc, w["k"], w["sink"], w["local"], scale, G)
-            c1 = time.perf_counter()
-            if r > 0:
-                times.append(c1 - c0)
-        times.sort()
-        cpu_s = times[len(times) // 2] * B
-        # sanity (not the parity oracle): same selected sets, outputs close
-        lo, hi = min(w["sink"], N), max(N - w["local"], min(w["sink"], N))
-        same_sets = True
-        for h in range(H):
-            want = set(range(lo)) | set(range(hi, N)) | set(ref_top[h].tolist())
-            got = plan.union_idx[0, h, :int(plan.union_count[0, h])].tolist()
-            same_sets = same_sets and got == sorted(want)
-        max_err = (plan.out[0].float().cpu() - ref_out).abs().max().item()
-        out["cpu_baseline"] = {
-            "value": round(step_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "us_per_step": round(cpu_s * 1e6, 1),
-            "cores": torch.get_num_threads(), "host_cpus": os.cpu_count(), "kind": "port",
-            "sample": "batch entry 0 of %d (all %d KV heads, full N=%d), median of %d runs, scaled x%d" % (
-                B, H, N, args.cpu_runs, B),
-            "union_sets_equal_gpu": bool(same_sets), "out_max_abs_diff_vs_gpu": round(max_err, 5)}
+    if not args.no_cpu and hasattr(w, "cpu_baseline"):
+        cpu_s, info = w.cpu_baseline(args.cpu_runs)
+        out["cpu_baseline"] = dict({"value": round(step_bytes / cpu_s / 1e9, 3), "unit": "GB/s",
+                                    "us_per_step": round(cpu_s * 1e6, 1)}, **info)
     print(json.dumps(out))
     return 0
 

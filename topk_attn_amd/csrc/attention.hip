@@ -185,56 +185,79 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
   }
 }
 
-constexpr int kCombineGroups = 8;  // split subsets reduced in parallel, then merged through LDS
+// lse_combine_kernel: one workgroup per output row.  The split maxima and sums go to LDS first (one
+// coalesced read), the weights 2^(m_s-M) are computed once, then 32 groups of 32 lanes (4 dims per lane,
+// 16-byte loads) add up the accumulators of every 32nd split and a last pass folds the 32 groups.
+constexpr int kCombineThreads = 1024;
+constexpr int kCombineLanes = kHeadDim / 4;                      // 32 lanes cover one accumulator row
+constexpr int kCombineGroups = kCombineThreads / kCombineLanes;  // 32 splits in flight
 
 template <int ODT>
-__global__ __launch_bounds__(kHeadDim * kCombineGroups) void lse_combine_kernel(CombineParams p) {
-  __shared__ float sh_m[kCombineGroups], sh_l[kCombineGroups][kHeadDim], sh_o[kCombineGroups][kHeadDim];
+__global__ __launch_bounds__(kCombineThreads) void lse_combine_kernel(CombineParams p) {
+  __shared__ float sh_w[TKA_MAX_SPLITS];                    // m_s, then the weight of split s
+  __shared__ float sh_red[kCombineThreads / kWave];
+  __shared__ f32x4 sh_o[kCombineGroups][kCombineLanes];
+  __shared__ float sh_stat[2];                              // M, L
   const int row = blockIdx.x;
-  const int d = threadIdx.x & (kHeadDim - 1);
-  const int g = threadIdx.x / kHeadDim;
-  const float* pm = p.part_m + (int64_t)row * p.num_splits;
-  const float* pl = p.part_l + (int64_t)row * p.num_splits;
-  const float* pa = p.part_acc + (int64_t)row * p.num_splits * kHeadDim;
-  float M = -INFINITY;
-  for (int s = g; s < p.num_splits; s += kCombineGroups) {
-    const float ls = pl[s], ms = pm[s];
-    if (ls > 0.0f) M = fmaxf(M, ms);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int S = p.num_splits;
+  const float* pm = p.part_m + (int64_t)row * S;
+  const float* pl = p.part_l + (int64_t)row * S;
+  const f32x4* pa = (const f32x4*)(p.part_acc + (int64_t)row * S * kHeadDim);
+
+  // M = max over non-empty splits
+  float ms = -INFINITY, ls = 0.0f;
+  if (tid < S) {
+    ls = pl[tid];
+    ms = ls > 0.0f ? pm[tid] : -INFINITY;
   }
-  float L = 0.0f, o = 0.0f;
-  for (int s = g; s < p.num_splits; s += kCombineGroups) {
-    const float ls = pl[s], ms = pm[s], as = pa[(int64_t)s * kHeadDim + d];
-    if (ls > 0.0f) {
-      const float w = __builtin_amdgcn_exp2f(ms - M);
-      L += ls * w;
-      o += as * w;
-    }
-  }
-  if (d == 0) sh_m[g] = M;
-  sh_l[g][d] = L;
-  sh_o[g][d] = o;
+  float mx = ms;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+  if (lane == 0) sh_red[wave] = mx;
   __syncthreads();
-  if (g != 0) return;
-  float Mt = -INFINITY;
+  float M = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < kCombineGroups; ++i) Mt = fmaxf(Mt, sh_m[i]);
-  float Lt = 0.0f, ot = 0.0f;
-  if (Mt != -INFINITY) {
+  for (int w = 0; w < kCombineThreads / kWave; ++w) M = fmaxf(M, sh_red[w]);
+  // weights and L
+  const float wgt = (ms != -INFINITY) ? __builtin_amdgcn_exp2f(ms - M) : 0.0f;
+  if (tid < S) sh_w[tid] = wgt;
+  float lsum = ls * wgt;
 #pragma unroll
-    for (int i = 0; i < kCombineGroups; ++i) {
-      const float mi = sh_m[i];
-      if (mi != -INFINITY) {
-        const float w = __builtin_amdgcn_exp2f(mi - Mt);
-        Lt += sh_l[i][d] * w;
-        ot += sh_o[i][d] * w;
-      }
+  for (int d = 32; d >= 1; d >>= 1) lsum += __shfl_xor(lsum, d, 64);
+  __syncthreads();  // sh_red read by everyone, sh_w written
+  if (lane == 0) sh_red[wave] = lsum;
+  __syncthreads();
+  if (tid == 0) {
+    float L = 0.0f;
+    for (int w = 0; w < kCombineThreads / kWave; ++w) L += sh_red[w];
+    sh_stat[0] = M;
+    sh_stat[1] = L;
+  }
+  // accumulators: group g takes splits g, g+32, ...
+  const int g = tid / kCombineLanes, dl = tid % kCombineLanes;
+  f32x4 o = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int s = g; s < S; s += kCombineGroups) {
+    const float w = sh_w[s];
+    if (w != 0.0f) {
+      const f32x4 a = pa[(int64_t)s * kCombineLanes + dl];
+      o += a * w;
     }
   }
-  const float r = Lt > 0.0f ? ot / Lt : 0.0f;
+  sh_o[g][dl] = o;
+  __syncthreads();
+  if (tid >= kHeadDim) return;
+  const float L = sh_stat[1];
+  float acc = 0.0f;
+  const float* so = (const float*)sh_o;
+#pragma unroll 8
+  for (int gg = 0; gg < kCombineGroups; ++gg) acc += so[gg * kHeadDim + tid];
+  const float r = L > 0.0f ? acc / L : 0.0f;
   const int bb = row / p.rows_per_batch, hh = row % p.rows_per_batch;
   uint16_t* out = (uint16_t*)p.out + (int64_t)bb * p.out_stride_b + (int64_t)hh * kHeadDim;
-  out[d] = Elem<ODT>::narrow(r);
-  if (p.out_lse && d == 0) p.out_lse[row] = Lt > 0.0f ? (Mt + __builtin_log2f(Lt)) * 0.69314718055994531f : -INFINITY;
+  out[tid] = Elem<ODT>::narrow(r);
+  if (p.out_lse && tid == 0) p.out_lse[row] = L > 0.0f ? (sh_stat[0] + __builtin_log2f(L)) * 0.69314718055994531f : -INFINITY;
 }
 
 template <int DT, int MODE>
@@ -271,9 +294,9 @@ int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream) {
 int launch_lse_combine(const CombineParams& p, hipStream_t stream) {
   LaunchTimer timer("lse_combine", stream);
   if (p.out_dtype == TKA_F16)
-    lse_combine_kernel<TKA_F16><<<(unsigned)p.rows, kHeadDim * kCombineGroups, 0, stream>>>(p);
+    lse_combine_kernel<TKA_F16><<<(unsigned)p.rows, kCombineThreads, 0, stream>>>(p);
   else
-    lse_combine_kernel<TKA_BF16><<<(unsigned)p.rows, kHeadDim * kCombineGroups, 0, stream>>>(p);
+    lse_combine_kernel<TKA_BF16><<<(unsigned)p.rows, kCombineThreads, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 

@@ -62,23 +62,29 @@ __device__ void find_threshold_bin(const uint32_t* sh_hist, uint32_t need, uint3
 
 // ---- bitonic sort of 1024*E composites, descending --------------------------------------------
 
-template <int M>
-__device__ __forceinline__ void cx_lane(uint64_t& v, bool keep_max) {
-  uint64_t o = lane_xor64<M>(v);
-  bool take = keep_max ? (o > v) : (o < v);
-  v = take ? o : v;
+// One compare-exchange stage whose partner sits M lanes away.  keep_max is the same for every element of
+// the thread (the stride and the merge size are multiples of E).  Composites are distinct (equal only
+// among the zero padding), so "partner greater" decides both directions with one 64-bit compare.
+template <int M, int E>
+__device__ __forceinline__ void stage_lanes(uint64_t (&v)[E], bool keep_max) {
+#pragma unroll
+  for (int s = 0; s < E; ++s) {
+    const uint64_t o = lane_xor64<M>(v[s]);
+    const bool take = (o > v[s]) == keep_max;
+    v[s] = take ? o : v[s];
+  }
 }
 
+// One compare-exchange stage inside the thread (STRIDE < E).
 template <int STRIDE, int E>
-__device__ __forceinline__ void cx_regs(uint64_t (&v)[E], int size) {
+__device__ __forceinline__ void stage_regs(uint64_t (&v)[E], int first, int size) {
   if constexpr (STRIDE < E) {
 #pragma unroll
     for (int s = 0; s < E; ++s) {
       if ((s & STRIDE) == 0) {
-        int e = threadIdx.x * E + s;
-        bool desc = (e & size) == 0;
-        uint64_t a = v[s], b = v[s ^ STRIDE];
-        bool sw = desc ? (b > a) : (b < a);
+        const bool desc = ((first + s) & size) == 0;
+        const uint64_t a = v[s], b = v[s ^ STRIDE];
+        const bool sw = (b > a) == desc;
         v[s] = sw ? b : a;
         v[s ^ STRIDE] = sw ? a : b;
       }
@@ -86,65 +92,78 @@ __device__ __forceinline__ void cx_regs(uint64_t (&v)[E], int size) {
   }
 }
 
-// Thread t holds elements t*E .. t*E+E-1.  sh is scratch for the cross-wave strides (1024*E entries).
-template <int E>
-__device__ void bitonic_sort_desc(uint64_t (&v)[E], uint64_t* sh) {
-  const int tid = threadIdx.x;
-  constexpr int N = kSelThreads * E;
-  for (int size = 2; size <= N; size <<= 1) {
-    for (int stride = size >> 1; stride >= 1; stride >>= 1) {
-      if (stride >= 64 * E) {
-        // partner in another wave: exchange through LDS
-        __syncthreads();
+// Bitonic sort, descending, of N composites held by the first N/E threads of the block (thread t holds
+// elements t*E .. t*E+E-1).  The network is unrolled at compile time: strides inside a thread are
+// register compare-exchanges, strides inside a wave use DPP / ds_swizzle / ds_bpermute, and only strides
+// of 64*E and more go through LDS (`sh`, N entries) with block barriers, which every thread must reach.
+template <int N, int E, int SIZE, int STRIDE>
+__device__ __forceinline__ void bitonic_net(uint64_t (&v)[E], uint64_t* sh, int tid, bool active) {
+  if constexpr (SIZE <= N) {
+    const int e0 = tid * E;
+    if constexpr (STRIDE >= 64 * E) {
+      __syncthreads();
+      if (active) {
 #pragma unroll
-        for (int s = 0; s < E; ++s) sh[tid * E + s] = v[s];
-        __syncthreads();
+        for (int s = 0; s < E; ++s) sh[e0 + s] = v[s];
+      }
+      __syncthreads();
+      if (active) {
+        const bool keep_max = ((e0 & STRIDE) == 0) == ((e0 & SIZE) == 0);
 #pragma unroll
         for (int s = 0; s < E; ++s) {
-          int e = tid * E + s;
-          uint64_t o = sh[e ^ stride];
-          bool keep_max = ((e & stride) == 0) == ((e & size) == 0);
-          bool take = keep_max ? (o > v[s]) : (o < v[s]);
+          const uint64_t o = sh[(e0 + s) ^ STRIDE];
+          const bool take = (o > v[s]) == keep_max;
           v[s] = take ? o : v[s];
         }
-      } else if (stride >= E) {
-        const int m = stride / E;  // lane distance
-#pragma unroll
-        for (int s = 0; s < E; ++s) {
-          int e = tid * E + s;
-          bool keep_max = ((e & stride) == 0) == ((e & size) == 0);
-          switch (m) {
-            case 1: cx_lane<1>(v[s], keep_max); break;
-            case 2: cx_lane<2>(v[s], keep_max); break;
-            case 4: cx_lane<4>(v[s], keep_max); break;
-            case 8: cx_lane<8>(v[s], keep_max); break;
-            case 16: cx_lane<16>(v[s], keep_max); break;
-            default: cx_lane<32>(v[s], keep_max); break;
-          }
-        }
-      } else {
-        // both elements in this thread (stride is 1, 2 or 4; compile-time register indices)
-        switch (stride) {
-          case 1: cx_regs<1, E>(v, size); break;
-          case 2: cx_regs<2, E>(v, size); break;
-          default: cx_regs<4, E>(v, size); break;
-        }
       }
+    } else if constexpr (STRIDE >= E) {
+      if (active) {
+        const bool keep_max = ((e0 & STRIDE) == 0) == ((e0 & SIZE) == 0);
+        stage_lanes<STRIDE / E, E>(v, keep_max);
+      }
+    } else {
+      if (active) stage_regs<STRIDE, E>(v, e0, SIZE);
     }
+    if constexpr (STRIDE > 1)
+      bitonic_net<N, E, SIZE, STRIDE / 2>(v, sh, tid, active);
+    else
+      bitonic_net<N, E, SIZE * 2, SIZE>(v, sh, tid, active);
   }
 }
 
-template <int E>
-__device__ void sort_lds_desc(uint64_t* sh_sort, uint64_t* sh_xchg) {
+// One element per thread up to 1024 (many waves hide the cross-lane latency), then 2, 4, 8 per thread.
+template <int N>
+__device__ __noinline__ void sort_lds_desc_n(uint64_t* sh_sort, uint64_t* sh_xchg) {
+  constexpr int E = N > kSelThreads ? N / kSelThreads : 1;
+  constexpr int NT = N / E;
   uint64_t v[E];
   const int tid = threadIdx.x;
+  const bool active = tid < NT;
+  if (active) {
 #pragma unroll
-  for (int s = 0; s < E; ++s) v[s] = sh_sort[tid * E + s];
-  bitonic_sort_desc<E>(v, sh_xchg);
+    for (int s = 0; s < E; ++s) v[s] = sh_sort[tid * E + s];
+  }
+  bitonic_net<N, E, 2, 1>(v, sh_xchg, tid, active);
   __syncthreads();
+  if (active) {
 #pragma unroll
-  for (int s = 0; s < E; ++s) sh_sort[tid * E + s] = v[s];
+    for (int s = 0; s < E; ++s) sh_sort[tid * E + s] = v[s];
+  }
   __syncthreads();
+}
+
+// Sorts sh_sort[0 .. kpad) descending; kpad is a power of two between 64 and 8192.
+__device__ void sort_lds_desc(uint64_t* sh_sort, uint64_t* sh_xchg, int kpad) {
+  switch (kpad) {
+    case 64: sort_lds_desc_n<64>(sh_sort, sh_xchg); break;
+    case 128: sort_lds_desc_n<128>(sh_sort, sh_xchg); break;
+    case 256: sort_lds_desc_n<256>(sh_sort, sh_xchg); break;
+    case 512: sort_lds_desc_n<512>(sh_sort, sh_xchg); break;
+    case 1024: sort_lds_desc_n<1024>(sh_sort, sh_xchg); break;
+    case 2048: sort_lds_desc_n<2048>(sh_sort, sh_xchg); break;
+    case 4096: sort_lds_desc_n<4096>(sh_sort, sh_xchg); break;
+    default: sort_lds_desc_n<8192>(sh_sort, sh_xchg); break;
+  }
 }
 
 // ---- kernels ----------------------------------------------------------------------------------
@@ -414,12 +433,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   if (!want_rank) return;
   __syncthreads();
 
-  switch (kpad / kSelThreads) {
-    case 1: sort_lds_desc<1>(sh_sort, sh_xchg); break;
-    case 2: sort_lds_desc<2>(sh_sort, sh_xchg); break;
-    case 4: sort_lds_desc<4>(sh_sort, sh_xchg); break;
-    default: sort_lds_desc<8>(sh_sort, sh_xchg); break;
-  }
+  sort_lds_desc(sh_sort, sh_xchg, kpad);
 
   const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
                                            : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
@@ -462,20 +476,16 @@ __global__ __launch_bounds__(kSelThreads) void index_union_kernel(UnionParams p,
     sh_sort[i] = c;
   }
   __syncthreads();
-  switch (kpad / kSelThreads) {
-    case 1: sort_lds_desc<1>(sh_sort, sh_xchg); break;
-    case 2: sort_lds_desc<2>(sh_sort, sh_xchg); break;
-    case 4: sort_lds_desc<4>(sh_sort, sh_xchg); break;
-    default: sort_lds_desc<8>(sh_sort, sh_xchg); break;
-  }
+  sort_lds_desc(sh_sort, sh_xchg, kpad);
   // count distinct non-zero entries; entry i is kept when it differs from entry i-1
   int32_t* out = p.out_idx + (int64_t)seg * (p.k + p.sink + p.local);
   const int cap = p.k + p.sink + p.local;
   // positions: a prefix count of "kept" flags.  kpad <= 8192: each thread scans its contiguous run.
-  const int per = kpad / kSelThreads;
+  const int per = kpad >= kSelThreads ? kpad / kSelThreads : 1;
   uint32_t mine = 0;
   for (int s = 0; s < per; ++s) {
     int i = tid * per + s;
+    if (i >= kpad) break;
     uint64_t c = sh_sort[i];
     if (c != 0 && (i == 0 || sh_sort[i - 1] != c)) ++mine;
   }
@@ -497,6 +507,7 @@ __global__ __launch_bounds__(kSelThreads) void index_union_kernel(UnionParams p,
   uint32_t pos = (uint32_t)lo + wbase + (pre - mine);
   for (int s = 0; s < per; ++s) {
     int i = tid * per + s;
+    if (i >= kpad) break;
     uint64_t c = sh_sort[i];
     if (c != 0 && (i == 0 || sh_sort[i - 1] != c)) out[pos++] = (int32_t)~(uint32_t)(c - 1u);
   }
@@ -509,7 +520,7 @@ __global__ __launch_bounds__(kSelThreads) void index_union_kernel(UnionParams p,
 }
 
 int kpad_for(int k) {
-  int kpad = kSelThreads;
+  int kpad = 64;
   while (kpad < k) kpad <<= 1;
   return kpad;
 }

@@ -60,30 +60,44 @@ def _q3(q):
     return q
 
 
+class GemvTopkPlan:
+    """Argument block, outputs and workspace of one fused GEMV + top-k configuration; run() is one C call."""
+
+    def __init__(self, q, keys, k, group=1, scale=1.0, num_chunks=1, return_scores=False):
+        _need_cuda(q, keys)
+        q = _q3(q)
+        B = q.shape[0]
+        sb, sn, sh, N, H = _kv_strides(keys, B)
+        if q.shape[1] != H * group:
+            raise ValueError("q heads != kv heads * group")
+        self.q, self.keys = q, keys
+        self.idx = torch.empty((B, H, num_chunks * k), dtype=torch.int32, device=q.device)
+        self.val = torch.empty((B, H, num_chunks * k), dtype=torch.float32, device=q.device)
+        self.scores = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if return_scores else None
+        a = L.GemvTopkArgs()
+        a.q, a.keys = q.data_ptr(), keys.data_ptr()
+        a.dtype, a.batch, a.num_kv_heads, a.group, a.head_dim = _dtype_code(keys), B, H, group, 128
+        a.k, a.num_chunks, a.seq_len = k, num_chunks, N
+        a.q_stride_b, a.key_stride_b, a.key_stride_n, a.key_stride_h = q.stride(0), sb, sn, sh
+        a.scale = scale
+        a.out_idx, a.out_val = self.idx.data_ptr(), self.val.data_ptr()
+        a.out_scores = self.scores.data_ptr() if self.scores is not None else None
+        need = L.lib().tka_gemv_topk_workspace_bytes(C.byref(a))
+        self.ws = _workspace(need, q.device)
+        a.workspace, a.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
+        self.args = a
+        self._fn = L.lib().tka_gemv_topk
+
+    def run(self):
+        self.args.stream = torch.cuda.current_stream().cuda_stream
+        L.check(self._fn(C.byref(self.args)), "tka_gemv_topk")
+        return self
+
+
 def gemv_topk(q, keys, k, group=1, scale=1.0, num_chunks=1, return_scores=False):
     """Fused GEMV + top-k.  Returns (idx int32 [B,Hkv,num_chunks*k], val fp32 same shape[, scores fp32 [B,Hkv,N]])."""
-    _need_cuda(q, keys)
-    q = _q3(q)
-    B = q.shape[0]
-    sb, sn, sh, N, H = _kv_strides(keys, B)
-    if q.shape[1] != H * group:
-        raise ValueError("q heads != kv heads * group")
-    idx = torch.empty((B, H, num_chunks * k), dtype=torch.int32, device=q.device)
-    val = torch.empty((B, H, num_chunks * k), dtype=torch.float32, device=q.device)
-    scores = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if return_scores else None
-    a = L.GemvTopkArgs()
-    a.q, a.keys = q.data_ptr(), keys.data_ptr()
-    a.dtype, a.batch, a.num_kv_heads, a.group, a.head_dim = _dtype_code(keys), B, H, group, 128
-    a.k, a.num_chunks, a.seq_len = k, num_chunks, N
-    a.q_stride_b, a.key_stride_b, a.key_stride_n, a.key_stride_h = q.stride(0), sb, sn, sh
-    a.scale = scale
-    a.out_idx, a.out_val = idx.data_ptr(), val.data_ptr()
-    a.out_scores = scores.data_ptr() if scores is not None else None
-    need = L.lib().tka_gemv_topk_workspace_bytes(C.byref(a))
-    ws = _workspace(need, q.device)
-    a.workspace, a.workspace_bytes, a.stream = ws.data_ptr(), ws.numel(), _stream()
-    L.check(L.lib().tka_gemv_topk(C.byref(a)), "tka_gemv_topk")
-    return (idx, val, scores) if return_scores else (idx, val)
+    plan = GemvTopkPlan(q, keys, k, group, scale, num_chunks, return_scores).run()
+    return (plan.idx, plan.val, plan.scores) if return_scores else (plan.idx, plan.val)
 
 
 def gemv_scores(q, keys, group=1, scale=1.0):
@@ -181,40 +195,57 @@ def index_union(idx, sink, local, seq_len):
     return out, cnt
 
 
+class FlashDecodePlan:
+    """Argument block, output and workspace of one split-K decode configuration; run() is one C call."""
+
+    def __init__(self, q, keys, values, scale, group=1, num_splits=0, kv_idx=None, kv_count=None, kv_logit=None,
+                 out_dtype=None, return_lse=False, softmax_mode=L.TKA_SOFTMAX_SCALED):
+        _need_cuda(q, keys, values, kv_idx, kv_count, kv_logit)
+        q = _q3(q)
+        B = q.shape[0]
+        sb, sn, sh, N, H = _kv_strides(keys, B)
+        if _kv_strides(values, B) != (sb, sn, sh, N, H):
+            raise ValueError("keys and values must share shape and strides")
+        out_dtype = out_dtype or q.dtype
+        self.q, self.keys, self.values = q, keys, values
+        self.out = torch.empty((B, H * group, 128), dtype=out_dtype, device=q.device)
+        self.lse = torch.empty((B, H * group), dtype=torch.float32, device=q.device) if return_lse else None
+        a = L.FlashDecodeArgs()
+        a.q, a.keys, a.values, a.out = q.data_ptr(), keys.data_ptr(), values.data_ptr(), self.out.data_ptr()
+        a.dtype, a.out_dtype = _dtype_code(keys), _DT[out_dtype]
+        a.batch, a.num_kv_heads, a.group, a.head_dim = B, H, group, 128
+        a.num_splits, a.softmax_mode = num_splits, softmax_mode
+        a.seq_len, a.q_stride_b, a.out_stride_b = N, q.stride(0), self.out.stride(0)
+        a.kv_stride_b, a.kv_stride_n, a.kv_stride_h = sb, sn, sh
+        a.scale = scale
+        if kv_idx is not None:
+            self.kv_idx = kv_idx.contiguous()
+            a.idx_len, a.kv_idx = self.kv_idx.shape[-1], self.kv_idx.data_ptr()
+            if kv_count is not None:
+                self.kv_count = kv_count.contiguous()
+                a.kv_count = self.kv_count.data_ptr()
+            if kv_logit is not None:
+                self.kv_logit = kv_logit.contiguous()
+                a.kv_logit = self.kv_logit.data_ptr()
+        a.out_lse = self.lse.data_ptr() if self.lse is not None else None
+        need = L.lib().tka_flash_decode_workspace_bytes(C.byref(a))
+        self.ws = _workspace(need, q.device)
+        a.workspace, a.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
+        self.args = a
+        self._fn = L.lib().tka_flash_decode
+
+    def run(self):
+        self.args.stream = torch.cuda.current_stream().cuda_stream
+        L.check(self._fn(C.byref(self.args)), "tka_flash_decode")
+        return self
+
+
 def flash_decode(q, keys, values, scale, group=1, num_splits=0, kv_idx=None, kv_count=None, kv_logit=None,
                  out_dtype=None, return_lse=False, softmax_mode=L.TKA_SOFTMAX_SCALED):
     """Split-K decode attention (dense, or over kv_idx [B,Hkv,L]).  Returns out [B,Hq,128] (and LSE fp32 [B,Hq])."""
-    _need_cuda(q, keys, values, kv_idx, kv_count, kv_logit)
-    q = _q3(q)
-    B = q.shape[0]
-    sb, sn, sh, N, H = _kv_strides(keys, B)
-    if _kv_strides(values, B) != (sb, sn, sh, N, H):
-        raise ValueError("keys and values must share shape and strides")
-    out_dtype = out_dtype or q.dtype
-    out = torch.empty((B, H * group, 128), dtype=out_dtype, device=q.device)
-    lse = torch.empty((B, H * group), dtype=torch.float32, device=q.device) if return_lse else None
-    a = L.FlashDecodeArgs()
-    a.q, a.keys, a.values, a.out = q.data_ptr(), keys.data_ptr(), values.data_ptr(), out.data_ptr()
-    a.dtype, a.out_dtype = _dtype_code(keys), _DT[out_dtype]
-    a.batch, a.num_kv_heads, a.group, a.head_dim, a.num_splits, a.softmax_mode = B, H, group, 128, num_splits, softmax_mode
-    a.seq_len, a.q_stride_b, a.out_stride_b = N, q.stride(0), out.stride(0)
-    a.kv_stride_b, a.kv_stride_n, a.kv_stride_h = sb, sn, sh
-    a.scale = scale
-    if kv_idx is not None:
-        kv_idx = kv_idx.contiguous()
-        a.idx_len, a.kv_idx = kv_idx.shape[-1], kv_idx.data_ptr()
-        if kv_count is not None:
-            kv_count = kv_count.contiguous()
-            a.kv_count = kv_count.data_ptr()
-        if kv_logit is not None:
-            kv_logit = kv_logit.contiguous()
-            a.kv_logit = kv_logit.data_ptr()
-    a.out_lse = lse.data_ptr() if lse is not None else None
-    need = L.lib().tka_flash_decode_workspace_bytes(C.byref(a))
-    ws = _workspace(need, q.device)
-    a.workspace, a.workspace_bytes, a.stream = ws.data_ptr(), ws.numel(), _stream()
-    L.check(L.lib().tka_flash_decode(C.byref(a)), "tka_flash_decode")
-    return (out, lse) if return_lse else out
+    plan = FlashDecodePlan(q, keys, values, scale, group, num_splits, kv_idx, kv_count, kv_logit, out_dtype,
+                           return_lse, softmax_mode).run()
+    return (plan.out, plan.lse) if return_lse else plan.out
 
 
 def lse_combine(part_m, part_l, part_acc, out_dtype=torch.float16, return_lse=False):
