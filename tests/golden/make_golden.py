@@ -1,0 +1,41 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/sparse_decode_small.npz: seeded inputs (bit patterns) and the oracle's outputs for one
+small end-to-end case per element type.  The reference repository holds no vectors of its own (all its data is
+generated at run time), so these fixtures freeze the oracle instead: a change in tka_oracle.c that alters any
+result fails tests/test_golden.py.  Run from the repository root:  python tests/golden/make_golden.py"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+import oracle  # noqa: E402
+
+
+def main():
+    out = {}
+    scale = float(np.float32(1.0 / np.sqrt(128.0)))
+    for tag, dtype, seed in (("f16", oracle.F16, 11), ("bf16", oracle.BF16, 12)):
+        rng = np.random.default_rng(seed)
+        N, H, G, k, sink, local = 128, 2, 4, 24, 4, 8
+        Kf = rng.standard_normal((N, H, 128))
+        Kf[rng.permutation(N)[:8]] *= 4.0                       # a few heavy hitters
+        levels = np.linspace(-2, 2, 16)
+        Kf[64:96] = levels[rng.integers(0, 16, (32, H, 128))]    # a stretch of 16-level keys: exact ties
+        q = oracle.to_bits(rng.standard_normal((H * G, 128)), dtype)
+        K = oracle.to_bits(Kf, dtype)
+        V = oracle.to_bits(rng.standard_normal((N, H, 128)), dtype)
+        outs, tidx, tval, unis, cnts = [], [], [], [], []
+        for h in range(H):
+            o, ti, tv, u = oracle.sparse_decode_step(q[h * G:(h + 1) * G], K[:, h], V[:, h], dtype, G, k, sink, local, scale)
+            outs.append(o); tidx.append(ti); tval.append(tv)
+            unis.append(np.pad(u, (0, k + sink + local - len(u)), constant_values=-1)); cnts.append(len(u))
+        out.update({tag + "_q": q, tag + "_K": K, tag + "_V": V, tag + "_out": np.stack(outs), tag + "_topk_idx": np.stack(tidx),
+                    tag + "_topk_val": np.stack(tval), tag + "_union": np.stack(unis), tag + "_union_count": np.array(cnts)})
+    out["params"] = np.array([128, 2, 4, 24, 4, 8], np.int64)
+    np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "sparse_decode_small.npz"), **out)
+
+
+if __name__ == "__main__":
+    main()

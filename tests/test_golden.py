@@ -1,0 +1,44 @@
+"""Committed fixtures (tests/golden/, written by make_golden.py): the oracle must still reproduce them, and on a
+GPU the library must match them through the C ABI."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+
+FIX = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sparse_decode_small.npz"))
+N, H, G, K_TOP, SINK, LOCAL = (int(x) for x in FIX["params"])
+SCALE = float(np.float32(1.0 / np.sqrt(128.0)))
+CASES = [("f16", oracle.F16), ("bf16", oracle.BF16)]
+
+
+@pytest.mark.parametrize("tag,dtype", CASES)
+def test_oracle_reproduces_fixture(tag, dtype):
+    q, K, V = FIX[tag + "_q"], FIX[tag + "_K"], FIX[tag + "_V"]
+    for h in range(H):
+        o, ti, tv, u = oracle.sparse_decode_step(q[h * G:(h + 1) * G], K[:, h], V[:, h], dtype, G, K_TOP, SINK, LOCAL, SCALE)
+        assert np.array_equal(ti, FIX[tag + "_topk_idx"][h])
+        assert np.array_equal(tv.view(np.uint32), FIX[tag + "_topk_val"][h].view(np.uint32))
+        assert len(u) == FIX[tag + "_union_count"][h] and np.array_equal(u, FIX[tag + "_union"][h][:len(u)])
+        assert np.abs(o - FIX[tag + "_out"][h]).max() < 1e-12
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,dtype", CASES)
+def test_gpu_matches_fixture(tag, dtype):
+    import torch
+    from tests.util import announce, f32_of, to_dev
+    from topk_attn_amd import ops
+    announce("golden fixture %s" % tag)
+    q, K, V = FIX[tag + "_q"], FIX[tag + "_K"], FIX[tag + "_V"]
+    out, tidx, tval, uidx, ucnt = ops.sparse_decode_step(to_dev(q[None], dtype), to_dev(K[None], dtype), to_dev(V[None], dtype),
+                                                         K_TOP, SINK, LOCAL, SCALE, G, out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    assert np.array_equal(tidx[0].cpu().numpy(), FIX[tag + "_topk_idx"])
+    assert np.array_equal(tval[0].cpu().numpy().view(np.uint32), FIX[tag + "_topk_val"].view(np.uint32))
+    cnt = ucnt[0].cpu().numpy()
+    assert np.array_equal(cnt, FIX[tag + "_union_count"])
+    for h in range(H):
+        assert np.array_equal(uidx[0, h, :cnt[h]].cpu().numpy(), FIX[tag + "_union"][h][:cnt[h]])
+    assert np.abs(f32_of(out)[0] - FIX[tag + "_out"].reshape(H * G, 128)).max() < 2e-3
