@@ -187,7 +187,26 @@ class FlashDecode:
         return kv + 2 * 32 * 128 * 2, kv, {}
 
 
+class PlainCopy:
+    """Calibration workload for the HBM traffic counters: a device-to-device copy of known size."""
+
+    def __init__(self, torch, dev, nbytes=1 << 30):
+        self.src = torch.ones(nbytes // 2, dtype=torch.float16, device=dev)
+        self.dst = torch.empty_like(self.src)
+        self.nbytes = nbytes
+        self.desc = "copy: %d bytes read + %d bytes written per step" % (nbytes, nbytes)
+        self.dominant = "(torch copy kernel)"
+
+    def step(self):
+        self.dst.copy_(self.src)
+
+    def bytes(self):
+        return 2 * self.nbytes, 2 * self.nbytes, {}
+
+
 def build_workload(name, torch, ops, dev, args):
+    if name == "copy":
+        return PlainCopy(torch, dev)
     if name == "c4":
         return SparseDecode(torch, ops, dev)
     if name == "c4-small":
@@ -208,7 +227,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c4-small", "c5"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c4-small", "c5", "copy"])
     ap.add_argument("--splits", type=int, default=0, help="c3: split count (0 = library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-runs", type=int, default=3)
@@ -251,7 +270,7 @@ def main():
     prof = ops.profile_read()
     ops.profile_enable(False)
     kern = {name: ms / max(n, 1) * 1e3 for name, (ms, n) in prof.items()}  # us per launch
-    dom_us = kern.get(w.dominant, float("nan"))
+    dom_us = kern.get(w.dominant, ms_per_step * 1e3)   # a workload with one foreign kernel: the step itself
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
 
     out = {
