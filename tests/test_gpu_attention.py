@@ -231,3 +231,37 @@ def test_sparse_decode_step(dtype, out_dt, B, H, G, N, k, sink, local):
             assert np.array_equal(tval[b, h].view(np.uint32), rv.view(np.uint32))
             assert ucnt[b, h] == len(ru) and np.array_equal(uidx[b, h, :len(ru)], ru)
             assert (np.abs(out[b, h * G:(h + 1) * G] - ro) < out_tol(ro, out_dt == torch.bfloat16)).all()
+
+
+@pytest.mark.parametrize("dtype,B,H,G,N,k,sink,local,kind", [
+    (oracle.F16, 2, 2, 4, 16384, 2048, 64, 512, "heavy"),
+    (oracle.BF16, 1, 2, 8, 40000, 1024, 16, 128, "levels"),
+    (oracle.F16, 1, 2, 1, 5000, 300, 8, 8, "equal"),
+    (oracle.F16, 1, 1, 2, 4099, 129, 0, 0, "heavy"),
+    (oracle.BF16, 1, 3, 4, 8000, 8000, 4, 4, "heavy")])
+def test_sparse_decode_step_union_only(dtype, B, H, G, N, k, sink, local, kind, out_dt=torch.float16):
+    """Production form of the step: no rank-ordered output.  The union list must still equal the oracle's bit for
+    bit — with heavy hitters, with 16-level keys (large tie buckets), with all keys equal (every token ties) and
+    with k = N."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step union-only dtype=%d B=%d H=%d G=%d N=%d k=%d %s" % (dtype, B, H, G, N, k, kind))
+    rng = np.random.default_rng(N + k)
+    if kind == "levels":
+        Kf = np.linspace(-2, 2, 16)[rng.integers(0, 16, (B, N, H, 128))]
+    elif kind == "equal":
+        Kf = np.broadcast_to(rng.standard_normal((1, 1, 1, 128)), (B, N, H, 128)).copy()
+    else:
+        Kf = rng.standard_normal((B, N, H, 128))
+        Kf[:, rng.permutation(N)[:max(1, N // 100)]] *= 4.0
+    q, K, V = randn_bits(rng, (B, H * G, 128), dtype), oracle.to_bits(Kf, dtype), randn_bits(rng, (B, N, H, 128), dtype)
+    out, tidx, tval, uidx, ucnt = ops.sparse_decode_step(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), k, sink,
+                                                         local, SCALE, G, out_dtype=out_dt, want_topk=False)
+    torch.cuda.synchronize()
+    assert tidx is None and tval is None
+    out, uidx, ucnt = f32_of(out), uidx.cpu().numpy(), ucnt.cpu().numpy()
+    for b in range(B):
+        for h in range(H):
+            ro, ri, rv, ru = oracle.sparse_decode_step(q[b, h * G:(h + 1) * G], K[b, :, h], V[b, :, h], dtype, G, k, sink,
+                                                       local, SCALE)
+            assert ucnt[b, h] == len(ru) and np.array_equal(uidx[b, h, :len(ru)], ru), "union differs (b=%d h=%d)" % (b, h)
+            assert (np.abs(out[b, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()

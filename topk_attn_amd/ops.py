@@ -335,9 +335,10 @@ class SparseDecodePlan:
         return self.out
 
 
-def sparse_decode_step(q, keys, values, k, sink, local, scale, group, out_dtype=None, num_splits=0):
-    """End-to-end decode step.  Returns (out, topk_idx, topk_val, union_idx, union_count)."""
-    plan = SparseDecodePlan(q, keys, values, k, sink, local, scale, group, out_dtype, num_splits)
+def sparse_decode_step(q, keys, values, k, sink, local, scale, group, out_dtype=None, num_splits=0, want_topk=True):
+    """End-to-end decode step.  Returns (out, topk_idx, topk_val, union_idx, union_count); without want_topk the
+    rank-ordered selection is not produced (None)."""
+    plan = SparseDecodePlan(q, keys, values, k, sink, local, scale, group, out_dtype, num_splits, want_topk=want_topk)
     plan.step()
     return plan.out, plan.topk_idx, plan.topk_val, plan.union_idx, plan.union_count
 
