@@ -235,7 +235,8 @@ def test_sparse_decode_step(dtype, out_dt, B, H, G, N, k, sink, local):
 
 @pytest.mark.parametrize("dtype,B,H,G,N,k,sink,local,kind", [
     (oracle.F16, 2, 2, 4, 16384, 2048, 64, 512, "heavy"),
-    (oracle.BF16, 1, 2, 8, 40000, 1024, 16, 128, "levels"),
+    (oracle.BF16, 1, 2, 8, 70000, 1024, 16, 128, "levels"),
+    (oracle.F16, 1, 2, 2, 66000, 2000, 8, 8, "equal"),
     (oracle.F16, 1, 2, 1, 5000, 300, 8, 8, "equal"),
     (oracle.F16, 1, 1, 2, 4099, 129, 0, 0, "heavy"),
     (oracle.BF16, 1, 3, 4, 8000, 8000, 4, 4, "heavy")])

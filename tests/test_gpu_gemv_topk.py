@@ -130,3 +130,69 @@ def test_two_level_cluster_reference_shape():
         # the reference's own check (gemv_topk.cu:138-170): set equality per (head, rank) slice
         for r in range(TOPC):
             assert set(out[h, r * K:(r + 1) * K]) == set(want[r * K:(r + 1) * K])
+
+
+# ---- long segments: sampled threshold + candidate lists, with the dense path as fallback ------------------
+
+def _mix32(x):
+    x &= 0xFFFFFFFF
+    x ^= x >> 16; x = (x * 0x7feb352d) & 0xFFFFFFFF
+    x ^= x >> 15; x = (x * 0x846ca68b) & 0xFFFFFFFF
+    x ^= x >> 16
+    return x
+
+
+def _sampled_positions(seg, n, samples=2048):
+    """Token positions the threshold estimate of a long segment looks at (one per stride, hashed offset)."""
+    stride = n // samples
+    return [i * stride + _mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) % stride for i in range(samples)]
+
+
+def _check_long(K, q, dtype, G, k, scale=SCALE):
+    from topk_attn_amd import ops
+    idx, val = ops.gemv_topk(to_dev(q, dtype), to_dev(K, dtype), k, group=G, scale=scale)
+    torch.cuda.synchronize()
+    idx, val = idx.cpu().numpy(), val.cpu().numpy()
+    B, N, H = K.shape[:3]
+    for b in range(B):
+        for h in range(H):
+            ref = oracle.scores_canonical(K[b, :, h, :], dtype, oracle.group_query(q[b, h * G:(h + 1) * G], dtype, G), scale)
+            ei, ev = oracle.topk_stable(ref, k)
+            assert np.array_equal(idx[b, h], ei), "indices differ (b=%d h=%d)" % (b, h)
+            assert np.array_equal(val[b, h].view(np.uint32), ev.view(np.uint32))
+
+
+def test_long_segment_candidates():
+    announce("gemv_topk long segment N=131072 k=2048 G=4 (candidate lists)")
+    rng = np.random.default_rng(31)
+    K = randn_bits(rng, (1, 131072, 2, 128), oracle.F16)
+    K[0, rng.permutation(131072)[:1300]] = oracle.to_bits(rng.standard_normal((1300, 2, 128)) * 4.0, oracle.F16)
+    _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 2048)
+
+
+def test_long_segment_all_equal_falls_back():
+    """Every key equal: every token passes the sampled threshold, the segment is redone by the dense path."""
+    announce("gemv_topk long segment all keys equal (fallback: too many candidates)")
+    rng = np.random.default_rng(32)
+    K = np.broadcast_to(randn_bits(rng, (1, 1, 1, 128), oracle.BF16), (1, 70001, 2, 128)).copy()
+    _check_long(K, randn_bits(rng, (1, 2, 128), oracle.BF16), oracle.BF16, 1, 1000)
+
+
+def test_long_segment_sample_hits_only_heavy_tokens_falls_back():
+    """Heavy tokens placed exactly where the threshold estimate samples: the threshold lands among them, fewer than
+    k tokens pass, and the segment is redone by the dense path.  One head is adversarial, the other ordinary."""
+    announce("gemv_topk long segment adversarial sample (fallback: too few candidates)")
+    rng = np.random.default_rng(33)
+    N, k, dtype = 131072, 4096, oracle.F16
+    Kf = rng.standard_normal((1, N, 2, 128)) * 0.05
+    qf = rng.standard_normal((1, 2, 128))
+    pos = _sampled_positions(0, N)                       # segment 0 = (batch 0, head 0)
+    Kf[0, pos, 0, :] = qf[0, 0] * rng.uniform(0.5, 1.5, (len(pos), 1))   # large positive scores, all distinct
+    _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k)
+
+
+def test_long_segment_bf16_levels_group8():
+    announce("gemv_topk long segment bf16 16-level keys N=262144 k=4096 G=8")
+    rng = np.random.default_rng(34)
+    K = oracle.to_bits(np.linspace(-2, 2, 16)[rng.integers(0, 16, (1, 262144, 1, 128))], oracle.BF16)
+    _check_long(K, randn_bits(rng, (1, 8, 128), oracle.BF16), oracle.BF16, 8, 4096)

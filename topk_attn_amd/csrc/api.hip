@@ -124,6 +124,12 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->group = a->group;
   g->num_chunks = a->num_chunks;
   g->scale = a->scale;
+  g->tau_key = nullptr;
+  g->tau_key_out = nullptr;
+  g->cand = nullptr;
+  g->cand_seg_stride = 0;
+  g->cand_cnt = nullptr;
+  g->seg_flags = nullptr;
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   g->tokens_per_wg = gemv_tokens_per_wg(rows, g->chunk_len);
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
@@ -169,13 +175,50 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     sp.local = u->local;
   }
 
-  int rc = launch_zero_u32(sp.hist, zero_words, stream);
-  if (rc != TKA_OK) return rc;
   GemvParams gp;
   fill_gemv_params(a, scores, sp.hist, &gp);
   gp.cluster_ids = cluster_ids;
+
+  int num_samples = 0, sample_rank = 0;
+  if (!a->out_scores) gemv_candidate_plan(chunk_len, a->k, &num_samples, &sample_rank);
+  if (num_samples == 0) {
+    // dense: clear histograms, GEMV with histogram, filter, finalize
+    int rc = launch_zero_u32(sp.hist, zero_words, stream);
+    if (rc != TKA_OK) return rc;
+    rc = launch_gemv_scores(gp, a->dtype, stream);
+    if (rc != TKA_OK) return rc;
+    return launch_select(sp, stream);
+  }
+
+  // Long segments: sampled threshold, GEMV that stores candidates only, selection straight from the
+  // candidate slices.  A segment whose candidates turn out too few (or far too many) is flagged and redone
+  // by the dense kernels, which otherwise exit at once.
+  GemvParams cp = gp;
+  cp.tau_key_out = sp.tau_key;
+  int rc = launch_sample_tau(cp, a->dtype, num_samples, sample_rank, stream);   // also clears the histograms
+  if (rc != TKA_OK) return rc;
+  cp.tau_key = sp.tau_key;
+  cp.cand = sp.list;
+  cp.cand_seg_stride = sp.list_stride;
+  cp.cand_cnt = sp.list_cnt;
+  cp.hist = nullptr;
+  rc = launch_gemv_scores(cp, a->dtype, stream);
+  if (rc != TKA_OK) return rc;
+  SelectParams sc = sp;
+  sc.hist = nullptr;
+  sc.parts = cp.wgs_per_chunk;
+  sc.part_len = cp.tokens_per_wg;
+  sc.list_stride = sp.list_stride;
+  sc.max_entries = (int)((chunk_len * (int64_t)sample_rank / num_samples) * 8);
+  rc = launch_select_finalize(sc, stream);
+  if (rc != TKA_OK) return rc;
+  // dense fallback for flagged segments: long runs per workgroup keep the (normally idle) grids small
+  gp.seg_flags = sp.seg_flags;
+  gp.tokens_per_wg = 4096;
+  gp.wgs_per_chunk = (int)((chunk_len + gp.tokens_per_wg - 1) / gp.tokens_per_wg);
   rc = launch_gemv_scores(gp, a->dtype, stream);
   if (rc != TKA_OK) return rc;
+  sp.check_flags = 1;
   return launch_select(sp, stream);
 }
 

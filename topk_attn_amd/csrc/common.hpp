@@ -19,6 +19,8 @@ constexpr int kHeadDim = TKA_HEAD_DIM;
 constexpr int kWave = 64;
 constexpr int kHistBits = 11;
 constexpr int kHistBins = 1 << kHistBits;  // first-level selection histogram: top 11 bits of the key
+constexpr int kGemvCandTokensPerWg = 256;  // tokens per GEMV workgroup on large problems (= slice length of candidate lists)
+constexpr int kGemvMaxSamples = 2048;      // sample size of the candidate-mode threshold estimate
 
 // ---- lane exchanges ---------------------------------------------------------------------------
 
@@ -119,6 +121,33 @@ __device__ __forceinline__ float key_score(uint32_t key) {
 }
 // 64-bit composite: all elements distinct, larger = earlier in (score desc, index asc) order.
 __device__ __forceinline__ uint64_t composite(uint32_t key, uint32_t idx) { return ((uint64_t)key << 32) | (uint32_t)~idx; }
+
+// ---- block-wide threshold search (1024 threads, 2048 bins) --------------------------------------
+
+// Finds the bin d with  count(bins > d) < need <= count(bins >= d)  in sh_hist[2048]; every one of the 1024
+// threads of the block must call it.  Results: sh_res[0] = d, sh_res[1] = count(bins > d), sh_res[2] = sh_hist[d].
+// sh_res is left untouched when the histogram holds fewer than `need` elements.
+__device__ __forceinline__ void find_threshold_bin_1024(const uint32_t* sh_hist, uint32_t need, uint32_t* sh_wtot, uint32_t* sh_res) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const uint32_t h0 = sh_hist[2 * tid], h1 = sh_hist[2 * tid + 1];
+  uint32_t v = h0 + h1;  // suffix sum over lanes >= lane
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    uint32_t t = __shfl_down(v, d, 64);
+    if (lane + d < 64) v += t;
+  }
+  if (lane == 0) sh_wtot[wave] = v;
+  __syncthreads();
+  uint32_t above = 0;
+  for (int w = wave + 1; w < 16; ++w) above += sh_wtot[w];
+  const uint32_t ge0 = above + v;   // count(bins >= 2*tid)
+  const uint32_t ge1 = ge0 - h0;    // count(bins >= 2*tid+1)
+  const uint32_t gt1 = ge1 - h1;    // count(bins >  2*tid+1)
+  if (ge1 >= need && gt1 < need) { sh_res[0] = 2 * tid + 1; sh_res[1] = gt1; sh_res[2] = h1; }
+  if (ge0 >= need && ge1 < need) { sh_res[0] = 2 * tid;     sh_res[1] = ge1; sh_res[2] = h0; }
+  __syncthreads();
+}
 
 // ---- host-side launch bookkeeping -------------------------------------------------------------
 

@@ -11,6 +11,13 @@ struct GemvParams {
   float* scores;        // [batch][num_kv_heads][num_chunks][chunk_len]
   const int32_t* cluster_ids;  // [batch*num_kv_heads*num_chunks] or nullptr: chunk c covers the tokens of that cluster
   uint32_t* hist;       // [batch*num_kv_heads*num_chunks][kHistBins] or nullptr; must be zero on entry
+  // candidate mode (cand != nullptr): only tokens with key >= tau_key[segment] are stored
+  const uint32_t* tau_key;    // [segments]
+  uint32_t* tau_key_out;      // [segments], written by the sample kernel
+  uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] composites, one slice per workgroup, ascending index
+  int64_t cand_seg_stride;    // entries between the slice arrays of consecutive segments
+  uint32_t* cand_cnt;         // [segments][wgs_per_chunk] entries in each slice
+  const uint32_t* seg_flags;  // nullptr, or [segments]: workgroups of segments whose flag is 0 exit at once
   int64_t chunk_len;    // tokens per chunk
   int64_t q_stride_b, key_stride_b, key_stride_n, key_stride_h;
   int batch, num_kv_heads, group, num_chunks;
@@ -18,6 +25,8 @@ struct GemvParams {
   float scale;
 };
 int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream);
+int launch_sample_tau(const GemvParams& p, int dtype, int num_samples, int sample_rank, hipStream_t stream);
+void gemv_candidate_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank);
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);
 
 // ---- stage 1: selection -----------------------------------------------------------------------
@@ -25,7 +34,12 @@ struct SelectParams {
   const float* scores;    // segment s starts at scores + s*seg_stride
   int64_t seg_len;
   int64_t seg_stride;
-  uint32_t* hist;         // [num_segments][kHistBins]
+  uint32_t* hist;         // [num_segments][kHistBins]; nullptr: the lists hold candidates above a sampled threshold
+  uint32_t* tau_key;      // [num_segments] candidate threshold (workspace)
+  uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment must be redone densely;
+                          // fallback launches (check_flags) skip segments whose flag is 0
+  int check_flags;
+  int max_entries;        // candidate mode: more listed entries than this also sends the segment to the dense path
   uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)
   uint64_t* list;         // [num_segments][list_stride] composites with bin >= threshold bin, slice p at p*part_len
   int64_t list_stride;
@@ -51,6 +65,8 @@ void select_plan(int64_t seg_len, int num_segments, SelectParams* p);
 int launch_zero_u32(uint32_t* ptr, size_t count, hipStream_t stream);
 int launch_select_hist(const SelectParams& p, hipStream_t stream);
 int launch_select(const SelectParams& p, hipStream_t stream);   // filter + finalize
+int launch_select_filter(const SelectParams& p, hipStream_t stream);
+int launch_select_finalize(const SelectParams& p, hipStream_t stream);
 
 struct UnionParams {
   const int32_t* idx;     // [num_segments][k]

@@ -31,34 +31,10 @@ namespace {
 
 constexpr int kSelThreads = 1024;
 constexpr int kSelWaves = kSelThreads / kWave;
-constexpr int kEndsInLds = 1024;   // slice offsets of one segment kept in LDS by the finalize kernel
+constexpr int kEndsInLds = 4096;   // slice offsets of one segment kept in LDS by the finalize kernel
 constexpr int kEntryCache = 8;     // listed entries per thread kept in registers by the finalize kernel
 
 // ---- block-wide helpers (1024 threads, 2048 bins) ---------------------------------------------
-
-// Finds the bin d with  count(bins > d) < need <= count(bins >= d)  in sh_hist[2048].
-// Results in sh_res[0] = d, sh_res[1] = count(bins > d), sh_res[2] = sh_hist[d].
-__device__ void find_threshold_bin(const uint32_t* sh_hist, uint32_t need, uint32_t* sh_wtot, uint32_t* sh_res) {
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const uint32_t h0 = sh_hist[2 * tid], h1 = sh_hist[2 * tid + 1];
-  uint32_t v = h0 + h1;  // suffix sum over lanes >= lane
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    uint32_t t = __shfl_down(v, d, 64);
-    if (lane + d < 64) v += t;
-  }
-  if (lane == 0) sh_wtot[wave] = v;
-  __syncthreads();
-  uint32_t above = 0;
-  for (int w = wave + 1; w < kSelWaves; ++w) above += sh_wtot[w];
-  const uint32_t ge0 = above + v;   // count(bins >= 2*tid)
-  const uint32_t ge1 = ge0 - h0;    // count(bins >= 2*tid+1)
-  const uint32_t gt1 = ge1 - h1;    // count(bins >  2*tid+1)
-  if (ge1 >= need && gt1 < need) { sh_res[0] = 2 * tid + 1; sh_res[1] = gt1; sh_res[2] = h1; }
-  if (ge0 >= need && ge1 < need) { sh_res[0] = 2 * tid;     sh_res[1] = ge1; sh_res[2] = h0; }
-  __syncthreads();
-}
 
 // ---- bitonic sort of 1024*E composites, descending --------------------------------------------
 
@@ -254,6 +230,7 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams
   const int tid = threadIdx.x;
   const int seg = blockIdx.y;
   const int part = blockIdx.x;
+  if (p.check_flags && p.seg_flags[seg] == 0) return;  // fallback launch: this segment needs nothing
 
   // this thread's run of scores first: the loads do not depend on the threshold
   const float* sc = p.scores + (int64_t)seg * p.seg_stride;
@@ -267,7 +244,7 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams
   sh_hist[2 * tid] = gh[2 * tid];
   sh_hist[2 * tid + 1] = gh[2 * tid + 1];
   __syncthreads();
-  find_threshold_bin(sh_hist, (uint32_t)p.k, sh_wtot, sh_res);
+  find_threshold_bin_1024(sh_hist, (uint32_t)p.k, sh_wtot, sh_res);
   const uint32_t b1 = sh_res[0];
 
   uint32_t mine = 0;
@@ -295,38 +272,48 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   const int tid = threadIdx.x;
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
+  if (p.check_flags && p.seg_flags[seg] == 0) return;  // fallback launch: this segment was already done
+  const bool from_hist = p.hist != nullptr;
 
-  // threshold bin, count above it, count inside it
-  {
+  // dense mode: threshold bin, count above it, count inside it
+  uint32_t b1 = 0, n_above = 0, n_bin = 0;
+  if (from_hist) {
     const uint32_t* gh = p.hist + (int64_t)seg * kHistBins;
     sh_hist[2 * tid] = gh[2 * tid];
     sh_hist[2 * tid + 1] = gh[2 * tid + 1];
     __syncthreads();
-    find_threshold_bin(sh_hist, k, sh_wtot, sh_res);
+    find_threshold_bin_1024(sh_hist, k, sh_wtot, sh_res);
+    b1 = sh_res[0], n_above = sh_res[1], n_bin = sh_res[2];
   }
-  const uint32_t b1 = sh_res[0], n_above = sh_res[1], n_bin = sh_res[2];
 
   // slice counts -> inclusive offsets (entries of the segment get one running index); kept in LDS when
   // they fit, in place in global memory otherwise
   __shared__ uint32_t sh_ends[kEndsInLds];
   uint32_t* g_ends = p.list_cnt + (int64_t)seg * p.parts;
   const bool ends_in_lds = p.parts <= kEndsInLds;
+  uint32_t n_listed = 0;
   {
-    uint32_t running = 0;
     for (int base = 0; base < p.parts; base += kSelThreads) {
       const int i = base + tid;
       const uint32_t c = i < p.parts ? g_ends[i] : 0u;
       uint32_t total;
       const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
       if (i < p.parts) {
-        if (ends_in_lds) sh_ends[i] = running + ex + c; else g_ends[i] = running + ex + c;
+        if (ends_in_lds) sh_ends[i] = n_listed + ex + c; else g_ends[i] = n_listed + ex + c;
       }
-      running += total;
+      n_listed += total;
     }
     __syncthreads();
   }
+  // candidate mode: the lists hold every token above a sampled threshold.  Fewer than k of them (the
+  // estimate was too high) or far too many (ties, skewed data) sends the segment to the dense path.
+  if (!from_hist) {
+    const bool redo = n_listed < k || n_listed > (uint32_t)p.max_entries;
+    if (tid == 0) p.seg_flags[seg] = redo ? 1u : 0u;
+    if (redo) return;
+  }
   const uint32_t* ends = ends_in_lds ? sh_ends : g_ends;
-  const uint32_t n_entries = n_above + n_bin;  // == ends[parts-1]
+  const uint32_t n_entries = n_listed;  // dense mode: == n_above + n_bin
   const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
   // entry v of the segment: slice s with ends[s-1] <= v < ends[s], position v - ends[s-1] in that slice
   auto fetch = [&](uint32_t v) -> uint64_t {
@@ -348,12 +335,13 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   auto entry = [&](uint32_t v) -> uint64_t { return fetch(v); };
 
   // Refine inside bin b1: the listed entries of that bin share their top 11 bits.  Take `need` of them.
-  uint32_t need = k - n_above;          // >= 1 by construction of b1
-  uint64_t prefix = b1;                 // value of the bits fixed so far
-  int fixed = kHistBits;                // number of top bits fixed
-  uint64_t threshold = 0;               // selected: composite >= threshold
-  bool done = (need == n_bin);          // whole bin taken
-  if (done) threshold = (uint64_t)b1 << (64 - kHistBits);
+  // (candidate mode starts from scratch: no bit fixed, k to take.)
+  uint32_t need = from_hist ? k - n_above : k;   // >= 1
+  uint64_t prefix = from_hist ? b1 : 0;          // value of the bits fixed so far
+  int fixed = from_hist ? kHistBits : 0;         // number of top bits fixed
+  uint64_t threshold = 0;                        // selected: composite >= threshold
+  bool done = from_hist ? (need == n_bin) : (need == n_entries);   // whole bin / whole list taken
+  if (done && from_hist) threshold = (uint64_t)b1 << (64 - kHistBits);
   while (!done) {
     const int bits = (64 - fixed) >= kHistBits ? kHistBits : (64 - fixed);
     const int shift = 64 - fixed - bits;
@@ -364,15 +352,15 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
 #pragma unroll
     for (int i = 0; i < kEntryCache; ++i) {
       const uint64_t c = cache[i];
-      if ((uint32_t)i * kSelThreads + tid < n_entries && (c >> (64 - fixed)) == prefix)
+      if ((uint32_t)i * kSelThreads + tid < n_entries && (fixed == 0 || (c >> (64 - fixed)) == prefix))
         atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
     }
     for (uint32_t v = kEntryCache * kSelThreads + tid; v < n_entries; v += kSelThreads) {
       const uint64_t c = entry(v);
-      if ((c >> (64 - fixed)) == prefix) atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
+      if (fixed == 0 || (c >> (64 - fixed)) == prefix) atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
     }
     __syncthreads();
-    find_threshold_bin(sh_hist, need, sh_wtot, sh_res);
+    find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
     const uint32_t d = sh_res[0], gt = sh_res[1], cnt = sh_res[2];
     need -= gt;
     prefix = (prefix << bits) | d;
@@ -528,20 +516,22 @@ int kpad_for(int k) {
 }  // namespace
 
 // Workspace layout (each part 256-byte aligned):
-//   hist [S][2048] u32 (cleared per call) | list_cnt [S][parts] u32 | list [S][parts*part_len] u64
+//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S] u32 | list_cnt [S][slices] u32 |
+//   list [S][slices*slice_len] u64      (slices: dense 4096/16384 scores, candidate mode one per GEMV workgroup)
 namespace {
 struct SelectLayout {
-  size_t hist, list_cnt, list, total;
+  size_t hist, flags, tau, list_cnt, list, total;
   int64_t list_stride;
 };
 SelectLayout select_layout(int num_segments, int64_t seg_len) {
   SelectLayout l;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t at = off; off += align_up(bytes, 256); return at; };
-  const int64_t min_part = 4 * kSelThreads;
-  const int64_t max_parts = (seg_len + min_part - 1) / min_part;
+  const int64_t max_parts = seg_len / 128 + 2;   // candidate mode: one slice per GEMV workgroup of >= 128 tokens
   l.list_stride = (seg_len + 16 * kSelThreads - 1) / (16 * kSelThreads) * (16 * kSelThreads);  // whole slices
   l.hist = take((size_t)num_segments * kHistBins * sizeof(uint32_t));
+  l.flags = take((size_t)num_segments * sizeof(uint32_t));
+  l.tau = take((size_t)num_segments * sizeof(uint32_t));
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
   l.total = off;
@@ -556,10 +546,12 @@ size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p
   const SelectLayout l = select_layout(num_segments, seg_len);
   unsigned char* c = (unsigned char*)ws;
   p->hist = (uint32_t*)(c + l.hist);
+  p->seg_flags = (uint32_t*)(c + l.flags);
+  p->tau_key = (uint32_t*)(c + l.tau);
   p->list_cnt = (uint32_t*)(c + l.list_cnt);
   p->list = (uint64_t*)(c + l.list);
   p->list_stride = l.list_stride;
-  return (size_t)num_segments * kHistBins;
+  return (size_t)num_segments * kHistBins;  // the flags follow the histograms; candidate mode writes them itself
 }
 
 // Slice per workgroup: 16384 scores (16 per thread) when that still gives every CU work, else 4096.
@@ -587,28 +579,40 @@ int launch_select_hist(const SelectParams& p, hipStream_t stream) {
   return hip_status(hipGetLastError());
 }
 
-int launch_select(const SelectParams& p, hipStream_t stream) {
-  const bool want_rank = p.out_idx != nullptr;
-  const int kpad = kpad_for(p.k);
-  const size_t lds = want_rank ? 2 * (size_t)kpad * sizeof(uint64_t) : 0;
+static int set_finalize_attr() {
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 130 * 1024);  // 2 x 8192 composites; 25 KB are static
     if (e != hipSuccess) return TKA_EHIP;
     attr_set = true;
   }
-  {
-    LaunchTimer timer("select_filter", stream);
-    const dim3 grid((unsigned)p.parts, (unsigned)p.num_segments);
-    if (p.part_len == 16 * kSelThreads)
-      select_filter_kernel<16><<<grid, kSelThreads, 0, stream>>>(p);
-    else
-      select_filter_kernel<4><<<grid, kSelThreads, 0, stream>>>(p);
-    if (hipGetLastError() != hipSuccess) return TKA_EHIP;
-  }
-  LaunchTimer timer("select_finalize", stream);
+  return TKA_OK;
+}
+
+int launch_select_filter(const SelectParams& p, hipStream_t stream) {
+  LaunchTimer timer(p.check_flags ? "select_filter_fallback" : "select_filter", stream);
+  const dim3 grid((unsigned)p.parts, (unsigned)p.num_segments);
+  if (p.part_len == 16 * kSelThreads)
+    select_filter_kernel<16><<<grid, kSelThreads, 0, stream>>>(p);
+  else
+    select_filter_kernel<4><<<grid, kSelThreads, 0, stream>>>(p);
+  return hip_status(hipGetLastError());
+}
+
+int launch_select_finalize(const SelectParams& p, hipStream_t stream) {
+  const bool want_rank = p.out_idx != nullptr;
+  const int kpad = kpad_for(p.k);
+  const size_t lds = want_rank ? 2 * (size_t)kpad * sizeof(uint64_t) : 0;
+  if (set_finalize_attr() != TKA_OK) return TKA_EHIP;
+  LaunchTimer timer(p.check_flags ? "select_finalize_fallback" : (p.hist ? "select_finalize" : "select_finalize_cand"), stream);
   select_finalize_kernel<<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(p, kpad);
   return hip_status(hipGetLastError());
+}
+
+int launch_select(const SelectParams& p, hipStream_t stream) {
+  int rc = launch_select_filter(p, stream);
+  if (rc != TKA_OK) return rc;
+  return launch_select_finalize(p, stream);
 }
 
 int launch_index_union(const UnionParams& p, hipStream_t stream) {
