@@ -142,10 +142,15 @@ def _mix32(x):
     return x
 
 
-def _sampled_positions(seg, n, samples=2048):
-    """Token positions the threshold estimate of a long segment looks at (one per stride, hashed offset)."""
-    stride = n // samples
-    return [i * stride + _mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) % stride for i in range(samples)]
+def _sampled_positions(seg, n, samples=512, split=4):
+    """Token positions the threshold estimate of a long segment looks at: `samples` per quarter of the segment,
+    one per stride, at a hashed offset inside the stride."""
+    stride = n // split // samples
+    pos = []
+    for quarter in range(split):
+        salt = ((seg * split + quarter) * 0x9e3779b9) & 0xFFFFFFFF
+        pos += [quarter * (n // split) + i * stride + _mix32((salt + i) & 0xFFFFFFFF) % stride for i in range(samples)]
+    return pos
 
 
 def _check_long(K, q, dtype, G, k, scale=SCALE):

@@ -180,7 +180,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   gp.cluster_ids = cluster_ids;
 
   int num_samples = 0, sample_rank = 0;
-  if (!a->out_scores) gemv_candidate_plan(chunk_len, a->k, &num_samples, &sample_rank);
+  if (!a->out_scores && gp.wgs_per_chunk <= select_cand_max_parts() && gp.tokens_per_wg == kGemvCandTokensPerWg)
+    gemv_candidate_plan(chunk_len, a->k, select_cand_capacity(), &num_samples, &sample_rank);
   if (num_samples == 0) {
     // dense: clear histograms, GEMV with histogram, filter, finalize
     int rc = launch_zero_u32(sp.hist, zero_words, stream);
@@ -209,8 +210,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   sc.parts = cp.wgs_per_chunk;
   sc.part_len = cp.tokens_per_wg;
   sc.list_stride = sp.list_stride;
-  sc.max_entries = (int)((chunk_len * (int64_t)sample_rank / num_samples) * 8);
-  rc = launch_select_finalize(sc, stream);
+  sc.max_entries = select_cand_capacity();
+  rc = launch_select_finalize_cand(sc, stream);
   if (rc != TKA_OK) return rc;
   // dense fallback for flagged segments: long runs per workgroup keep the (normally idle) grids small
   gp.seg_flags = sp.seg_flags;

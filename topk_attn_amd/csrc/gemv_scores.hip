@@ -28,6 +28,7 @@ constexpr int kGemvUnroll = 8;                                         // loads 
 constexpr int kGemvRowsPerIter = (kGemvThreads / 16) * kGemvUnroll;    // 128 tokens per WG iteration
 constexpr int kCandMaxIters = kGemvCandTokensPerWg / kGemvRowsPerIter; // iterations of a candidate-mode workgroup
 constexpr int kCandSubLists = kCandMaxIters * kGemvWaves;
+constexpr int kTauSplit = 4;   // sample workgroups (and thresholds) per segment
 
 // Group query of this lane in fp32: ((q0 + q1) + q2) + ... in ascending head order, dims 8j..8j+7.
 template <int DT>
@@ -87,7 +88,12 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
                           chunk_base * p.key_stride_n + 8 * j;
   float* sc_out = CAND ? nullptr : p.scores + seg * p.chunk_len;
-  const uint32_t tau = CAND ? p.tau_key[seg] : 0u;
+  uint32_t tau = 0u;
+  if (CAND) {   // lowest of the quarter thresholds: every quarter then passes at least its own share
+    tau = ~0u;
+#pragma unroll
+    for (int w = 0; w < kTauSplit; ++w) tau = min(tau, p.tau_key[seg * kTauSplit + w]);
+  }
 
   int it = 0;
   for (int64_t base = t_begin; base < t_end; base += kGemvRowsPerIter, ++it) {
@@ -154,15 +160,19 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
 
 constexpr int kTauThreads = 1024;
 constexpr int kTauRowGroups = kTauThreads / 16;
+constexpr int kTauUnroll = 8;            // rows per row group and round: 512 samples per round
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {  // integer hash for the sample jitter
   x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
   return x;
 }
 
-// One workgroup per segment: scores of num_samples tokens (one per stride of chunk_len/num_samples tokens, at
-// a hashed offset inside the stride so that periodic data cannot alias with the sampling), then the
-// sample_rank-th largest key by radix select in LDS -> tau_key[segment].
+// kTauSplit workgroups per segment (a single CU cannot pull its share of rows fast enough): each scores
+// num_samples tokens of its quarter of the segment (one per stride, at a hashed offset inside the stride so
+// that periodic data cannot alias with the sampling) and takes the sample_rank-th largest key by radix select
+// in LDS -> tau_key[segment][quarter].  About sample_rank/num_samples of the quarter's tokens lie at or above
+// that key wherever the large scores sit in the segment; the GEMV uses the lowest of the four, so that the
+// number of tokens that pass is at least the sum of the four shares.
 template <int DT>
 __global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, int num_samples, int sample_rank) {
   __shared__ uint32_t sh_keys[kGemvMaxSamples];
@@ -172,13 +182,14 @@ __global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, i
 
   const int tid = threadIdx.x;
   const int j = tid & 15, rg = tid >> 4;
-  const int seg = blockIdx.x;
+  const int seg = blockIdx.y;
+  const int quarter = blockIdx.x;
   const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
   const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
 
   // the dense fallback, should this segment need it, finds its histogram cleared
-  if (p.hist) {
+  if (p.hist && quarter == 0) {
     p.hist[(int64_t)seg * kHistBins + 2 * tid] = 0u;
     p.hist[(int64_t)seg * kHistBins + 2 * tid + 1] = 0u;
   }
@@ -187,30 +198,34 @@ __global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, i
   load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
                           chunk_base * p.key_stride_n + 8 * j;
-  const int64_t stride = p.chunk_len / num_samples;
+  const int64_t quarter_len = p.chunk_len / kTauSplit;
+  const int64_t stride = quarter_len / num_samples;
+  kbase += (int64_t)quarter * quarter_len * p.key_stride_n;
 
-  for (int base = 0; base < num_samples; base += kTauRowGroups * kGemvUnroll) {
-    u32x4 kv[kGemvUnroll];
+  // kTauUnroll rows in flight per row group: the kernel is one latency chain per batch of loads
+  for (int base = 0; base < num_samples; base += kTauRowGroups * kTauUnroll) {
+    u32x4 kv[kTauUnroll];
 #pragma unroll
-    for (int u = 0; u < kGemvUnroll; ++u) {
-      const int i = base + rg * kGemvUnroll + u;                       // sample number (num_samples is a multiple of 512)
-      const int64_t t = (int64_t)i * stride + (int64_t)(mix32((uint32_t)seg * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
+    for (int u = 0; u < kTauUnroll; ++u) {
+      const int i = base + rg * kTauUnroll + u;                        // sample number (num_samples is a multiple of 512)
+      const int64_t t = (int64_t)i * stride + (int64_t)(mix32(((uint32_t)seg * kTauSplit + quarter) * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
       kv[u] = *(const u32x4*)(kbase + t * p.key_stride_n);
     }
     float mine = 0.0f;
 #pragma unroll
-    for (int u = 0; u < kGemvUnroll; ++u) {
+    for (int u = 0; u < kTauUnroll; ++u) {
       const float s = row_score<DT>(qf, kv[u], p.scale);
       if (j == u) mine = s;
     }
-    if (j < kGemvUnroll) sh_keys[base + rg * kGemvUnroll + j] = score_key(mine);
+    if (j < kTauUnroll) sh_keys[base + rg * kTauUnroll + j] = score_key(mine);
   }
 
-  // sample_rank-th largest of sh_keys[0 .. num_samples): 11 + 11 + 10 bits
+  // sample_rank-th largest of sh_keys[0 .. num_samples), resolved to its top 22 bits: the threshold only has
+  // to lie at or below that order statistic, so the low 10 bits are left at zero
   uint32_t need = (uint32_t)sample_rank, prefix = 0;
   int fixed = 0;
-  while (fixed < 32) {
-    const int bits = 32 - fixed >= kHistBits ? kHistBits : 32 - fixed;
+  while (fixed < 2 * kHistBits) {
+    const int bits = kHistBits;
     const int shift = 32 - fixed - bits;
     __syncthreads();
     sh_hist[2 * tid] = 0;
@@ -226,7 +241,8 @@ __global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, i
     prefix = (prefix << bits) | sh_res[0];
     fixed += bits;
   }
-  if (tid == 0) p.tau_key_out[seg] = prefix;
+  prefix <<= (32 - fixed);
+  if (tid == 0) p.tau_key_out[seg * kTauSplit + quarter] = prefix;
 }
 
 }  // namespace
@@ -246,7 +262,7 @@ int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
 }
 
 int launch_sample_tau(const GemvParams& p, int dtype, int num_samples, int sample_rank, hipStream_t stream) {
-  const unsigned segs = (unsigned)(p.batch * p.num_kv_heads * p.num_chunks);
+  const dim3 segs(kTauSplit, (unsigned)(p.batch * p.num_kv_heads * p.num_chunks));
   LaunchTimer timer("sample_tau", stream);
   if (dtype == TKA_F16)
     sample_tau_kernel<TKA_F16><<<segs, kTauThreads, 0, stream>>>(p, num_samples, sample_rank);
@@ -263,20 +279,27 @@ int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len) {
   return total_rows <= 65536 ? 128 : kGemvCandTokensPerWg;
 }
 
-// Candidate-mode plan for one segment length and k: number of samples and the rank of the order statistic
-// used as threshold, or 0 samples when pruning does not pay (short segments, k a large share of the segment).
-// With s samples the number of true top-k members among them is about Binomial(s, k/n): mean m = k*s/n.
-// Rank r = m + 6*sqrt(m) + 2 makes "fewer than k tokens pass" a six-sigma event; about n*r/s tokens pass.
-void gemv_candidate_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank) {
+// Candidate-mode plan for one segment length and k: samples per sampling workgroup and the rank of the order
+// statistic each of them takes as its threshold, or 0 samples when pruning does not pay (short segments, k a
+// large share of the segment, more candidates than the selection kernel holds).
+// With S = kTauSplit * s samples in all and m = k*S/n, R = m + 6*sqrt(m) + 2 is the total rank: the share of
+// tokens that pass concentrates around R/S with relative deviation 1/sqrt(R), which puts "fewer than k pass"
+// (the segment is then redone densely) four to five deviations out.  Taking the lowest of the four
+// thresholds passes about a quarter more than R/S.
+void gemv_candidate_plan(int64_t chunk_len, int k, int max_candidates, int* num_samples, int* sample_rank) {
   *num_samples = 0;
   *sample_rank = 0;
   if (chunk_len < 65536 || (int64_t)k * 16 > chunk_len) return;
-  const int s = kGemvMaxSamples;
-  const double m = (double)k * s / (double)chunk_len;
+  int rounds = (int)(chunk_len / 262144);   // more samples on long segments keep the candidate share near k/n
+  rounds = rounds < 1 ? 1 : (rounds > 4 ? 4 : rounds);
+  const int s = kTauRowGroups * kTauUnroll * rounds;
+  const double S = (double)s * kTauSplit;
+  const double m = (double)k * S / (double)chunk_len;
   double root = 0.0;
   while ((root + 1.0) * (root + 1.0) <= m) root += 1.0;   // floor(sqrt(m))
-  const int r = (int)(m + 6.0 * (root + 1.0) + 2.0);
-  if (r * 8 > s) return;  // more than an eighth of the segment would pass: not worth it
+  const int r = ((int)(m + 6.0 * (root + 1.0) + 2.0) + kTauSplit - 1) / kTauSplit;
+  const double expected = (double)chunk_len * r / s * 1.25;
+  if (expected * 1.3 > (double)max_candidates) return;
   *num_samples = s;
   *sample_rank = r;
 }

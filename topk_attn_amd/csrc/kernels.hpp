@@ -26,7 +26,7 @@ struct GemvParams {
 };
 int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream);
 int launch_sample_tau(const GemvParams& p, int dtype, int num_samples, int sample_rank, hipStream_t stream);
-void gemv_candidate_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank);
+void gemv_candidate_plan(int64_t chunk_len, int k, int max_candidates, int* num_samples, int* sample_rank);
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);
 
 // ---- stage 1: selection -----------------------------------------------------------------------
@@ -67,6 +67,9 @@ int launch_select_hist(const SelectParams& p, hipStream_t stream);
 int launch_select(const SelectParams& p, hipStream_t stream);   // filter + finalize
 int launch_select_filter(const SelectParams& p, hipStream_t stream);
 int launch_select_finalize(const SelectParams& p, hipStream_t stream);
+int launch_select_finalize_cand(const SelectParams& p, hipStream_t stream);   // candidate slices -> outputs, or a flag
+int select_cand_max_parts();   // most candidate slices per segment
+int select_cand_capacity();    // most candidates per segment
 
 struct UnionParams {
   const int32_t* idx;     // [num_segments][k]

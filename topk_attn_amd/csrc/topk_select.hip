@@ -32,7 +32,7 @@ namespace {
 constexpr int kSelThreads = 1024;
 constexpr int kSelWaves = kSelThreads / kWave;
 constexpr int kEndsInLds = 4096;   // slice offsets of one segment kept in LDS by the finalize kernel
-constexpr int kEntryCache = 8;     // listed entries per thread kept in registers by the finalize kernel
+constexpr int kEntryCache = 16;    // listed entries per thread kept in registers by the finalize kernel
 
 // ---- block-wide helpers (1024 threads, 2048 bins) ---------------------------------------------
 
@@ -259,6 +259,44 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams
   if (tid == 0) p.list_cnt[(int64_t)seg * p.parts + part] = total;
 }
 
+
+// Union list of one segment outside the selected middle part: the sink ids, the local window behind
+// `mid` selected ids, -1 padding, and the count.
+__device__ __forceinline__ void write_union_edges(int32_t* uo, const SelectParams& p, int seg, uint32_t lo, uint32_t hi, uint32_t mid) {
+  const int tid = threadIdx.x;
+  const int64_t n = p.seg_len;
+  const int cap = p.k + p.sink + p.local;
+  for (uint32_t t = tid; t < lo; t += kSelThreads) uo[t] = (int32_t)t;
+  const uint32_t mid_end = lo + mid;
+  for (int64_t t = (int64_t)hi + tid; t < n; t += kSelThreads) uo[mid_end + (t - hi)] = (int32_t)t;
+  const uint32_t count = mid_end + (uint32_t)(n - hi);
+  for (int i = (int)count + tid; i < cap; i += kSelThreads) uo[i] = -1;
+  if (tid == 0) p.union_count[seg] = (int32_t)count;
+}
+
+// Rank-ordered outputs of one segment from the sorted composites in sh_sort[0 .. k).
+__device__ __forceinline__ void write_rank_outputs(const uint64_t* sh_sort, const SelectParams& p, int seg) {
+  const int tid = threadIdx.x;
+  const uint32_t k = (uint32_t)p.k;
+  const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
+                                           : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
+  int32_t* oi = p.out_idx + (int64_t)seg * p.out_stride;
+  float* ov = p.out_val ? p.out_val + (int64_t)seg * p.out_stride : nullptr;
+  for (uint32_t r = tid; r < k; r += kSelThreads) {
+    uint64_t c = sh_sort[r];
+    oi[r] = (int32_t)(~(uint32_t)c + idx_base);
+    if (ov) ov[r] = key_score((uint32_t)(c >> 32));
+  }
+  if (p.out_expand) {
+    int32_t* oe = p.out_expand + (int64_t)seg * p.k * p.expand;
+    const uint32_t total = k * (uint32_t)p.expand;
+    for (uint32_t e = tid; e < total; e += kSelThreads) {
+      uint32_t jj = e / (uint32_t)p.expand, ii = e % (uint32_t)p.expand;
+      oe[e] = (int32_t)(~(uint32_t)sh_sort[jj] * (uint32_t)p.expand + ii);
+    }
+  }
+}
+
 // Dynamic LDS of select_finalize_kernel (rank mode only): kpad composites (sort buffer), then kpad
 // composites (cross-wave exchange buffer).
 __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectParams p, int kpad) {
@@ -273,11 +311,10 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
   if (p.check_flags && p.seg_flags[seg] == 0) return;  // fallback launch: this segment was already done
-  const bool from_hist = p.hist != nullptr;
 
-  // dense mode: threshold bin, count above it, count inside it
-  uint32_t b1 = 0, n_above = 0, n_bin = 0;
-  if (from_hist) {
+  // threshold bin, count above it, count inside it
+  uint32_t b1, n_above, n_bin;
+  {
     const uint32_t* gh = p.hist + (int64_t)seg * kHistBins;
     sh_hist[2 * tid] = gh[2 * tid];
     sh_hist[2 * tid + 1] = gh[2 * tid + 1];
@@ -305,15 +342,8 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
     }
     __syncthreads();
   }
-  // candidate mode: the lists hold every token above a sampled threshold.  Fewer than k of them (the
-  // estimate was too high) or far too many (ties, skewed data) sends the segment to the dense path.
-  if (!from_hist) {
-    const bool redo = n_listed < k || n_listed > (uint32_t)p.max_entries;
-    if (tid == 0) p.seg_flags[seg] = redo ? 1u : 0u;
-    if (redo) return;
-  }
   const uint32_t* ends = ends_in_lds ? sh_ends : g_ends;
-  const uint32_t n_entries = n_listed;  // dense mode: == n_above + n_bin
+  const uint32_t n_entries = n_listed;  // == n_above + n_bin
   const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
   // entry v of the segment: slice s with ends[s-1] <= v < ends[s], position v - ends[s-1] in that slice
   auto fetch = [&](uint32_t v) -> uint64_t {
@@ -335,13 +365,11 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   auto entry = [&](uint32_t v) -> uint64_t { return fetch(v); };
 
   // Refine inside bin b1: the listed entries of that bin share their top 11 bits.  Take `need` of them.
-  // (candidate mode starts from scratch: no bit fixed, k to take.)
-  uint32_t need = from_hist ? k - n_above : k;   // >= 1
-  uint64_t prefix = from_hist ? b1 : 0;          // value of the bits fixed so far
-  int fixed = from_hist ? kHistBits : 0;         // number of top bits fixed
-  uint64_t threshold = 0;                        // selected: composite >= threshold
-  bool done = from_hist ? (need == n_bin) : (need == n_entries);   // whole bin / whole list taken
-  if (done && from_hist) threshold = (uint64_t)b1 << (64 - kHistBits);
+  uint32_t need = k - n_above;   // >= 1
+  uint64_t prefix = b1;          // value of the bits fixed so far
+  int fixed = kHistBits;         // number of top bits fixed
+  bool done = need == n_bin;     // whole bin taken
+  uint64_t threshold = (uint64_t)b1 << (64 - kHistBits);   // selected: composite >= threshold
   while (!done) {
     const int bits = (64 - fixed) >= kHistBits ? kHistBits : (64 - fixed);
     const int shift = 64 - fixed - bits;
@@ -352,12 +380,12 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
 #pragma unroll
     for (int i = 0; i < kEntryCache; ++i) {
       const uint64_t c = cache[i];
-      if ((uint32_t)i * kSelThreads + tid < n_entries && (fixed == 0 || (c >> (64 - fixed)) == prefix))
+      if ((uint32_t)i * kSelThreads + tid < n_entries && (c >> (64 - fixed)) == prefix)
         atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
     }
     for (uint32_t v = kEntryCache * kSelThreads + tid; v < n_entries; v += kSelThreads) {
       const uint64_t c = entry(v);
-      if (fixed == 0 || (c >> (64 - fixed)) == prefix) atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
+      if ((c >> (64 - fixed)) == prefix) atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
     }
     __syncthreads();
     find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
@@ -409,37 +437,213 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
       run_mid += total;
     }
   }
-  if (want_union) {
-    const int cap = p.k + p.sink + p.local;
-    for (uint32_t t = tid; t < lo; t += kSelThreads) uo[t] = (int32_t)t;
-    const uint32_t mid_end = lo + run_mid;
-    for (int64_t t = (int64_t)hi + tid; t < n; t += kSelThreads) uo[mid_end + (t - hi)] = (int32_t)t;
-    const uint32_t count = mid_end + (uint32_t)(n - hi);
-    for (int i = (int)count + tid; i < cap; i += kSelThreads) uo[i] = -1;
-    if (tid == 0) p.union_count[seg] = (int32_t)count;
-  }
+  if (want_union) write_union_edges(uo, p, seg, lo, hi, run_mid);
   if (!want_rank) return;
   __syncthreads();
 
   sort_lds_desc(sh_sort, sh_xchg, kpad);
+  write_rank_outputs(sh_sort, p, seg);
+}
 
-  const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
-                                           : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
-  int32_t* oi = p.out_idx + (int64_t)seg * p.out_stride;
-  float* ov = p.out_val ? p.out_val + (int64_t)seg * p.out_stride : nullptr;
-  for (uint32_t r = tid; r < k; r += kSelThreads) {
-    uint64_t c = sh_sort[r];
-    oi[r] = (int32_t)(~(uint32_t)c + idx_base);
-    if (ov) ov[r] = key_score((uint32_t)(c >> 32));
+// ---- finalize of the candidate mode -------------------------------------------------------------
+
+constexpr int kCandCap = 16384;    // candidates of one segment held in LDS (128 KB of composites)
+constexpr int kCandPerThread = kCandCap / kSelThreads;
+constexpr int kCandMaxParts = 4096;
+constexpr int kSmallBucket = 64;   // a threshold bucket of this many entries or fewer is ranked by one wave
+
+// Candidate mode: the slices hold every token whose key reached the sampled threshold, ascending in token
+// index inside and across slices.  One workgroup per segment copies them into LDS (entry v of the segment
+// at position v), finds the k-th largest composite by radix passes that start below the common prefix of
+// the smallest and largest candidate, and walks the entries once in index order.
+// A segment with fewer than k candidates, or more than fit, is flagged for the dense kernels instead.
+// Dynamic LDS: kCandCap composites; rank mode reuses them as sort and exchange buffers.
+__global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(SelectParams p, int kpad) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint64_t* sh_ent = (uint64_t*)smem;
+  __shared__ uint32_t sh_hist[kHistBins];
+  __shared__ uint32_t sh_ends[kCandMaxParts];
+  __shared__ uint32_t sh_wtot[kSelWaves];
+  __shared__ uint32_t sh_res[4];
+  __shared__ uint64_t sh_wmin[kSelWaves], sh_wmax[kSelWaves];
+  __shared__ uint64_t sh_small[kSmallBucket];
+  __shared__ uint32_t sh_small_cnt;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int seg = blockIdx.x;
+  const uint32_t k = (uint32_t)p.k;
+
+  // slice counts -> inclusive offsets
+  const uint32_t* g_cnt = p.list_cnt + (int64_t)seg * p.parts;
+  uint32_t n_entries = 0;
+  for (int base = 0; base < p.parts; base += kSelThreads) {
+    const int i = base + tid;
+    const uint32_t c = i < p.parts ? g_cnt[i] : 0u;
+    uint32_t total;
+    const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
+    if (i < p.parts) sh_ends[i] = n_entries + ex + c;
+    n_entries += total;
   }
-  if (p.out_expand) {
-    int32_t* oe = p.out_expand + (int64_t)seg * p.k * p.expand;
-    const uint32_t total = k * (uint32_t)p.expand;
-    for (uint32_t e = tid; e < total; e += kSelThreads) {
-      uint32_t jj = e / (uint32_t)p.expand, ii = e % (uint32_t)p.expand;
-      oe[e] = (int32_t)(~(uint32_t)sh_sort[jj] * (uint32_t)p.expand + ii);
+  const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
+  const bool redo = n_entries < k || n_entries > cap;
+  if (tid == 0) {
+    p.seg_flags[seg] = redo ? 1u : 0u;
+    sh_small_cnt = 0;
+  }
+  if (redo) return;
+  __syncthreads();
+
+  // copy the slices into LDS: 16 lanes per slice, 8 slices in flight per lane group
+  {
+    const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
+    const int sub = tid & 15, grp = tid >> 4;
+    constexpr int kGroups = kSelThreads / 16, kInFlight = 8;
+    for (int s0 = 0; s0 < p.parts; s0 += kGroups * kInFlight) {
+      uint64_t first[kInFlight];
+      uint32_t start[kInFlight], cnt[kInFlight];
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const int sl = s0 + u * kGroups + grp;
+        start[u] = cnt[u] = 0;
+        first[u] = 0;
+        if (sl < p.parts) {
+          start[u] = sl ? sh_ends[sl - 1] : 0u;
+          cnt[u] = sh_ends[sl] - start[u];
+          if ((uint32_t)sub < cnt[u]) first[u] = lists[(int64_t)sl * p.part_len + sub];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        if ((uint32_t)sub < cnt[u]) sh_ent[start[u] + sub] = first[u];
+        if (cnt[u] > 16u) {
+          const int sl = s0 + u * kGroups + grp;
+          for (uint32_t j = 16u + sub; j < cnt[u]; j += 16u) sh_ent[start[u] + j] = lists[(int64_t)sl * p.part_len + j];
+        }
+      }
     }
   }
+  __syncthreads();
+
+  // this thread's share for the radix passes: entries tid, tid + 1024, ...
+  uint64_t mine[kCandPerThread];
+  uint64_t cmin = ~0ull, cmax = 0ull;
+#pragma unroll
+  for (int i = 0; i < kCandPerThread; ++i) {
+    const uint32_t v = (uint32_t)i * kSelThreads + tid;
+    const bool ok = v < n_entries;
+    mine[i] = ok ? sh_ent[v] : 0ull;
+    if (ok) {
+      cmin = mine[i] < cmin ? mine[i] : cmin;
+      cmax = mine[i] > cmax ? mine[i] : cmax;
+    }
+  }
+
+  uint64_t threshold = 0;   // selected: composite >= threshold
+  if (n_entries > k) {
+    // common prefix of all candidates: the passes start below it
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const uint64_t a = __shfl_xor(cmin, d, 64), b = __shfl_xor(cmax, d, 64);
+      cmin = a < cmin ? a : cmin;
+      cmax = b > cmax ? b : cmax;
+    }
+    if (lane == 0) { sh_wmin[wave] = cmin; sh_wmax[wave] = cmax; }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kSelWaves; ++w) {
+      const uint64_t a = sh_wmin[w], b = sh_wmax[w];
+      cmin = a < cmin ? a : cmin;
+      cmax = b > cmax ? b : cmax;
+    }
+    int fixed = __builtin_clzll(cmin ^ cmax);            // composites are distinct and n_entries >= 2: < 64
+    uint64_t prefix = fixed ? cmax >> (64 - fixed) : 0ull;
+    uint32_t need = k;
+    bool done = false;
+    while (!done) {
+      const int bits = (64 - fixed) >= kHistBits ? kHistBits : (64 - fixed);
+      const int shift = 64 - fixed - bits;
+      __syncthreads();
+      sh_hist[2 * tid] = 0;
+      sh_hist[2 * tid + 1] = 0;
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < kCandPerThread; ++i) {
+        const uint64_t c = mine[i];
+        if ((uint32_t)i * kSelThreads + tid < n_entries && (fixed == 0 || (c >> (64 - fixed)) == prefix))
+          atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
+      }
+      __syncthreads();
+      find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
+      const uint32_t d = sh_res[0], gt = sh_res[1], cnt = sh_res[2];
+      need -= gt;
+      prefix = (prefix << bits) | d;
+      fixed += bits;
+      if (cnt == need || fixed == 64) {
+        threshold = fixed == 64 ? prefix : (prefix << (64 - fixed));
+        done = true;
+      } else if (cnt <= (uint32_t)kSmallBucket) {
+        // few entries left in the threshold bucket: every wave ranks them and picks the need-th largest
+#pragma unroll
+        for (int i = 0; i < kCandPerThread; ++i) {
+          const uint64_t c = mine[i];
+          if ((uint32_t)i * kSelThreads + tid < n_entries && (c >> (64 - fixed)) == prefix) sh_small[atomicAdd(&sh_small_cnt, 1u)] = c;
+        }
+        __syncthreads();
+        const uint64_t e = (uint32_t)lane < cnt ? sh_small[lane] : 0ull;
+        uint32_t greater = 0;
+        for (uint32_t j = 0; j < cnt; ++j) greater += sh_small[j] > e ? 1u : 0u;
+        const uint64_t hit = __ballot((uint32_t)lane < cnt && greater == need - 1u);
+        threshold = __shfl(e, (int)__builtin_ctzll(hit), 64);
+        done = true;
+      }
+    }
+  }
+
+  // Walk in index order: thread t takes the run of `per` consecutive entries starting at t*per.
+  const bool want_rank = p.out_idx != nullptr;
+  const bool want_union = p.union_idx != nullptr;
+  const int64_t n = p.seg_len;
+  const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
+  const uint32_t hi = (uint32_t)(n - p.local > lo ? n - p.local : lo);
+  const uint32_t per = (n_entries + kSelThreads - 1) / kSelThreads;
+  uint64_t run[kCandPerThread];
+  uint32_t sel_mask = 0, mid_mask = 0;
+#pragma unroll
+  for (int i = 0; i < kCandPerThread; ++i) {
+    const uint32_t v = (uint32_t)tid * per + i;
+    const bool ok = (uint32_t)i < per && v < n_entries;
+    run[i] = ok ? sh_ent[v] : 0ull;
+    const bool sel = ok && run[i] >= threshold;
+    const uint32_t idx = ~(uint32_t)run[i];
+    sel_mask |= (sel ? 1u : 0u) << i;
+    mid_mask |= (sel && idx >= lo && idx < hi ? 1u : 0u) << i;
+  }
+  // one scan for both counts (each total is at most 16384)
+  uint32_t totals;
+  const uint32_t ex = block_exclusive_scan(((uint32_t)__builtin_popcount(sel_mask) << 16) | (uint32_t)__builtin_popcount(mid_mask), sh_wtot, &totals);
+  if (want_union) {
+    int32_t* uo = p.union_idx + (int64_t)seg * (p.k + p.sink + p.local);
+    uint32_t pos = lo + (ex & 0xffffu);
+#pragma unroll
+    for (int i = 0; i < kCandPerThread; ++i)
+      if (mid_mask >> i & 1u) uo[pos++] = (int32_t)~(uint32_t)run[i];
+    write_union_edges(uo, p, seg, lo, hi, totals & 0xffffu);
+  }
+  if (!want_rank) return;
+  uint64_t* sh_sort = sh_ent;
+  uint64_t* sh_xchg = sh_ent + kpad;
+  __syncthreads();   // every thread holds its run in registers: the entries may be overwritten
+  {
+    uint32_t pos = ex >> 16;
+#pragma unroll
+    for (int i = 0; i < kCandPerThread; ++i)
+      if (sel_mask >> i & 1u) sh_sort[pos++] = run[i];
+    for (int i = (int)k + tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite
+  }
+  __syncthreads();
+  sort_lds_desc(sh_sort, sh_xchg, kpad);
+  write_rank_outputs(sh_sort, p, seg);
 }
 
 // Ascending duplicate-free union of the selected ids with [0,sink) and [n-local,n).
@@ -516,7 +720,7 @@ int kpad_for(int k) {
 }  // namespace
 
 // Workspace layout (each part 256-byte aligned):
-//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S] u32 | list_cnt [S][slices] u32 |
+//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S][4] u32 | list_cnt [S][slices] u32 |
 //   list [S][slices*slice_len] u64      (slices: dense 4096/16384 scores, candidate mode one per GEMV workgroup)
 namespace {
 struct SelectLayout {
@@ -531,7 +735,7 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   l.list_stride = (seg_len + 16 * kSelThreads - 1) / (16 * kSelThreads) * (16 * kSelThreads);  // whole slices
   l.hist = take((size_t)num_segments * kHistBins * sizeof(uint32_t));
   l.flags = take((size_t)num_segments * sizeof(uint32_t));
-  l.tau = take((size_t)num_segments * sizeof(uint32_t));
+  l.tau = take((size_t)num_segments * 4 * sizeof(uint32_t));   // one threshold per sampled quarter
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
   l.total = off;
@@ -604,8 +808,25 @@ int launch_select_finalize(const SelectParams& p, hipStream_t stream) {
   const int kpad = kpad_for(p.k);
   const size_t lds = want_rank ? 2 * (size_t)kpad * sizeof(uint64_t) : 0;
   if (set_finalize_attr() != TKA_OK) return TKA_EHIP;
-  LaunchTimer timer(p.check_flags ? "select_finalize_fallback" : (p.hist ? "select_finalize" : "select_finalize_cand"), stream);
+  LaunchTimer timer(p.check_flags ? "select_finalize_fallback" : "select_finalize", stream);
   select_finalize_kernel<<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(p, kpad);
+  return hip_status(hipGetLastError());
+}
+
+int select_cand_max_parts() { return kCandMaxParts; }
+int select_cand_capacity() { return kCandCap; }
+
+int launch_select_finalize_cand(const SelectParams& p, hipStream_t stream) {
+  if (p.parts > kCandMaxParts || p.k > kCandCap / 2) return TKA_EINVAL;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_cand_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       kCandCap * (int)sizeof(uint64_t));
+    if (e != hipSuccess) return TKA_EHIP;
+    attr_set = true;
+  }
+  LaunchTimer timer("select_finalize_cand", stream);
+  select_finalize_cand_kernel<<<(unsigned)p.num_segments, kSelThreads, kCandCap * sizeof(uint64_t), stream>>>(p, kpad_for(p.k));
   return hip_status(hipGetLastError());
 }
 
