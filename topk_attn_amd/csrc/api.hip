@@ -129,7 +129,6 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->cand = nullptr;
   g->cand_seg_stride = 0;
   g->cand_cnt = nullptr;
-  g->seg_flags = nullptr;
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   g->tokens_per_wg = gemv_tokens_per_wg(rows, g->chunk_len);
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
@@ -192,17 +191,17 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   }
 
   // Long segments: sampled threshold, GEMV that stores candidates only, selection straight from the
-  // candidate slices.  A segment whose candidates turn out too few (or far too many) is flagged and redone
-  // by the dense kernels, which otherwise exit at once.
+  // candidate slices.  A segment whose candidates turn out too few (or too many) is flagged and redone
+  // by the fallback kernel, which otherwise exits at once.
   GemvParams cp = gp;
+  cp.hist = nullptr;
   cp.tau_key_out = sp.tau_key;
-  int rc = launch_sample_tau(cp, a->dtype, num_samples, sample_rank, stream);   // also clears the histograms
+  int rc = launch_sample_tau(cp, a->dtype, num_samples, sample_rank, stream);
   if (rc != TKA_OK) return rc;
   cp.tau_key = sp.tau_key;
   cp.cand = sp.list;
   cp.cand_seg_stride = sp.list_stride;
   cp.cand_cnt = sp.list_cnt;
-  cp.hist = nullptr;
   rc = launch_gemv_scores(cp, a->dtype, stream);
   if (rc != TKA_OK) return rc;
   SelectParams sc = sp;
@@ -213,14 +212,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   sc.max_entries = select_cand_capacity();
   rc = launch_select_finalize_cand(sc, stream);
   if (rc != TKA_OK) return rc;
-  // dense fallback for flagged segments: long runs per workgroup keep the (normally idle) grids small
-  gp.seg_flags = sp.seg_flags;
-  gp.tokens_per_wg = 4096;
-  gp.wgs_per_chunk = (int)((chunk_len + gp.tokens_per_wg - 1) / gp.tokens_per_wg);
-  rc = launch_gemv_scores(gp, a->dtype, stream);
-  if (rc != TKA_OK) return rc;
-  sp.check_flags = 1;
-  return launch_select(sp, stream);
+  // flagged segments are redone by one workgroup each; the launch is idle otherwise
+  return launch_select_fallback(gp, sp, a->dtype, stream);
 }
 
 int check_flash(const tka_flash_decode_args* a) {

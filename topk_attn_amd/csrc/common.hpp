@@ -107,6 +107,31 @@ struct Elem<TKA_BF16> {
   }
 };
 
+// ---- canonical row score (gemv_topk.cu:303-332) ------------------------------------------------
+
+// Group query of this lane in fp32: ((q0 + q1) + q2) + ... in ascending head order, dims 8j..8j+7.
+template <int DT>
+__device__ __forceinline__ void load_group_query(const void* q, int64_t q_stride_b, int b, int h, int group, int j, float (&qf)[8]) {
+  const uint16_t* qb = (const uint16_t*)q + (int64_t)b * q_stride_b + (int64_t)h * group * kHeadDim + 8 * j;
+  u32x4 v = *(const u32x4*)qb;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) qf[i] = Elem<DT>::get(v, i);
+  for (int g = 1; g < group; ++g) {
+    u32x4 w = *(const u32x4*)(qb + (int64_t)g * kHeadDim);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] = qf[i] + Elem<DT>::get(w, i);
+  }
+}
+
+// Canonical score of the row in `kv` for the lane's 8 dims: fma chain, DPP butterfly, one multiply.
+template <int DT>
+__device__ __forceinline__ float row_score(const float (&qf)[8], const u32x4& kv, float scale) {
+  float acc = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc = __builtin_fmaf(qf[i], Elem<DT>::get(kv, i), acc);
+  return row16_sum(acc) * scale;
+}
+
 // ---- score key --------------------------------------------------------------------------------
 
 // Order-preserving fp32 -> uint32 (bigger score, bigger key); -0.0 == +0.0; NaN is the lowest key.

@@ -30,29 +30,6 @@ constexpr int kCandMaxIters = kGemvCandTokensPerWg / kGemvRowsPerIter; // iterat
 constexpr int kCandSubLists = kCandMaxIters * kGemvWaves;
 constexpr int kTauSplit = 4;   // sample workgroups (and thresholds) per segment
 
-// Group query of this lane in fp32: ((q0 + q1) + q2) + ... in ascending head order, dims 8j..8j+7.
-template <int DT>
-__device__ __forceinline__ void load_group_query(const void* q, int64_t q_stride_b, int b, int h, int group, int j, float (&qf)[8]) {
-  const uint16_t* qb = (const uint16_t*)q + (int64_t)b * q_stride_b + (int64_t)h * group * kHeadDim + 8 * j;
-  u32x4 v = *(const u32x4*)qb;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) qf[i] = Elem<DT>::get(v, i);
-  for (int g = 1; g < group; ++g) {
-    u32x4 w = *(const u32x4*)(qb + (int64_t)g * kHeadDim);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) qf[i] = qf[i] + Elem<DT>::get(w, i);
-  }
-}
-
-// Canonical score of the row in `kv` for the lane's 8 dims: fma chain, DPP butterfly, one multiply.
-template <int DT>
-__device__ __forceinline__ float row_score(const float (&qf)[8], const u32x4& kv, float scale) {
-  float acc = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) acc = __builtin_fmaf(qf[i], Elem<DT>::get(kv, i), acc);
-  return row16_sum(acc) * scale;
-}
-
 template <int DT, bool CAND>
 __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p) {
   __shared__ uint32_t sh_hist[CAND ? 1 : kHistBins];
@@ -67,7 +44,6 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
   const int chunk = blockIdx.x / p.wgs_per_chunk;
   const int wg_in_chunk = blockIdx.x % p.wgs_per_chunk;
   const int64_t seg = ((int64_t)b * p.num_kv_heads + h) * p.num_chunks + chunk;
-  if (p.seg_flags && p.seg_flags[seg] == 0) return;  // fallback launch: this segment needs nothing
   // tokens are counted inside the chunk; the chunk starts at chunk*chunk_len, or at the start of the
   // cluster chosen for this (head, rank) in two-level selection
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
@@ -188,12 +164,6 @@ __global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, i
   const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
 
-  // the dense fallback, should this segment need it, finds its histogram cleared
-  if (p.hist && quarter == 0) {
-    p.hist[(int64_t)seg * kHistBins + 2 * tid] = 0u;
-    p.hist[(int64_t)seg * kHistBins + 2 * tid + 1] = 0u;
-  }
-
   float qf[8];
   load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
@@ -250,7 +220,7 @@ __global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, i
 int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
   dim3 grid((unsigned)(p.num_chunks * p.wgs_per_chunk), (unsigned)p.num_kv_heads, (unsigned)p.batch);
   const bool cand = p.cand != nullptr;
-  LaunchTimer timer(cand ? "gemv_scores_cand" : (p.seg_flags ? "gemv_scores_fallback" : "gemv_scores"), stream);
+  LaunchTimer timer(cand ? "gemv_scores_cand" : "gemv_scores", stream);
   if (dtype == TKA_F16) {
     if (cand) gemv_scores_kernel<TKA_F16, true><<<grid, kGemvThreads, 0, stream>>>(p);
     else gemv_scores_kernel<TKA_F16, false><<<grid, kGemvThreads, 0, stream>>>(p);
@@ -290,8 +260,7 @@ void gemv_candidate_plan(int64_t chunk_len, int k, int max_candidates, int* num_
   *num_samples = 0;
   *sample_rank = 0;
   if (chunk_len < 65536 || (int64_t)k * 16 > chunk_len) return;
-  int rounds = (int)(chunk_len / 262144);   // more samples on long segments keep the candidate share near k/n
-  rounds = rounds < 1 ? 1 : (rounds > 4 ? 4 : rounds);
+  const int rounds = chunk_len >= 1048576 ? 4 : (chunk_len >= 524288 ? 2 : 1);   // more samples on long segments keep the candidate share near k/n
   const int s = kTauRowGroups * kTauUnroll * rounds;
   const double S = (double)s * kTauSplit;
   const double m = (double)k * S / (double)chunk_len;

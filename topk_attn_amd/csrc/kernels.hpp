@@ -8,7 +8,7 @@ namespace tka {
 struct GemvParams {
   const void* q;        // [batch][num_kv_heads*group][128]
   const void* keys;
-  float* scores;        // [batch][num_kv_heads][num_chunks][chunk_len]
+  float* scores;        // [batch][num_kv_heads][num_chunks][chunk_len]; selection kernels also read them
   const int32_t* cluster_ids;  // [batch*num_kv_heads*num_chunks] or nullptr: chunk c covers the tokens of that cluster
   uint32_t* hist;       // [batch*num_kv_heads*num_chunks][kHistBins] or nullptr; must be zero on entry
   // candidate mode (cand != nullptr): only tokens with key >= tau_key[segment] are stored
@@ -17,7 +17,6 @@ struct GemvParams {
   uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] composites, one slice per workgroup, ascending index
   int64_t cand_seg_stride;    // entries between the slice arrays of consecutive segments
   uint32_t* cand_cnt;         // [segments][wgs_per_chunk] entries in each slice
-  const uint32_t* seg_flags;  // nullptr, or [segments]: workgroups of segments whose flag is 0 exit at once
   int64_t chunk_len;    // tokens per chunk
   int64_t q_stride_b, key_stride_b, key_stride_n, key_stride_h;
   int batch, num_kv_heads, group, num_chunks;
@@ -36,10 +35,8 @@ struct SelectParams {
   int64_t seg_stride;
   uint32_t* hist;         // [num_segments][kHistBins]; nullptr: the lists hold candidates above a sampled threshold
   uint32_t* tau_key;      // [num_segments] candidate threshold (workspace)
-  uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment must be redone densely;
-                          // fallback launches (check_flags) skip segments whose flag is 0
-  int check_flags;
-  int max_entries;        // candidate mode: more listed entries than this also sends the segment to the dense path
+  uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment must be redone by the fallback kernel
+  int max_entries;        // candidate mode: more listed entries than this also sends the segment to the fallback kernel
   uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)
   uint64_t* list;         // [num_segments][list_stride] composites with bin >= threshold bin, slice p at p*part_len
   int64_t list_stride;
@@ -68,6 +65,8 @@ int launch_select(const SelectParams& p, hipStream_t stream);   // filter + fina
 int launch_select_filter(const SelectParams& p, hipStream_t stream);
 int launch_select_finalize(const SelectParams& p, hipStream_t stream);
 int launch_select_finalize_cand(const SelectParams& p, hipStream_t stream);   // candidate slices -> outputs, or a flag
+// One workgroup per flagged segment redoes scores and selection on its own; the others exit at once.
+int launch_select_fallback(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
 int select_cand_max_parts();   // most candidate slices per segment
 int select_cand_capacity();    // most candidates per segment
 

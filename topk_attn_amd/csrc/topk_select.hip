@@ -24,123 +24,16 @@
 #include <stdlib.h>
 
 #include "kernels.hpp"
+#include "bitonic.hpp"
 
 namespace tka {
 
 namespace {
 
-constexpr int kSelThreads = 1024;
+constexpr int kSelThreads = kSortThreads;
 constexpr int kSelWaves = kSelThreads / kWave;
 constexpr int kEndsInLds = 4096;   // slice offsets of one segment kept in LDS by the finalize kernel
 constexpr int kEntryCache = 16;    // listed entries per thread kept in registers by the finalize kernel
-
-// ---- block-wide helpers (1024 threads, 2048 bins) ---------------------------------------------
-
-// ---- bitonic sort of 1024*E composites, descending --------------------------------------------
-
-// One compare-exchange stage whose partner sits M lanes away.  keep_max is the same for every element of
-// the thread (the stride and the merge size are multiples of E).  Composites are distinct (equal only
-// among the zero padding), so "partner greater" decides both directions with one 64-bit compare.
-template <int M, int E>
-__device__ __forceinline__ void stage_lanes(uint64_t (&v)[E], bool keep_max) {
-#pragma unroll
-  for (int s = 0; s < E; ++s) {
-    const uint64_t o = lane_xor64<M>(v[s]);
-    const bool take = (o > v[s]) == keep_max;
-    v[s] = take ? o : v[s];
-  }
-}
-
-// One compare-exchange stage inside the thread (STRIDE < E).
-template <int STRIDE, int E>
-__device__ __forceinline__ void stage_regs(uint64_t (&v)[E], int first, int size) {
-  if constexpr (STRIDE < E) {
-#pragma unroll
-    for (int s = 0; s < E; ++s) {
-      if ((s & STRIDE) == 0) {
-        const bool desc = ((first + s) & size) == 0;
-        const uint64_t a = v[s], b = v[s ^ STRIDE];
-        const bool sw = (b > a) == desc;
-        v[s] = sw ? b : a;
-        v[s ^ STRIDE] = sw ? a : b;
-      }
-    }
-  }
-}
-
-// Bitonic sort, descending, of N composites held by the first N/E threads of the block (thread t holds
-// elements t*E .. t*E+E-1).  The network is unrolled at compile time: strides inside a thread are
-// register compare-exchanges, strides inside a wave use DPP / ds_swizzle / ds_bpermute, and only strides
-// of 64*E and more go through LDS (`sh`, N entries) with block barriers, which every thread must reach.
-template <int N, int E, int SIZE, int STRIDE>
-__device__ __forceinline__ void bitonic_net(uint64_t (&v)[E], uint64_t* sh, int tid, bool active) {
-  if constexpr (SIZE <= N) {
-    const int e0 = tid * E;
-    if constexpr (STRIDE >= 64 * E) {
-      __syncthreads();
-      if (active) {
-#pragma unroll
-        for (int s = 0; s < E; ++s) sh[e0 + s] = v[s];
-      }
-      __syncthreads();
-      if (active) {
-        const bool keep_max = ((e0 & STRIDE) == 0) == ((e0 & SIZE) == 0);
-#pragma unroll
-        for (int s = 0; s < E; ++s) {
-          const uint64_t o = sh[(e0 + s) ^ STRIDE];
-          const bool take = (o > v[s]) == keep_max;
-          v[s] = take ? o : v[s];
-        }
-      }
-    } else if constexpr (STRIDE >= E) {
-      if (active) {
-        const bool keep_max = ((e0 & STRIDE) == 0) == ((e0 & SIZE) == 0);
-        stage_lanes<STRIDE / E, E>(v, keep_max);
-      }
-    } else {
-      if (active) stage_regs<STRIDE, E>(v, e0, SIZE);
-    }
-    if constexpr (STRIDE > 1)
-      bitonic_net<N, E, SIZE, STRIDE / 2>(v, sh, tid, active);
-    else
-      bitonic_net<N, E, SIZE * 2, SIZE>(v, sh, tid, active);
-  }
-}
-
-// One element per thread up to 1024 (many waves hide the cross-lane latency), then 2, 4, 8 per thread.
-template <int N>
-__device__ __noinline__ void sort_lds_desc_n(uint64_t* sh_sort, uint64_t* sh_xchg) {
-  constexpr int E = N > kSelThreads ? N / kSelThreads : 1;
-  constexpr int NT = N / E;
-  uint64_t v[E];
-  const int tid = threadIdx.x;
-  const bool active = tid < NT;
-  if (active) {
-#pragma unroll
-    for (int s = 0; s < E; ++s) v[s] = sh_sort[tid * E + s];
-  }
-  bitonic_net<N, E, 2, 1>(v, sh_xchg, tid, active);
-  __syncthreads();
-  if (active) {
-#pragma unroll
-    for (int s = 0; s < E; ++s) sh_sort[tid * E + s] = v[s];
-  }
-  __syncthreads();
-}
-
-// Sorts sh_sort[0 .. kpad) descending; kpad is a power of two between 64 and 8192.
-__device__ void sort_lds_desc(uint64_t* sh_sort, uint64_t* sh_xchg, int kpad) {
-  switch (kpad) {
-    case 64: sort_lds_desc_n<64>(sh_sort, sh_xchg); break;
-    case 128: sort_lds_desc_n<128>(sh_sort, sh_xchg); break;
-    case 256: sort_lds_desc_n<256>(sh_sort, sh_xchg); break;
-    case 512: sort_lds_desc_n<512>(sh_sort, sh_xchg); break;
-    case 1024: sort_lds_desc_n<1024>(sh_sort, sh_xchg); break;
-    case 2048: sort_lds_desc_n<2048>(sh_sort, sh_xchg); break;
-    case 4096: sort_lds_desc_n<4096>(sh_sort, sh_xchg); break;
-    default: sort_lds_desc_n<8192>(sh_sort, sh_xchg); break;
-  }
-}
 
 // ---- kernels ----------------------------------------------------------------------------------
 
@@ -230,7 +123,6 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams
   const int tid = threadIdx.x;
   const int seg = blockIdx.y;
   const int part = blockIdx.x;
-  if (p.check_flags && p.seg_flags[seg] == 0) return;  // fallback launch: this segment needs nothing
 
   // this thread's run of scores first: the loads do not depend on the threshold
   const float* sc = p.scores + (int64_t)seg * p.seg_stride;
@@ -310,7 +202,6 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   const int tid = threadIdx.x;
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
-  if (p.check_flags && p.seg_flags[seg] == 0) return;  // fallback launch: this segment was already done
 
   // threshold bin, count above it, count inside it
   uint32_t b1, n_above, n_bin;
@@ -646,6 +537,151 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(Selec
   write_rank_outputs(sh_sort, p, seg);
 }
 
+// ---- fallback of the candidate mode ---------------------------------------------------------------
+
+// One workgroup per segment; all but the flagged segments exit at once, so the launch normally costs its
+// overhead only.  A flagged segment is redone from the keys by its workgroup alone: scores in the canonical
+// order (stored, and a histogram of the top key bits kept in LDS), radix passes over the stored scores until
+// the k-th largest key is fixed, then one walk in index order that takes every key above the threshold
+// bucket and the first `need` keys inside it.  Exact for any data; slow (one CU streams the segment), which
+// is acceptable for an event that the sampling makes rare.
+// Dynamic LDS (rank mode only): kpad composites (sort buffer), then kpad composites (exchange buffer).
+template <int DT>
+__global__ __launch_bounds__(kSelThreads) void select_fallback_kernel(GemvParams g, SelectParams p, int kpad) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint64_t* sh_sort = (uint64_t*)smem;
+  uint64_t* sh_xchg = sh_sort + kpad;
+  __shared__ uint32_t sh_hist[kHistBins];
+  __shared__ uint32_t sh_wtot[kSelWaves];
+  __shared__ uint32_t sh_res[4];
+
+  const int tid = threadIdx.x;
+  const int seg = blockIdx.x;
+  if (p.seg_flags[seg] == 0) return;
+  const uint32_t k = (uint32_t)p.k;
+  const int64_t n = p.seg_len;
+  float* sc = g.scores + (int64_t)seg * p.seg_stride;
+
+  sh_hist[2 * tid] = 0;
+  sh_hist[2 * tid + 1] = 0;
+  __syncthreads();
+
+  // scores of the whole segment: 64 row groups of 16 lanes, 8 rows in flight each
+  {
+    const int j = tid & 15, rg = tid >> 4;
+    const int chunk = seg % g.num_chunks, bh = seg / g.num_chunks;
+    const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
+    const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
+    float qf[8];
+    load_group_query<DT>(g.q, g.q_stride_b, b, h, g.group, j, qf);
+    const uint16_t* kbase = (const uint16_t*)g.keys + (int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h +
+                            chunk_base * g.key_stride_n + 8 * j;
+    constexpr int kRows = 8;
+    for (int64_t base = 0; base < n; base += (kSelThreads / 16) * kRows) {
+      u32x4 kv[kRows];
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        const int64_t t = base + rg * kRows + u;
+        kv[u] = *(const u32x4*)(kbase + (t < n ? t : n - 1) * g.key_stride_n);
+      }
+      float mine = 0.0f;
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        const float s = row_score<DT>(qf, kv[u], g.scale);
+        if (j == u) mine = s;
+      }
+      const int64_t t = base + rg * kRows + j;
+      if (j < kRows && t < n) {
+        sc[t] = mine;
+        atomicAdd(&sh_hist[score_key(mine) >> (32 - kHistBits)], 1u);
+      }
+    }
+  }
+  __syncthreads();   // also orders this workgroup's score stores before its loads below
+
+  // radix passes: `prefix` = value of the top `fixed` key bits of the k-th largest key, `need` = how many
+  // keys of that bucket belong to the top k
+  const bool vec_ok = (((uintptr_t)sc) & 15u) == 0;
+  uint32_t need = k, prefix = 0;
+  int fixed = 0;
+  bool whole = false;   // the bucket is taken whole
+  while (!whole && fixed < 32) {
+    const int bits = (32 - fixed) >= kHistBits ? kHistBits : (32 - fixed);
+    const int shift = 32 - fixed - bits;
+    if (fixed) {
+      __syncthreads();
+      sh_hist[2 * tid] = 0;
+      sh_hist[2 * tid + 1] = 0;
+      __syncthreads();
+      for (int64_t first = (int64_t)tid * 4; first < n; first += 4 * kSelThreads) {
+        uint32_t keys[4], vm;
+        load_keys<4>(sc, first, n, vec_ok, keys, &vm);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if ((vm >> e & 1u) && (keys[e] >> (32 - fixed)) == prefix) atomicAdd(&sh_hist[(keys[e] >> shift) & ((1u << bits) - 1u)], 1u);
+      }
+      __syncthreads();
+    }
+    find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
+    const uint32_t d = sh_res[0], gt = sh_res[1], cnt = sh_res[2];
+    need -= gt;
+    prefix = (prefix << bits) | d;
+    fixed += bits;
+    whole = cnt == need;
+  }
+
+  // walk in index order
+  const bool want_rank = p.out_idx != nullptr;
+  const bool want_union = p.union_idx != nullptr;
+  const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
+  const uint32_t hi = (uint32_t)(n - p.local > lo ? n - p.local : lo);
+  int32_t* uo = want_union ? p.union_idx + (int64_t)seg * (p.k + p.sink + p.local) : nullptr;
+  if (want_rank) {
+    __syncthreads();
+    for (int i = tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite
+  }
+  uint32_t run_bucket = 0, run_sel = 0, run_mid = 0;
+  for (int64_t base = 0; base < n; base += 4 * kSelThreads) {
+    const int64_t first = base + (int64_t)tid * 4;
+    uint32_t keys[4], vm;
+    load_keys<4>(sc, first, n, vec_ok, keys, &vm);
+    uint32_t above = 0, inside = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t top = keys[e] >> (32 - fixed);
+      above |= ((vm >> e & 1u) && top > prefix ? 1u : 0u) << e;
+      inside |= ((vm >> e & 1u) && top == prefix ? 1u : 0u) << e;
+    }
+    uint32_t total;
+    uint32_t rank_in_bucket = run_bucket + block_exclusive_scan((uint32_t)__builtin_popcount(inside), sh_wtot, &total);
+    run_bucket += total;
+    uint32_t sel = above, mid = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (inside >> e & 1u) {
+        sel |= (rank_in_bucket < need ? 1u : 0u) << e;
+        ++rank_in_bucket;
+      }
+      const uint32_t idx = (uint32_t)(first + e);
+      mid |= ((sel >> e & 1u) && idx >= lo && idx < hi ? 1u : 0u) << e;
+    }
+    const uint32_t ex = block_exclusive_scan(((uint32_t)__builtin_popcount(sel) << 16) | (uint32_t)__builtin_popcount(mid), sh_wtot, &total);
+    uint32_t pos_sel = run_sel + (ex >> 16), pos_mid = lo + run_mid + (ex & 0xffffu);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (want_rank && (sel >> e & 1u)) sh_sort[pos_sel++] = composite(keys[e], (uint32_t)(first + e));
+      if (want_union && (mid >> e & 1u)) uo[pos_mid++] = (int32_t)(first + e);
+    }
+    run_sel += total >> 16;
+    run_mid += total & 0xffffu;
+  }
+  if (want_union) write_union_edges(uo, p, seg, lo, hi, run_mid);
+  if (!want_rank) return;
+  __syncthreads();
+  sort_lds_desc(sh_sort, sh_xchg, kpad);
+  write_rank_outputs(sh_sort, p, seg);
+}
+
 // Ascending duplicate-free union of the selected ids with [0,sink) and [n-local,n).
 // One workgroup per segment; the middle part is sorted ascending with the same bitonic network
 // (ids complemented so that "descending" composites are ascending ids).
@@ -794,7 +830,7 @@ static int set_finalize_attr() {
 }
 
 int launch_select_filter(const SelectParams& p, hipStream_t stream) {
-  LaunchTimer timer(p.check_flags ? "select_filter_fallback" : "select_filter", stream);
+  LaunchTimer timer("select_filter", stream);
   const dim3 grid((unsigned)p.parts, (unsigned)p.num_segments);
   if (p.part_len == 16 * kSelThreads)
     select_filter_kernel<16><<<grid, kSelThreads, 0, stream>>>(p);
@@ -808,7 +844,7 @@ int launch_select_finalize(const SelectParams& p, hipStream_t stream) {
   const int kpad = kpad_for(p.k);
   const size_t lds = want_rank ? 2 * (size_t)kpad * sizeof(uint64_t) : 0;
   if (set_finalize_attr() != TKA_OK) return TKA_EHIP;
-  LaunchTimer timer(p.check_flags ? "select_finalize_fallback" : "select_finalize", stream);
+  LaunchTimer timer("select_finalize", stream);
   select_finalize_kernel<<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(p, kpad);
   return hip_status(hipGetLastError());
 }
@@ -827,6 +863,26 @@ int launch_select_finalize_cand(const SelectParams& p, hipStream_t stream) {
   }
   LaunchTimer timer("select_finalize_cand", stream);
   select_finalize_cand_kernel<<<(unsigned)p.num_segments, kSelThreads, kCandCap * sizeof(uint64_t), stream>>>(p, kpad_for(p.k));
+  return hip_status(hipGetLastError());
+}
+
+int launch_select_fallback(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
+  const bool want_rank = p.out_idx != nullptr;
+  const int kpad = kpad_for(p.k);
+  const size_t lds = want_rank ? 2 * (size_t)kpad * sizeof(uint64_t) : 0;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)select_fallback_kernel<TKA_F16>, hipFuncAttributeMaxDynamicSharedMemorySize, 130 * 1024);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)select_fallback_kernel<TKA_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, 130 * 1024);
+    if (e != hipSuccess) return TKA_EHIP;
+    attr_set = true;
+  }
+  LaunchTimer timer("select_fallback", stream);
+  if (dtype == TKA_F16)
+    select_fallback_kernel<TKA_F16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad);
+  else
+    select_fallback_kernel<TKA_BF16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad);
   return hip_status(hipGetLastError());
 }
 
