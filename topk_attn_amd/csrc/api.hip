@@ -128,7 +128,6 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->tau_key_out = nullptr;
   g->cand = nullptr;
   g->cand_seg_stride = 0;
-  g->cand_cnt = nullptr;
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   g->tokens_per_wg = gemv_tokens_per_wg(rows, g->chunk_len);
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
@@ -201,7 +200,6 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   cp.tau_key = sp.tau_key;
   cp.cand = sp.list;
   cp.cand_seg_stride = sp.list_stride;
-  cp.cand_cnt = sp.list_cnt;
   rc = launch_gemv_scores(cp, a->dtype, stream);
   if (rc != TKA_OK) return rc;
   SelectParams sc = sp;

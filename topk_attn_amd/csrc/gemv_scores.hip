@@ -13,9 +13,10 @@
 //              and callers that want all scores);
 //   candidate  a threshold tau per segment is known beforehand (sample_tau_kernel: an order statistic of a
 //              strided sample of the segment, chosen so that about 2k tokens pass); only tokens with
-//              key >= tau are stored, in index order, in the workgroup's own slice.  The selection kernel
-//              checks that at least k tokens passed and otherwise flags the segment for the dense path,
-//              so the result is exact whatever the data.
+//              key >= tau are stored, in index order, in the workgroup's own slice (the count rides in the
+//              first entry: one partial line per workgroup).  The selection kernel checks that at least k
+//              tokens passed and otherwise flags the segment for the fallback kernel, so the result is
+//              exact whatever the data.
 #include "kernels.hpp"
 
 namespace tka {
@@ -115,10 +116,16 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
       before += s < sub ? c : 0u;
       total += c;
     }
-    const int64_t slice = seg * p.wgs_per_chunk + wg_in_chunk;
-    if (sub < kCandSubLists && (uint32_t)r < sh_ccnt[sub])
-      p.cand[seg * p.cand_seg_stride + (int64_t)wg_in_chunk * p.tokens_per_wg + before + r] = sh_cand[sub][r];
-    if (tid == 0) p.cand_cnt[slice] = total;
+    // Slice format: word = key << 32 | count << 8 | token - first token of the slice; only slot 0 carries the
+    // count (0 .. 256), so a workgroup with few candidates writes a single line and nothing else
+    uint64_t* slice = p.cand + seg * p.cand_seg_stride + (int64_t)wg_in_chunk * p.tokens_per_wg;
+    if (sub < kCandSubLists && (uint32_t)r < sh_ccnt[sub]) {
+      const uint64_t c = sh_cand[sub][r];
+      const uint32_t pos = before + r;
+      const uint32_t rel = ~(uint32_t)c - (uint32_t)t_begin;
+      slice[pos] = (c & 0xffffffff00000000ull) | (pos == 0 ? total << 8 : 0u) | rel;
+    }
+    if (tid == 0 && total == 0) slice[0] = 0ull;
     return;
   }
 

@@ -14,9 +14,9 @@ struct GemvParams {
   // candidate mode (cand != nullptr): only tokens with key >= tau_key[segment] are stored
   const uint32_t* tau_key;    // [segments]
   uint32_t* tau_key_out;      // [segments], written by the sample kernel
-  uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] composites, one slice per workgroup, ascending index
+  uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] one slice per workgroup, ascending index:
+                              // key << 32 | count << 8 | token offset in the slice (count in entry 0 only)
   int64_t cand_seg_stride;    // entries between the slice arrays of consecutive segments
-  uint32_t* cand_cnt;         // [segments][wgs_per_chunk] entries in each slice
   int64_t chunk_len;    // tokens per chunk
   int64_t q_stride_b, key_stride_b, key_stride_n, key_stride_h;
   int batch, num_kv_heads, group, num_chunks;

@@ -344,8 +344,8 @@ constexpr int kCandMaxParts = 4096;
 constexpr int kSmallBucket = 64;   // a threshold bucket of this many entries or fewer is ranked by one wave
 
 // Candidate mode: the slices hold every token whose key reached the sampled threshold, ascending in token
-// index inside and across slices.  One workgroup per segment copies them into LDS (entry v of the segment
-// at position v), finds the k-th largest composite by radix passes that start below the common prefix of
+// index inside and across slices (format: GemvParams::cand).  One workgroup per segment copies them into LDS
+// as composites (entry v of the segment at position v), finds the k-th largest composite by radix passes that start below the common prefix of
 // the smallest and largest candidate, and walks the entries once in index order.
 // A segment with fewer than k candidates, or more than fit, is flagged for the dense kernels instead.
 // Dynamic LDS: kCandCap composites; rank mode reuses them as sort and exchange buffers.
@@ -353,7 +353,8 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(Selec
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint64_t* sh_ent = (uint64_t*)smem;
   __shared__ uint32_t sh_hist[kHistBins];
-  __shared__ uint32_t sh_ends[kCandMaxParts];
+  constexpr int kGroups = kSelThreads / 16, kInFlight = 8, kRound = kGroups * kInFlight;   // 512 slices per round
+  __shared__ uint32_t sh_cnt[kRound], sh_start[kRound];
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
   __shared__ uint64_t sh_wmin[kSelWaves], sh_wmax[kSelWaves];
@@ -365,55 +366,52 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(Selec
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
 
-  // slice counts -> inclusive offsets
-  const uint32_t* g_cnt = p.list_cnt + (int64_t)seg * p.parts;
+  // Copy the slices into LDS, kRound slices at a time: 16 lanes per slice load its first 16 entries (entry 0
+  // carries the slice's count; entries beyond the count are stale memory and ignored), the counts are
+  // scanned into start positions, and the entries go to their place.  One memory round trip per round.
+  const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
+  const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
+  const int sub = tid & 15, grp = tid >> 4;
   uint32_t n_entries = 0;
-  for (int base = 0; base < p.parts; base += kSelThreads) {
-    const int i = base + tid;
-    const uint32_t c = i < p.parts ? g_cnt[i] : 0u;
+  for (int s0 = 0; s0 < p.parts; s0 += kRound) {
+    uint64_t first[kInFlight];
+    uint32_t cnt[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int sl = s0 + u * kGroups + grp;
+      first[u] = sl < p.parts ? lists[(int64_t)sl * p.part_len + sub] : 0ull;
+    }
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      cnt[u] = ((uint32_t)__shfl((int)(uint32_t)first[u], lane & ~15, 64) >> 8) & 0x1ffu;
+      if (sub == 0) sh_cnt[u * kGroups + grp] = cnt[u];
+    }
+    __syncthreads();
     uint32_t total;
+    const uint32_t c = tid < kRound ? sh_cnt[tid] : 0u;
     const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
-    if (i < p.parts) sh_ends[i] = n_entries + ex + c;
+    if (tid < kRound) sh_start[tid] = n_entries + ex;
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int sl = s0 + u * kGroups + grp;
+      const uint32_t start = sh_start[u * kGroups + grp];
+      const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
+      if ((uint32_t)sub < cnt[u] && start + sub < cap)
+        sh_ent[start + sub] = (first[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)first[u] & 0xffu));
+      for (uint32_t j = 16u + sub; j < cnt[u] && start + j < cap; j += 16u) {   // rare: a slice with more than 16 candidates
+        const uint64_t w = lists[(int64_t)sl * p.part_len + j];
+        sh_ent[start + j] = (w & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w & 0xffu));
+      }
+    }
     n_entries += total;
   }
-  const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
   const bool redo = n_entries < k || n_entries > cap;
   if (tid == 0) {
     p.seg_flags[seg] = redo ? 1u : 0u;
     sh_small_cnt = 0;
   }
   if (redo) return;
-  __syncthreads();
-
-  // copy the slices into LDS: 16 lanes per slice, 8 slices in flight per lane group
-  {
-    const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
-    const int sub = tid & 15, grp = tid >> 4;
-    constexpr int kGroups = kSelThreads / 16, kInFlight = 8;
-    for (int s0 = 0; s0 < p.parts; s0 += kGroups * kInFlight) {
-      uint64_t first[kInFlight];
-      uint32_t start[kInFlight], cnt[kInFlight];
-#pragma unroll
-      for (int u = 0; u < kInFlight; ++u) {
-        const int sl = s0 + u * kGroups + grp;
-        start[u] = cnt[u] = 0;
-        first[u] = 0;
-        if (sl < p.parts) {
-          start[u] = sl ? sh_ends[sl - 1] : 0u;
-          cnt[u] = sh_ends[sl] - start[u];
-          if ((uint32_t)sub < cnt[u]) first[u] = lists[(int64_t)sl * p.part_len + sub];
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < kInFlight; ++u) {
-        if ((uint32_t)sub < cnt[u]) sh_ent[start[u] + sub] = first[u];
-        if (cnt[u] > 16u) {
-          const int sl = s0 + u * kGroups + grp;
-          for (uint32_t j = 16u + sub; j < cnt[u]; j += 16u) sh_ent[start[u] + j] = lists[(int64_t)sl * p.part_len + j];
-        }
-      }
-    }
-  }
   __syncthreads();
 
   // this thread's share for the radix passes: entries tid, tid + 1024, ...
