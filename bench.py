@@ -271,8 +271,8 @@ def main():
     ops.profile_enable(False)
     kern = {name: ms / max(n, 1) * 1e3 for name, (ms, n) in prof.items()}  # us per launch
     dominant = w.dominant
-    if dominant == "gemv_scores" and "gemv_scores_cand" in kern:
-        dominant = "gemv_scores_cand"                   # long segments run the candidate-mode GEMV
+    if dominant == "gemv_scores" and "gemv_candidates" in kern:
+        dominant = "gemv_candidates"                    # long segments run the candidate-mode GEMV
     dom_us = kern.get(dominant, ms_per_step * 1e3)     # a workload with one foreign kernel: the step itself
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
 

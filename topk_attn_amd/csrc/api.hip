@@ -1,4 +1,5 @@
 // C ABI of the library: argument validation (before any HIP call), workspace carving, launch sequence.
+#include <atomic>
 #include <stdio.h>
 #include <string.h>
 
@@ -124,8 +125,9 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->group = a->group;
   g->num_chunks = a->num_chunks;
   g->scale = a->scale;
-  g->tau_key = nullptr;
-  g->tau_key_out = nullptr;
+  g->tau_words = nullptr;
+  g->epoch = 0;
+  g->num_samples = g->sample_rank = g->sample_wgs = g->early_wgs = 0;
   g->cand = nullptr;
   g->cand_seg_stride = 0;
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
@@ -192,15 +194,16 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // Long segments: sampled threshold, GEMV that stores candidates only, selection straight from the
   // candidate slices.  A segment whose candidates turn out too few (or too many) is flagged and redone
   // by the fallback kernel, which otherwise exits at once.
+  static std::atomic<uint32_t> call_counter{0};
   GemvParams cp = gp;
   cp.hist = nullptr;
-  cp.tau_key_out = sp.tau_key;
-  int rc = launch_sample_tau(cp, a->dtype, num_samples, sample_rank, stream);
-  if (rc != TKA_OK) return rc;
-  cp.tau_key = sp.tau_key;
+  cp.tau_words = sp.tau_words;
+  cp.epoch = call_counter.fetch_add(1, std::memory_order_relaxed) | 0x80000000u;   // never 0, the cleared state
+  cp.num_samples = num_samples;
+  cp.sample_rank = sample_rank;
   cp.cand = sp.list;
   cp.cand_seg_stride = sp.list_stride;
-  rc = launch_gemv_scores(cp, a->dtype, stream);
+  int rc = launch_gemv_candidates(cp, a->dtype, stream);
   if (rc != TKA_OK) return rc;
   SelectParams sc = sp;
   sc.hist = nullptr;

@@ -8,15 +8,17 @@
 // What the kernel WRITES decides how close it gets to the streaming rate.  Measured on MI355X (2.1 GB of
 // keys): no writes 306 us; 4 B of score per row (1.6 % of the bytes) +45 us; 2 B per row +35 us; the
 // histogram flush (150 memory-side atomics per 256-token workgroup) +40 us; the same stores into a buffer
-// that stays in L2 +2 us.  The cost follows the volume that reaches HBM.  Hence two modes:
-//   dense      every score is stored and a first-level histogram is flushed (short segments, the fallback,
-//              and callers that want all scores);
-//   candidate  a threshold tau per segment is known beforehand (sample_tau_kernel: an order statistic of a
-//              strided sample of the segment, chosen so that about 2k tokens pass); only tokens with
-//              key >= tau are stored, in index order, in the workgroup's own slice (the count rides in the
-//              first entry: one partial line per workgroup).  The selection kernel checks that at least k
-//              tokens passed and otherwise flags the segment for the fallback kernel, so the result is
-//              exact whatever the data.
+// that stays in L2 +2 us.  The cost follows the volume that reaches HBM.  Hence two kernels:
+//   dense      every score is stored and a first-level histogram is flushed (short segments and callers that
+//              want all scores);
+//   candidate  a threshold tau per segment comes from an order statistic of a strided sample of the segment,
+//              chosen so that about 2k tokens pass; only tokens with key >= tau are stored, in index order,
+//              in the workgroup's own slice (the count rides in the first entry: one partial line per
+//              workgroup).  The selection kernel checks that at least k tokens passed and otherwise flags
+//              the segment for the fallback kernel, so the result is exact whatever the data.
+//              The sampling runs inside the same launch: the first workgroups of the grid score the samples
+//              and publish the thresholds, the streaming workgroups need them only when their rows are
+//              scored and wait (bounded) for them then.
 #include "kernels.hpp"
 
 namespace tka {
@@ -27,15 +29,14 @@ constexpr int kGemvThreads = 256;
 constexpr int kGemvWaves = kGemvThreads / kWave;
 constexpr int kGemvUnroll = 8;                                         // loads in flight per lane
 constexpr int kGemvRowsPerIter = (kGemvThreads / 16) * kGemvUnroll;    // 128 tokens per WG iteration
-constexpr int kCandMaxIters = kGemvCandTokensPerWg / kGemvRowsPerIter; // iterations of a candidate-mode workgroup
-constexpr int kCandSubLists = kCandMaxIters * kGemvWaves;
-constexpr int kTauSplit = 4;   // sample workgroups (and thresholds) per segment
+constexpr int kTauSplit = 4;           // sampling workgroups (and thresholds) per segment
+constexpr int kTauSpinLimit = 1 << 16;
+constexpr int kEarlySlices = 3;       // slices of a streaming workgroup that starts before the thresholds are published // polls of a streaming workgroup for its thresholds before it gives up
+static_assert(kGemvCandTokensPerWg == kGemvThreads, "candidate mode: one thread per token in the epilogue");
 
-template <int DT, bool CAND>
+template <int DT>
 __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p) {
-  __shared__ uint32_t sh_hist[CAND ? 1 : kHistBins];
-  __shared__ uint64_t sh_cand[CAND ? kCandSubLists : 1][32];   // per (iteration, wave): ascending index
-  __shared__ uint32_t sh_ccnt[kCandSubLists];
+  __shared__ uint32_t sh_hist[kHistBins];
 
   const int tid = threadIdx.x;
   const int j = tid & 15;            // lane inside the row: dims 8j..8j+7
@@ -52,11 +53,10 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
   int64_t t_end = t_begin + p.tokens_per_wg;
   if (t_end > p.chunk_len) t_end = p.chunk_len;
 
-  const bool do_hist = !CAND && p.hist != nullptr;
+  const bool do_hist = p.hist != nullptr;
   if (do_hist) {
     for (int i = tid; i < kHistBins; i += kGemvThreads) sh_hist[i] = 0;
   }
-  if (CAND && tid < kCandSubLists) sh_ccnt[tid] = 0;
   __syncthreads();
 
   float qf[8];
@@ -64,16 +64,9 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
 
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
                           chunk_base * p.key_stride_n + 8 * j;
-  float* sc_out = CAND ? nullptr : p.scores + seg * p.chunk_len;
-  uint32_t tau = 0u;
-  if (CAND) {   // lowest of the quarter thresholds: every quarter then passes at least its own share
-    tau = ~0u;
-#pragma unroll
-    for (int w = 0; w < kTauSplit; ++w) tau = min(tau, p.tau_key[seg * kTauSplit + w]);
-  }
+  float* sc_out = p.scores + seg * p.chunk_len;
 
-  int it = 0;
-  for (int64_t base = t_begin; base < t_end; base += kGemvRowsPerIter, ++it) {
+  for (int64_t base = t_begin; base < t_end; base += kGemvRowsPerIter) {
     // row group rg owns 8 consecutive tokens per iteration: load u brings token base + rg*8 + u
     u32x4 kv[kGemvUnroll];
 #pragma unroll
@@ -88,45 +81,12 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
       const float s = row_score<DT>(qf, kv[u], p.scale);
       if (j == u) mine = s;
     }
-    // lane j < 8 of row group rg now holds the score of token base + rg*8 + j: a wave covers 32
-    // consecutive tokens, in lane order
+    // lane j < 8 of row group rg now holds the score of token base + rg*8 + j
     const int64_t t = base + rg * kGemvUnroll + j;
-    const bool owner = j < kGemvUnroll && t < t_end;
-    const uint32_t key = score_key(mine);
-    if (CAND) {
-      const bool pass = owner && key >= tau;
-      const unsigned long long mask = __ballot(pass);
-      const int lane = tid & 63, wave = tid >> 6;
-      if (pass) sh_cand[it * kGemvWaves + wave][__popcll(mask & ((1ull << lane) - 1ull))] = composite(key, (uint32_t)t);
-      if (lane == 0) sh_ccnt[it * kGemvWaves + wave] = (uint32_t)__popcll(mask);
-    } else if (owner) {
+    if (j < kGemvUnroll && t < t_end) {
       sc_out[t] = mine;
-      if (do_hist) atomicAdd(&sh_hist[key >> (32 - kHistBits)], 1u);
+      if (do_hist) atomicAdd(&sh_hist[score_key(mine) >> (32 - kHistBits)], 1u);
     }
-  }
-
-  if (CAND) {
-    // (iteration, wave) sub-lists are in token order one after the other: concatenate them into the slice
-    __syncthreads();
-    const int sub = tid >> 5, r = tid & 31;   // 8 sub-lists x 32 slots = 256 threads
-    uint32_t before = 0, total = 0;
-#pragma unroll
-    for (int s = 0; s < kCandSubLists; ++s) {
-      const uint32_t c = sh_ccnt[s];
-      before += s < sub ? c : 0u;
-      total += c;
-    }
-    // Slice format: word = key << 32 | count << 8 | token - first token of the slice; only slot 0 carries the
-    // count (0 .. 256), so a workgroup with few candidates writes a single line and nothing else
-    uint64_t* slice = p.cand + seg * p.cand_seg_stride + (int64_t)wg_in_chunk * p.tokens_per_wg;
-    if (sub < kCandSubLists && (uint32_t)r < sh_ccnt[sub]) {
-      const uint64_t c = sh_cand[sub][r];
-      const uint32_t pos = before + r;
-      const uint32_t rel = ~(uint32_t)c - (uint32_t)t_begin;
-      slice[pos] = (c & 0xffffffff00000000ull) | (pos == 0 ? total << 8 : 0u) | rel;
-    }
-    if (tid == 0 && total == 0) slice[0] = 0ull;
-    return;
   }
 
   if (do_hist) {
@@ -139,25 +99,248 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
   }
 }
 
-// ---- pilot: threshold of the candidate mode -----------------------------------------------------
-
-constexpr int kTauThreads = 1024;
-constexpr int kTauRowGroups = kTauThreads / 16;
-constexpr int kTauUnroll = 8;            // rows per row group and round: 512 samples per round
+// ---- candidate mode -----------------------------------------------------------------------------
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {  // integer hash for the sample jitter
   x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
   return x;
 }
 
-// kTauSplit workgroups per segment (a single CU cannot pull its share of rows fast enough): each scores
-// num_samples tokens of its quarter of the segment (one per stride, at a hashed offset inside the stride so
-// that periodic data cannot alias with the sampling) and takes the sample_rank-th largest key by radix select
-// in LDS -> tau_key[segment][quarter].  About sample_rank/num_samples of the quarter's tokens lie at or above
-// that key wherever the large scores sit in the segment; the GEMV uses the lowest of the four, so that the
-// number of tokens that pass is at least the sum of the four shares.
+// Token (inside its quarter of the segment) of sample i: one per stride, at a hashed offset inside the stride
+// so that periodic data cannot alias with the sampling.
+__device__ __forceinline__ int64_t sample_token(int seg, int quarter, int i, int64_t stride) {
+  return (int64_t)i * stride + (int64_t)(mix32(((uint32_t)seg * kTauSplit + quarter) * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
+}
+
+// A threshold word is (epoch << 32) | key: the epoch of the call tells a published threshold from whatever
+// the workspace held before.
+__device__ __forceinline__ void publish_tau(uint64_t* word, uint32_t epoch, uint32_t key) {
+  __hip_atomic_store(word, ((uint64_t)epoch << 32) | key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Sampling workgroup (256 threads) of one quarter of one segment: scores p.num_samples tokens and publishes the
+// p.sample_rank-th largest key.  About sample_rank/num_samples of the quarter's tokens lie at or above that key
+// wherever the large scores sit in the segment.  sh: num_samples + 256 + 8 words.
 template <int DT>
-__global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, int num_samples, int sample_rank) {
+__device__ __forceinline__ void sample_quarter(const GemvParams& p, int seg, int quarter, uint32_t* sh) {
+  uint32_t* sh_keys = sh;
+  uint32_t* sh_hist = sh + p.num_samples;   // 256 bins
+  uint32_t* sh_wtot = sh_hist + 256;        // 4 wave totals, then bin and count above it
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int j = tid & 15, rg = tid >> 4;
+  const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
+  const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
+  const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
+  float qf[8];
+  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  const int64_t quarter_len = p.chunk_len / kTauSplit;
+  const int64_t stride = quarter_len / p.num_samples;
+  const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
+                          (chunk_base + (int64_t)quarter * quarter_len) * p.key_stride_n + 8 * j;
+  for (int base = 0; base < p.num_samples; base += kGemvRowsPerIter) {
+    u32x4 kv[kGemvUnroll];
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u)
+      kv[u] = *(const u32x4*)(kbase + sample_token(seg, quarter, base + rg * kGemvUnroll + u, stride) * p.key_stride_n);
+    float mine = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      const float s = row_score<DT>(qf, kv[u], p.scale);
+      if (j == u) mine = s;
+    }
+    if (j < kGemvUnroll) sh_keys[base + rg * kGemvUnroll + j] = score_key(mine);
+  }
+  // sample_rank-th largest key: four 8-bit radix passes, thread t owns bin t
+  uint32_t need = (uint32_t)p.sample_rank, prefix = 0;
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    __syncthreads();
+    sh_hist[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < p.num_samples; i += kGemvThreads) {
+      const uint32_t key = sh_keys[i];
+      if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&sh_hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    const uint32_t mine = sh_hist[tid];
+    uint32_t ge = mine;   // count in bins >= tid, first inside the wave
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const uint32_t t = __shfl_down(ge, d, 64);
+      if (lane + d < 64) ge += t;
+    }
+    if (lane == 0) sh_wtot[wave] = ge;
+    __syncthreads();
+    for (int w = wave + 1; w < kGemvWaves; ++w) ge += sh_wtot[w];
+    if (ge >= need && ge - mine < need) { sh_wtot[4] = (uint32_t)tid; sh_wtot[5] = ge - mine; }
+    __syncthreads();
+    prefix = (prefix << 8) | sh_wtot[4];
+    need -= sh_wtot[5];
+  }
+  if (tid == 0) publish_tau(p.tau_words + (int64_t)seg * kTauSplit + quarter, p.epoch, prefix);
+}
+
+// Scores of one slice (up to 256 tokens from sbase on) as keys into LDS: lane j < 8 of row group rg writes the
+// key of token it*128 + rg*8 + j to keys_out[it*128].  FULL: the slice has all 256 tokens; the eight rows of
+// a lane then differ by a uniform offset and one lane offset serves all loads.  Otherwise rows past the end
+// are clamped to the last one, lane by lane.
+template <int DT, bool FULL>
+__device__ __forceinline__ void stream_slice(const unsigned char* sbase, uint32_t row_bytes, int n_local, const float (&qf)[8],
+                                             float scale, uint32_t* keys_out) {
+  const int j = threadIdx.x & 15, rg = threadIdx.x >> 4;
+  const uint32_t voff = (uint32_t)(rg * kGemvUnroll) * row_bytes + 16u * (uint32_t)j;
+  for (int it = 0; it < kGemvThreads / kGemvRowsPerIter; ++it) {
+    u32x4 kv[kGemvUnroll];
+    if constexpr (FULL) {
+      const unsigned char* ibase = sbase + (uint64_t)(it * kGemvRowsPerIter) * row_bytes;   // uniform
+#pragma unroll
+      for (int u = 0; u < kGemvUnroll; ++u)
+        kv[u] = __builtin_nontemporal_load((const u32x4*)(ibase + (uint64_t)u * row_bytes + voff));
+    } else {
+#pragma unroll
+      for (int u = 0; u < kGemvUnroll; ++u) {
+        int lt = it * kGemvRowsPerIter + rg * kGemvUnroll + u;
+        lt = lt < n_local ? lt : n_local - 1;
+        kv[u] = __builtin_nontemporal_load((const u32x4*)(sbase + ((uint32_t)lt * row_bytes + 16u * (uint32_t)j)));
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // all eight loads go out before the first score is computed
+    float mine = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      const float sc = row_score<DT>(qf, kv[u], scale);
+      if (j == u) mine = sc;
+    }
+    if (j < kGemvUnroll) keys_out[it * kGemvRowsPerIter] = score_key(mine);
+  }
+}
+
+// Grid: p.sample_wgs sampling workgroups first (so that they are resident before any workgroup that waits for
+// them), then the streaming workgroups.  Slices (256 tokens) are numbered segment-major.  The first
+// p.early_wgs streaming workgroups take kEarlySlices consecutive slices each, all later ones a single slice:
+// the workgroups that start together with the sampling would otherwise sit idle on their CU until the
+// thresholds arrive; with more rows to stream they reach that point when the thresholds are there.
+template <int DT>
+__global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void gemv_candidates_kernel(GemvParams p) {
+  __shared__ uint32_t sh[(kEarlySlices * kGemvThreads > kGemvMaxSamplesInline + 256 ? kEarlySlices * kGemvThreads : kGemvMaxSamplesInline + 256) + 8];
+  const int tid = threadIdx.x;
+  if ((int)blockIdx.x < p.sample_wgs) {
+    __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
+    sample_quarter<DT>(p, (int)blockIdx.x / kTauSplit, (int)blockIdx.x % kTauSplit, sh);
+    return;
+  }
+  uint32_t* sh_key = sh;                               // keys of this workgroup's tokens, slice after slice
+  uint32_t* sh_wcnt = sh + kEarlySlices * kGemvThreads; // candidates per wave
+  __shared__ uint32_t sh_tau[2 * kTauSplit];            // the segment's thresholds and whether each one has arrived
+
+  const int j = tid & 15;            // lane inside the row: dims 8j..8j+7
+  const int rg = tid >> 4;           // row group 0..15 inside the workgroup
+  const int lane = tid & 63, wave = tid >> 6;
+  const int64_t w = (int64_t)blockIdx.x - p.sample_wgs;
+  const int num_slices = w < p.early_wgs ? kEarlySlices : 1;
+  const int64_t first_slice = w < p.early_wgs ? w * kEarlySlices : (int64_t)p.early_wgs * kEarlySlices + (w - p.early_wgs);
+
+  const int64_t first_seg = first_slice / p.wgs_per_chunk;
+  const int first_wg = (int)(first_slice % p.wgs_per_chunk);
+
+  const uint32_t row_bytes = (uint32_t)p.key_stride_n * 2u;
+  {
+    int64_t seg = first_seg;
+    int wg_in_chunk = first_wg;
+    for (int s = 0; s < num_slices; ++s) {
+      const int chunk = (int)(seg % p.num_chunks);
+      const int64_t bh = seg / p.num_chunks;
+      const int h = (int)(bh % p.num_kv_heads), b = (int)(bh / p.num_kv_heads);
+      const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
+      const int64_t t_begin = (int64_t)wg_in_chunk * kGemvThreads;
+      const int n_local = (int)(p.chunk_len - t_begin < kGemvThreads ? p.chunk_len - t_begin : kGemvThreads);
+      float qf[8];
+      load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+      // uniform base of the slice + 32-bit lane offsets: one address register per load
+      const unsigned char* sbase = (const unsigned char*)p.keys +
+                                   2 * ((int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h + (chunk_base + t_begin) * p.key_stride_n);
+      uint32_t* keys_out = sh_key + s * kGemvThreads + rg * kGemvUnroll + j;
+      if (n_local == kGemvThreads)
+        stream_slice<DT, true>(sbase, row_bytes, n_local, qf, p.scale, keys_out);
+      else
+        stream_slice<DT, false>(sbase, row_bytes, n_local, qf, p.scale, keys_out);
+      if (++wg_in_chunk == p.wgs_per_chunk) { wg_in_chunk = 0; ++seg; }
+    }
+  }
+  __syncthreads();
+
+  uint32_t tau = 0;
+  bool tau_ready = false;
+  int64_t tau_seg = first_seg, seg = first_seg;
+  int wg_in_chunk = first_wg;
+  for (int s = 0; s < num_slices; ++s) {
+    const int64_t t_begin = (int64_t)wg_in_chunk * kGemvThreads;
+    int64_t t_end = t_begin + kGemvThreads;
+    if (t_end > p.chunk_len) t_end = p.chunk_len;
+    // Thresholds of the slice's segment: lanes 0..3 fetch one word each and hand them on through LDS (every
+    // wave asking for itself makes a hot spot of the few words).  A bounded wait: a workgroup that never sees
+    // its thresholds stores no candidates, and the selection kernel then flags the segment for the fallback
+    // kernel.
+    if (s == 0 || seg != tau_seg) {
+      tau_seg = seg;
+      if (s) __syncthreads();   // the previous slice's thresholds have been read
+      if (tid < kTauSplit) {
+        const uint64_t* word = p.tau_words + seg * kTauSplit + tid;
+        uint64_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int spin = 0; (uint32_t)(v >> 32) != p.epoch && spin < kTauSpinLimit; ++spin) {
+          __builtin_amdgcn_s_sleep(16);
+          v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        sh_tau[tid] = (uint32_t)v;
+        sh_tau[kTauSplit + tid] = (uint32_t)(v >> 32) == p.epoch ? 1u : 0u;
+      }
+      __syncthreads();
+      tau = ~0u;
+      tau_ready = true;
+#pragma unroll
+      for (int q = 0; q < kTauSplit; ++q) {   // lowest of the four: every quarter then passes at least its own share
+        tau = min(tau, sh_tau[q]);
+        tau_ready = tau_ready && sh_tau[kTauSplit + q] != 0u;
+      }
+    }
+
+    // thread t owns token t_begin + t: candidates in index order into the slice.
+    // Slice format: word = key << 32 | count << 8 | token - first token of the slice; only entry 0 carries
+    // the count (0 .. 256), so a workgroup with few candidates writes a single line and nothing else.
+    const uint32_t key = sh_key[s * kGemvThreads + tid];
+    const bool pass = tau_ready && t_begin + tid < t_end && key >= tau;
+    const unsigned long long mask = __ballot(pass);
+    if (s) __syncthreads();   // the previous slice's counts have been read
+    if (lane == 0) sh_wcnt[wave] = (uint32_t)__popcll(mask);
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int v = 0; v < kGemvWaves; ++v) {
+      const uint32_t c = sh_wcnt[v];
+      before += v < wave ? c : 0u;
+      total += c;
+    }
+    uint64_t* slice = p.cand + seg * p.cand_seg_stride + (int64_t)wg_in_chunk * kGemvThreads;
+    if (pass) {
+      const uint32_t pos = before + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+      slice[pos] = ((uint64_t)key << 32) | (pos == 0 ? total << 8 : 0u) | (uint32_t)tid;
+    }
+    if (tid == 0 && total == 0) slice[0] = 0ull;
+    if (++wg_in_chunk == p.wgs_per_chunk) { wg_in_chunk = 0; ++seg; }
+  }
+}
+
+// ---- stand-alone sampling kernel (long segments: more samples than the streaming grid's workgroups take) --
+
+constexpr int kTauThreads = 1024;
+constexpr int kTauRowGroups = kTauThreads / 16;
+constexpr int kTauUnroll = 8;            // rows per row group and round: 512 samples per round
+
+// kTauSplit workgroups of 1024 threads per segment: as sample_quarter, for 1024 or 2048 samples per quarter.
+template <int DT>
+__global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p) {
+  const int num_samples = p.num_samples, sample_rank = p.sample_rank;
   __shared__ uint32_t sh_keys[kGemvMaxSamples];
   __shared__ uint32_t sh_hist[kHistBins];
   __shared__ uint32_t sh_wtot[kTauThreads / kWave];
@@ -185,7 +368,7 @@ __global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, i
 #pragma unroll
     for (int u = 0; u < kTauUnroll; ++u) {
       const int i = base + rg * kTauUnroll + u;                        // sample number (num_samples is a multiple of 512)
-      const int64_t t = (int64_t)i * stride + (int64_t)(mix32(((uint32_t)seg * kTauSplit + quarter) * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
+      const int64_t t = sample_token(seg, quarter, i, stride);
       kv[u] = *(const u32x4*)(kbase + t * p.key_stride_n);
     }
     float mine = 0.0f;
@@ -219,32 +402,52 @@ __global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p, i
     fixed += bits;
   }
   prefix <<= (32 - fixed);
-  if (tid == 0) p.tau_key_out[seg * kTauSplit + quarter] = prefix;
+  if (tid == 0) publish_tau(p.tau_words + (int64_t)seg * kTauSplit + quarter, p.epoch, prefix);
 }
 
 }  // namespace
 
 int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
   dim3 grid((unsigned)(p.num_chunks * p.wgs_per_chunk), (unsigned)p.num_kv_heads, (unsigned)p.batch);
-  const bool cand = p.cand != nullptr;
-  LaunchTimer timer(cand ? "gemv_scores_cand" : "gemv_scores", stream);
-  if (dtype == TKA_F16) {
-    if (cand) gemv_scores_kernel<TKA_F16, true><<<grid, kGemvThreads, 0, stream>>>(p);
-    else gemv_scores_kernel<TKA_F16, false><<<grid, kGemvThreads, 0, stream>>>(p);
-  } else {
-    if (cand) gemv_scores_kernel<TKA_BF16, true><<<grid, kGemvThreads, 0, stream>>>(p);
-    else gemv_scores_kernel<TKA_BF16, false><<<grid, kGemvThreads, 0, stream>>>(p);
-  }
+  LaunchTimer timer("gemv_scores", stream);
+  if (dtype == TKA_F16)
+    gemv_scores_kernel<TKA_F16><<<grid, kGemvThreads, 0, stream>>>(p);
+  else
+    gemv_scores_kernel<TKA_BF16><<<grid, kGemvThreads, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 
-int launch_sample_tau(const GemvParams& p, int dtype, int num_samples, int sample_rank, hipStream_t stream) {
-  const dim3 segs(kTauSplit, (unsigned)(p.batch * p.num_kv_heads * p.num_chunks));
-  LaunchTimer timer("sample_tau", stream);
+// Candidate mode.  p.num_samples <= kGemvMaxSamplesInline: the sampling workgroups are part of the launch;
+// more: the stand-alone sampling kernel goes first.
+int launch_gemv_candidates(const GemvParams& p0, int dtype, hipStream_t stream) {
+  GemvParams p = p0;
+  const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
+  if (p.tokens_per_wg != kGemvThreads || p.num_samples < 1 || p.num_samples % kGemvRowsPerIter) return TKA_EINVAL;
+  if (p.num_samples > kGemvMaxSamplesInline) {
+    if (p.num_samples > kGemvMaxSamples || p.num_samples % (kTauRowGroups * kTauUnroll)) return TKA_EINVAL;
+    const dim3 grid(kTauSplit, (unsigned)segs);
+    LaunchTimer timer("sample_tau", stream);
+    if (dtype == TKA_F16)
+      sample_tau_kernel<TKA_F16><<<grid, kTauThreads, 0, stream>>>(p);
+    else
+      sample_tau_kernel<TKA_BF16><<<grid, kTauThreads, 0, stream>>>(p);
+    if (hipGetLastError() != hipSuccess) return TKA_EHIP;
+    p.sample_wgs = 0;
+  } else {
+    p.sample_wgs = (int)(segs * kTauSplit);
+  }
+  // early workgroups: as many as the GPU holds at once (256 CUs x 8), when the sampling runs beside them
+  const int64_t slices = segs * p.wgs_per_chunk;
+  int64_t early = p.sample_wgs ? 2048 : 0;
+  if (early > slices / (2 * kEarlySlices)) early = slices / (2 * kEarlySlices);
+  p.early_wgs = (int)early;
+  const int64_t wgs = p.sample_wgs + early + (slices - early * kEarlySlices);
+  if (wgs > 0x7fffffffLL) return TKA_EUNSUPPORTED;
+  LaunchTimer timer("gemv_candidates", stream);
   if (dtype == TKA_F16)
-    sample_tau_kernel<TKA_F16><<<segs, kTauThreads, 0, stream>>>(p, num_samples, sample_rank);
+    gemv_candidates_kernel<TKA_F16><<<(unsigned)wgs, kGemvThreads, 0, stream>>>(p);
   else
-    sample_tau_kernel<TKA_BF16><<<segs, kTauThreads, 0, stream>>>(p, num_samples, sample_rank);
+    gemv_candidates_kernel<TKA_BF16><<<(unsigned)wgs, kGemvThreads, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 
@@ -268,7 +471,7 @@ void gemv_candidate_plan(int64_t chunk_len, int k, int max_candidates, int* num_
   *sample_rank = 0;
   if (chunk_len < 65536 || (int64_t)k * 16 > chunk_len) return;
   const int rounds = chunk_len >= 1048576 ? 4 : (chunk_len >= 524288 ? 2 : 1);   // more samples on long segments keep the candidate share near k/n
-  const int s = kTauRowGroups * kTauUnroll * rounds;
+  const int s = kGemvMaxSamplesInline * rounds;
   const double S = (double)s * kTauSplit;
   const double m = (double)k * S / (double)chunk_len;
   double root = 0.0;

@@ -11,9 +11,12 @@ struct GemvParams {
   float* scores;        // [batch][num_kv_heads][num_chunks][chunk_len]; selection kernels also read them
   const int32_t* cluster_ids;  // [batch*num_kv_heads*num_chunks] or nullptr: chunk c covers the tokens of that cluster
   uint32_t* hist;       // [batch*num_kv_heads*num_chunks][kHistBins] or nullptr; must be zero on entry
-  // candidate mode (cand != nullptr): only tokens with key >= tau_key[segment] are stored
-  const uint32_t* tau_key;    // [segments]
-  uint32_t* tau_key_out;      // [segments], written by the sample kernel
+  // candidate mode: only tokens whose key reaches the lowest of the segment's four thresholds are stored
+  uint64_t* tau_words;        // [segments][4] (epoch << 32) | threshold key, one per sampled quarter
+  uint32_t epoch;             // tells this call's thresholds from older contents of tau_words (never 0)
+  int num_samples, sample_rank;   // per quarter
+  int sample_wgs;             // sampling workgroups at the front of the candidate grid (set by the launcher)
+  int early_wgs;              // streaming workgroups behind them that take several slices each (set by the launcher)
   uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] one slice per workgroup, ascending index:
                               // key << 32 | count << 8 | token offset in the slice (count in entry 0 only)
   int64_t cand_seg_stride;    // entries between the slice arrays of consecutive segments
@@ -24,7 +27,7 @@ struct GemvParams {
   float scale;
 };
 int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream);
-int launch_sample_tau(const GemvParams& p, int dtype, int num_samples, int sample_rank, hipStream_t stream);
+int launch_gemv_candidates(const GemvParams& p, int dtype, hipStream_t stream);   // thresholds + candidate slices
 void gemv_candidate_plan(int64_t chunk_len, int k, int max_candidates, int* num_samples, int* sample_rank);
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);
 
@@ -34,7 +37,7 @@ struct SelectParams {
   int64_t seg_len;
   int64_t seg_stride;
   uint32_t* hist;         // [num_segments][kHistBins]; nullptr: the lists hold candidates above a sampled threshold
-  uint32_t* tau_key;      // [num_segments] candidate threshold (workspace)
+  uint64_t* tau_words;    // [num_segments][4] candidate thresholds (workspace); the candidate selection kernel clears them
   uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment must be redone by the fallback kernel
   int max_entries;        // candidate mode: more listed entries than this also sends the segment to the fallback kernel
   uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)

@@ -411,6 +411,8 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(Selec
     p.seg_flags[seg] = redo ? 1u : 0u;
     sh_small_cnt = 0;
   }
+  // the thresholds are spent: a replay of the same launches (a captured graph) must not take them for its own
+  if (tid < 4) p.tau_words[(int64_t)seg * 4 + tid] = 0ull;
   if (redo) return;
   __syncthreads();
 
@@ -754,7 +756,7 @@ int kpad_for(int k) {
 }  // namespace
 
 // Workspace layout (each part 256-byte aligned):
-//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S][4] u32 | list_cnt [S][slices] u32 |
+//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S][4] u64 | list_cnt [S][slices] u32 |
 //   list [S][slices*slice_len] u64      (slices: dense 4096/16384 scores, candidate mode one per GEMV workgroup)
 namespace {
 struct SelectLayout {
@@ -769,7 +771,7 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   l.list_stride = (seg_len + 16 * kSelThreads - 1) / (16 * kSelThreads) * (16 * kSelThreads);  // whole slices
   l.hist = take((size_t)num_segments * kHistBins * sizeof(uint32_t));
   l.flags = take((size_t)num_segments * sizeof(uint32_t));
-  l.tau = take((size_t)num_segments * 4 * sizeof(uint32_t));   // one threshold per sampled quarter
+  l.tau = take((size_t)num_segments * 4 * sizeof(uint64_t));   // one threshold word per sampled quarter
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
   l.total = off;
@@ -785,7 +787,7 @@ size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p
   unsigned char* c = (unsigned char*)ws;
   p->hist = (uint32_t*)(c + l.hist);
   p->seg_flags = (uint32_t*)(c + l.flags);
-  p->tau_key = (uint32_t*)(c + l.tau);
+  p->tau_words = (uint64_t*)(c + l.tau);
   p->list_cnt = (uint32_t*)(c + l.list_cnt);
   p->list = (uint64_t*)(c + l.list);
   p->list_stride = l.list_stride;
