@@ -50,7 +50,7 @@ class SparseDecode:
     """c4 (and a small variant): the end-to-end step."""
 
     def __init__(self, torch, ops, dev, batch=8, hkv=8, group=4, seq_len=131072, k=2048, sink=64, local=512,
-                 dtype="float16", out_dtype="bfloat16", heavy=0.01, seed=4, name="c4"):
+                 dtype="float16", out_dtype="bfloat16", heavy=0.01, seed=4, name="c4", num_splits=0):
         self.torch, self.name = torch, name
         g = torch.Generator(device=dev)
         g.manual_seed(seed)
@@ -68,7 +68,7 @@ class SparseDecode:
         # production configuration: the attention consumes the union list; the optional rank-ordered top-k
         # output (a sort per KV head) is not requested
         self.plan = ops.SparseDecodePlan(self.q, self.K, self.V, k, sink, local, SCALE, G,
-                                         out_dtype=getattr(torch, out_dtype), want_topk=False)
+                                         out_dtype=getattr(torch, out_dtype), num_splits=num_splits, want_topk=False)
         self.desc = "%s: B=%d Hq=%d Hkv=%d D=128 N=%d %s k=%d sink=%d local=%d out=%s" % (
             name, B, H * G, H, N, dtype, k, sink, local, out_dtype)
         self.dominant = "gemv_scores"
@@ -208,7 +208,7 @@ def build_workload(name, torch, ops, dev, args):
     if name == "copy":
         return PlainCopy(torch, dev)
     if name == "c4":
-        return SparseDecode(torch, ops, dev)
+        return SparseDecode(torch, ops, dev, num_splits=args.splits)
     if name == "c4-small":
         return SparseDecode(torch, ops, dev, batch=2, seq_len=16384, name="c4-small")
     if name == "c1":
@@ -228,7 +228,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c4-small", "c5", "copy"])
-    ap.add_argument("--splits", type=int, default=0, help="c3: split count (0 = library default)")
+    ap.add_argument("--splits", type=int, default=0, help="c3, c4: split count of the attention (0 = library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-runs", type=int, default=3)
     args = ap.parse_args()

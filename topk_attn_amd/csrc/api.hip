@@ -192,8 +192,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   }
 
   // Long segments: sampled threshold, GEMV that stores candidates only, selection straight from the
-  // candidate slices.  A segment whose candidates turn out too few (or too many) is flagged and redone
-  // by the fallback kernel, which otherwise exits at once.
+  // candidate slices.  A segment whose candidates turn out too few (or too many) is redone from the keys by
+  // its selection workgroup.
   static std::atomic<uint32_t> call_counter{0};
   GemvParams cp = gp;
   cp.hist = nullptr;
@@ -211,10 +211,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   sc.part_len = cp.tokens_per_wg;
   sc.list_stride = sp.list_stride;
   sc.max_entries = select_cand_capacity();
-  rc = launch_select_finalize_cand(sc, stream);
-  if (rc != TKA_OK) return rc;
-  // flagged segments are redone by one workgroup each; the launch is idle otherwise
-  return launch_select_fallback(gp, sp, a->dtype, stream);
+  sc.scores = scores;
+  return launch_select_finalize_cand(gp, sc, a->dtype, stream);
 }
 
 int check_flash(const tka_flash_decode_args* a) {

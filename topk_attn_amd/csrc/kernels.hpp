@@ -38,8 +38,8 @@ struct SelectParams {
   int64_t seg_stride;
   uint32_t* hist;         // [num_segments][kHistBins]; nullptr: the lists hold candidates above a sampled threshold
   uint64_t* tau_words;    // [num_segments][4] candidate thresholds (workspace); the candidate selection kernel clears them
-  uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment must be redone by the fallback kernel
-  int max_entries;        // candidate mode: more listed entries than this also sends the segment to the fallback kernel
+  uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment was redone from the keys
+  int max_entries;        // candidate mode: a segment with more candidates than this is also redone from the keys
   uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)
   uint64_t* list;         // [num_segments][list_stride] composites with bin >= threshold bin, slice p at p*part_len
   int64_t list_stride;
@@ -67,9 +67,8 @@ int launch_select_hist(const SelectParams& p, hipStream_t stream);
 int launch_select(const SelectParams& p, hipStream_t stream);   // filter + finalize
 int launch_select_filter(const SelectParams& p, hipStream_t stream);
 int launch_select_finalize(const SelectParams& p, hipStream_t stream);
-int launch_select_finalize_cand(const SelectParams& p, hipStream_t stream);   // candidate slices -> outputs, or a flag
-// One workgroup per flagged segment redoes scores and selection on its own; the others exit at once.
-int launch_select_fallback(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
+// Candidate slices -> outputs; a segment whose slices cannot be used is redone from the keys by its workgroup.
+int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
 int select_cand_max_parts();   // most candidate slices per segment
 int select_cand_capacity();    // most candidates per segment
 

@@ -336,228 +336,19 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   write_rank_outputs(sh_sort, p, seg);
 }
 
-// ---- finalize of the candidate mode -------------------------------------------------------------
-
-constexpr int kCandCap = 16384;    // candidates of one segment held in LDS (128 KB of composites)
-constexpr int kCandPerThread = kCandCap / kSelThreads;
-constexpr int kCandMaxParts = 4096;
-constexpr int kSmallBucket = 64;   // a threshold bucket of this many entries or fewer is ranked by one wave
-
-// Candidate mode: the slices hold every token whose key reached the sampled threshold, ascending in token
-// index inside and across slices (format: GemvParams::cand).  One workgroup per segment copies them into LDS
-// as composites (entry v of the segment at position v), finds the k-th largest composite by radix passes that start below the common prefix of
-// the smallest and largest candidate, and walks the entries once in index order.
-// A segment with fewer than k candidates, or more than fit, is flagged for the dense kernels instead.
-// Dynamic LDS: kCandCap composites; rank mode reuses them as sort and exchange buffers.
-__global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(SelectParams p, int kpad) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint64_t* sh_ent = (uint64_t*)smem;
-  __shared__ uint32_t sh_hist[kHistBins];
-  constexpr int kGroups = kSelThreads / 16, kInFlight = 8, kRound = kGroups * kInFlight;   // 512 slices per round
-  __shared__ uint32_t sh_cnt[kRound], sh_start[kRound];
-  __shared__ uint32_t sh_wtot[kSelWaves];
-  __shared__ uint32_t sh_res[4];
-  __shared__ uint64_t sh_wmin[kSelWaves], sh_wmax[kSelWaves];
-  __shared__ uint64_t sh_small[kSmallBucket];
-  __shared__ uint32_t sh_small_cnt;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int seg = blockIdx.x;
-  const uint32_t k = (uint32_t)p.k;
-
-  // Copy the slices into LDS, kRound slices at a time: 16 lanes per slice load its first 16 entries (entry 0
-  // carries the slice's count; entries beyond the count are stale memory and ignored), the counts are
-  // scanned into start positions, and the entries go to their place.  One memory round trip per round.
-  const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
-  const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
-  const int sub = tid & 15, grp = tid >> 4;
-  uint32_t n_entries = 0;
-  for (int s0 = 0; s0 < p.parts; s0 += kRound) {
-    uint64_t first[kInFlight];
-    uint32_t cnt[kInFlight];
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u) {
-      const int sl = s0 + u * kGroups + grp;
-      first[u] = sl < p.parts ? lists[(int64_t)sl * p.part_len + sub] : 0ull;
-    }
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u) {
-      cnt[u] = ((uint32_t)__shfl((int)(uint32_t)first[u], lane & ~15, 64) >> 8) & 0x1ffu;
-      if (sub == 0) sh_cnt[u * kGroups + grp] = cnt[u];
-    }
-    __syncthreads();
-    uint32_t total;
-    const uint32_t c = tid < kRound ? sh_cnt[tid] : 0u;
-    const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
-    if (tid < kRound) sh_start[tid] = n_entries + ex;
-    __syncthreads();
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u) {
-      const int sl = s0 + u * kGroups + grp;
-      const uint32_t start = sh_start[u * kGroups + grp];
-      const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
-      if ((uint32_t)sub < cnt[u] && start + sub < cap)
-        sh_ent[start + sub] = (first[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)first[u] & 0xffu));
-      for (uint32_t j = 16u + sub; j < cnt[u] && start + j < cap; j += 16u) {   // rare: a slice with more than 16 candidates
-        const uint64_t w = lists[(int64_t)sl * p.part_len + j];
-        sh_ent[start + j] = (w & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w & 0xffu));
-      }
-    }
-    n_entries += total;
-  }
-  const bool redo = n_entries < k || n_entries > cap;
-  if (tid == 0) {
-    p.seg_flags[seg] = redo ? 1u : 0u;
-    sh_small_cnt = 0;
-  }
-  // the thresholds are spent: a replay of the same launches (a captured graph) must not take them for its own
-  if (tid < 4) p.tau_words[(int64_t)seg * 4 + tid] = 0ull;
-  if (redo) return;
-  __syncthreads();
-
-  // this thread's share for the radix passes: entries tid, tid + 1024, ...
-  uint64_t mine[kCandPerThread];
-  uint64_t cmin = ~0ull, cmax = 0ull;
-#pragma unroll
-  for (int i = 0; i < kCandPerThread; ++i) {
-    const uint32_t v = (uint32_t)i * kSelThreads + tid;
-    const bool ok = v < n_entries;
-    mine[i] = ok ? sh_ent[v] : 0ull;
-    if (ok) {
-      cmin = mine[i] < cmin ? mine[i] : cmin;
-      cmax = mine[i] > cmax ? mine[i] : cmax;
-    }
-  }
-
-  uint64_t threshold = 0;   // selected: composite >= threshold
-  if (n_entries > k) {
-    // common prefix of all candidates: the passes start below it
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const uint64_t a = __shfl_xor(cmin, d, 64), b = __shfl_xor(cmax, d, 64);
-      cmin = a < cmin ? a : cmin;
-      cmax = b > cmax ? b : cmax;
-    }
-    if (lane == 0) { sh_wmin[wave] = cmin; sh_wmax[wave] = cmax; }
-    __syncthreads();
-#pragma unroll
-    for (int w = 0; w < kSelWaves; ++w) {
-      const uint64_t a = sh_wmin[w], b = sh_wmax[w];
-      cmin = a < cmin ? a : cmin;
-      cmax = b > cmax ? b : cmax;
-    }
-    int fixed = __builtin_clzll(cmin ^ cmax);            // composites are distinct and n_entries >= 2: < 64
-    uint64_t prefix = fixed ? cmax >> (64 - fixed) : 0ull;
-    uint32_t need = k;
-    bool done = false;
-    while (!done) {
-      const int bits = (64 - fixed) >= kHistBits ? kHistBits : (64 - fixed);
-      const int shift = 64 - fixed - bits;
-      __syncthreads();
-      sh_hist[2 * tid] = 0;
-      sh_hist[2 * tid + 1] = 0;
-      __syncthreads();
-#pragma unroll
-      for (int i = 0; i < kCandPerThread; ++i) {
-        const uint64_t c = mine[i];
-        if ((uint32_t)i * kSelThreads + tid < n_entries && (fixed == 0 || (c >> (64 - fixed)) == prefix))
-          atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
-      }
-      __syncthreads();
-      find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
-      const uint32_t d = sh_res[0], gt = sh_res[1], cnt = sh_res[2];
-      need -= gt;
-      prefix = (prefix << bits) | d;
-      fixed += bits;
-      if (cnt == need || fixed == 64) {
-        threshold = fixed == 64 ? prefix : (prefix << (64 - fixed));
-        done = true;
-      } else if (cnt <= (uint32_t)kSmallBucket) {
-        // few entries left in the threshold bucket: every wave ranks them and picks the need-th largest
-#pragma unroll
-        for (int i = 0; i < kCandPerThread; ++i) {
-          const uint64_t c = mine[i];
-          if ((uint32_t)i * kSelThreads + tid < n_entries && (c >> (64 - fixed)) == prefix) sh_small[atomicAdd(&sh_small_cnt, 1u)] = c;
-        }
-        __syncthreads();
-        const uint64_t e = (uint32_t)lane < cnt ? sh_small[lane] : 0ull;
-        uint32_t greater = 0;
-        for (uint32_t j = 0; j < cnt; ++j) greater += sh_small[j] > e ? 1u : 0u;
-        const uint64_t hit = __ballot((uint32_t)lane < cnt && greater == need - 1u);
-        threshold = __shfl(e, (int)__builtin_ctzll(hit), 64);
-        done = true;
-      }
-    }
-  }
-
-  // Walk in index order: thread t takes the run of `per` consecutive entries starting at t*per.
-  const bool want_rank = p.out_idx != nullptr;
-  const bool want_union = p.union_idx != nullptr;
-  const int64_t n = p.seg_len;
-  const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
-  const uint32_t hi = (uint32_t)(n - p.local > lo ? n - p.local : lo);
-  const uint32_t per = (n_entries + kSelThreads - 1) / kSelThreads;
-  uint64_t run[kCandPerThread];
-  uint32_t sel_mask = 0, mid_mask = 0;
-#pragma unroll
-  for (int i = 0; i < kCandPerThread; ++i) {
-    const uint32_t v = (uint32_t)tid * per + i;
-    const bool ok = (uint32_t)i < per && v < n_entries;
-    run[i] = ok ? sh_ent[v] : 0ull;
-    const bool sel = ok && run[i] >= threshold;
-    const uint32_t idx = ~(uint32_t)run[i];
-    sel_mask |= (sel ? 1u : 0u) << i;
-    mid_mask |= (sel && idx >= lo && idx < hi ? 1u : 0u) << i;
-  }
-  // one scan for both counts (each total is at most 16384)
-  uint32_t totals;
-  const uint32_t ex = block_exclusive_scan(((uint32_t)__builtin_popcount(sel_mask) << 16) | (uint32_t)__builtin_popcount(mid_mask), sh_wtot, &totals);
-  if (want_union) {
-    int32_t* uo = p.union_idx + (int64_t)seg * (p.k + p.sink + p.local);
-    uint32_t pos = lo + (ex & 0xffffu);
-#pragma unroll
-    for (int i = 0; i < kCandPerThread; ++i)
-      if (mid_mask >> i & 1u) uo[pos++] = (int32_t)~(uint32_t)run[i];
-    write_union_edges(uo, p, seg, lo, hi, totals & 0xffffu);
-  }
-  if (!want_rank) return;
-  uint64_t* sh_sort = sh_ent;
-  uint64_t* sh_xchg = sh_ent + kpad;
-  __syncthreads();   // every thread holds its run in registers: the entries may be overwritten
-  {
-    uint32_t pos = ex >> 16;
-#pragma unroll
-    for (int i = 0; i < kCandPerThread; ++i)
-      if (sel_mask >> i & 1u) sh_sort[pos++] = run[i];
-    for (int i = (int)k + tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite
-  }
-  __syncthreads();
-  sort_lds_desc(sh_sort, sh_xchg, kpad);
-  write_rank_outputs(sh_sort, p, seg);
-}
-
 // ---- fallback of the candidate mode ---------------------------------------------------------------
 
-// One workgroup per segment; all but the flagged segments exit at once, so the launch normally costs its
-// overhead only.  A flagged segment is redone from the keys by its workgroup alone: scores in the canonical
-// order (stored, and a histogram of the top key bits kept in LDS), radix passes over the stored scores until
-// the k-th largest key is fixed, then one walk in index order that takes every key above the threshold
-// bucket and the first `need` keys inside it.  Exact for any data; slow (one CU streams the segment), which
-// is acceptable for an event that the sampling makes rare.
-// Dynamic LDS (rank mode only): kpad composites (sort buffer), then kpad composites (exchange buffer).
+// A segment whose candidate slices cannot be used (fewer than k candidates, or more than fit) is redone from
+// the keys by its workgroup alone: scores in the canonical order (stored, and a histogram of the top key bits
+// kept in LDS), radix passes over the stored scores until the k-th largest key is fixed, then one walk in
+// index order that takes every key above the threshold bucket and the first `need` keys inside it.  Exact for
+// any data; slow (one CU streams the segment), which is acceptable for an event that the sampling makes rare.
+// sh_sort: 2*kpad composites (rank mode only).  Every thread of the block must call it.
 template <int DT>
-__global__ __launch_bounds__(kSelThreads) void select_fallback_kernel(GemvParams g, SelectParams p, int kpad) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint64_t* sh_sort = (uint64_t*)smem;
+__device__ __forceinline__ void fallback_segment(const GemvParams& g, const SelectParams& p, int seg, int kpad, uint64_t* sh_sort,
+                                                 uint32_t* sh_hist, uint32_t* sh_wtot, uint32_t* sh_res) {
   uint64_t* sh_xchg = sh_sort + kpad;
-  __shared__ uint32_t sh_hist[kHistBins];
-  __shared__ uint32_t sh_wtot[kSelWaves];
-  __shared__ uint32_t sh_res[4];
-
   const int tid = threadIdx.x;
-  const int seg = blockIdx.x;
-  if (p.seg_flags[seg] == 0) return;
   const uint32_t k = (uint32_t)p.k;
   const int64_t n = p.seg_len;
   float* sc = g.scores + (int64_t)seg * p.seg_stride;
@@ -677,6 +468,213 @@ __global__ __launch_bounds__(kSelThreads) void select_fallback_kernel(GemvParams
   }
   if (want_union) write_union_edges(uo, p, seg, lo, hi, run_mid);
   if (!want_rank) return;
+  __syncthreads();
+  sort_lds_desc(sh_sort, sh_xchg, kpad);
+  write_rank_outputs(sh_sort, p, seg);
+}
+
+// ---- finalize of the candidate mode -------------------------------------------------------------
+
+constexpr int kCandCap = 16384;    // candidates of one segment held in LDS (128 KB of composites)
+constexpr int kCandPerThread = kCandCap / kSelThreads;
+constexpr int kCandMaxParts = 4096;
+constexpr int kSmallBucket = 64;   // a threshold bucket of this many entries or fewer is ranked by one wave
+
+// Candidate mode: the slices hold every token whose key reached the sampled threshold, ascending in token
+// index inside and across slices (format: GemvParams::cand).  One workgroup per segment copies them into LDS
+// as composites (entry v of the segment at position v), finds the k-th largest composite by radix passes that start below the common prefix of
+// the smallest and largest candidate, and walks the entries once in index order.
+// A segment with fewer than k candidates, or more than fit, is redone by fallback_segment (and flagged in
+// seg_flags, for the curious).
+// Dynamic LDS: kCandCap composites; rank mode reuses them as sort and exchange buffers.
+template <int DT>
+__global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvParams g, SelectParams p, int kpad) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint64_t* sh_ent = (uint64_t*)smem;
+  __shared__ uint32_t sh_hist[kHistBins];
+  constexpr int kGroups = kSelThreads / 16, kInFlight = 8, kRound = kGroups * kInFlight;   // 512 slices per round
+  __shared__ uint32_t sh_cnt[kRound], sh_start[kRound];
+  __shared__ uint32_t sh_wtot[kSelWaves];
+  __shared__ uint32_t sh_res[4];
+  __shared__ uint64_t sh_wmin[kSelWaves], sh_wmax[kSelWaves];
+  __shared__ uint64_t sh_small[kSmallBucket];
+  __shared__ uint32_t sh_small_cnt;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int seg = blockIdx.x;
+  const uint32_t k = (uint32_t)p.k;
+
+  // Copy the slices into LDS, kRound slices at a time: 16 lanes per slice load its first 16 entries (entry 0
+  // carries the slice's count; entries beyond the count are stale memory and ignored), the counts are
+  // scanned into start positions, and the entries go to their place.  One memory round trip per round.
+  const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
+  const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
+  const int sub = tid & 15, grp = tid >> 4;
+  uint32_t n_entries = 0;
+  for (int s0 = 0; s0 < p.parts; s0 += kRound) {
+    uint64_t first[kInFlight];
+    uint32_t cnt[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int sl = s0 + u * kGroups + grp;
+      first[u] = sl < p.parts ? lists[(int64_t)sl * p.part_len + sub] : 0ull;
+    }
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      cnt[u] = ((uint32_t)__shfl((int)(uint32_t)first[u], lane & ~15, 64) >> 8) & 0x1ffu;
+      if (sub == 0) sh_cnt[u * kGroups + grp] = cnt[u];
+    }
+    __syncthreads();
+    uint32_t total;
+    const uint32_t c = tid < kRound ? sh_cnt[tid] : 0u;
+    const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
+    if (tid < kRound) sh_start[tid] = n_entries + ex;
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int sl = s0 + u * kGroups + grp;
+      const uint32_t start = sh_start[u * kGroups + grp];
+      const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
+      if ((uint32_t)sub < cnt[u] && start + sub < cap)
+        sh_ent[start + sub] = (first[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)first[u] & 0xffu));
+      for (uint32_t j = 16u + sub; j < cnt[u] && start + j < cap; j += 16u) {   // rare: a slice with more than 16 candidates
+        const uint64_t w = lists[(int64_t)sl * p.part_len + j];
+        sh_ent[start + j] = (w & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w & 0xffu));
+      }
+    }
+    n_entries += total;
+  }
+  const bool redo = n_entries < k || n_entries > cap;
+  if (tid == 0) {
+    p.seg_flags[seg] = redo ? 1u : 0u;
+    sh_small_cnt = 0;
+  }
+  // the thresholds are spent: a replay of the same launches (a captured graph) must not take them for its own
+  if (tid < 4) p.tau_words[(int64_t)seg * 4 + tid] = 0ull;
+  if (redo) {
+    __syncthreads();
+    fallback_segment<DT>(g, p, seg, kpad, sh_ent, sh_hist, sh_wtot, sh_res);
+    return;
+  }
+  __syncthreads();
+
+  // this thread's share for the radix passes: entries tid, tid + 1024, ...
+  uint64_t mine[kCandPerThread];
+  uint64_t cmin = ~0ull, cmax = 0ull;
+#pragma unroll
+  for (int i = 0; i < kCandPerThread; ++i) {
+    const uint32_t v = (uint32_t)i * kSelThreads + tid;
+    const bool ok = v < n_entries;
+    mine[i] = ok ? sh_ent[v] : 0ull;
+    if (ok) {
+      cmin = mine[i] < cmin ? mine[i] : cmin;
+      cmax = mine[i] > cmax ? mine[i] : cmax;
+    }
+  }
+
+  uint64_t threshold = 0;   // selected: composite >= threshold
+  if (n_entries > k) {
+    // common prefix of all candidates: the passes start below it
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const uint64_t a = __shfl_xor(cmin, d, 64), b = __shfl_xor(cmax, d, 64);
+      cmin = a < cmin ? a : cmin;
+      cmax = b > cmax ? b : cmax;
+    }
+    if (lane == 0) { sh_wmin[wave] = cmin; sh_wmax[wave] = cmax; }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kSelWaves; ++w) {
+      const uint64_t a = sh_wmin[w], b = sh_wmax[w];
+      cmin = a < cmin ? a : cmin;
+      cmax = b > cmax ? b : cmax;
+    }
+    int fixed = __builtin_clzll(cmin ^ cmax);            // composites are distinct and n_entries >= 2: < 64
+    uint64_t prefix = fixed ? cmax >> (64 - fixed) : 0ull;
+    uint32_t need = k;
+    bool done = false;
+    while (!done) {
+      const int bits = (64 - fixed) >= kHistBits ? kHistBits : (64 - fixed);
+      const int shift = 64 - fixed - bits;
+      __syncthreads();
+      sh_hist[2 * tid] = 0;
+      sh_hist[2 * tid + 1] = 0;
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < kCandPerThread; ++i) {
+        const uint64_t c = mine[i];
+        if ((uint32_t)i * kSelThreads + tid < n_entries && (fixed == 0 || (c >> (64 - fixed)) == prefix))
+          atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
+      }
+      __syncthreads();
+      find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
+      const uint32_t d = sh_res[0], gt = sh_res[1], cnt = sh_res[2];
+      need -= gt;
+      prefix = (prefix << bits) | d;
+      fixed += bits;
+      if (cnt == need || fixed == 64) {
+        threshold = fixed == 64 ? prefix : (prefix << (64 - fixed));
+        done = true;
+      } else if (cnt <= (uint32_t)kSmallBucket) {
+        // few entries left in the threshold bucket: every wave ranks them and picks the need-th largest
+#pragma unroll
+        for (int i = 0; i < kCandPerThread; ++i) {
+          const uint64_t c = mine[i];
+          if ((uint32_t)i * kSelThreads + tid < n_entries && (c >> (64 - fixed)) == prefix) sh_small[atomicAdd(&sh_small_cnt, 1u)] = c;
+        }
+        __syncthreads();
+        const uint64_t e = (uint32_t)lane < cnt ? sh_small[lane] : 0ull;
+        uint32_t greater = 0;
+        for (uint32_t j = 0; j < cnt; ++j) greater += sh_small[j] > e ? 1u : 0u;
+        const uint64_t hit = __ballot((uint32_t)lane < cnt && greater == need - 1u);
+        threshold = __shfl(e, (int)__builtin_ctzll(hit), 64);
+        done = true;
+      }
+    }
+  }
+
+  // Walk in index order: thread t takes the run of `per` consecutive entries starting at t*per.
+  const bool want_rank = p.out_idx != nullptr;
+  const bool want_union = p.union_idx != nullptr;
+  const int64_t n = p.seg_len;
+  const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
+  const uint32_t hi = (uint32_t)(n - p.local > lo ? n - p.local : lo);
+  const uint32_t per = (n_entries + kSelThreads - 1) / kSelThreads;
+  uint64_t run[kCandPerThread];
+  uint32_t sel_mask = 0, mid_mask = 0;
+#pragma unroll
+  for (int i = 0; i < kCandPerThread; ++i) {
+    const uint32_t v = (uint32_t)tid * per + i;
+    const bool ok = (uint32_t)i < per && v < n_entries;
+    run[i] = ok ? sh_ent[v] : 0ull;
+    const bool sel = ok && run[i] >= threshold;
+    const uint32_t idx = ~(uint32_t)run[i];
+    sel_mask |= (sel ? 1u : 0u) << i;
+    mid_mask |= (sel && idx >= lo && idx < hi ? 1u : 0u) << i;
+  }
+  // one scan for both counts (each total is at most 16384)
+  uint32_t totals;
+  const uint32_t ex = block_exclusive_scan(((uint32_t)__builtin_popcount(sel_mask) << 16) | (uint32_t)__builtin_popcount(mid_mask), sh_wtot, &totals);
+  if (want_union) {
+    int32_t* uo = p.union_idx + (int64_t)seg * (p.k + p.sink + p.local);
+    uint32_t pos = lo + (ex & 0xffffu);
+#pragma unroll
+    for (int i = 0; i < kCandPerThread; ++i)
+      if (mid_mask >> i & 1u) uo[pos++] = (int32_t)~(uint32_t)run[i];
+    write_union_edges(uo, p, seg, lo, hi, totals & 0xffffu);
+  }
+  if (!want_rank) return;
+  uint64_t* sh_sort = sh_ent;
+  uint64_t* sh_xchg = sh_ent + kpad;
+  __syncthreads();   // every thread holds its run in registers: the entries may be overwritten
+  {
+    uint32_t pos = ex >> 16;
+#pragma unroll
+    for (int i = 0; i < kCandPerThread; ++i)
+      if (sel_mask >> i & 1u) sh_sort[pos++] = run[i];
+    for (int i = (int)k + tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite
+  }
   __syncthreads();
   sort_lds_desc(sh_sort, sh_xchg, kpad);
   write_rank_outputs(sh_sort, p, seg);
@@ -852,37 +850,24 @@ int launch_select_finalize(const SelectParams& p, hipStream_t stream) {
 int select_cand_max_parts() { return kCandMaxParts; }
 int select_cand_capacity() { return kCandCap; }
 
-int launch_select_finalize_cand(const SelectParams& p, hipStream_t stream) {
+int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
   if (p.parts > kCandMaxParts || p.k > kCandCap / 2) return TKA_EINVAL;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_cand_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_cand_kernel<TKA_F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        kCandCap * (int)sizeof(uint64_t));
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)select_finalize_cand_kernel<TKA_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kCandCap * (int)sizeof(uint64_t));
     if (e != hipSuccess) return TKA_EHIP;
     attr_set = true;
   }
   LaunchTimer timer("select_finalize_cand", stream);
-  select_finalize_cand_kernel<<<(unsigned)p.num_segments, kSelThreads, kCandCap * sizeof(uint64_t), stream>>>(p, kpad_for(p.k));
-  return hip_status(hipGetLastError());
-}
-
-int launch_select_fallback(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
-  const bool want_rank = p.out_idx != nullptr;
-  const int kpad = kpad_for(p.k);
-  const size_t lds = want_rank ? 2 * (size_t)kpad * sizeof(uint64_t) : 0;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)select_fallback_kernel<TKA_F16>, hipFuncAttributeMaxDynamicSharedMemorySize, 130 * 1024);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)select_fallback_kernel<TKA_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, 130 * 1024);
-    if (e != hipSuccess) return TKA_EHIP;
-    attr_set = true;
-  }
-  LaunchTimer timer("select_fallback", stream);
+  const size_t lds = kCandCap * sizeof(uint64_t);
   if (dtype == TKA_F16)
-    select_fallback_kernel<TKA_F16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad);
+    select_finalize_cand_kernel<TKA_F16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
   else
-    select_fallback_kernel<TKA_BF16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad);
+    select_finalize_cand_kernel<TKA_BF16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
   return hip_status(hipGetLastError());
 }
 
