@@ -21,6 +21,10 @@
 // No workgroup waits for another: the hand-off between 2 and 3 is the kernel boundary (a device-scope
 // fence per workgroup would write back the whole L2 of its XCD each time).
 // Traffic: 4 B read per score, 8 B written and read per listed element (about k + one bin per segment).
+//
+// Long segments skip 1 and 2: the GEMV stores only the tokens above a sampled threshold (candidate
+// slices), and select_finalize_cand_kernel does step 3 on them from LDS, or, when the slices cannot be
+// used, redoes the segment from the keys (fallback_segment).
 #include <stdlib.h>
 
 #include "kernels.hpp"
