@@ -201,3 +201,75 @@ def test_long_segment_bf16_levels_group8():
     rng = np.random.default_rng(34)
     K = oracle.to_bits(np.linspace(-2, 2, 16)[rng.integers(0, 16, (1, 262144, 1, 128))], oracle.BF16)
     _check_long(K, randn_bits(rng, (1, 8, 128), oracle.BF16), oracle.BF16, 8, 4096)
+
+
+def test_long_segment_chunked_shared_kv():
+    """Two chunks of 65536 tokens of a KV cache shared by the batch: per-chunk thresholds, per-chunk top-k."""
+    from topk_attn_amd import ops
+    announce("gemv_topk long chunks N=131072 chunks=2 k=512 shared KV B=2")
+    rng = np.random.default_rng(35)
+    dtype, N, k, chunks = oracle.F16, 131072, 512, 2
+    K = randn_bits(rng, (N, 2, 128), dtype)
+    q = randn_bits(rng, (2, 2, 128), dtype)
+    idx, val = ops.gemv_topk(to_dev(q, dtype), to_dev(K, dtype), k, group=1, scale=SCALE, num_chunks=chunks)
+    torch.cuda.synchronize()
+    idx, val = idx.cpu().numpy(), val.cpu().numpy()
+    chunk = N // chunks
+    for b in range(2):
+        for h in range(2):
+            ref = oracle.scores_canonical(K[:, h, :], dtype, oracle.group_query(q[b, h:h + 1], dtype, 1), SCALE)
+            for c in range(chunks):
+                ei, ev = oracle.topk_stable(ref[c * chunk:(c + 1) * chunk], k)
+                assert np.array_equal(idx[b, h, c * k:(c + 1) * k], ei + c * chunk), "indices differ (b=%d h=%d c=%d)" % (b, h, c)
+                assert np.array_equal(val[b, h, c * k:(c + 1) * k].view(np.uint32), ev.view(np.uint32))
+
+
+def test_long_segment_ragged_length():
+    """Segment length that is no multiple of the 256-token slice (nor of 4): the last slice is partial."""
+    announce("gemv_topk long segment N=100003 k=1500 bf16 G=2")
+    rng = np.random.default_rng(36)
+    K = randn_bits(rng, (1, 100003, 2, 128), oracle.BF16)
+    _check_long(K, randn_bits(rng, (1, 4, 128), oracle.BF16), oracle.BF16, 2, 1500)
+
+
+def test_two_level_long_clusters():
+    """Two-level selection whose clusters are long enough for the sampled-threshold path (cluster ids pick the
+    segments)."""
+    from topk_attn_amd import ops
+    announce("cluster_gemv_topk CSZ=4 CLEN=65536 TOPC=2 k=300")
+    rng = np.random.default_rng(37)
+    H, CSZ, CLEN, TOPC, K = 2, 4, 65536, 2, 300
+    cen = rng.uniform(-0.5, 0.5, (H, CSZ, 128))
+    keys = np.empty((CSZ * CLEN, H, 128), dtype=np.float32)
+    for c in range(CSZ):
+        keys[c * CLEN:(c + 1) * CLEN] = cen[:, c][None] + 0.05 * rng.standard_normal((CLEN, H, 128), dtype=np.float32)
+    cen_b, keys_b = oracle.to_bits(cen, oracle.F16), oracle.to_bits(keys, oracle.F16)
+    q_b = oracle.to_bits(rng.uniform(-0.5, 0.5, (H, 128)), oracle.F16)
+    out = ops.cluster_gemv_topk(to_dev(q_b, oracle.F16), to_dev(cen_b, oracle.F16), to_dev(keys_b, oracle.F16),
+                                TOPC, CLEN, K, 1.0)
+    torch.cuda.synchronize()
+    out = out.cpu().numpy()
+    for h in range(H):
+        want = oracle.cluster_topk(q_b[h], cen_b[h], keys_b[:, h, :], oracle.F16, TOPC, CLEN, K, 1.0)
+        assert np.array_equal(out[h], want)
+
+
+def test_long_segment_plan_reuse():
+    """One plan (one workspace) run three times with a new query each time: thresholds of an earlier run must
+    never be taken for the current one."""
+    from topk_attn_amd import ops
+    announce("gemv_topk long segment, plan reused with changing queries")
+    rng = np.random.default_rng(38)
+    dtype, N, k = oracle.F16, 80000, 1000
+    K = randn_bits(rng, (1, N, 1, 128), dtype)
+    qd = to_dev(randn_bits(rng, (1, 1, 128), dtype), dtype)
+    plan = ops.GemvTopkPlan(qd, to_dev(K, dtype), k, group=1, scale=SCALE)
+    for it in range(3):
+        q = oracle.to_bits(rng.standard_normal((1, 1, 128)) * (1.0 + it), dtype)
+        qd.copy_(to_dev(q, dtype))
+        plan.run()
+        torch.cuda.synchronize()
+        ref = oracle.scores_canonical(K[0, :, 0, :], dtype, oracle.group_query(q[0], dtype, 1), SCALE)
+        ei, ev = oracle.topk_stable(ref, k)
+        assert np.array_equal(plan.idx[0, 0].cpu().numpy(), ei), "indices differ on run %d" % it
+        assert np.array_equal(plan.val[0, 0].cpu().numpy().view(np.uint32), ev.view(np.uint32))
