@@ -498,6 +498,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   __shared__ uint32_t sh_hist[kHistBins];
   constexpr int kGroups = kSelThreads / 16, kInFlight = 8, kRound = kGroups * kInFlight;   // 512 slices per round
   __shared__ uint32_t sh_cnt[kRound], sh_start[kRound];
+  __shared__ uint32_t sh_pos[kCandMaxParts + 1];   // start positions of all slices (segments with more than kRound slices)
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
   __shared__ uint64_t sh_wmin[kSelWaves], sh_wmax[kSelWaves];
@@ -509,45 +510,88 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
 
-  // Copy the slices into LDS, kRound slices at a time: 16 lanes per slice load its first 16 entries (entry 0
-  // carries the slice's count; entries beyond the count are stale memory and ignored), the counts are
-  // scanned into start positions, and the entries go to their place.  One memory round trip per round.
+  // Copy the slices into LDS.  Up to kRound slices: 16 lanes per slice load its first 16 entries (entry 0 carries
+  // the slice's count; entries beyond the count are stale memory and ignored), the counts are scanned into
+  // start positions, and the entries go to their place: one memory round trip.
   const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
   const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
   const int sub = tid & 15, grp = tid >> 4;
   uint32_t n_entries = 0;
-  for (int s0 = 0; s0 < p.parts; s0 += kRound) {
-    uint64_t first[kInFlight];
-    uint32_t cnt[kInFlight];
+  if (p.parts <= kRound) {
+    for (int s0 = 0; s0 < p.parts; s0 += kRound) {
+      uint64_t first[kInFlight];
+      uint32_t cnt[kInFlight];
 #pragma unroll
-    for (int u = 0; u < kInFlight; ++u) {
-      const int sl = s0 + u * kGroups + grp;
-      first[u] = sl < p.parts ? lists[(int64_t)sl * p.part_len + sub] : 0ull;
-    }
+      for (int u = 0; u < kInFlight; ++u) {
+        const int sl = s0 + u * kGroups + grp;
+        first[u] = sl < p.parts ? lists[(int64_t)sl * p.part_len + sub] : 0ull;
+      }
 #pragma unroll
-    for (int u = 0; u < kInFlight; ++u) {
-      cnt[u] = ((uint32_t)__shfl((int)(uint32_t)first[u], lane & ~15, 64) >> 8) & 0x1ffu;
-      if (sub == 0) sh_cnt[u * kGroups + grp] = cnt[u];
+      for (int u = 0; u < kInFlight; ++u) {
+        cnt[u] = ((uint32_t)__shfl((int)(uint32_t)first[u], lane & ~15, 64) >> 8) & 0x1ffu;
+        if (sub == 0) sh_cnt[u * kGroups + grp] = cnt[u];
+      }
+      __syncthreads();
+      uint32_t total;
+      const uint32_t c = tid < kRound ? sh_cnt[tid] : 0u;
+      const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
+      if (tid < kRound) sh_start[tid] = n_entries + ex;
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const int sl = s0 + u * kGroups + grp;
+        const uint32_t start = sh_start[u * kGroups + grp];
+        const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
+        if ((uint32_t)sub < cnt[u] && start + sub < cap)
+          sh_ent[start + sub] = (first[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)first[u] & 0xffu));
+        for (uint32_t j = 16u + sub; j < cnt[u] && start + j < cap; j += 16u) {   // rare: a slice with more than 16 candidates
+          const uint64_t w = lists[(int64_t)sl * p.part_len + j];
+          sh_ent[start + j] = (w & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w & 0xffu));
+        }
+      }
+      n_entries += total;
     }
-    __syncthreads();
+  } else {
+    // many slices: all counts first (one round trip), one scan, then the entries with no barrier in between
+    uint32_t c4[4], sum = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int sl = 4 * tid + q;
+      c4[q] = sl < p.parts ? ((uint32_t)lists[(int64_t)sl * p.part_len] >> 8) & 0x1ffu : 0u;
+      sum += c4[q];
+    }
     uint32_t total;
-    const uint32_t c = tid < kRound ? sh_cnt[tid] : 0u;
-    const uint32_t ex = block_exclusive_scan(c, sh_wtot, &total);
-    if (tid < kRound) sh_start[tid] = n_entries + ex;
-    __syncthreads();
+    uint32_t running = block_exclusive_scan(sum, sh_wtot, &total);
 #pragma unroll
-    for (int u = 0; u < kInFlight; ++u) {
-      const int sl = s0 + u * kGroups + grp;
-      const uint32_t start = sh_start[u * kGroups + grp];
-      const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
-      if ((uint32_t)sub < cnt[u] && start + sub < cap)
-        sh_ent[start + sub] = (first[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)first[u] & 0xffu));
-      for (uint32_t j = 16u + sub; j < cnt[u] && start + j < cap; j += 16u) {   // rare: a slice with more than 16 candidates
-        const uint64_t w = lists[(int64_t)sl * p.part_len + j];
-        sh_ent[start + j] = (w & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w & 0xffu));
+    for (int q = 0; q < 4; ++q) {
+      sh_pos[4 * tid + q] = running;
+      running += c4[q];
+    }
+    if (tid == kSelThreads - 1) sh_pos[kCandMaxParts] = total;
+    n_entries = total;
+    __syncthreads();
+    for (int s0 = 0; s0 < p.parts; s0 += kRound) {
+      uint64_t w[kInFlight];
+      uint32_t start[kInFlight], cnt[kInFlight];
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const int sl = s0 + u * kGroups + grp;
+        start[u] = sl < p.parts ? sh_pos[sl] : 0u;
+        cnt[u] = sl < p.parts ? sh_pos[sl + 1] - start[u] : 0u;
+        w[u] = (uint32_t)sub < cnt[u] ? lists[(int64_t)sl * p.part_len + sub] : 0ull;
+      }
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const int sl = s0 + u * kGroups + grp;
+        const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
+        if ((uint32_t)sub < cnt[u] && start[u] + sub < cap)
+          sh_ent[start[u] + sub] = (w[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w[u] & 0xffu));
+        for (uint32_t j = 16u + sub; j < cnt[u] && start[u] + j < cap; j += 16u) {
+          const uint64_t x = lists[(int64_t)sl * p.part_len + j];
+          sh_ent[start[u] + j] = (x & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)x & 0xffu));
+        }
       }
     }
-    n_entries += total;
   }
   const bool redo = n_entries < k || n_entries > cap;
   if (tid == 0) {
