@@ -132,7 +132,7 @@ def test_two_level_cluster_reference_shape():
             assert set(out[h, r * K:(r + 1) * K]) == set(want[r * K:(r + 1) * K])
 
 
-# ---- long segments: sampled threshold + candidate lists, with the dense path as fallback ------------------
+# ---- long segments: sampled threshold + candidate slices; a segment they fail is redone from the keys ----
 
 def _mix32(x):
     x &= 0xFFFFFFFF
@@ -142,15 +142,11 @@ def _mix32(x):
     return x
 
 
-def _sampled_positions(seg, n, samples=512, split=4):
-    """Token positions the threshold estimate of a long segment looks at: `samples` per quarter of the segment,
-    one per stride, at a hashed offset inside the stride."""
-    stride = n // split // samples
-    pos = []
-    for quarter in range(split):
-        salt = ((seg * split + quarter) * 0x9e3779b9) & 0xFFFFFFFF
-        pos += [quarter * (n // split) + i * stride + _mix32((salt + i) & 0xFFFFFFFF) % stride for i in range(samples)]
-    return pos
+def _sampled_positions(seg, n, samples=2048):
+    """Token positions the threshold estimate of a long segment looks at: one per stride of n/samples tokens, at a
+    hashed offset inside the stride (2048 samples for segments below 512K tokens)."""
+    stride = n // samples
+    return [i * stride + _mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) % stride for i in range(samples)]
 
 
 def _check_long(K, q, dtype, G, k, scale=SCALE):
@@ -176,7 +172,7 @@ def test_long_segment_candidates():
 
 
 def test_long_segment_all_equal_falls_back():
-    """Every key equal: every token passes the sampled threshold, the segment is redone by the dense path."""
+    """Every key equal: every token passes the sampled threshold, the segment is redone from the keys."""
     announce("gemv_topk long segment all keys equal (fallback: too many candidates)")
     rng = np.random.default_rng(32)
     K = np.broadcast_to(randn_bits(rng, (1, 1, 1, 128), oracle.BF16), (1, 70001, 2, 128)).copy()
@@ -185,7 +181,7 @@ def test_long_segment_all_equal_falls_back():
 
 def test_long_segment_sample_hits_only_heavy_tokens_falls_back():
     """Heavy tokens placed exactly where the threshold estimate samples: the threshold lands among them, fewer than
-    k tokens pass, and the segment is redone by the dense path.  One head is adversarial, the other ordinary."""
+    k tokens pass, and the segment is redone from the keys.  One head is adversarial, the other ordinary."""
     announce("gemv_topk long segment adversarial sample (fallback: too few candidates)")
     rng = np.random.default_rng(33)
     N, k, dtype = 131072, 4096, oracle.F16

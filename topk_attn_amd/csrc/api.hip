@@ -126,6 +126,8 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->num_chunks = a->num_chunks;
   g->scale = a->scale;
   g->tau_words = nullptr;
+  g->sample_flags = nullptr;
+  g->sample_pool = nullptr;
   g->epoch = 0;
   g->num_samples = g->sample_rank = g->sample_wgs = g->early_wgs = 0;
   g->cand = nullptr;
@@ -198,6 +200,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   GemvParams cp = gp;
   cp.hist = nullptr;
   cp.tau_words = sp.tau_words;
+  cp.sample_flags = sp.sample_flags;
+  cp.sample_pool = sp.sample_pool;
   cp.epoch = call_counter.fetch_add(1, std::memory_order_relaxed) | 0x80000000u;   // never 0, the cleared state
   cp.num_samples = num_samples;
   cp.sample_rank = sample_rank;

@@ -20,8 +20,7 @@ constexpr int kWave = 64;
 constexpr int kHistBits = 11;
 constexpr int kHistBins = 1 << kHistBits;  // first-level selection histogram: top 11 bits of the key
 constexpr int kGemvCandTokensPerWg = 256;  // tokens per GEMV workgroup on large problems (= slice length of candidate lists)
-constexpr int kGemvMaxSamples = 2048;        // most samples per quarter segment of the candidate-mode threshold estimate
-constexpr int kGemvMaxSamplesInline = 512;   // samples per quarter that the streaming launch takes itself
+constexpr int kGemvMaxSamples = 8192;      // most samples per segment of the candidate-mode threshold estimate
 
 // ---- lane exchanges ---------------------------------------------------------------------------
 

@@ -16,9 +16,9 @@
 //              in the workgroup's own slice (the count rides in the first entry: one partial line per
 //              workgroup).  The selection kernel checks that at least k tokens passed and otherwise flags
 //              the segment for the fallback kernel, so the result is exact whatever the data.
-//              The sampling runs inside the same launch: the first workgroups of the grid score the samples
-//              and publish the thresholds, the streaming workgroups need them only when their rows are
-//              scored and wait (bounded) for them then.
+//              The sampling runs inside the same launch: the first workgroups of the grid score the samples,
+//              the last of them to finish publishes the threshold, and the streaming workgroups need it only
+//              when their rows are scored and wait (bounded) for it then.
 #include "kernels.hpp"
 
 namespace tka {
@@ -29,9 +29,8 @@ constexpr int kGemvThreads = 256;
 constexpr int kGemvWaves = kGemvThreads / kWave;
 constexpr int kGemvUnroll = 8;                                         // loads in flight per lane
 constexpr int kGemvRowsPerIter = (kGemvThreads / 16) * kGemvUnroll;    // 128 tokens per WG iteration
-constexpr int kTauSplit = 4;           // sampling workgroups (and thresholds) per segment
-constexpr int kTauSpinLimit = 1 << 16;
-constexpr int kEarlySlices = 3;       // slices of a streaming workgroup that starts before the thresholds are published // polls of a streaming workgroup for its thresholds before it gives up
+constexpr int kTauSpinLimit = 1 << 16; // polls of a streaming workgroup for its threshold before it gives up
+constexpr int kEarlySlices = 3;        // slices of a streaming workgroup that starts before the threshold is published
 static_assert(kGemvCandTokensPerWg == kGemvThreads, "candidate mode: one thread per token in the epilogue");
 
 template <int DT>
@@ -106,26 +105,26 @@ __device__ __forceinline__ uint32_t mix32(uint32_t x) {  // integer hash for the
   return x;
 }
 
-// Token (inside its quarter of the segment) of sample i: one per stride, at a hashed offset inside the stride
-// so that periodic data cannot alias with the sampling.
-__device__ __forceinline__ int64_t sample_token(int seg, int quarter, int i, int64_t stride) {
-  return (int64_t)i * stride + (int64_t)(mix32(((uint32_t)seg * kTauSplit + quarter) * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
+// Token of sample i of a segment: one per stride, at a hashed offset inside the stride so that periodic data
+// cannot alias with the sampling.
+__device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) {
+  return (int64_t)i * stride + (int64_t)(mix32((uint32_t)seg * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
 }
 
-// A threshold word is (epoch << 32) | key: the epoch of the call tells a published threshold from whatever
-// the workspace held before.
-__device__ __forceinline__ void publish_tau(uint64_t* word, uint32_t epoch, uint32_t key) {
-  __hip_atomic_store(word, ((uint64_t)epoch << 32) | key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Sampling workgroup (256 threads) of one quarter of one segment: scores p.num_samples tokens and publishes the
-// p.sample_rank-th largest key.  About sample_rank/num_samples of the quarter's tokens lie at or above that key
-// wherever the large scores sit in the segment.  sh: num_samples + 256 + 8 words.
+// Sampling workgroup (256 threads): scores 128 of the segment's p.num_samples sample tokens (one round of
+// loads) and stores their keys in the segment's pool.  The workgroup that arrives last (epoch-valued arrival
+// flags, so that the workspace needs no clearing) takes the p.sample_rank-th largest key of the whole pool and
+// publishes it as the segment's threshold word, (epoch << 32) | key.  The sample is spread evenly over the
+// segment, so about sample_rank/num_samples of the segment's tokens lie at or above that key wherever the
+// large scores sit.
+// Ordering between workgroups: the keys are agent-scope atomic stores, their completion and a barrier precede
+// the workgroup's arrival flag; the last workgroup reads the pool with agent-scope atomic loads after it has
+// seen every flag.
+// sh: 2048 + 8 words.
 template <int DT>
-__device__ __forceinline__ void sample_quarter(const GemvParams& p, int seg, int quarter, uint32_t* sh) {
-  uint32_t* sh_keys = sh;
-  uint32_t* sh_hist = sh + p.num_samples;   // 256 bins
-  uint32_t* sh_wtot = sh_hist + 256;        // 4 wave totals, then bin and count above it
+__device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int part, uint32_t* sh) {
+  uint32_t* sh_hist = sh;                   // 2048 bins
+  uint32_t* sh_wtot = sh_hist + kHistBins;  // 4 wave totals, bin and count above it, "last" flag
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int j = tid & 15, rg = tid >> 4;
@@ -134,37 +133,76 @@ __device__ __forceinline__ void sample_quarter(const GemvParams& p, int seg, int
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
   float qf[8];
   load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
-  const int64_t quarter_len = p.chunk_len / kTauSplit;
-  const int64_t stride = quarter_len / p.num_samples;
+  const int64_t stride = p.chunk_len / p.num_samples;
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
-                          (chunk_base + (int64_t)quarter * quarter_len) * p.key_stride_n + 8 * j;
-  for (int base = 0; base < p.num_samples; base += kGemvRowsPerIter) {
+                          chunk_base * p.key_stride_n + 8 * j;
+  uint32_t* pool = p.sample_pool + (int64_t)seg * p.num_samples;
+  {
+    const int first = part * kGemvRowsPerIter + rg * kGemvUnroll;
     u32x4 kv[kGemvUnroll];
 #pragma unroll
     for (int u = 0; u < kGemvUnroll; ++u)
-      kv[u] = *(const u32x4*)(kbase + sample_token(seg, quarter, base + rg * kGemvUnroll + u, stride) * p.key_stride_n);
+      kv[u] = *(const u32x4*)(kbase + sample_token(seg, first + u, stride) * p.key_stride_n);
     float mine = 0.0f;
 #pragma unroll
     for (int u = 0; u < kGemvUnroll; ++u) {
-      const float s = row_score<DT>(qf, kv[u], p.scale);
-      if (j == u) mine = s;
+      const float sc = row_score<DT>(qf, kv[u], p.scale);
+      if (j == u) mine = sc;
     }
-    if (j < kGemvUnroll) sh_keys[base + rg * kGemvUnroll + j] = score_key(mine);
+    if (j < kGemvUnroll) __hip_atomic_store(pool + first + j, score_key(mine), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  // sample_rank-th largest key: four 8-bit radix passes, thread t owns bin t
+  // The keys went out as agent-scope atomic stores (performed at the point of coherence); what the counter
+  // update needs is that they have completed, not a write-back of the L2 (an agent-scope release fence walks
+  // the whole L2 every time a wave executes it: 4096 of them cost 150 us here).
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's key stores have completed
+  __syncthreads();
+  if (wave == 0) {
+    // Arrival flags, one word per sampling workgroup (a shared counter costs 0.4 us per arrival: the adds to
+    // one word are served one after the other).  Set my flag, wait until it has completed, read all flags:
+    // of two workgroups that finish together at least the one whose flag completed later sees both, so
+    // somebody always sees all of them; if two do, both publish the same threshold.
+    const int parts = p.num_samples / kGemvRowsPerIter;   // <= 64
+    uint32_t* flags = p.sample_flags + (int64_t)seg * (kGemvMaxSamples / kGemvRowsPerIter);
+    if (lane == 0) __hip_atomic_store(flags + part, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const uint32_t f = lane < parts ? __hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : p.epoch;
+    const bool all = __ballot(f == p.epoch) == ~0ull;
+    if (lane == 0) sh_wtot[6] = all ? 1u : 0u;
+  }
+  __syncthreads();
+  if (sh_wtot[6] == 0u) return;
+
+  // sample_rank-th largest key of the pool, to its top 22 bits (the threshold only has to lie at or below that
+  // order statistic): two 11-bit radix passes, thread t owns bins 8t .. 8t+7
+  // the pool once into registers, all loads in flight together (one at a time they cost 2-3 us each)
+  constexpr int kPerThread = kGemvMaxSamples / kGemvThreads;
+  uint32_t keys[kPerThread];
+#pragma unroll
+  for (int u = 0; u < kPerThread; ++u) {
+    const int i = u * kGemvThreads + tid;
+    keys[u] = i < p.num_samples ? __hip_atomic_load(pool + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+  }
   uint32_t need = (uint32_t)p.sample_rank, prefix = 0;
-  for (int pass = 0; pass < 4; ++pass) {
-    const int shift = 24 - 8 * pass;
+  for (int pass = 0; pass < 2; ++pass) {
+    const int shift = pass ? 32 - 2 * kHistBits : 32 - kHistBits;
     __syncthreads();
-    sh_hist[tid] = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sh_hist[8 * tid + e] = 0;
     __syncthreads();
-    for (int i = tid; i < p.num_samples; i += kGemvThreads) {
-      const uint32_t key = sh_keys[i];
-      if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&sh_hist[(key >> shift) & 255u], 1u);
+#pragma unroll
+    for (int u = 0; u < kPerThread; ++u) {
+      const uint32_t key = keys[u];
+      if (u * kGemvThreads + tid < p.num_samples && (pass == 0 || (key >> (32 - kHistBits)) == prefix))
+        atomicAdd(&sh_hist[(key >> shift) & (kHistBins - 1)], 1u);
     }
     __syncthreads();
-    const uint32_t mine = sh_hist[tid];
-    uint32_t ge = mine;   // count in bins >= tid, first inside the wave
+    uint32_t h[8], mine = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      h[e] = sh_hist[8 * tid + e];
+      mine += h[e];
+    }
+    uint32_t ge = mine;   // count in the bins of threads >= tid, first inside the wave
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
       const uint32_t t = __shfl_down(ge, d, 64);
@@ -173,12 +211,25 @@ __device__ __forceinline__ void sample_quarter(const GemvParams& p, int seg, int
     if (lane == 0) sh_wtot[wave] = ge;
     __syncthreads();
     for (int w = wave + 1; w < kGemvWaves; ++w) ge += sh_wtot[w];
-    if (ge >= need && ge - mine < need) { sh_wtot[4] = (uint32_t)tid; sh_wtot[5] = ge - mine; }
+    if (ge >= need && ge - mine < need) {   // the bin sits among this thread's eight: walk them from the top
+      uint32_t above = ge - mine;
+      int bin = 0;
+      bool found = false;
+#pragma unroll
+      for (int e = 7; e >= 0; --e) {
+        if (!found && above + h[e] >= need) { bin = 8 * tid + e; found = true; }
+        if (!found) above += h[e];
+      }
+      sh_wtot[4] = (uint32_t)bin;
+      sh_wtot[5] = above;
+    }
     __syncthreads();
-    prefix = (prefix << 8) | sh_wtot[4];
+    prefix = (prefix << kHistBits) | sh_wtot[4];
     need -= sh_wtot[5];
   }
-  if (tid == 0) publish_tau(p.tau_words + (int64_t)seg * kTauSplit + quarter, p.epoch, prefix);
+  prefix <<= 32 - 2 * kHistBits;
+  if (tid == 0)
+    __hip_atomic_store(p.tau_words + seg, ((uint64_t)p.epoch << 32) | prefix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Scores of one slice (up to 256 tokens from sbase on) as keys into LDS: lane j < 8 of row group rg writes the
@@ -223,16 +274,18 @@ __device__ __forceinline__ void stream_slice(const unsigned char* sbase, uint32_
 // thresholds arrive; with more rows to stream they reach that point when the thresholds are there.
 template <int DT>
 __global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void gemv_candidates_kernel(GemvParams p) {
-  __shared__ uint32_t sh[(kEarlySlices * kGemvThreads > kGemvMaxSamplesInline + 256 ? kEarlySlices * kGemvThreads : kGemvMaxSamplesInline + 256) + 8];
+  __shared__ uint32_t sh[kHistBins + 8];   // streaming: keys of kEarlySlices * 256 tokens + wave counts; sampling: histogram
+  static_assert(kEarlySlices * kGemvThreads <= kHistBins, "LDS of the streaming role");
   const int tid = threadIdx.x;
   if ((int)blockIdx.x < p.sample_wgs) {
     __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
-    sample_quarter<DT>(p, (int)blockIdx.x / kTauSplit, (int)blockIdx.x % kTauSplit, sh);
+    const int parts = p.num_samples / kGemvRowsPerIter;
+    sample_role<DT>(p, (int)blockIdx.x / parts, (int)blockIdx.x % parts, sh);
     return;
   }
   uint32_t* sh_key = sh;                               // keys of this workgroup's tokens, slice after slice
   uint32_t* sh_wcnt = sh + kEarlySlices * kGemvThreads; // candidates per wave
-  __shared__ uint32_t sh_tau[2 * kTauSplit];            // the segment's thresholds and whether each one has arrived
+  __shared__ uint32_t sh_tau[2];                        // the segment's threshold and whether it has arrived
 
   const int j = tid & 15;            // lane inside the row: dims 8j..8j+7
   const int rg = tid >> 4;           // row group 0..15 inside the workgroup
@@ -278,31 +331,25 @@ __global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8,
     const int64_t t_begin = (int64_t)wg_in_chunk * kGemvThreads;
     int64_t t_end = t_begin + kGemvThreads;
     if (t_end > p.chunk_len) t_end = p.chunk_len;
-    // Thresholds of the slice's segment: lanes 0..3 fetch one word each and hand them on through LDS (every
-    // wave asking for itself makes a hot spot of the few words).  A bounded wait: a workgroup that never sees
-    // its thresholds stores no candidates, and the selection kernel then flags the segment for the fallback
-    // kernel.
+    // Threshold of the slice's segment: one lane fetches the word and hands it on through LDS (every wave
+    // asking for itself makes a hot spot of the few words).  A bounded wait: a workgroup that never sees its
+    // threshold stores no candidates, and the selection kernel then redoes the segment from the keys.
     if (s == 0 || seg != tau_seg) {
       tau_seg = seg;
-      if (s) __syncthreads();   // the previous slice's thresholds have been read
-      if (tid < kTauSplit) {
-        const uint64_t* word = p.tau_words + seg * kTauSplit + tid;
+      if (s) __syncthreads();   // the previous slice's threshold has been read
+      if (tid == 0) {
+        const uint64_t* word = p.tau_words + seg;
         uint64_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         for (int spin = 0; (uint32_t)(v >> 32) != p.epoch && spin < kTauSpinLimit; ++spin) {
           __builtin_amdgcn_s_sleep(16);
           v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        sh_tau[tid] = (uint32_t)v;
-        sh_tau[kTauSplit + tid] = (uint32_t)(v >> 32) == p.epoch ? 1u : 0u;
+        sh_tau[0] = (uint32_t)v;
+        sh_tau[1] = (uint32_t)(v >> 32) == p.epoch ? 1u : 0u;
       }
       __syncthreads();
-      tau = ~0u;
-      tau_ready = true;
-#pragma unroll
-      for (int q = 0; q < kTauSplit; ++q) {   // lowest of the four: every quarter then passes at least its own share
-        tau = min(tau, sh_tau[q]);
-        tau_ready = tau_ready && sh_tau[kTauSplit + q] != 0u;
-      }
+      tau = sh_tau[0];
+      tau_ready = sh_tau[1] != 0u;
     }
 
     // thread t owns token t_begin + t: candidates in index order into the slice.
@@ -331,80 +378,6 @@ __global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8,
   }
 }
 
-// ---- stand-alone sampling kernel (long segments: more samples than the streaming grid's workgroups take) --
-
-constexpr int kTauThreads = 1024;
-constexpr int kTauRowGroups = kTauThreads / 16;
-constexpr int kTauUnroll = 8;            // rows per row group and round: 512 samples per round
-
-// kTauSplit workgroups of 1024 threads per segment: as sample_quarter, for 1024 or 2048 samples per quarter.
-template <int DT>
-__global__ __launch_bounds__(kTauThreads) void sample_tau_kernel(GemvParams p) {
-  const int num_samples = p.num_samples, sample_rank = p.sample_rank;
-  __shared__ uint32_t sh_keys[kGemvMaxSamples];
-  __shared__ uint32_t sh_hist[kHistBins];
-  __shared__ uint32_t sh_wtot[kTauThreads / kWave];
-  __shared__ uint32_t sh_res[4];
-
-  const int tid = threadIdx.x;
-  const int j = tid & 15, rg = tid >> 4;
-  const int seg = blockIdx.y;
-  const int quarter = blockIdx.x;
-  const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
-  const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
-  const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
-
-  float qf[8];
-  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
-  const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
-                          chunk_base * p.key_stride_n + 8 * j;
-  const int64_t quarter_len = p.chunk_len / kTauSplit;
-  const int64_t stride = quarter_len / num_samples;
-  kbase += (int64_t)quarter * quarter_len * p.key_stride_n;
-
-  // kTauUnroll rows in flight per row group: the kernel is one latency chain per batch of loads
-  for (int base = 0; base < num_samples; base += kTauRowGroups * kTauUnroll) {
-    u32x4 kv[kTauUnroll];
-#pragma unroll
-    for (int u = 0; u < kTauUnroll; ++u) {
-      const int i = base + rg * kTauUnroll + u;                        // sample number (num_samples is a multiple of 512)
-      const int64_t t = sample_token(seg, quarter, i, stride);
-      kv[u] = *(const u32x4*)(kbase + t * p.key_stride_n);
-    }
-    float mine = 0.0f;
-#pragma unroll
-    for (int u = 0; u < kTauUnroll; ++u) {
-      const float s = row_score<DT>(qf, kv[u], p.scale);
-      if (j == u) mine = s;
-    }
-    if (j < kTauUnroll) sh_keys[base + rg * kTauUnroll + j] = score_key(mine);
-  }
-
-  // sample_rank-th largest of sh_keys[0 .. num_samples), resolved to its top 22 bits: the threshold only has
-  // to lie at or below that order statistic, so the low 10 bits are left at zero
-  uint32_t need = (uint32_t)sample_rank, prefix = 0;
-  int fixed = 0;
-  while (fixed < 2 * kHistBits) {
-    const int bits = kHistBits;
-    const int shift = 32 - fixed - bits;
-    __syncthreads();
-    sh_hist[2 * tid] = 0;
-    sh_hist[2 * tid + 1] = 0;
-    __syncthreads();
-    for (int i = tid; i < num_samples; i += kTauThreads) {
-      const uint32_t key = sh_keys[i];
-      if (fixed == 0 || (key >> (32 - fixed)) == prefix) atomicAdd(&sh_hist[(key >> shift) & ((1u << bits) - 1u)], 1u);
-    }
-    __syncthreads();
-    find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
-    need -= sh_res[1];
-    prefix = (prefix << bits) | sh_res[0];
-    fixed += bits;
-  }
-  prefix <<= (32 - fixed);
-  if (tid == 0) publish_tau(p.tau_words + (int64_t)seg * kTauSplit + quarter, p.epoch, prefix);
-}
-
 }  // namespace
 
 int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
@@ -417,28 +390,17 @@ int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
   return hip_status(hipGetLastError());
 }
 
-// Candidate mode.  p.num_samples <= kGemvMaxSamplesInline: the sampling workgroups are part of the launch;
-// more: the stand-alone sampling kernel goes first.
+// Candidate mode: sampling workgroups (128 samples each) at the front of the grid, then the streaming ones.
 int launch_gemv_candidates(const GemvParams& p0, int dtype, hipStream_t stream) {
   GemvParams p = p0;
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  if (p.tokens_per_wg != kGemvThreads || p.num_samples < 1 || p.num_samples % kGemvRowsPerIter) return TKA_EINVAL;
-  if (p.num_samples > kGemvMaxSamplesInline) {
-    if (p.num_samples > kGemvMaxSamples || p.num_samples % (kTauRowGroups * kTauUnroll)) return TKA_EINVAL;
-    const dim3 grid(kTauSplit, (unsigned)segs);
-    LaunchTimer timer("sample_tau", stream);
-    if (dtype == TKA_F16)
-      sample_tau_kernel<TKA_F16><<<grid, kTauThreads, 0, stream>>>(p);
-    else
-      sample_tau_kernel<TKA_BF16><<<grid, kTauThreads, 0, stream>>>(p);
-    if (hipGetLastError() != hipSuccess) return TKA_EHIP;
-    p.sample_wgs = 0;
-  } else {
-    p.sample_wgs = (int)(segs * kTauSplit);
-  }
-  // early workgroups: as many as the GPU holds at once (256 CUs x 8), when the sampling runs beside them
+  if (p.tokens_per_wg != kGemvThreads || p.num_samples < kGemvRowsPerIter || p.num_samples % kGemvRowsPerIter ||
+      p.num_samples > kGemvMaxSamples || p.sample_rank < 1 || p.sample_rank > p.num_samples)
+    return TKA_EINVAL;
+  p.sample_wgs = (int)(segs * (p.num_samples / kGemvRowsPerIter));
+  // early workgroups: as many as the GPU holds at once (256 CUs x 8)
   const int64_t slices = segs * p.wgs_per_chunk;
-  int64_t early = p.sample_wgs ? 2048 : 0;
+  int64_t early = 2048;
   if (early > slices / (2 * kEarlySlices)) early = slices / (2 * kEarlySlices);
   p.early_wgs = (int)early;
   const int64_t wgs = p.sample_wgs + early + (slices - early * kEarlySlices);
@@ -459,26 +421,25 @@ int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len) {
   return total_rows <= 65536 ? 128 : kGemvCandTokensPerWg;
 }
 
-// Candidate-mode plan for one segment length and k: samples per sampling workgroup and the rank of the order
-// statistic each of them takes as its threshold, or 0 samples when pruning does not pay (short segments, k a
-// large share of the segment, more candidates than the selection kernel holds).
-// With S = kTauSplit * s samples in all and m = k*S/n, R = m + 6*sqrt(m) + 2 is the total rank: the share of
-// tokens that pass concentrates around R/S with relative deviation 1/sqrt(R), which puts "fewer than k pass"
-// (the segment is then redone densely) four to five deviations out.  Taking the lowest of the four
-// thresholds passes about a quarter more than R/S.
+// Candidate-mode plan for one segment length and k: samples per segment and the rank of the order statistic
+// that becomes the threshold, or 0 samples when pruning does not pay (short segments, k a large share of the
+// segment, more candidates than the selection kernel holds).
+// With S samples spread evenly over the n tokens and m = k*S/n, the rank is R = m + 6*sqrt(m) + 2.  The share of
+// tokens at or above the R-th largest sample concentrates around R/S with relative deviation 1/sqrt(R), so
+// "fewer than k pass" (the segment is then redone from the keys) lies more than four deviations out, and about
+// n*R/S candidates are stored.
 void gemv_candidate_plan(int64_t chunk_len, int k, int max_candidates, int* num_samples, int* sample_rank) {
   *num_samples = 0;
   *sample_rank = 0;
   if (chunk_len < 65536 || (int64_t)k * 16 > chunk_len) return;
-  const int rounds = chunk_len >= 1048576 ? 4 : (chunk_len >= 524288 ? 2 : 1);   // more samples on long segments keep the candidate share near k/n
-  const int s = kGemvMaxSamplesInline * rounds;
-  const double S = (double)s * kTauSplit;
-  const double m = (double)k * S / (double)chunk_len;
+  // more samples on long segments keep the candidate count near k
+  const int s = chunk_len >= 1048576 ? kGemvMaxSamples : (chunk_len >= 524288 ? kGemvMaxSamples / 2 : kGemvMaxSamples / 4);
+  const double m = (double)k * s / (double)chunk_len;
   double root = 0.0;
   while ((root + 1.0) * (root + 1.0) <= m) root += 1.0;   // floor(sqrt(m))
-  const int r = ((int)(m + 6.0 * (root + 1.0) + 2.0) + kTauSplit - 1) / kTauSplit;
-  const double expected = (double)chunk_len * r / s * 1.25;
-  if (expected * 1.3 > (double)max_candidates) return;
+  const int r = (int)(m + 6.0 * (root + 1.0) + 2.0);
+  const double expected = (double)chunk_len * r / s;
+  if (expected * 1.5 > (double)max_candidates) return;
   *num_samples = s;
   *sample_rank = r;
 }

@@ -11,10 +11,12 @@ struct GemvParams {
   float* scores;        // [batch][num_kv_heads][num_chunks][chunk_len]; selection kernels also read them
   const int32_t* cluster_ids;  // [batch*num_kv_heads*num_chunks] or nullptr: chunk c covers the tokens of that cluster
   uint32_t* hist;       // [batch*num_kv_heads*num_chunks][kHistBins] or nullptr; must be zero on entry
-  // candidate mode: only tokens whose key reaches the lowest of the segment's four thresholds are stored
-  uint64_t* tau_words;        // [segments][4] (epoch << 32) | threshold key, one per sampled quarter
-  uint32_t epoch;             // tells this call's thresholds from older contents of tau_words (never 0)
-  int num_samples, sample_rank;   // per quarter
+  // candidate mode: only tokens whose key reaches the segment's sampled threshold are stored
+  uint64_t* tau_words;        // [segments] (epoch << 32) | threshold key
+  uint32_t* sample_flags;     // [segments][64] epoch of the call in which that sampling workgroup last arrived
+  uint32_t* sample_pool;      // [segments][num_samples] keys of the sampled tokens
+  uint32_t epoch;             // tells this call's words from older contents of the workspace (never 0)
+  int num_samples, sample_rank;   // per segment
   int sample_wgs;             // sampling workgroups at the front of the candidate grid (set by the launcher)
   int early_wgs;              // streaming workgroups behind them that take several slices each (set by the launcher)
   uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] one slice per workgroup, ascending index:
@@ -37,7 +39,9 @@ struct SelectParams {
   int64_t seg_len;
   int64_t seg_stride;
   uint32_t* hist;         // [num_segments][kHistBins]; nullptr: the lists hold candidates above a sampled threshold
-  uint64_t* tau_words;    // [num_segments][4] candidate thresholds (workspace); the candidate selection kernel clears them
+  uint64_t* tau_words;    // [num_segments] candidate thresholds (workspace); the candidate selection kernel clears them
+  uint32_t* sample_flags; // [num_segments][64] arrival flags of the sampling workgroups (workspace)
+  uint32_t* sample_pool;  // [num_segments][kGemvMaxSamples] sampled keys (workspace)
   uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment was redone from the keys
   int max_entries;        // candidate mode: a segment with more candidates than this is also redone from the keys
   uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)

@@ -598,8 +598,10 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     p.seg_flags[seg] = redo ? 1u : 0u;
     sh_small_cnt = 0;
   }
-  // the thresholds are spent: a replay of the same launches (a captured graph) must not take them for its own
-  if (tid < 4) p.tau_words[(int64_t)seg * 4 + tid] = 0ull;
+  // the threshold and the arrival flags are spent: a replay of the same launches (a captured graph) must not
+  // take them for its own
+  if (tid >= 64 && tid < 128) p.sample_flags[(int64_t)seg * 64 + (tid - 64)] = 0u;
+  if (tid == 0) p.tau_words[seg] = 0ull;
   if (redo) {
     __syncthreads();
     fallback_segment<DT>(g, p, seg, kpad, sh_ent, sh_hist, sh_wtot, sh_res);
@@ -802,11 +804,11 @@ int kpad_for(int k) {
 }  // namespace
 
 // Workspace layout (each part 256-byte aligned):
-//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S][4] u64 | list_cnt [S][slices] u32 |
+//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S] u64 | arrival flags [S][64] u32 | sample pool [S][8192] u32 | list_cnt [S][slices] u32 |
 //   list [S][slices*slice_len] u64      (slices: dense 4096/16384 scores, candidate mode one per GEMV workgroup)
 namespace {
 struct SelectLayout {
-  size_t hist, flags, tau, list_cnt, list, total;
+  size_t hist, flags, tau, ctr, pool, list_cnt, list, total;
   int64_t list_stride;
 };
 SelectLayout select_layout(int num_segments, int64_t seg_len) {
@@ -817,7 +819,9 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   l.list_stride = (seg_len + 16 * kSelThreads - 1) / (16 * kSelThreads) * (16 * kSelThreads);  // whole slices
   l.hist = take((size_t)num_segments * kHistBins * sizeof(uint32_t));
   l.flags = take((size_t)num_segments * sizeof(uint32_t));
-  l.tau = take((size_t)num_segments * 4 * sizeof(uint64_t));   // one threshold word per sampled quarter
+  l.tau = take((size_t)num_segments * sizeof(uint64_t));
+  l.ctr = take((size_t)num_segments * 64 * sizeof(uint32_t));
+  l.pool = take((size_t)num_segments * kGemvMaxSamples * sizeof(uint32_t));
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
   l.total = off;
@@ -834,6 +838,8 @@ size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p
   p->hist = (uint32_t*)(c + l.hist);
   p->seg_flags = (uint32_t*)(c + l.flags);
   p->tau_words = (uint64_t*)(c + l.tau);
+  p->sample_flags = (uint32_t*)(c + l.ctr);
+  p->sample_pool = (uint32_t*)(c + l.pool);
   p->list_cnt = (uint32_t*)(c + l.list_cnt);
   p->list = (uint64_t*)(c + l.list);
   p->list_stride = l.list_stride;
