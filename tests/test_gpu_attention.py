@@ -266,3 +266,9 @@ def test_sparse_decode_step_union_only(dtype, B, H, G, N, k, sink, local, kind, 
                                                        local, SCALE)
             assert ucnt[b, h] == len(ru) and np.array_equal(uidx[b, h, :len(ru)], ru), "union differs (b=%d h=%d)" % (b, h)
             assert (np.abs(out[b, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
+
+
+def test_sparse_decode_step_forced_redo(monkeypatch):
+    """Union mode of the path that redoes a segment from the keys (TKA_FORCE_SEGMENT_REDO), 16-level keys."""
+    monkeypatch.setenv("TKA_FORCE_SEGMENT_REDO", "1")
+    test_sparse_decode_step_union_only(oracle.BF16, 1, 2, 4, 66001, 1500, 32, 100, "levels")

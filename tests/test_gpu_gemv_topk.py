@@ -269,3 +269,14 @@ def test_long_segment_plan_reuse():
         ei, ev = oracle.topk_stable(ref, k)
         assert np.array_equal(plan.idx[0, 0].cpu().numpy(), ei), "indices differ on run %d" % it
         assert np.array_equal(plan.val[0, 0].cpu().numpy().view(np.uint32), ev.view(np.uint32))
+
+
+def test_long_segment_forced_redo(monkeypatch):
+    """TKA_FORCE_SEGMENT_REDO sends every long segment through the path that redoes it from the keys — here on
+    ordinary data with heavy hitters, in rank mode, with a ragged length."""
+    announce("gemv_topk long segment, every segment redone from the keys (N=70001 k=3000 G=4)")
+    monkeypatch.setenv("TKA_FORCE_SEGMENT_REDO", "1")
+    rng = np.random.default_rng(39)
+    K = randn_bits(rng, (1, 70001, 2, 128), oracle.F16)
+    K[0, rng.permutation(70001)[:700]] = oracle.to_bits(rng.standard_normal((700, 2, 128)) * 4.0, oracle.F16)
+    _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 3000)

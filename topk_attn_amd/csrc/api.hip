@@ -214,7 +214,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   sc.parts = cp.wgs_per_chunk;
   sc.part_len = cp.tokens_per_wg;
   sc.list_stride = sp.list_stride;
-  sc.max_entries = select_cand_capacity();
+  // TKA_FORCE_SEGMENT_REDO (testing): no candidate count is acceptable, every segment is redone from the keys
+  sc.max_entries = getenv("TKA_FORCE_SEGMENT_REDO") ? 0 : select_cand_capacity();
   sc.scores = scores;
   return launch_select_finalize_cand(gp, sc, a->dtype, stream);
 }

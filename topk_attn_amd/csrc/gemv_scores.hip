@@ -431,7 +431,7 @@ int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len) {
 void gemv_candidate_plan(int64_t chunk_len, int k, int max_candidates, int* num_samples, int* sample_rank) {
   *num_samples = 0;
   *sample_rank = 0;
-  if (chunk_len < 65536 || (int64_t)k * 16 > chunk_len) return;
+  if (chunk_len < kCandMinSegLen || (int64_t)k * 16 > chunk_len) return;
   // more samples on long segments keep the candidate count near k
   const int s = chunk_len >= 1048576 ? kGemvMaxSamples : (chunk_len >= 524288 ? kGemvMaxSamples / 2 : kGemvMaxSamples / 4);
   const double m = (double)k * s / (double)chunk_len;

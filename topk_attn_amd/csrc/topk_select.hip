@@ -371,7 +371,7 @@ __device__ __forceinline__ void fallback_segment(const GemvParams& g, const Sele
     load_group_query<DT>(g.q, g.q_stride_b, b, h, g.group, j, qf);
     const uint16_t* kbase = (const uint16_t*)g.keys + (int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h +
                             chunk_base * g.key_stride_n + 8 * j;
-    constexpr int kRows = 8;
+    constexpr int kRows = 16;   // rows in flight per lane: one CU has to pull the whole segment
     for (int64_t base = 0; base < n; base += (kSelThreads / 16) * kRows) {
       u32x4 kv[kRows];
 #pragma unroll
@@ -379,6 +379,7 @@ __device__ __forceinline__ void fallback_segment(const GemvParams& g, const Sele
         const int64_t t = base + rg * kRows + u;
         kv[u] = *(const u32x4*)(kbase + (t < n ? t : n - 1) * g.key_stride_n);
       }
+      __builtin_amdgcn_sched_barrier(0);   // all loads go out before the first score is computed
       float mine = 0.0f;
 #pragma unroll
       for (int u = 0; u < kRows; ++u) {
@@ -820,8 +821,9 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   l.hist = take((size_t)num_segments * kHistBins * sizeof(uint32_t));
   l.flags = take((size_t)num_segments * sizeof(uint32_t));
   l.tau = take((size_t)num_segments * sizeof(uint64_t));
-  l.ctr = take((size_t)num_segments * 64 * sizeof(uint32_t));
-  l.pool = take((size_t)num_segments * kGemvMaxSamples * sizeof(uint32_t));
+  const size_t cand_segs = seg_len >= kCandMinSegLen ? (size_t)num_segments : 0;   // sampling state: long segments only
+  l.ctr = take(cand_segs * 64 * sizeof(uint32_t));
+  l.pool = take(cand_segs * kGemvMaxSamples * sizeof(uint32_t));
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
   l.total = off;
