@@ -146,19 +146,20 @@ class GemvTopk:
 class CenterTopk:
     """c2: centre-only top-k with expansion."""
 
-    def __init__(self, torch, ops, dev):
+    def __init__(self, torch, ops, dev, centroids=4096, expand=64):
         g = torch.Generator(device=dev)
         g.manual_seed(2)
-        H, Cn = 32, 4096
-        self.ops, self.H, self.Cn, self.top_c, self.clen = ops, H, Cn, 64, 64
+        H, Cn = 32, centroids
+        self.ops, self.H, self.Cn, self.top_c, self.clen = ops, H, Cn, 64, expand
         cen = torch.randn((H, Cn, 128), generator=g, device=dev) + 0.5 * torch.randn((H, 1, 128), generator=g, device=dev)
         self.cen = cen.half()
         self.q = torch.randn((H, 128), generator=g, device=dev).half()
-        self.desc = "c2: 32 heads x 4096 centroids fp16, top-64, expand x64"
+        self.plan = ops.CenterTopkPlan(self.q, self.cen, self.top_c, self.clen, SCALE)
+        self.desc = "c2: 32 heads x %d centroids fp16, top-64, expand x%d" % (Cn, expand)
         self.dominant = "gemv_scores"
 
     def step(self):
-        self.out = self.ops.center_topk_expand(self.q, self.cen, self.top_c, self.clen, SCALE)
+        self.plan.run()
 
     def bytes(self):
         gemv = self.H * self.Cn * 128 * 2
@@ -215,6 +216,8 @@ def build_workload(name, torch, ops, dev, args):
         return GemvTopk(torch, ops, dev, 1, 1, 1, 32768, 2048, "float16", 1, "c1")
     if name == "c2":
         return CenterTopk(torch, ops, dev)
+    if name == "c2-ref":   # the problem of the reference's recorded latencies (center_only_topk/gemv_topk.cu:2-7)
+        return CenterTopk(torch, ops, dev, centroids=1024, expand=128)
     if name == "c3":
         return FlashDecode(torch, ops, dev, args.splits)
     if name == "c5":
@@ -235,7 +238,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c4-small", "c5", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c5", "copy"])
     ap.add_argument("--splits", type=int, default=0, help="c3, c4: split count of the attention (0 = library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-runs", type=int, default=3)

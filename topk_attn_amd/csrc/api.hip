@@ -181,6 +181,14 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   fill_gemv_params(a, scores, sp.hist, &gp);
   gp.cluster_ids = cluster_ids;
 
+  // Short segments: one launch, each workgroup scores and selects its own segment.  One CU pulls about
+  // 55 GB/s, so beyond 2048 rows (0.5 MB) the separate GEMV launch with many workgroups per segment wins.
+  if (!a->out_scores && chunk_len <= kFusedMaxSegLen) {
+    SelectParams sf = sp;
+    sf.from_keys = 1;
+    return launch_select_finalize_cand(gp, sf, a->dtype, stream);
+  }
+
   int num_samples = 0, sample_rank = 0;
   if (!a->out_scores && gp.wgs_per_chunk <= select_cand_max_parts() && gp.tokens_per_wg == kGemvCandTokensPerWg)
     gemv_candidate_plan(chunk_len, a->k, select_cand_capacity(), &num_samples, &sample_rank);

@@ -515,10 +515,41 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   // the slice's count; entries beyond the count are stale memory and ignored), the counts are scanned into
   // start positions, and the entries go to their place: one memory round trip.
   const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
-  const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;
+  const uint64_t* lists = p.from_keys ? nullptr : p.list + (int64_t)seg * p.list_stride;
   const int sub = tid & 15, grp = tid >> 4;
   uint32_t n_entries = 0;
-  if (p.parts <= kRound) {
+  if (p.from_keys) {
+    // Short segments: no GEMV launch before this one.  The workgroup scores its segment itself (64 row groups
+    // of 16 lanes, 8 rows in flight each, canonical order) and every token becomes an entry.
+    const int j = tid & 15, rg = tid >> 4;
+    const int chunk = seg % g.num_chunks, bh = seg / g.num_chunks;
+    const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
+    const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
+    float qf[8];
+    load_group_query<DT>(g.q, g.q_stride_b, b, h, g.group, j, qf);
+    const uint16_t* kbase = (const uint16_t*)g.keys + (int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h +
+                            chunk_base * g.key_stride_n + 8 * j;
+    const int n = (int)p.seg_len;
+    constexpr int kRows = 8;
+    for (int base = 0; base < n; base += (kSelThreads / 16) * kRows) {
+      u32x4 kv[kRows];
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        const int t = base + rg * kRows + u;
+        kv[u] = *(const u32x4*)(kbase + (int64_t)(t < n ? t : n - 1) * g.key_stride_n);
+      }
+      __builtin_amdgcn_sched_barrier(0);   // all loads go out before the first score is computed
+      float mine = 0.0f;
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        const float sc = row_score<DT>(qf, kv[u], g.scale);
+        if (j == u) mine = sc;
+      }
+      const int t = base + rg * kRows + j;
+      if (j < kRows && t < n) sh_ent[t] = composite(score_key(mine), (uint32_t)t);
+    }
+    n_entries = (uint32_t)n;
+  } else   if (p.parts <= kRound) {
     for (int s0 = 0; s0 < p.parts; s0 += kRound) {
       uint64_t first[kInFlight];
       uint32_t cnt[kInFlight];
@@ -594,18 +625,28 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
       }
     }
   }
-  const bool redo = n_entries < k || n_entries > cap;
-  if (tid == 0) {
-    p.seg_flags[seg] = redo ? 1u : 0u;
-    sh_small_cnt = 0;
+  const bool redo = !p.from_keys && (n_entries < k || n_entries > cap);
+  if (tid == 0) sh_small_cnt = 0;
+  if (!p.from_keys) {
+    if (tid == 0) p.seg_flags[seg] = redo ? 1u : 0u;
+    // the threshold and the arrival flags are spent: a replay of the same launches (a captured graph) must not
+    // take them for its own
+    if (tid >= 64 && tid < 128) p.sample_flags[(int64_t)seg * 64 + (tid - 64)] = 0u;
+    if (tid == 0) p.tau_words[seg] = 0ull;
   }
-  // the threshold and the arrival flags are spent: a replay of the same launches (a captured graph) must not
-  // take them for its own
-  if (tid >= 64 && tid < 128) p.sample_flags[(int64_t)seg * 64 + (tid - 64)] = 0u;
-  if (tid == 0) p.tau_words[seg] = 0ull;
   if (redo) {
     __syncthreads();
     fallback_segment<DT>(g, p, seg, kpad, sh_ent, sh_hist, sh_wtot, sh_res);
+    return;
+  }
+  if (p.from_keys && p.out_idx != nullptr && p.union_idx == nullptr && n_entries <= 2u * kSelThreads) {
+    // a short segment whose caller wants rank order only: sorting all of it is quicker than selecting first
+    uint32_t npad = 64;
+    while (npad < n_entries) npad <<= 1;
+    for (uint32_t i = n_entries + tid; i < npad; i += kSelThreads) sh_ent[i] = 0;   // pad: below every real composite
+    __syncthreads();
+    sort_lds_desc(sh_ent, sh_ent + npad, (int)npad);
+    write_rank_outputs(sh_ent, p, seg);
     return;
   }
   __syncthreads();
@@ -907,7 +948,8 @@ int select_cand_max_parts() { return kCandMaxParts; }
 int select_cand_capacity() { return kCandCap; }
 
 int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
-  if (p.parts > kCandMaxParts || p.k > kCandCap / 2) return TKA_EINVAL;
+  if (p.from_keys ? p.seg_len > kCandCap : p.parts > kCandMaxParts) return TKA_EINVAL;
+  if (p.k > kCandCap / 2) return TKA_EINVAL;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)select_finalize_cand_kernel<TKA_F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -918,7 +960,7 @@ int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int 
     if (e != hipSuccess) return TKA_EHIP;
     attr_set = true;
   }
-  LaunchTimer timer("select_finalize_cand", stream);
+  LaunchTimer timer(p.from_keys ? "gemv_topk_fused" : "select_finalize_cand", stream);
   const size_t lds = kCandCap * sizeof(uint64_t);
   if (dtype == TKA_F16)
     select_finalize_cand_kernel<TKA_F16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));

@@ -140,26 +140,38 @@ def topk(scores, k):
     return idx, val
 
 
+class CenterTopkPlan:
+    """Argument block, outputs and workspace of one centre-only selection; run() is one C call."""
+
+    def __init__(self, q, centers, top_c, cluster_len, scale=1.0):
+        _need_cuda(q, centers)
+        if not centers.is_contiguous() or not q.is_contiguous():
+            raise ValueError("q and centers must be contiguous")
+        H, Cn, _ = centers.shape
+        self.q, self.centers = q, centers
+        self.out = torch.empty((H, top_c * cluster_len), dtype=torch.int32, device=q.device)
+        self.cen = torch.empty((H, top_c), dtype=torch.int32, device=q.device)
+        self.val = torch.empty((H, top_c), dtype=torch.float32, device=q.device)
+        a = self.args = L.CenterTopkArgs()
+        a.q, a.centers, a.dtype = q.data_ptr(), centers.data_ptr(), _dtype_code(centers)
+        a.num_heads, a.num_centers, a.top_c, a.cluster_len, a.head_dim = H, Cn, top_c, cluster_len, 128
+        a.scale = scale
+        a.out_idx, a.out_centers, a.out_center_val = self.out.data_ptr(), self.cen.data_ptr(), self.val.data_ptr()
+        need = L.lib().tka_center_topk_expand_workspace_bytes(C.byref(a))
+        self.ws = _workspace(need, q.device)
+        a.workspace, a.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
+
+    def run(self):
+        self.args.stream = _stream()
+        L.check(L.lib().tka_center_topk_expand(C.byref(self.args)), "tka_center_topk_expand")
+        return self
+
+
 def center_topk_expand(q, centers, top_c, cluster_len, scale=1.0):
     """Centre-only selection.  q [H,128], centers [H,C,128] contiguous.
     Returns (token ids int32 [H, top_c*cluster_len], centre ids int32 [H,top_c], centre scores fp32 [H,top_c])."""
-    _need_cuda(q, centers)
-    if not centers.is_contiguous() or not q.is_contiguous():
-        raise ValueError("q and centers must be contiguous")
-    H, Cn, _ = centers.shape
-    out = torch.empty((H, top_c * cluster_len), dtype=torch.int32, device=q.device)
-    cen = torch.empty((H, top_c), dtype=torch.int32, device=q.device)
-    val = torch.empty((H, top_c), dtype=torch.float32, device=q.device)
-    a = L.CenterTopkArgs()
-    a.q, a.centers, a.dtype = q.data_ptr(), centers.data_ptr(), _dtype_code(centers)
-    a.num_heads, a.num_centers, a.top_c, a.cluster_len, a.head_dim = H, Cn, top_c, cluster_len, 128
-    a.scale = scale
-    a.out_idx, a.out_centers, a.out_center_val = out.data_ptr(), cen.data_ptr(), val.data_ptr()
-    need = L.lib().tka_center_topk_expand_workspace_bytes(C.byref(a))
-    ws = _workspace(need, q.device)
-    a.workspace, a.workspace_bytes, a.stream = ws.data_ptr(), ws.numel(), _stream()
-    L.check(L.lib().tka_center_topk_expand(C.byref(a)), "tka_center_topk_expand")
-    return out, cen, val
+    plan = CenterTopkPlan(q, centers, top_c, cluster_len, scale).run()
+    return plan.out, plan.cen, plan.val
 
 
 def cluster_gemv_topk(q, centers, keys, top_c, cluster_len, k, scale=1.0):
