@@ -189,6 +189,16 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     return launch_select_finalize_cand(gp, sf, a->dtype, stream);
   }
 
+  // Segments that fit in LDS whole: GEMV that stores plain scores (no histogram), then one selection launch.
+  if (chunk_len <= select_cand_capacity()) {
+    gp.hist = nullptr;
+    int rc = launch_gemv_scores(gp, a->dtype, stream);
+    if (rc != TKA_OK) return rc;
+    SelectParams sw = sp;
+    sw.from_scores = 1;
+    return launch_select_finalize_cand(gp, sw, a->dtype, stream);
+  }
+
   int num_samples = 0, sample_rank = 0;
   if (!a->out_scores && gp.wgs_per_chunk <= select_cand_max_parts() && gp.tokens_per_wg == kGemvCandTokensPerWg)
     gemv_candidate_plan(chunk_len, a->k, select_cand_capacity(), &num_samples, &sample_rank);
@@ -403,6 +413,12 @@ int tka_topk_f32(const tka_topk_args* a) {
   sp.num_segments = a->num_segments;
   sp.k = a->k;
   sp.segs_per_row = 1;
+  if (a->seg_len <= select_cand_capacity()) {   // the segment fits in LDS whole: one launch
+    GemvParams none;
+    memset(&none, 0, sizeof none);
+    sp.from_scores = 1;
+    return launch_select_finalize_cand(none, sp, TKA_F16, stream);
+  }
   rc = launch_zero_u32(sp.hist, zero_words, stream);
   if (rc != TKA_OK) return rc;
   rc = launch_select_hist(sp, stream);

@@ -74,6 +74,22 @@ __device__ __forceinline__ uint64_t lane_xor64(uint64_t v) {
   return ((uint64_t)hi << 32) | lo;
 }
 
+// Inclusive prefix sum over the 64 lanes of the wave: four DPP row shifts, then the row totals are carried
+// forward with row_bcast:15 (rows 1, 3) and row_bcast:31 (rows 2, 3).  Lanes without a source add 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_add_u32(uint32_t v) {
+  return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+  v = dpp_add_u32<0x111, 0xf>(v);   // row_shr:1
+  v = dpp_add_u32<0x112, 0xf>(v);   // row_shr:2
+  v = dpp_add_u32<0x114, 0xf>(v);   // row_shr:4
+  v = dpp_add_u32<0x118, 0xf>(v);   // row_shr:8
+  v = dpp_add_u32<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
+  v = dpp_add_u32<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 __device__ __forceinline__ int lane_id() {
   return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }
@@ -158,12 +174,10 @@ __device__ __forceinline__ void find_threshold_bin_1024(const uint32_t* sh_hist,
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const uint32_t h0 = sh_hist[2 * tid], h1 = sh_hist[2 * tid + 1];
-  uint32_t v = h0 + h1;  // suffix sum over lanes >= lane
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    uint32_t t = __shfl_down(v, d, 64);
-    if (lane + d < 64) v += t;
-  }
+  const uint32_t mine = h0 + h1;
+  const uint32_t inc = wave_inclusive_scan(mine);
+  const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)inc, 63);
+  const uint32_t v = wave_total - inc + mine;  // suffix sum over lanes >= lane
   if (lane == 0) sh_wtot[wave] = v;
   __syncthreads();
   uint32_t above = 0;

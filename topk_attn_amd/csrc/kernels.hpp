@@ -45,6 +45,7 @@ struct SelectParams {
   uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment was redone from the keys
   int max_entries;        // candidate mode: a segment with more candidates than this is also redone from the keys
   int from_keys;          // candidate selection kernel: no slices, the workgroup scores its (short) segment itself
+  int from_scores;        // candidate selection kernel: no slices, the entries are all scores of the segment (<= 16384)
   uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)
   uint64_t* list;         // [num_segments][list_stride] composites with bin >= threshold bin, slice p at p*part_len
   int64_t list_stride;

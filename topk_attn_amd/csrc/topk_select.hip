@@ -49,12 +49,7 @@ __global__ __launch_bounds__(256) void zero_u32_kernel(uint32_t* p, size_t n) {
 // Exclusive prefix of v over the 1024 threads of the block; *total = block sum.  Two barriers.
 __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* sh_wtot, uint32_t* total) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint32_t inc = v;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    uint32_t t = __shfl_up(inc, d, 64);
-    if (lane >= d) inc += t;
-  }
+  const uint32_t inc = wave_inclusive_scan(v);
   __syncthreads();  // sh_wtot may still be read by the previous call
   if (lane == 63) sh_wtot[wave] = inc;
   __syncthreads();
@@ -502,12 +497,12 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   __shared__ uint32_t sh_pos[kCandMaxParts + 1];   // start positions of all slices (segments with more than kRound slices)
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
-  __shared__ uint64_t sh_wmin[kSelWaves], sh_wmax[kSelWaves];
+  __shared__ uint32_t sh_kminmax[2];
   __shared__ uint64_t sh_small[kSmallBucket];
   __shared__ uint32_t sh_small_cnt;
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
 
@@ -515,7 +510,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   // the slice's count; entries beyond the count are stale memory and ignored), the counts are scanned into
   // start positions, and the entries go to their place: one memory round trip.
   const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
-  const uint64_t* lists = p.from_keys ? nullptr : p.list + (int64_t)seg * p.list_stride;
+  const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;   // (not read when the entries come from keys or scores)
   const int sub = tid & 15, grp = tid >> 4;
   uint32_t n_entries = 0;
   if (p.from_keys) {
@@ -547,6 +542,19 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
       }
       const int t = base + rg * kRows + j;
       if (j < kRows && t < n) sh_ent[t] = composite(score_key(mine), (uint32_t)t);
+    }
+    n_entries = (uint32_t)n;
+  } else if (p.from_scores) {
+    // Segments that fit in LDS whole: the GEMV launch stored plain scores, every one of them becomes an entry.
+    const float* sc = p.scores + (int64_t)seg * p.seg_stride;
+    const bool vec_ok = (((uintptr_t)sc) & 15u) == 0;
+    const int64_t n = p.seg_len;
+    for (int64_t first = (int64_t)tid * 4; first < n; first += 4 * kSelThreads) {
+      uint32_t keys[4], vm;
+      load_keys<4>(sc, first, n, vec_ok, keys, &vm);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (vm >> e & 1u) sh_ent[first + e] = composite(keys[e], (uint32_t)(first + e));
     }
     n_entries = (uint32_t)n;
   } else   if (p.parts <= kRound) {
@@ -625,9 +633,14 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
       }
     }
   }
-  const bool redo = !p.from_keys && (n_entries < k || n_entries > cap);
-  if (tid == 0) sh_small_cnt = 0;
-  if (!p.from_keys) {
+  const bool whole = p.from_keys || p.from_scores;   // the entries are the whole segment, not candidate slices
+  const bool redo = !whole && (n_entries < k || n_entries > cap);
+  if (tid == 0) {
+    sh_small_cnt = 0;
+    sh_kminmax[0] = ~0u;
+    sh_kminmax[1] = 0u;
+  }
+  if (!whole) {
     if (tid == 0) p.seg_flags[seg] = redo ? 1u : 0u;
     // the threshold and the arrival flags are spent: a replay of the same launches (a captured graph) must not
     // take them for its own
@@ -639,7 +652,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     fallback_segment<DT>(g, p, seg, kpad, sh_ent, sh_hist, sh_wtot, sh_res);
     return;
   }
-  if (p.from_keys && p.out_idx != nullptr && p.union_idx == nullptr && n_entries <= 2u * kSelThreads) {
+  if (whole && p.out_idx != nullptr && p.union_idx == nullptr && n_entries <= 2u * kSelThreads) {
     // a short segment whose caller wants rank order only: sorting all of it is quicker than selecting first
     uint32_t npad = 64;
     while (npad < n_entries) npad <<= 1;
@@ -653,37 +666,36 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
 
   // this thread's share for the radix passes: entries tid, tid + 1024, ...
   uint64_t mine[kCandPerThread];
-  uint64_t cmin = ~0ull, cmax = 0ull;
+  uint32_t kmin = ~0u, kmax = 0u;   // smallest and largest key among the entries
 #pragma unroll
   for (int i = 0; i < kCandPerThread; ++i) {
     const uint32_t v = (uint32_t)i * kSelThreads + tid;
     const bool ok = v < n_entries;
     mine[i] = ok ? sh_ent[v] : 0ull;
     if (ok) {
-      cmin = mine[i] < cmin ? mine[i] : cmin;
-      cmax = mine[i] > cmax ? mine[i] : cmax;
+      kmin = min(kmin, (uint32_t)(mine[i] >> 32));
+      kmax = max(kmax, (uint32_t)(mine[i] >> 32));
     }
   }
 
   uint64_t threshold = 0;   // selected: composite >= threshold
   if (n_entries > k) {
-    // common prefix of all candidates: the passes start below it
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const uint64_t a = __shfl_xor(cmin, d, 64), b = __shfl_xor(cmax, d, 64);
-      cmin = a < cmin ? a : cmin;
-      cmax = b > cmax ? b : cmax;
+    // common prefix of all keys: the passes start below it (all keys equal: they start at the index bits)
+    kmin = min(kmin, lane_xor<1>(kmin));   kmax = max(kmax, lane_xor<1>(kmax));
+    kmin = min(kmin, lane_xor<2>(kmin));   kmax = max(kmax, lane_xor<2>(kmax));
+    kmin = min(kmin, lane_xor<4>(kmin));   kmax = max(kmax, lane_xor<4>(kmax));
+    kmin = min(kmin, lane_xor<8>(kmin));   kmax = max(kmax, lane_xor<8>(kmax));
+    kmin = min(kmin, lane_xor<16>(kmin));  kmax = max(kmax, lane_xor<16>(kmax));
+    kmin = min(kmin, lane_xor<32>(kmin));  kmax = max(kmax, lane_xor<32>(kmax));
+    if (lane == 0) {
+      atomicMin(&sh_kminmax[0], kmin);
+      atomicMax(&sh_kminmax[1], kmax);
     }
-    if (lane == 0) { sh_wmin[wave] = cmin; sh_wmax[wave] = cmax; }
     __syncthreads();
-#pragma unroll
-    for (int w = 0; w < kSelWaves; ++w) {
-      const uint64_t a = sh_wmin[w], b = sh_wmax[w];
-      cmin = a < cmin ? a : cmin;
-      cmax = b > cmax ? b : cmax;
-    }
-    int fixed = __builtin_clzll(cmin ^ cmax);            // composites are distinct and n_entries >= 2: < 64
-    uint64_t prefix = fixed ? cmax >> (64 - fixed) : 0ull;
+    kmin = sh_kminmax[0];
+    kmax = sh_kminmax[1];
+    int fixed = kmin == kmax ? 32 : __builtin_clz(kmin ^ kmax);
+    uint64_t prefix = fixed ? (uint64_t)(kmax >> (32 - fixed)) : 0ull;
     uint32_t need = k;
     bool done = false;
     while (!done) {
@@ -948,7 +960,7 @@ int select_cand_max_parts() { return kCandMaxParts; }
 int select_cand_capacity() { return kCandCap; }
 
 int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
-  if (p.from_keys ? p.seg_len > kCandCap : p.parts > kCandMaxParts) return TKA_EINVAL;
+  if ((p.from_keys || p.from_scores) ? p.seg_len > kCandCap : p.parts > kCandMaxParts) return TKA_EINVAL;
   if (p.k > kCandCap / 2) return TKA_EINVAL;
   static bool attr_set = false;
   if (!attr_set) {
@@ -960,7 +972,7 @@ int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int 
     if (e != hipSuccess) return TKA_EHIP;
     attr_set = true;
   }
-  LaunchTimer timer(p.from_keys ? "gemv_topk_fused" : "select_finalize_cand", stream);
+  LaunchTimer timer(p.from_keys ? "gemv_topk_fused" : (p.from_scores ? "select_whole" : "select_finalize_cand"), stream);
   const size_t lds = kCandCap * sizeof(uint64_t);
   if (dtype == TKA_F16)
     select_finalize_cand_kernel<TKA_F16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
