@@ -515,7 +515,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   uint32_t n_entries = 0;
   if (p.from_keys) {
     // Short segments: no GEMV launch before this one.  The workgroup scores its segment itself (64 row groups
-    // of 16 lanes, 8 rows in flight each, canonical order) and every token becomes an entry.
+    // of 16 lanes, 16 rows in flight each, canonical order) and every token becomes an entry.
     const int j = tid & 15, rg = tid >> 4;
     const int chunk = seg % g.num_chunks, bh = seg / g.num_chunks;
     const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
@@ -525,7 +525,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     const uint16_t* kbase = (const uint16_t*)g.keys + (int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h +
                             chunk_base * g.key_stride_n + 8 * j;
     const int n = (int)p.seg_len;
-    constexpr int kRows = 8;
+    constexpr int kRows = 16;   // rows in flight per lane
     for (int base = 0; base < n; base += (kSelThreads / 16) * kRows) {
       u32x4 kv[kRows];
 #pragma unroll
@@ -973,7 +973,18 @@ int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int 
     attr_set = true;
   }
   LaunchTimer timer(p.from_keys ? "gemv_topk_fused" : (p.from_scores ? "select_whole" : "select_finalize_cand"), stream);
-  const size_t lds = kCandCap * sizeof(uint64_t);
+  // entries of the segment; rank mode reuses the buffer as sort + exchange buffers (2 x kpad, or 2 x the padded
+  // segment when a short segment is sorted whole).  Short segments leave room for two workgroups per CU.
+  size_t entries = kCandCap;
+  if (p.from_keys || p.from_scores) {
+    entries = (size_t)p.seg_len;
+    if (p.out_idx) {
+      size_t pad = (size_t)kpad_for(p.k);
+      if (!p.union_idx && p.seg_len <= 2 * kSelThreads) pad = (size_t)kpad_for((int)p.seg_len);
+      if (entries < 2 * pad) entries = 2 * pad;
+    }
+  }
+  const size_t lds = entries * sizeof(uint64_t);
   if (dtype == TKA_F16)
     select_finalize_cand_kernel<TKA_F16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
   else
