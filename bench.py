@@ -115,7 +115,7 @@ class SparseDecode:
 class GemvTopk:
     """c1 / c5: fused GEMV + top-k alone."""
 
-    def __init__(self, torch, ops, dev, batch, hkv, group, seq_len, k, dtype, seed, name, levels=False):
+    def __init__(self, torch, ops, dev, batch, hkv, group, seq_len, k, dtype, seed, name, levels=False, rotate=0):
         g = torch.Generator(device=dev)
         g.manual_seed(seed)
         dt = getattr(torch, dtype)
@@ -131,12 +131,19 @@ class GemvTopk:
                     self.K[b, t0:t1] = lv[ids].to(dt)
         else:
             self.K = randn16(torch, (batch, seq_len, hkv, 128), dt, g, dev)
-        self.plan = ops.GemvTopkPlan(self.q, self.K, k, group=group, scale=SCALE)
-        self.desc = "%s: B=%d Hkv=%d G=%d D=128 N=%d %s k=%d (GEMV + top-k only)" % (name, batch, hkv, group, seq_len, dtype, k)
+        # rotate > 0: that many copies of the keys, one plan each, taken in turn, so that a key set much smaller
+        # than the Infinity Cache is read from HBM every step
+        self.plans = [ops.GemvTopkPlan(self.q, self.K, k, group=group, scale=SCALE)]
+        self.copies = [self.K.clone() for _ in range(max(rotate - 1, 0))]
+        self.plans += [ops.GemvTopkPlan(self.q, Kc, k, group=group, scale=SCALE) for Kc in self.copies]
+        self.turn = 0
+        self.desc = "%s: B=%d Hkv=%d G=%d D=128 N=%d %s k=%d (GEMV + top-k only)%s" % (
+            name, batch, hkv, group, seq_len, dtype, k, ", %d rotating key sets" % rotate if rotate > 1 else "")
         self.dominant = "gemv_scores"
 
     def step(self):
-        self.plan.run()
+        self.plans[self.turn % len(self.plans)].run()
+        self.turn += 1
 
     def bytes(self):
         gemv = self.B * self.N * self.H * 128 * 2
@@ -146,7 +153,7 @@ class GemvTopk:
 class CenterTopk:
     """c2: centre-only top-k with expansion."""
 
-    def __init__(self, torch, ops, dev, centroids=4096, expand=64):
+    def __init__(self, torch, ops, dev, centroids=4096, expand=64, rotate=0):
         g = torch.Generator(device=dev)
         g.manual_seed(2)
         H, Cn = 32, centroids
@@ -154,12 +161,17 @@ class CenterTopk:
         cen = torch.randn((H, Cn, 128), generator=g, device=dev) + 0.5 * torch.randn((H, 1, 128), generator=g, device=dev)
         self.cen = cen.half()
         self.q = torch.randn((H, 128), generator=g, device=dev).half()
-        self.plan = ops.CenterTopkPlan(self.q, self.cen, self.top_c, self.clen, SCALE)
-        self.desc = "c2: 32 heads x %d centroids fp16, top-64, expand x%d" % (Cn, expand)
+        self.plans = [ops.CenterTopkPlan(self.q, self.cen, self.top_c, self.clen, SCALE)]
+        self.copies = [self.cen.clone() for _ in range(max(rotate - 1, 0))]
+        self.plans += [ops.CenterTopkPlan(self.q, c, self.top_c, self.clen, SCALE) for c in self.copies]
+        self.turn = 0
+        self.desc = "c2: 32 heads x %d centroids fp16, top-64, expand x%d%s" % (
+            Cn, expand, ", %d rotating centroid sets" % rotate if rotate > 1 else "")
         self.dominant = "gemv_scores"
 
     def step(self):
-        self.plan.run()
+        self.plans[self.turn % len(self.plans)].run()
+        self.turn += 1
 
     def bytes(self):
         gemv = self.H * self.Cn * 128 * 2
@@ -213,11 +225,11 @@ def build_workload(name, torch, ops, dev, args):
     if name == "c4-small":
         return SparseDecode(torch, ops, dev, batch=2, seq_len=16384, name="c4-small")
     if name == "c1":
-        return GemvTopk(torch, ops, dev, 1, 1, 1, 32768, 2048, "float16", 1, "c1")
+        return GemvTopk(torch, ops, dev, 1, 1, 1, 32768, 2048, "float16", 1, "c1", rotate=args.rotate)
     if name == "c2":
-        return CenterTopk(torch, ops, dev)
+        return CenterTopk(torch, ops, dev, rotate=args.rotate)
     if name == "c2-ref":   # the problem of the reference's recorded latencies (center_only_topk/gemv_topk.cu:2-7)
-        return CenterTopk(torch, ops, dev, centroids=1024, expand=128)
+        return CenterTopk(torch, ops, dev, centroids=1024, expand=128, rotate=args.rotate)
     if name == "c3":
         return FlashDecode(torch, ops, dev, args.splits)
     if name == "c5":
@@ -240,6 +252,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c5", "copy"])
     ap.add_argument("--splits", type=int, default=0, help="c3, c4: split count of the attention (0 = library default)")
+    ap.add_argument("--rotate", type=int, default=0,
+                    help="c1, c2, c2-ref: number of key sets taken in turn (working set beyond the Infinity Cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-runs", type=int, default=3)
     args = ap.parse_args()
