@@ -272,3 +272,42 @@ def test_sparse_decode_step_forced_redo(monkeypatch):
     """Union mode of the path that redoes a segment from the keys (TKA_FORCE_SEGMENT_REDO), 16-level keys."""
     monkeypatch.setenv("TKA_FORCE_SEGMENT_REDO", "1")
     test_sparse_decode_step_union_only(oracle.BF16, 1, 2, 4, 66001, 1500, 32, 100, "levels")
+
+
+def test_sparse_decode_step_graph_replay():
+    """The step captured in a HIP graph and replayed with a new query each time (long segments: the sampled
+    thresholds and arrival flags of one replay must never serve the next).  Every replay is compared with the
+    eager result for the same query, with eager work in between."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step captured in a graph, 3 replays with changing queries (N=70000 k=1024 G=4)")
+    rng = np.random.default_rng(77)
+    dtype, B, H, G, N, k, sink, local = oracle.F16, 1, 2, 4, 70000, 1024, 16, 128
+    Kf = rng.standard_normal((B, N, H, 128))
+    Kf[:, rng.permutation(N)[:N // 100]] *= 4.0
+    q = to_dev(randn_bits(rng, (B, H * G, 128), dtype), dtype)
+    K, V = to_dev(oracle.to_bits(Kf, dtype), dtype), to_dev(randn_bits(rng, (B, N, H, 128), dtype), dtype)
+    plan = ops.SparseDecodePlan(q, K, V, k, sink, local, SCALE, G, out_dtype=torch.float16, want_topk=False)
+    plan.step()                      # warm-up outside the capture (one-time function attributes)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        plan.step()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            plan.step()
+    torch.cuda.synchronize()
+    for it in range(3):
+        q.copy_(to_dev(oracle.to_bits(rng.standard_normal((B, H * G, 128)) * (1.0 + 0.5 * it), dtype), dtype))
+        plan.step()                  # eager, default stream
+        torch.cuda.synchronize()
+        want_out, want_idx, want_cnt = plan.out.clone(), plan.union_idx.clone(), plan.union_count.clone()
+        plan.out.zero_()
+        plan.union_idx.fill_(-7)
+        plan.union_count.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(plan.union_count, want_cnt), "replay %d: union counts differ" % it
+        assert torch.equal(plan.union_idx, want_idx), "replay %d: union lists differ" % it
+        assert torch.equal(plan.out, want_out), "replay %d: outputs differ" % it
