@@ -56,6 +56,17 @@ def test_small_shapes(dtype):
     _run_flat(dtype, 1, 1, 8, 130, 130, seed=4)
 
 
+def test_whole_segment_routes_edges():
+    """Segments that one workgroup scores itself (up to 2048 rows) or that fit in LDS whole (up to 16384): k = n,
+    k = 1, the largest k, odd lengths, chunks, both dtypes."""
+    announce("gemv_topk whole-segment routes: edge shapes")
+    _run_flat(oracle.BF16, 1, 1, 8, 2048, 2048, seed=40)            # k = n, sorted whole
+    _run_flat(oracle.F16, 2, 2, 1, 2047, 1, seed=41)                # k = 1
+    _run_flat(oracle.F16, 1, 2, 2, 16384, 8192, seed=42)            # largest segment and k of the LDS route
+    _run_flat(oracle.BF16, 1, 3, 4, 6000, 1500, seed=43, num_chunks=3, levels=True)   # chunks of 2000, ties
+    _run_flat(oracle.F16, 1, 1, 1, 2049, 700, seed=44)              # first length past the one-launch route
+
+
 def test_grouped_batched():
     announce("gemv_topk B=2 Hkv=8 G=4 N=16384 k=2048 fp16")
     _run_flat(oracle.F16, 2, 8, 4, 16384, 2048, seed=5)
