@@ -200,7 +200,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   }
 
   int num_samples = 0, sample_rank = 0;
-  if (!a->out_scores && gp.wgs_per_chunk <= select_cand_max_parts() && gp.tokens_per_wg == kGemvCandTokensPerWg)
+  const int64_t cand_slices = (chunk_len + kGemvCandTokensPerWg - 1) / kGemvCandTokensPerWg;
+  if (!a->out_scores && cand_slices <= select_cand_max_parts())
     gemv_candidate_plan(chunk_len, a->k, select_cand_capacity(), &num_samples, &sample_rank);
   if (num_samples == 0) {
     // dense: clear histograms, GEMV with histogram, filter, finalize
@@ -217,6 +218,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   static std::atomic<uint32_t> call_counter{0};
   GemvParams cp = gp;
   cp.hist = nullptr;
+  cp.tokens_per_wg = kGemvCandTokensPerWg;
+  cp.wgs_per_chunk = (int)cand_slices;
   cp.tau_words = sp.tau_words;
   cp.sample_flags = sp.sample_flags;
   cp.sample_pool = sp.sample_pool;

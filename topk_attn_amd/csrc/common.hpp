@@ -19,7 +19,8 @@ constexpr int kHeadDim = TKA_HEAD_DIM;
 constexpr int kWave = 64;
 constexpr int kHistBits = 11;
 constexpr int kHistBins = 1 << kHistBits;  // first-level selection histogram: top 11 bits of the key
-constexpr int kGemvCandTokensPerWg = 256;  // tokens per GEMV workgroup on large problems (= slice length of candidate lists)
+constexpr int kGemvDenseTokensPerWg = 256; // tokens per workgroup of the dense GEMV on large problems
+constexpr int kGemvCandTokensPerWg = 512;  // tokens (and threads) per streaming workgroup of the candidate GEMV = slice length
 constexpr int64_t kFusedMaxSegLen = 2048;   // segments up to this length are scored and selected by one workgroup in one launch
 constexpr int64_t kCandMinSegLen = 65536;   // shorter segments never take the candidate mode
 constexpr int kGemvMaxSamples = 8192;      // most samples per segment of the candidate-mode threshold estimate

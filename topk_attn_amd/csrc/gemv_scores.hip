@@ -26,12 +26,13 @@ namespace tka {
 namespace {
 
 constexpr int kGemvThreads = 256;
-constexpr int kGemvWaves = kGemvThreads / kWave;
 constexpr int kGemvUnroll = 8;                                         // loads in flight per lane
 constexpr int kGemvRowsPerIter = (kGemvThreads / 16) * kGemvUnroll;    // 128 tokens per WG iteration
 constexpr int kTauSpinLimit = 1 << 16; // polls of a streaming workgroup for its threshold before it gives up
 constexpr int kEarlySlices = 3;        // slices of a streaming workgroup that starts before the threshold is published
-static_assert(kGemvCandTokensPerWg == kGemvThreads, "candidate mode: one thread per token in the epilogue");
+constexpr int kCandThreads = kGemvCandTokensPerWg;                     // candidate kernel: one thread per token of the slice
+constexpr int kCandWaves = kCandThreads / kWave;
+constexpr int kCandRowsPerIter = (kCandThreads / 16) * kGemvUnroll;    // 256 tokens per WG iteration
 
 template <int DT>
 __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p) {
@@ -111,7 +112,7 @@ __device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) 
   return (int64_t)i * stride + (int64_t)(mix32((uint32_t)seg * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
 }
 
-// Sampling workgroup (256 threads): scores 128 of the segment's p.num_samples sample tokens (one round of
+// Sampling workgroup: scores 256 of the segment's p.num_samples sample tokens (one round of
 // loads) and stores their keys in the segment's pool.  The workgroup that arrives last (epoch-valued arrival
 // flags, so that the workspace needs no clearing) takes the p.sample_rank-th largest key of the whole pool and
 // publishes it as the segment's threshold word, (epoch << 32) | key.  The sample is spread evenly over the
@@ -120,11 +121,11 @@ __device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) 
 // Ordering between workgroups: the keys are agent-scope atomic stores, their completion and a barrier precede
 // the workgroup's arrival flag; the last workgroup reads the pool with agent-scope atomic loads after it has
 // seen every flag.
-// sh: 2048 + 8 words.
+// sh: 2048 + 16 words.
 template <int DT>
 __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int part, uint32_t* sh) {
   uint32_t* sh_hist = sh;                   // 2048 bins
-  uint32_t* sh_wtot = sh_hist + kHistBins;  // 4 wave totals, bin and count above it, "last" flag
+  uint32_t* sh_wtot = sh_hist + kHistBins;  // 8 wave totals, then [8] bin, [9] count above it, [10] "last" flag
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int j = tid & 15, rg = tid >> 4;
@@ -138,7 +139,7 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
                           chunk_base * p.key_stride_n + 8 * j;
   uint32_t* pool = p.sample_pool + (int64_t)seg * p.num_samples;
   {
-    const int first = part * kGemvRowsPerIter + rg * kGemvUnroll;
+    const int first = part * kCandRowsPerIter + rg * kGemvUnroll;
     u32x4 kv[kGemvUnroll];
 #pragma unroll
     for (int u = 0; u < kGemvUnroll; ++u)
@@ -161,25 +162,26 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
     // one word are served one after the other).  Set my flag, wait until it has completed, read all flags:
     // of two workgroups that finish together at least the one whose flag completed later sees both, so
     // somebody always sees all of them; if two do, both publish the same threshold.
-    const int parts = p.num_samples / kGemvRowsPerIter;   // <= 64
-    uint32_t* flags = p.sample_flags + (int64_t)seg * (kGemvMaxSamples / kGemvRowsPerIter);
+    const int parts = p.num_samples / kCandRowsPerIter;   // <= 64
+    uint32_t* flags = p.sample_flags + (int64_t)seg * (kGemvMaxSamples / kCandRowsPerIter);
     if (lane == 0) __hip_atomic_store(flags + part, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const uint32_t f = lane < parts ? __hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : p.epoch;
     const bool all = __ballot(f == p.epoch) == ~0ull;
-    if (lane == 0) sh_wtot[6] = all ? 1u : 0u;
+    if (lane == 0) sh_wtot[10] = all ? 1u : 0u;
   }
   __syncthreads();
-  if (sh_wtot[6] == 0u) return;
+  if (sh_wtot[10] == 0u) return;
 
   // sample_rank-th largest key of the pool, to its top 22 bits (the threshold only has to lie at or below that
-  // order statistic): two 11-bit radix passes, thread t owns bins 8t .. 8t+7
+  // order statistic): two 11-bit radix passes, thread t owns bins 4t .. 4t+3
   // the pool once into registers, all loads in flight together (one at a time they cost 2-3 us each)
-  constexpr int kPerThread = kGemvMaxSamples / kGemvThreads;
+  constexpr int kPerThread = kGemvMaxSamples / kCandThreads;
+  constexpr int kBinsPerThread = kHistBins / kCandThreads;
   uint32_t keys[kPerThread];
 #pragma unroll
   for (int u = 0; u < kPerThread; ++u) {
-    const int i = u * kGemvThreads + tid;
+    const int i = u * kCandThreads + tid;
     keys[u] = i < p.num_samples ? __hip_atomic_load(pool + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
   }
   uint32_t need = (uint32_t)p.sample_rank, prefix = 0;
@@ -187,19 +189,19 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
     const int shift = pass ? 32 - 2 * kHistBits : 32 - kHistBits;
     __syncthreads();
 #pragma unroll
-    for (int e = 0; e < 8; ++e) sh_hist[8 * tid + e] = 0;
+    for (int e = 0; e < kBinsPerThread; ++e) sh_hist[kBinsPerThread * tid + e] = 0;
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < kPerThread; ++u) {
       const uint32_t key = keys[u];
-      if (u * kGemvThreads + tid < p.num_samples && (pass == 0 || (key >> (32 - kHistBits)) == prefix))
+      if (u * kCandThreads + tid < p.num_samples && (pass == 0 || (key >> (32 - kHistBits)) == prefix))
         atomicAdd(&sh_hist[(key >> shift) & (kHistBins - 1)], 1u);
     }
     __syncthreads();
-    uint32_t h[8], mine = 0;
+    uint32_t h[kBinsPerThread], mine = 0;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      h[e] = sh_hist[8 * tid + e];
+    for (int e = 0; e < kBinsPerThread; ++e) {
+      h[e] = sh_hist[kBinsPerThread * tid + e];
       mine += h[e];
     }
     uint32_t ge = mine;   // count in the bins of threads >= tid, first inside the wave
@@ -210,22 +212,22 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
     }
     if (lane == 0) sh_wtot[wave] = ge;
     __syncthreads();
-    for (int w = wave + 1; w < kGemvWaves; ++w) ge += sh_wtot[w];
-    if (ge >= need && ge - mine < need) {   // the bin sits among this thread's eight: walk them from the top
+    for (int w = wave + 1; w < kCandWaves; ++w) ge += sh_wtot[w];
+    if (ge >= need && ge - mine < need) {   // the bin sits among this thread's four: walk them from the top
       uint32_t above = ge - mine;
       int bin = 0;
       bool found = false;
 #pragma unroll
-      for (int e = 7; e >= 0; --e) {
-        if (!found && above + h[e] >= need) { bin = 8 * tid + e; found = true; }
+      for (int e = kBinsPerThread - 1; e >= 0; --e) {
+        if (!found && above + h[e] >= need) { bin = kBinsPerThread * tid + e; found = true; }
         if (!found) above += h[e];
       }
-      sh_wtot[4] = (uint32_t)bin;
-      sh_wtot[5] = above;
+      sh_wtot[8] = (uint32_t)bin;
+      sh_wtot[9] = above;
     }
     __syncthreads();
-    prefix = (prefix << kHistBits) | sh_wtot[4];
-    need -= sh_wtot[5];
+    prefix = (prefix << kHistBits) | sh_wtot[8];
+    need -= sh_wtot[9];
   }
   prefix <<= 32 - 2 * kHistBits;
   if (tid == 0)
@@ -241,17 +243,17 @@ __device__ __forceinline__ void stream_slice(const unsigned char* sbase, uint32_
                                              float scale, uint32_t* keys_out) {
   const int j = threadIdx.x & 15, rg = threadIdx.x >> 4;
   const uint32_t voff = (uint32_t)(rg * kGemvUnroll) * row_bytes + 16u * (uint32_t)j;
-  for (int it = 0; it < kGemvThreads / kGemvRowsPerIter; ++it) {
+  for (int it = 0; it < kCandThreads / kCandRowsPerIter; ++it) {
     u32x4 kv[kGemvUnroll];
     if constexpr (FULL) {
-      const unsigned char* ibase = sbase + (uint64_t)(it * kGemvRowsPerIter) * row_bytes;   // uniform
+      const unsigned char* ibase = sbase + (uint64_t)(it * kCandRowsPerIter) * row_bytes;   // uniform
 #pragma unroll
       for (int u = 0; u < kGemvUnroll; ++u)
         kv[u] = __builtin_nontemporal_load((const u32x4*)(ibase + (uint64_t)u * row_bytes + voff));
     } else {
 #pragma unroll
       for (int u = 0; u < kGemvUnroll; ++u) {
-        int lt = it * kGemvRowsPerIter + rg * kGemvUnroll + u;
+        int lt = it * kCandRowsPerIter + rg * kGemvUnroll + u;
         lt = lt < n_local ? lt : n_local - 1;
         kv[u] = __builtin_nontemporal_load((const u32x4*)(sbase + ((uint32_t)lt * row_bytes + 16u * (uint32_t)j)));
       }
@@ -263,7 +265,7 @@ __device__ __forceinline__ void stream_slice(const unsigned char* sbase, uint32_
       const float sc = row_score<DT>(qf, kv[u], scale);
       if (j == u) mine = sc;
     }
-    if (j < kGemvUnroll) keys_out[it * kGemvRowsPerIter] = score_key(mine);
+    if (j < kGemvUnroll) keys_out[it * kCandRowsPerIter] = score_key(mine);
   }
 }
 
@@ -273,18 +275,18 @@ __device__ __forceinline__ void stream_slice(const unsigned char* sbase, uint32_
 // the workgroups that start together with the sampling would otherwise sit idle on their CU until the
 // thresholds arrive; with more rows to stream they reach that point when the thresholds are there.
 template <int DT>
-__global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void gemv_candidates_kernel(GemvParams p) {
-  __shared__ uint32_t sh[kHistBins + 8];   // streaming: keys of kEarlySlices * 256 tokens + wave counts; sampling: histogram
-  static_assert(kEarlySlices * kGemvThreads <= kHistBins, "LDS of the streaming role");
+__global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void gemv_candidates_kernel(GemvParams p) {
+  __shared__ uint32_t sh[kHistBins + 16];   // streaming: keys of kEarlySlices * 256 tokens + wave counts; sampling: histogram
+  static_assert(kEarlySlices * kCandThreads <= kHistBins, "LDS of the streaming role");
   const int tid = threadIdx.x;
   if ((int)blockIdx.x < p.sample_wgs) {
     __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
-    const int parts = p.num_samples / kGemvRowsPerIter;
+    const int parts = p.num_samples / kCandRowsPerIter;
     sample_role<DT>(p, (int)blockIdx.x / parts, (int)blockIdx.x % parts, sh);
     return;
   }
   uint32_t* sh_key = sh;                               // keys of this workgroup's tokens, slice after slice
-  uint32_t* sh_wcnt = sh + kEarlySlices * kGemvThreads; // candidates per wave
+  uint32_t* sh_wcnt = sh + kEarlySlices * kCandThreads; // candidates per wave
   __shared__ uint32_t sh_tau[2];                        // the segment's threshold and whether it has arrived
 
   const int j = tid & 15;            // lane inside the row: dims 8j..8j+7
@@ -306,15 +308,15 @@ __global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8,
       const int64_t bh = seg / p.num_chunks;
       const int h = (int)(bh % p.num_kv_heads), b = (int)(bh / p.num_kv_heads);
       const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
-      const int64_t t_begin = (int64_t)wg_in_chunk * kGemvThreads;
-      const int n_local = (int)(p.chunk_len - t_begin < kGemvThreads ? p.chunk_len - t_begin : kGemvThreads);
+      const int64_t t_begin = (int64_t)wg_in_chunk * kCandThreads;
+      const int n_local = (int)(p.chunk_len - t_begin < kCandThreads ? p.chunk_len - t_begin : kCandThreads);
       float qf[8];
       load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
       // uniform base of the slice + 32-bit lane offsets: one address register per load
       const unsigned char* sbase = (const unsigned char*)p.keys +
                                    2 * ((int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h + (chunk_base + t_begin) * p.key_stride_n);
-      uint32_t* keys_out = sh_key + s * kGemvThreads + rg * kGemvUnroll + j;
-      if (n_local == kGemvThreads)
+      uint32_t* keys_out = sh_key + s * kCandThreads + rg * kGemvUnroll + j;
+      if (n_local == kCandThreads)
         stream_slice<DT, true>(sbase, row_bytes, n_local, qf, p.scale, keys_out);
       else
         stream_slice<DT, false>(sbase, row_bytes, n_local, qf, p.scale, keys_out);
@@ -328,8 +330,8 @@ __global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8,
   int64_t tau_seg = first_seg, seg = first_seg;
   int wg_in_chunk = first_wg;
   for (int s = 0; s < num_slices; ++s) {
-    const int64_t t_begin = (int64_t)wg_in_chunk * kGemvThreads;
-    int64_t t_end = t_begin + kGemvThreads;
+    const int64_t t_begin = (int64_t)wg_in_chunk * kCandThreads;
+    int64_t t_end = t_begin + kCandThreads;
     if (t_end > p.chunk_len) t_end = p.chunk_len;
     // Threshold of the slice's segment: one lane fetches the word and hands it on through LDS (every wave
     // asking for itself makes a hot spot of the few words).  A bounded wait: a workgroup that never sees its
@@ -353,9 +355,9 @@ __global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8,
     }
 
     // thread t owns token t_begin + t: candidates in index order into the slice.
-    // Slice format: word = key << 32 | count << 8 | token - first token of the slice; only entry 0 carries
-    // the count (0 .. 256), so a workgroup with few candidates writes a single line and nothing else.
-    const uint32_t key = sh_key[s * kGemvThreads + tid];
+    // Slice format: word = key << 32 | count << 9 | token - first token of the slice; only entry 0 carries
+    // the count (0 .. 512), so a workgroup with few candidates writes a single line and nothing else.
+    const uint32_t key = sh_key[s * kCandThreads + tid];
     const bool pass = tau_ready && t_begin + tid < t_end && key >= tau;
     const unsigned long long mask = __ballot(pass);
     if (s) __syncthreads();   // the previous slice's counts have been read
@@ -363,15 +365,15 @@ __global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(8,
     __syncthreads();
     uint32_t before = 0, total = 0;
 #pragma unroll
-    for (int v = 0; v < kGemvWaves; ++v) {
+    for (int v = 0; v < kCandWaves; ++v) {
       const uint32_t c = sh_wcnt[v];
       before += v < wave ? c : 0u;
       total += c;
     }
-    uint64_t* slice = p.cand + seg * p.cand_seg_stride + (int64_t)wg_in_chunk * kGemvThreads;
+    uint64_t* slice = p.cand + seg * p.cand_seg_stride + (int64_t)wg_in_chunk * kCandThreads;
     if (pass) {
       const uint32_t pos = before + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-      slice[pos] = ((uint64_t)key << 32) | (pos == 0 ? total << 8 : 0u) | (uint32_t)tid;
+      slice[pos] = ((uint64_t)key << 32) | (pos == 0 ? total << 9 : 0u) | (uint32_t)tid;
     }
     if (tid == 0 && total == 0) slice[0] = 0ull;
     if (++wg_in_chunk == p.wgs_per_chunk) { wg_in_chunk = 0; ++seg; }
@@ -390,26 +392,26 @@ int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
   return hip_status(hipGetLastError());
 }
 
-// Candidate mode: sampling workgroups (128 samples each) at the front of the grid, then the streaming ones.
+// Candidate mode: sampling workgroups (256 samples each) at the front of the grid, then the streaming ones.
 int launch_gemv_candidates(const GemvParams& p0, int dtype, hipStream_t stream) {
   GemvParams p = p0;
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  if (p.tokens_per_wg != kGemvThreads || p.num_samples < kGemvRowsPerIter || p.num_samples % kGemvRowsPerIter ||
+  if (p.tokens_per_wg != kCandThreads || p.num_samples < kCandRowsPerIter || p.num_samples % kCandRowsPerIter ||
       p.num_samples > kGemvMaxSamples || p.sample_rank < 1 || p.sample_rank > p.num_samples)
     return TKA_EINVAL;
-  p.sample_wgs = (int)(segs * (p.num_samples / kGemvRowsPerIter));
-  // early workgroups: as many as the GPU holds at once (256 CUs x 8)
+  p.sample_wgs = (int)(segs * (p.num_samples / kCandRowsPerIter));
+  // early workgroups: as many as the GPU holds at once (256 CUs x 4 workgroups of 8 waves)
   const int64_t slices = segs * p.wgs_per_chunk;
-  int64_t early = 2048;
+  int64_t early = 1024;
   if (early > slices / (2 * kEarlySlices)) early = slices / (2 * kEarlySlices);
   p.early_wgs = (int)early;
   const int64_t wgs = p.sample_wgs + early + (slices - early * kEarlySlices);
   if (wgs > 0x7fffffffLL) return TKA_EUNSUPPORTED;
   LaunchTimer timer("gemv_candidates", stream);
   if (dtype == TKA_F16)
-    gemv_candidates_kernel<TKA_F16><<<(unsigned)wgs, kGemvThreads, 0, stream>>>(p);
+    gemv_candidates_kernel<TKA_F16><<<(unsigned)wgs, kCandThreads, 0, stream>>>(p);
   else
-    gemv_candidates_kernel<TKA_BF16><<<(unsigned)wgs, kGemvThreads, 0, stream>>>(p);
+    gemv_candidates_kernel<TKA_BF16><<<(unsigned)wgs, kCandThreads, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 
@@ -418,7 +420,7 @@ int launch_gemv_candidates(const GemvParams& p0, int dtype, hipStream_t stream) 
 // gets a workgroup.
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len) {
   (void)chunk_len;
-  return total_rows <= 65536 ? 128 : kGemvCandTokensPerWg;
+  return total_rows <= 65536 ? 128 : kGemvDenseTokensPerWg;
 }
 
 // Candidate-mode plan for one segment length and k: samples per segment and the rank of the order statistic

@@ -20,7 +20,7 @@ struct GemvParams {
   int sample_wgs;             // sampling workgroups at the front of the candidate grid (set by the launcher)
   int early_wgs;              // streaming workgroups behind them that take several slices each (set by the launcher)
   uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] one slice per workgroup, ascending index:
-                              // key << 32 | count << 8 | token offset in the slice (count in entry 0 only)
+                              // key << 32 | count << 9 | token offset in the slice (count in entry 0 only)
   int64_t cand_seg_stride;    // entries between the slice arrays of consecutive segments
   int64_t chunk_len;    // tokens per chunk
   int64_t q_stride_b, key_stride_b, key_stride_n, key_stride_h;

@@ -492,7 +492,8 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint64_t* sh_ent = (uint64_t*)smem;
   __shared__ uint32_t sh_hist[kHistBins];
-  constexpr int kGroups = kSelThreads / 16, kInFlight = 8, kRound = kGroups * kInFlight;   // 512 slices per round
+  constexpr int kSliceLanes = 32;   // lanes that copy one slice (a slice of 512 tokens holds about 18 candidates)
+  constexpr int kGroups = kSelThreads / kSliceLanes, kInFlight = 8, kRound = kGroups * kInFlight;   // 256 slices per round
   __shared__ uint32_t sh_cnt[kRound], sh_start[kRound];
   __shared__ uint32_t sh_pos[kCandMaxParts + 1];   // start positions of all slices (segments with more than kRound slices)
   __shared__ uint32_t sh_wtot[kSelWaves];
@@ -506,12 +507,12 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
 
-  // Copy the slices into LDS.  Up to kRound slices: 16 lanes per slice load its first 16 entries (entry 0 carries
+  // Copy the slices into LDS.  Up to kRound slices: 32 lanes per slice load its first 32 entries (entry 0 carries
   // the slice's count; entries beyond the count are stale memory and ignored), the counts are scanned into
   // start positions, and the entries go to their place: one memory round trip.
   const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
   const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;   // (not read when the entries come from keys or scores)
-  const int sub = tid & 15, grp = tid >> 4;
+  const int sub = tid & (kSliceLanes - 1), grp = tid / kSliceLanes;
   uint32_t n_entries = 0;
   if (p.from_keys) {
     // Short segments: no GEMV launch before this one.  The workgroup scores its segment itself (64 row groups
@@ -568,7 +569,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
       }
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
-        cnt[u] = ((uint32_t)__shfl((int)(uint32_t)first[u], lane & ~15, 64) >> 8) & 0x1ffu;
+        cnt[u] = ((uint32_t)__shfl((int)(uint32_t)first[u], lane & ~(kSliceLanes - 1), 64) >> 9) & 0x3ffu;
         if (sub == 0) sh_cnt[u * kGroups + grp] = cnt[u];
       }
       __syncthreads();
@@ -583,10 +584,10 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
         const uint32_t start = sh_start[u * kGroups + grp];
         const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
         if ((uint32_t)sub < cnt[u] && start + sub < cap)
-          sh_ent[start + sub] = (first[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)first[u] & 0xffu));
-        for (uint32_t j = 16u + sub; j < cnt[u] && start + j < cap; j += 16u) {   // rare: a slice with more than 16 candidates
+          sh_ent[start + sub] = (first[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)first[u] & 0x1ffu));
+        for (uint32_t j = kSliceLanes + sub; j < cnt[u] && start + j < cap; j += kSliceLanes) {   // rare: a slice with more than 32 candidates
           const uint64_t w = lists[(int64_t)sl * p.part_len + j];
-          sh_ent[start + j] = (w & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w & 0xffu));
+          sh_ent[start + j] = (w & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w & 0x1ffu));
         }
       }
       n_entries += total;
@@ -597,7 +598,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int sl = 4 * tid + q;
-      c4[q] = sl < p.parts ? ((uint32_t)lists[(int64_t)sl * p.part_len] >> 8) & 0x1ffu : 0u;
+      c4[q] = sl < p.parts ? ((uint32_t)lists[(int64_t)sl * p.part_len] >> 9) & 0x3ffu : 0u;
       sum += c4[q];
     }
     uint32_t total;
@@ -625,10 +626,10 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
         const int sl = s0 + u * kGroups + grp;
         const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
         if ((uint32_t)sub < cnt[u] && start[u] + sub < cap)
-          sh_ent[start[u] + sub] = (w[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w[u] & 0xffu));
-        for (uint32_t j = 16u + sub; j < cnt[u] && start[u] + j < cap; j += 16u) {
+          sh_ent[start[u] + sub] = (w[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w[u] & 0x1ffu));
+        for (uint32_t j = kSliceLanes + sub; j < cnt[u] && start[u] + j < cap; j += kSliceLanes) {
           const uint64_t x = lists[(int64_t)sl * p.part_len + j];
-          sh_ent[start[u] + j] = (x & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)x & 0xffu));
+          sh_ent[start[u] + j] = (x & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)x & 0x1ffu));
         }
       }
     }
