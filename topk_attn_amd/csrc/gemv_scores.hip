@@ -234,8 +234,8 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
     __hip_atomic_store(p.tau_words + seg, ((uint64_t)p.epoch << 32) | prefix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Scores of one slice (up to 256 tokens from sbase on) as keys into LDS: lane j < 8 of row group rg writes the
-// key of token it*128 + rg*8 + j to keys_out[it*128].  FULL: the slice has all 256 tokens; the eight rows of
+// Scores of one slice (up to 512 tokens from sbase on) as keys into LDS: lane j < 8 of row group rg writes the
+// key of token it*256 + rg*8 + j to keys_out[it*256].  FULL: the slice has all 512 tokens; the eight rows of
 // a lane then differ by a uniform offset and one lane offset serves all loads.  Otherwise rows past the end
 // are clamped to the last one, lane by lane.
 template <int DT, bool FULL>
@@ -270,13 +270,13 @@ __device__ __forceinline__ void stream_slice(const unsigned char* sbase, uint32_
 }
 
 // Grid: p.sample_wgs sampling workgroups first (so that they are resident before any workgroup that waits for
-// them), then the streaming workgroups.  Slices (256 tokens) are numbered segment-major.  The first
+// them), then the streaming workgroups.  Slices (512 tokens) are numbered segment-major.  The first
 // p.early_wgs streaming workgroups take kEarlySlices consecutive slices each, all later ones a single slice:
 // the workgroups that start together with the sampling would otherwise sit idle on their CU until the
 // thresholds arrive; with more rows to stream they reach that point when the thresholds are there.
 template <int DT>
 __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void gemv_candidates_kernel(GemvParams p) {
-  __shared__ uint32_t sh[kHistBins + 16];   // streaming: keys of kEarlySlices * 256 tokens + wave counts; sampling: histogram
+  __shared__ uint32_t sh[kHistBins + 16];   // streaming: keys of kEarlySlices * 512 tokens + wave counts; sampling: histogram
   static_assert(kEarlySlices * kCandThreads <= kHistBins, "LDS of the streaming role");
   const int tid = threadIdx.x;
   if ((int)blockIdx.x < p.sample_wgs) {
