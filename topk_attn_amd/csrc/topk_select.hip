@@ -188,6 +188,106 @@ __device__ __forceinline__ void write_rank_outputs(const uint64_t* sh_sort, cons
   }
 }
 
+// Rank order of the k selected composites in sh_sort[0 .. k) (any order on entry; [k, kpad) must be zero), descending
+// on exit.  Instead of a bitonic network over all of them: key minus smallest key, cut to its 11 leading bits,
+// gives up to 2048 buckets in rank order; a histogram and one suffix scan give every bucket its first rank; the
+// composites are scattered to their bucket (sh_xchg) and each one counts the larger members of its own bucket.
+// Buckets are small on ordinary data (k / (occupied buckets)); when one exceeds kRankBucketMax (heavy ties in
+// the score AND neighbouring indices, or k < 3) the bitonic network does the job instead.
+// sh_xchg: kpad composites; sh_hist, sh_off: 2048 words each; sh_mm: 2 composites + 1 word.  All 1024 threads call.
+constexpr uint32_t kRankBucketMax = 96;
+__device__ __forceinline__ void rank_sort_desc(uint64_t* sh_sort, uint64_t* sh_xchg, uint32_t k, int kpad, uint32_t* sh_hist,
+                                               uint32_t* sh_off, uint32_t* sh_wtot, uint64_t* sh_mm) {
+  if (kpad <= 1024) {   // a small network (one composite per thread) is quicker than the bucket bookkeeping
+    sort_lds_desc(sh_sort, sh_xchg, kpad);
+    return;
+  }
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  constexpr int kMaxPer = TKA_MAX_TOPK / kSelThreads;   // 8 composites per thread at most
+  uint32_t* sh_big = (uint32_t*)(sh_mm + 2);
+  uint64_t c[kMaxPer];
+  uint64_t cmin = ~0ull, cmax = 0ull;
+#pragma unroll
+  for (int e = 0; e < kMaxPer; ++e) {
+    const uint32_t i = (uint32_t)e * kSelThreads + tid;
+    c[e] = i < k ? sh_sort[i] : 0ull;
+    if (i < k) {
+      cmin = c[e] < cmin ? c[e] : cmin;
+      cmax = c[e] > cmax ? c[e] : cmax;
+    }
+  }
+  if (tid == 0) { sh_mm[0] = ~0ull; sh_mm[1] = 0ull; *sh_big = 0u; }
+  sh_hist[2 * tid] = 0;
+  sh_hist[2 * tid + 1] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint64_t a = __shfl_xor(cmin, d, 64), b = __shfl_xor(cmax, d, 64);
+    cmin = a < cmin ? a : cmin;
+    cmax = b > cmax ? b : cmax;
+  }
+  if (lane == 0) {
+    atomicMin((unsigned long long*)&sh_mm[0], (unsigned long long)cmin);
+    atomicMax((unsigned long long*)&sh_mm[1], (unsigned long long)cmax);
+  }
+  __syncthreads();
+  cmin = sh_mm[0];
+  cmax = sh_mm[1];
+  // buckets are linear in (key - smallest key): the bits of a float key that two scores share say little once
+  // the scores straddle a power of two
+  const uint64_t base = cmin & 0xffffffff00000000ull;
+  const int fixed = cmax - base == 0 ? 64 - kHistBits : __builtin_clzll(cmax - base);
+  const int bits = (64 - fixed) >= kHistBits ? kHistBits : (64 - fixed);
+  const int shift = 64 - fixed - bits;
+  uint32_t slot[kMaxPer];
+#pragma unroll
+  for (int e = 0; e < kMaxPer; ++e) {
+    const uint32_t i = (uint32_t)e * kSelThreads + tid;
+    slot[e] = i < k ? atomicAdd(&sh_hist[(uint32_t)((c[e] - base) >> shift)], 1u) : 0u;
+  }
+  __syncthreads();
+  // first rank of every bucket: number of composites in higher buckets (thread t owns buckets 2t, 2t+1)
+  {
+    const uint32_t h0 = sh_hist[2 * tid], h1 = sh_hist[2 * tid + 1];
+    const uint32_t mine = h0 + h1;
+    const uint32_t inc = wave_inclusive_scan(mine);
+    const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)inc, 63);
+    const uint32_t ge = wave_total - inc + mine;   // this wave's composites in buckets >= 2t
+    if (lane == 0) sh_wtot[wave] = ge;
+    if (h0 > kRankBucketMax || h1 > kRankBucketMax) *sh_big = 1u;
+    __syncthreads();
+    uint32_t above = 0;
+    for (int w = wave + 1; w < kSelWaves; ++w) above += sh_wtot[w];
+    sh_off[2 * tid + 1] = above + ge - mine;        // buckets > 2t+1
+    sh_off[2 * tid] = above + ge - h0;              // buckets > 2t
+  }
+  __syncthreads();
+  if (*sh_big != 0u || k < 3u) {
+    sort_lds_desc(sh_sort, sh_xchg, kpad);
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < kMaxPer; ++e) {
+    const uint32_t i = (uint32_t)e * kSelThreads + tid;
+    if (i < k) sh_xchg[sh_off[(uint32_t)((c[e] - base) >> shift)] + slot[e]] = c[e];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < kMaxPer; ++e) {
+    const uint32_t i = (uint32_t)e * kSelThreads + tid;
+    if (i < k) {
+      const uint64_t x = sh_xchg[i];
+      const uint32_t bin = (uint32_t)((x - base) >> shift);
+      const uint32_t first = sh_off[bin], cnt = sh_hist[bin];
+      uint32_t larger = 0;
+      for (uint32_t j = 0; j < cnt; ++j) larger += sh_xchg[first + j] > x ? 1u : 0u;
+      sh_sort[first + larger] = x;
+    }
+  }
+  __syncthreads();
+}
+
 // Dynamic LDS of select_finalize_kernel (rank mode only): kpad composites (sort buffer), then kpad
 // composites (cross-wave exchange buffer).
 __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectParams p, int kpad) {
@@ -331,7 +431,8 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
   if (!want_rank) return;
   __syncthreads();
 
-  sort_lds_desc(sh_sort, sh_xchg, kpad);
+  __shared__ uint64_t sh_mm[3];
+  rank_sort_desc(sh_sort, sh_xchg, k, kpad, sh_hist, sh_ends, sh_wtot, sh_mm);   // (the slice offsets are spent)
   write_rank_outputs(sh_sort, p, seg);
 }
 
@@ -342,10 +443,11 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
 // kept in LDS), radix passes over the stored scores until the k-th largest key is fixed, then one walk in
 // index order that takes every key above the threshold bucket and the first `need` keys inside it.  Exact for
 // any data; slow (one CU streams the segment), which is acceptable for an event that the sampling makes rare.
-// sh_sort: 2*kpad composites (rank mode only).  Every thread of the block must call it.
+// sh_sort: 2*kpad composites (rank mode only); sh_hist, sh_off: 2048 words each.  Every thread of the block must call it.
 template <int DT>
 __device__ __forceinline__ void fallback_segment(const GemvParams& g, const SelectParams& p, int seg, int kpad, uint64_t* sh_sort,
-                                                 uint32_t* sh_hist, uint32_t* sh_wtot, uint32_t* sh_res) {
+                                                 uint32_t* sh_hist, uint32_t* sh_off, uint32_t* sh_wtot, uint32_t* sh_res,
+                                                 uint64_t* sh_mm) {
   uint64_t* sh_xchg = sh_sort + kpad;
   const int tid = threadIdx.x;
   const uint32_t k = (uint32_t)p.k;
@@ -469,7 +571,7 @@ __device__ __forceinline__ void fallback_segment(const GemvParams& g, const Sele
   if (want_union) write_union_edges(uo, p, seg, lo, hi, run_mid);
   if (!want_rank) return;
   __syncthreads();
-  sort_lds_desc(sh_sort, sh_xchg, kpad);
+  rank_sort_desc(sh_sort, sh_xchg, k, kpad, sh_hist, sh_off, sh_wtot, sh_mm);
   write_rank_outputs(sh_sort, p, seg);
 }
 
@@ -499,6 +601,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
   __shared__ uint32_t sh_kminmax[2];
+  __shared__ uint64_t sh_mm[3];
   __shared__ uint64_t sh_small[kSmallBucket];
   __shared__ uint32_t sh_small_cnt;
 
@@ -650,7 +753,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   }
   if (redo) {
     __syncthreads();
-    fallback_segment<DT>(g, p, seg, kpad, sh_ent, sh_hist, sh_wtot, sh_res);
+    fallback_segment<DT>(g, p, seg, kpad, sh_ent, sh_hist, sh_pos, sh_wtot, sh_res, sh_mm);
     return;
   }
   if (whole && p.out_idx != nullptr && p.union_idx == nullptr && n_entries <= 2u * kSelThreads) {
@@ -659,7 +762,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     while (npad < n_entries) npad <<= 1;
     for (uint32_t i = n_entries + tid; i < npad; i += kSelThreads) sh_ent[i] = 0;   // pad: below every real composite
     __syncthreads();
-    sort_lds_desc(sh_ent, sh_ent + npad, (int)npad);
+    sort_lds_desc(sh_ent, sh_ent + npad, (int)npad);   // (measured quicker here than the bucketed rank sort)
     write_rank_outputs(sh_ent, p, seg);
     return;
   }
@@ -695,8 +798,15 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     __syncthreads();
     kmin = sh_kminmax[0];
     kmax = sh_kminmax[1];
-    int fixed = kmin == kmax ? 32 : __builtin_clz(kmin ^ kmax);
-    uint64_t prefix = fixed ? (uint64_t)(kmax >> (32 - fixed)) : 0ull;
+    // Radix passes on the composites relative to the smallest key: their leading bits are zero down to the
+    // width of the key range, and the 11 bits below spread the candidates evenly (shared bits of the float
+    // keys themselves say little once the scores straddle a power of two).
+    const uint64_t base = (uint64_t)kmin << 32;
+#pragma unroll
+    for (int i = 0; i < kCandPerThread; ++i)
+      if ((uint32_t)i * kSelThreads + tid < n_entries) mine[i] -= base;
+    int fixed = kmin == kmax ? 32 : __builtin_clz(kmax - kmin);
+    uint64_t prefix = 0ull;
     uint32_t need = k;
     bool done = false;
     while (!done) {
@@ -737,6 +847,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
         done = true;
       }
     }
+    threshold += base;   // back from the relative composites
   }
 
   // Walk in index order: thread t takes the run of `per` consecutive entries starting at t*per.
@@ -781,7 +892,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     for (int i = (int)k + tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite
   }
   __syncthreads();
-  sort_lds_desc(sh_sort, sh_xchg, kpad);
+  rank_sort_desc(sh_sort, sh_xchg, k, kpad, sh_hist, sh_pos, sh_wtot, sh_mm);   // (the slice positions are spent)
   write_rank_outputs(sh_sort, p, seg);
 }
 
