@@ -241,12 +241,19 @@ __global__ __launch_bounds__(kCombineThreads) void lse_combine_kernel(CombinePar
   // accumulators: group g takes splits g, g+32, ...
   const int g = tid / kCombineLanes, dl = tid % kCombineLanes;
   f32x4 o = (f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int s = g; s < S; s += kCombineGroups) {
-    const float w = sh_w[s];
-    if (w != 0.0f) {
-      const f32x4 a = pa[(int64_t)s * kCombineLanes + dl];
-      o += a * w;
+  // four splits per trip, loads first: a load behind the weight test would make every trip a memory round trip
+  for (int s0 = g; s0 < S; s0 += 4 * kCombineGroups) {
+    f32x4 a[4];
+    float w[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int s = s0 + u * kCombineGroups;
+      w[u] = s < S ? sh_w[s] : 0.0f;
+      a[u] = pa[(int64_t)(s < S ? s : g) * kCombineLanes + dl];
     }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (w[u] != 0.0f) o += a[u] * w[u];   // the accumulator of an empty split is never looked at
   }
   sh_o[g][dl] = o;
   __syncthreads();
