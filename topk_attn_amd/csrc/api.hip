@@ -269,7 +269,8 @@ void flash_plan(const tka_flash_decode_args* a, int* splits, int* tokens_per_spl
   const int64_t len = a->kv_idx ? a->idx_len : a->seq_len;
   int64_t want = a->num_splits;
   if (want <= 0) {
-    want = 2048 / ((int64_t)a->batch * a->num_kv_heads);
+    // measured: the dense scan likes about 2048 workgroups, the gathered form about one resident set (3 per CU)
+    want = (a->kv_idx ? 1024 : 2048) / ((int64_t)a->batch * a->num_kv_heads);
     if (want < 1) want = 1;
   }
   int64_t tps = (len + want - 1) / want;
