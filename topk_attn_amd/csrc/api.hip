@@ -201,7 +201,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
 
   int num_samples = 0, sample_rank = 0;
   const int64_t cand_slices = (chunk_len + kGemvCandTokensPerWg - 1) / kGemvCandTokensPerWg;
-  if (!a->out_scores && cand_slices <= select_cand_max_parts())
+  // (the candidate kernel addresses the rows of a slice with 32-bit byte offsets)
+  if (!a->out_scores && cand_slices <= select_cand_max_parts() && a->key_stride_n < (int64_t)1 << 21)
     gemv_candidate_plan(chunk_len, a->k, select_cand_capacity(), &num_samples, &sample_rank);
   if (num_samples == 0) {
     // dense: clear histograms, GEMV with histogram, filter, finalize
