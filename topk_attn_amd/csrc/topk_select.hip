@@ -27,6 +27,10 @@
 // used, redoes the segment from the keys (fallback_segment).
 #include <stdlib.h>
 
+#include <mutex>
+#include <utility>
+#include <vector>
+
 #include "kernels.hpp"
 #include "bitonic.hpp"
 
@@ -1038,14 +1042,22 @@ int launch_select_hist(const SelectParams& p, hipStream_t stream) {
   return hip_status(hipGetLastError());
 }
 
-static int set_finalize_attr() {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 130 * 1024);  // 2 x 8192 composites; 25 KB are static
-    if (e != hipSuccess) return TKA_EHIP;
-    attr_set = true;
-  }
+// Raises a kernel's dynamic-LDS limit once per (kernel, device); safe to call from several host threads.
+static int allow_dynamic_lds(const void* kernel, int bytes) {
+  static std::mutex guard;
+  static std::vector<std::pair<const void*, int>> done;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return TKA_EHIP;
+  std::lock_guard<std::mutex> lock(guard);
+  for (const auto& d : done)
+    if (d.first == kernel && d.second == device) return TKA_OK;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return TKA_EHIP;
+  done.emplace_back(kernel, device);
   return TKA_OK;
+}
+
+static int set_finalize_attr() {
+  return allow_dynamic_lds((const void*)select_finalize_kernel, 130 * 1024);   // 2 x 8192 composites; 25 KB are static
 }
 
 int launch_select_filter(const SelectParams& p, hipStream_t stream) {
@@ -1074,16 +1086,9 @@ int select_cand_capacity() { return kCandCap; }
 int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
   if ((p.from_keys || p.from_scores) ? p.seg_len > kCandCap : p.parts > kCandMaxParts) return TKA_EINVAL;
   if (p.k > kCandCap / 2) return TKA_EINVAL;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)select_finalize_cand_kernel<TKA_F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       kCandCap * (int)sizeof(uint64_t));
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)select_finalize_cand_kernel<TKA_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kCandCap * (int)sizeof(uint64_t));
-    if (e != hipSuccess) return TKA_EHIP;
-    attr_set = true;
-  }
+  if (allow_dynamic_lds((const void*)select_finalize_cand_kernel<TKA_F16>, kCandCap * (int)sizeof(uint64_t)) != TKA_OK ||
+      allow_dynamic_lds((const void*)select_finalize_cand_kernel<TKA_BF16>, kCandCap * (int)sizeof(uint64_t)) != TKA_OK)
+    return TKA_EHIP;
   LaunchTimer timer(p.from_keys ? "gemv_topk_fused" : (p.from_scores ? "select_whole" : "select_finalize_cand"), stream);
   // entries of the segment; rank mode reuses the buffer as sort + exchange buffers (2 x kpad, or 2 x the padded
   // segment when a short segment is sorted whole).  Short segments leave room for two workgroups per CU.
@@ -1113,12 +1118,7 @@ int launch_select(const SelectParams& p, hipStream_t stream) {
 int launch_index_union(const UnionParams& p, hipStream_t stream) {
   const int kpad = kpad_for(p.k);
   const size_t lds = 2 * (size_t)kpad * sizeof(uint64_t);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)index_union_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
-    if (e != hipSuccess) return TKA_EHIP;
-    attr_set = true;
-  }
+  if (allow_dynamic_lds((const void*)index_union_kernel, 144 * 1024) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("index_union", stream);
   index_union_kernel<<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(p, kpad);
   return hip_status(hipGetLastError());
