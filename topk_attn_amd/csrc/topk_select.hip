@@ -718,23 +718,26 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     if (tid == kSelThreads - 1) sh_pos[kCandMaxParts] = total;
     n_entries = total;
     __syncthreads();
-    for (int s0 = 0; s0 < p.parts; s0 += kRound) {
+    // long segments are sparse in candidates per slice: 8 lanes per slice, 1024 slices per trip
+    constexpr int kLanes2 = 8, kGroups2 = kSelThreads / kLanes2, kRound2 = kGroups2 * kInFlight;
+    const int sub2 = tid & (kLanes2 - 1), grp2 = tid / kLanes2;
+    for (int s0 = 0; s0 < p.parts; s0 += kRound2) {
       uint64_t w[kInFlight];
       uint32_t start[kInFlight], cnt[kInFlight];
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
-        const int sl = s0 + u * kGroups + grp;
+        const int sl = s0 + u * kGroups2 + grp2;
         start[u] = sl < p.parts ? sh_pos[sl] : 0u;
         cnt[u] = sl < p.parts ? sh_pos[sl + 1] - start[u] : 0u;
-        w[u] = (uint32_t)sub < cnt[u] ? lists[(int64_t)sl * p.part_len + sub] : 0ull;
+        w[u] = (uint32_t)sub2 < cnt[u] ? lists[(int64_t)sl * p.part_len + sub2] : 0ull;
       }
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
-        const int sl = s0 + u * kGroups + grp;
+        const int sl = s0 + u * kGroups2 + grp2;
         const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
-        if ((uint32_t)sub < cnt[u] && start[u] + sub < cap)
-          sh_ent[start[u] + sub] = (w[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w[u] & 0x1ffu));
-        for (uint32_t j = kSliceLanes + sub; j < cnt[u] && start[u] + j < cap; j += kSliceLanes) {
+        if ((uint32_t)sub2 < cnt[u] && start[u] + sub2 < cap)
+          sh_ent[start[u] + sub2] = (w[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w[u] & 0x1ffu));
+        for (uint32_t j = kLanes2 + sub2; j < cnt[u] && start[u] + j < cap; j += kLanes2) {
           const uint64_t x = lists[(int64_t)sl * p.part_len + j];
           sh_ent[start[u] + j] = (x & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)x & 0x1ffu));
         }
