@@ -78,6 +78,25 @@ def test_shared_kv_chunked():
     _run_flat(oracle.F16, 2, 4, 1, 8192, 128, seed=6, shared_kv=True, num_chunks=4, scale=1.0)
 
 
+@pytest.mark.parametrize("B,H", [(2, 32), (3, 22), (5, 13), (8, 8), (9, 8), (17, 4)])
+def test_shared_kv_batch_tiles(B, H):
+    """Keys shared by the batch are scored for several batch entries per pass (tiles of 2, 4 or 8 entries, with
+    a ragged last tile) and the 256 or more short segments are selected one per wavefront."""
+    announce("gemv_topk shared KV batch tiles B=%d H=%d N=8192 chunks=4 k=128" % (B, H))
+    _run_flat(oracle.F16, B, H, 1, 8192, 128, seed=60 + B, shared_kv=True, num_chunks=4, scale=1.0)
+
+
+def test_many_short_segments_routes():
+    """256 or more segments of at most 2048 rows: plain scores + one wavefront per segment; both dtypes, grouped
+    queries, odd lengths, ties, keys per sequence and shared."""
+    announce("gemv_topk many short segments")
+    _run_flat(oracle.BF16, 8, 8, 2, 8000, 500, seed=70, num_chunks=4)                      # per-sequence keys
+    _run_flat(oracle.BF16, 6, 11, 4, 4000, 1000, seed=71, shared_kv=True, num_chunks=4, levels=True)   # ties, k = n
+    _run_flat(oracle.F16, 16, 16, 1, 1999, 1024, seed=72, shared_kv=True)                  # odd length, largest k
+    _run_flat(oracle.F16, 8, 32, 1, 300, 7, seed=73, shared_kv=True)                       # tiny segments
+    _run_flat(oracle.F16, 3, 2, 1, 12000, 300, seed=74, shared_kv=True)                    # shared keys, one workgroup per segment
+
+
 def test_tie_stress_bf16_levels():
     """K quantised to 16 levels: many exact score ties; indices must still match bit for bit."""
     announce("gemv_topk tie stress bf16 N=65536 G=8 k=4096")

@@ -85,6 +85,49 @@ def test_strided_segments():
         assert np.array_equal(idx[r].cpu().numpy(), ei)
 
 
+def _short_segment_rows(rng, n):
+    """Rows that stress every radix pass of a short segment: ties in the key, in its leading bits, specials."""
+    levels = np.linspace(-2, 2, 16).astype(np.float32)
+    tiny = (1.0 + np.arange(n) % 5 * 2.0 ** -23).astype(np.float32)        # keys that differ in the last bits only
+    close = (1.0 + rng.integers(0, 1 << 12, n) * 2.0 ** -23).astype(np.float32)
+    special = rng.standard_normal(n).astype(np.float32)
+    special[::7] = 0.0
+    special[3::7] = -0.0
+    special[5::97] = np.inf
+    special[11::89] = -np.inf
+    special[13::101] = np.nan
+    wide = (rng.standard_normal(n) * 10.0 ** rng.integers(-30, 30, n)).astype(np.float32)
+    return [rng.standard_normal(n).astype(np.float32), np.full(n, -3.25, np.float32), levels[rng.integers(0, 16, n)], tiny,
+            close, special, wide, np.arange(n, dtype=np.float32), -np.arange(n, dtype=np.float32),
+            np.abs(rng.standard_normal(n)).astype(np.float32), np.full(n, np.nan, np.float32)]
+
+
+@pytest.mark.parametrize("n,k", [(2048, 128), (2048, 1024), (2048, 2048 // 2 - 1), (2048, 1), (2047, 33), (1024, 64),
+                                 (1280, 512), (777, 777), (64, 5), (3, 2), (1, 1)])
+def test_short_segments(n, k):
+    """Segments of at most 2048 scores, many per call (the operator's chunks): adversarial rows and random ones."""
+    announce("topk short segments n=%d k=%d" % (n, k))
+    rng = np.random.default_rng(n * 7 + k)
+    rows = _short_segment_rows(rng, n)
+    rows += [rng.standard_normal(n).astype(np.float32) for _ in range(256)]   # enough segments for the wavefront route
+    _check(np.stack(rows), k)
+
+
+def test_short_segments_many():
+    """4096 segments in one call (32 batch entries x 32 heads x 4 chunks of the operator)."""
+    announce("topk short segments 4096 x 2048, k=128")
+    from topk_attn_amd import ops
+    rng = np.random.default_rng(99)
+    x = rng.standard_normal((4096, 2048)).astype(np.float32)
+    x[:, ::3] = np.round(x[:, ::3], 1)      # ties across the rank boundary
+    idx, val = ops.topk(torch.from_numpy(x).cuda(), 128)
+    torch.cuda.synchronize()
+    idx, val = idx.cpu().numpy(), val.cpu().numpy()
+    order = np.lexsort((np.broadcast_to(np.arange(2048), x.shape), -x), axis=1)[:, :128]
+    assert np.array_equal(idx, order.astype(np.int32))
+    assert np.array_equal(val, np.take_along_axis(x, order, axis=1))
+
+
 def test_rejects_bad_k():
     from topk_attn_amd import ops, TkaError
     s = torch.zeros(2, 100, device="cuda")

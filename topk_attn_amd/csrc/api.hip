@@ -137,6 +137,19 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
 }
 
+// Short segments in numbers: one wavefront per segment selects (no workgroup barriers; a compute unit works on
+// many segments at a time).
+int wave_select_min_segments() {
+  static const int v = [] {
+    const char* e = getenv("TKA_WAVE_MIN_SEGS");
+    return e && *e ? atoi(e) : 256;
+  }();
+  return v;
+}
+bool wave_select_fits(int64_t seg_len, int k, int64_t segments) {
+  return seg_len <= select_wave_max_len() && k <= select_wave_max_k() && segments >= wave_select_min_segments();
+}
+
 struct UnionOut {
   int32_t* idx;
   int32_t* count;
@@ -145,8 +158,9 @@ struct UnionOut {
 
 // Runs clear + GEMV (+histogram) + select.  `ws` holds [scores][select workspace].
 // a->out_idx == nullptr skips the rank-order sort (then `u` must ask for the union list).
+// `any_order`: the caller does not need out_idx / out_val in rank order (a route may still deliver it).
 int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, const int32_t* cluster_ids = nullptr,
-                  const UnionOut* u = nullptr) {
+                  const UnionOut* u = nullptr, bool any_order = false) {
   hipStream_t stream = (hipStream_t)a->stream;
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
@@ -181,6 +195,19 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   fill_gemv_params(a, scores, sp.hist, &gp);
   gp.cluster_ids = cluster_ids;
 
+  // Keys shared by the batch are read once for several batch entries.
+  const bool shared_keys = a->key_stride_b == 0 && a->batch >= 2 && !cluster_ids;
+
+  // Many short segments: plain scores, then one wavefront per segment selects.
+  if (a->out_idx && !u && wave_select_fits(chunk_len, a->k, segs)) {
+    gp.hist = nullptr;
+    int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);
+    if (rc != TKA_OK) return rc;
+    SelectParams sw = sp;
+    sw.unordered = any_order ? 1 : 0;
+    return launch_select_wave(sw, stream);
+  }
+
   // Short segments: one launch, each workgroup scores and selects its own segment.  One CU pulls about
   // 55 GB/s, so beyond 2048 rows (0.5 MB) the separate GEMV launch with many workgroups per segment wins.
   if (!a->out_scores && chunk_len <= kFusedMaxSegLen) {
@@ -192,7 +219,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // Segments that fit in LDS whole: GEMV that stores plain scores (no histogram), then one selection launch.
   if (chunk_len <= select_cand_capacity()) {
     gp.hist = nullptr;
-    int rc = launch_gemv_scores(gp, a->dtype, stream);
+    int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);
     if (rc != TKA_OK) return rc;
     SelectParams sw = sp;
     sw.from_scores = 1;
@@ -384,6 +411,7 @@ int tka_gemv_scores(const tka_gemv_topk_args* a) {
   if (rc != TKA_OK) return rc;
   GemvParams gp;
   fill_gemv_params(a, a->out_scores, nullptr, &gp);
+  if (a->key_stride_b == 0 && a->batch >= 2) return launch_gemv_scores_shared(gp, a->dtype, (hipStream_t)a->stream);
   return launch_gemv_scores(gp, a->dtype, (hipStream_t)a->stream);
 }
 
@@ -418,6 +446,7 @@ int tka_topk_f32(const tka_topk_args* a) {
   sp.num_segments = a->num_segments;
   sp.k = a->k;
   sp.segs_per_row = 1;
+  if (wave_select_fits(a->seg_len, a->k, a->num_segments)) return launch_select_wave(sp, stream);
   if (a->seg_len <= select_cand_capacity()) {   // the segment fits in LDS whole: one launch
     GemvParams none;
     memset(&none, 0, sizeof none);
@@ -700,7 +729,7 @@ static int ra_launch(const tka_ra_args* a) {
   const size_t gemv_ws = tka_gemv_topk_workspace_bytes(&g);
   g.workspace = ws;
   g.workspace_bytes = gemv_ws;
-  rc = run_gemv_topk(&g, nullptr, 0);
+  rc = run_gemv_topk(&g, nullptr, 0, nullptr, nullptr, true);   // (softmax and the weighted sum take any order)
   if (rc != TKA_OK) return rc;
   return run_flash(&f, ws + gemv_ws);
 }

@@ -99,6 +99,127 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
   }
 }
 
+// ---- one key stream for a batch of queries ------------------------------------------------------------
+
+// Value of lane (lane ^ 4) of the 16-lane row: row_half_mirror (lane ^ 7) then quad_perm [3,2,1,0] (lane ^ 3).
+__device__ __forceinline__ float row_xor4(float x) { return dpp_f32<0x1B>(dpp_f32<0x141>(x)); }
+
+// The 16-lane sums of BQ partial products per lane, in the canonical tree (xor 8, 4, 2, 1), as a reduce-scatter:
+// at each level a lane keeps the half of its values whose query index has the lane's bit set (or clear) and hands
+// the other half to its partner, so the adds are the ones of row16_sum (addition commutes) at about a third of
+// the instructions.  Lane j returns the sum of query j / (16 / BQ).
+template <int BQ>
+__device__ __forceinline__ float row16_reduce_scatter(const float (&acc)[BQ], int j) {
+  const bool b3 = (j & 8) != 0, b2 = (j & 4) != 0, b1 = (j & 2) != 0;
+  float r;
+  if constexpr (BQ == 8) {
+    float r1[4], r2[2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r1[i] = (b3 ? acc[i + 4] : acc[i]) + dpp_f32<0x128>(b3 ? acc[i] : acc[i + 4]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) r2[i] = (b2 ? r1[i + 2] : r1[i]) + row_xor4(b2 ? r1[i] : r1[i + 2]);
+    r = (b1 ? r2[1] : r2[0]) + dpp_f32<0x4E>(b1 ? r2[0] : r2[1]);
+  } else if constexpr (BQ == 4) {
+    float r1[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) r1[i] = (b3 ? acc[i + 2] : acc[i]) + dpp_f32<0x128>(b3 ? acc[i] : acc[i + 2]);
+    r = (b2 ? r1[1] : r1[0]) + row_xor4(b2 ? r1[0] : r1[1]);
+    r = r + dpp_f32<0x4E>(r);
+  } else {
+    static_assert(BQ == 2, "row16_reduce_scatter: 2, 4 or 8 queries");
+    r = (b3 ? acc[1] : acc[0]) + dpp_f32<0x128>(b3 ? acc[0] : acc[1]);
+    r = r + row_xor4(r);
+    r = r + dpp_f32<0x4E>(r);
+  }
+  return r + dpp_f32<0xB1>(r);
+}
+
+// Keys shared by every batch entry (key_stride_b == 0: the operator of the reference holds one KV cache for
+// the whole batch, retrieval_attention.cu:681-683): a workgroup scores its rows for BQ batch entries at once,
+// so the keys are read once per BQ entries instead of once per entry.  Each score is the canonical one
+// (fma chain over the lane's 8 dims, the 16-lane tree, one multiply) of its (entry, row).  16 row groups of
+// 16 lanes, 8 rows in flight per group; after the reduce-scatter lane j holds the scores of entry
+// j / (16 / BQ) for the 8 rows and stores BQ / 2 of them.
+// PACKED (fp16, one query head per KV head): the queries stay in their 16-bit form, four registers per entry,
+// and the widening is part of the multiply-add instruction.
+// Grid: 1-D over (head, row tile, batch tile), batch tile fastest, dealt so that the tiles that share rows run
+// on the same XCD (same L2) at about the same time.
+template <int DT, int BQ, bool PACKED>
+__global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(4, 8))) void gemv_scores_shared_kernel(
+    GemvParams p, int row_tiles, int batch_tiles) {
+  constexpr int LPQ = 16 / BQ;       // lanes that end up with the same entry
+  constexpr int RPL = 8 / LPQ;       // rows each of them stores
+  const int tid = threadIdx.x;
+  const int j = tid & 15, rg = tid >> 4;
+  uint32_t id = blockIdx.x;
+  if (gridDim.x % 8 == 0) id = (id % 8) * (gridDim.x / 8) + id / 8;
+  const int bt = (int)(id % (uint32_t)batch_tiles);
+  const int tile = (int)((id / (uint32_t)batch_tiles) % (uint32_t)row_tiles);
+  const int h = (int)(id / ((uint32_t)batch_tiles * (uint32_t)row_tiles));
+  const int b0 = bt * BQ;
+  const int64_t n = p.chunk_len * p.num_chunks;
+  const int64_t t_begin = (int64_t)tile * p.tokens_per_wg;
+  int64_t t_end = t_begin + p.tokens_per_wg;
+  if (t_end > n) t_end = n;
+
+  float qf[PACKED ? 1 : BQ][8];
+  u32x4 qp[PACKED ? BQ : 1];
+#pragma unroll
+  for (int q = 0; q < BQ; ++q) {
+    const int b = b0 + q < p.batch ? b0 + q : p.batch - 1;
+    if constexpr (PACKED)
+      qp[q] = *(const u32x4*)((const uint16_t*)p.q + (int64_t)b * p.q_stride_b + (int64_t)h * kHeadDim + 8 * j);
+    else
+      load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf[q]);
+  }
+  const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)h * p.key_stride_h + 8 * j;
+  const int my_b = b0 + j / LPQ;
+  const int my_row0 = (j % LPQ) * RPL;
+  float* my_out = p.scores + ((int64_t)(my_b < p.batch ? my_b : 0) * p.num_kv_heads + h) * n;
+
+  for (int64_t base = t_begin; base < t_end; base += kGemvRowsPerIter) {
+    u32x4 kv[kGemvUnroll];
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      const int64_t t = base + rg * kGemvUnroll + u;
+      const int64_t tc = t < t_end ? t : t_end - 1;
+      kv[u] = *(const u32x4*)(kbase + tc * p.key_stride_n);
+    }
+    float mine[RPL];
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) mine[i] = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      float acc[BQ];
+#pragma unroll
+      for (int q = 0; q < BQ; ++q) {
+        acc[q] = 0.0f;
+        if constexpr (PACKED) {
+          // (the empty asm keeps the compiler from widening all queries to fp32 ahead of the loop, which
+          // would take 8 registers per entry instead of 4)
+          asm volatile("" : "+v"(qp[q]));
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[q] = __builtin_fmaf(Elem<DT>::get(qp[q], i), Elem<DT>::get(kv[u], i), acc[q]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[q] = __builtin_fmaf(qf[q][i], Elem<DT>::get(kv[u], i), acc[q]);
+        }
+      }
+      const float s = row16_reduce_scatter<BQ>(acc, j) * p.scale;
+      if (u / RPL * RPL == my_row0) mine[u % RPL] = s;
+      // one row at a time: its BQ independent chains are parallelism enough, and interleaving the rows costs
+      // more registers than the file has for four waves
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const int64_t t0 = base + rg * kGemvUnroll + my_row0;
+    if (my_b < p.batch) {
+#pragma unroll
+      for (int i = 0; i < RPL; ++i)
+        if (t0 + i < t_end) my_out[t0 + i] = mine[i];
+    }
+  }
+}
+
 // ---- candidate mode -----------------------------------------------------------------------------
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {  // integer hash for the sample jitter
@@ -389,6 +510,37 @@ int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream) {
     gemv_scores_kernel<TKA_F16><<<grid, kGemvThreads, 0, stream>>>(p);
   else
     gemv_scores_kernel<TKA_BF16><<<grid, kGemvThreads, 0, stream>>>(p);
+  return hip_status(hipGetLastError());
+}
+
+// Shared keys (key_stride_b == 0), plain scores [batch][head][seq_len] (no histogram, no cluster bases).
+int launch_gemv_scores_shared(const GemvParams& p0, int dtype, hipStream_t stream) {
+  if (p0.key_stride_b != 0 || p0.cluster_ids || !p0.scores) return TKA_EINVAL;
+  GemvParams p = p0;
+  const int64_t n = p.chunk_len * p.num_chunks;
+  p.tokens_per_wg = 256;
+  // fp16 queries of single heads stay packed: 8 entries per pass fit the registers; otherwise 4 (fp32 queries)
+  const bool packed = dtype == TKA_F16 && p.group == 1;
+  const int bq = packed && p.batch >= 5 ? 8 : p.batch >= 3 ? 4 : 2;
+  const int64_t row_tiles = (n + p.tokens_per_wg - 1) / p.tokens_per_wg;
+  const int64_t batch_tiles = (p.batch + bq - 1) / bq;
+  const int64_t wgs = row_tiles * batch_tiles * p.num_kv_heads;
+  if (wgs > 0x7fffffffLL) return TKA_EUNSUPPORTED;
+  LaunchTimer timer("gemv_scores_shared", stream);
+#define TKA_LAUNCH_SHARED(DT, BQ, PACKED) \
+  gemv_scores_shared_kernel<DT, BQ, PACKED><<<(unsigned)wgs, kGemvThreads, 0, stream>>>(p, (int)row_tiles, (int)batch_tiles)
+  if (packed) {
+    if (bq == 8) TKA_LAUNCH_SHARED(TKA_F16, 8, true);
+    else if (bq == 4) TKA_LAUNCH_SHARED(TKA_F16, 4, true);
+    else TKA_LAUNCH_SHARED(TKA_F16, 2, true);
+  } else if (dtype == TKA_F16) {
+    if (bq == 4) TKA_LAUNCH_SHARED(TKA_F16, 4, false);
+    else TKA_LAUNCH_SHARED(TKA_F16, 2, false);
+  } else {
+    if (bq == 4) TKA_LAUNCH_SHARED(TKA_BF16, 4, false);
+    else TKA_LAUNCH_SHARED(TKA_BF16, 2, false);
+  }
+#undef TKA_LAUNCH_SHARED
   return hip_status(hipGetLastError());
 }
 
