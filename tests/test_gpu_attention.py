@@ -34,7 +34,7 @@ def _dense_ref(q, K, V, dtype, G, scale):
 
 @pytest.mark.parametrize("dtype,B,H,G,N,splits", [
     (oracle.F16, 1, 8, 4, 4096, 0), (oracle.F16, 2, 2, 1, 1000, 3), (oracle.BF16, 1, 2, 8, 3333, 7),
-    (oracle.F16, 1, 1, 2, 77, 1), (oracle.BF16, 2, 4, 4, 2048, 64)])
+    (oracle.F16, 1, 1, 2, 77, 1), (oracle.BF16, 2, 4, 4, 2048, 64), (oracle.BF16, 3, 2, 1, 700, 1)])
 def test_flash_decode_dense(dtype, B, H, G, N, splits):
     from topk_attn_amd import ops
     announce("flash_decode dense dtype=%d B=%d H=%d G=%d N=%d splits=%d" % (dtype, B, H, G, N, splits))
@@ -163,6 +163,26 @@ def test_retrieval_attention_op(topk):
         for h in range(0, H, 5):
             ref, _, _ = oracle.retrieval_attention(q[b, h], K[:, h], V[:, h], dtype, 4, topk, 1.0)
             assert np.abs(got[b, h] - ref).max() < TOL
+
+
+@pytest.mark.parametrize("B,topk", [(9, 128), (33, 1024), (2, 32)])
+def test_retrieval_attention_op_batches(B, topk):
+    """Batches whose keys are scored several entries per pass (with a ragged last tile), selected one segment per
+    wavefront, and, from 32 entries on, attended by one workgroup per row without a combine launch."""
+    from topk_attn_amd import retrieval_attention_cpp as ra
+    announce("retrieval_attention op B=%d topk=%d" % (B, topk))
+    rng = np.random.default_rng(B)
+    dtype = oracle.F16
+    H, N = 32, 8192
+    q, K, V = randn_bits(rng, (B, H, 128), dtype, 0.1), randn_bits(rng, (N, H, 128), dtype, 0.1), randn_bits(rng, (N, H, 128), dtype, 0.1)
+    out = torch.zeros((B, H, 128), dtype=torch.float16, device="cuda")
+    getattr(ra, "retrieval_attention_%d" % topk)(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), out)
+    torch.cuda.synchronize()
+    got = f32_of(out)
+    for b in sorted({0, 1, B // 2, B - 2, B - 1}):
+        for h in range(b % 7, H, 7):
+            ref, _, _ = oracle.retrieval_attention(q[b, h], K[:, h], V[:, h], dtype, 4, topk, 1.0)
+            assert np.abs(got[b, h] - ref).max() < TOL, "b=%d h=%d" % (b, h)
 
 
 def test_retrieval_attention_variants_agree():

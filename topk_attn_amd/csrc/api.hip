@@ -353,8 +353,15 @@ int run_flash(const tka_flash_decode_args* a, void* workspace) {
   ap.tokens_per_split = tps;
   ap.scale_log2e = a->scale * 1.44269504088896340736f;
   // grouped queries go to the matrix cores; one query head per KV head (and supplied logits) stay on VALU
-  int rc = (a->group >= 2 && !a->kv_logit) ? launch_attn_partial_mfma(ap, a->dtype, stream)
-                                           : launch_attn_partial(ap, a->dtype, stream);
+  const bool mfma = a->group >= 2 && !a->kv_logit;
+  if (!mfma && splits == 1) {   // nothing to combine: the kernel writes the result itself
+    ap.out = a->out;
+    ap.out_lse = a->out_lse;
+    ap.out_stride_b = a->out_stride_b;
+    ap.out_dtype = a->out_dtype;
+    return launch_attn_partial(ap, a->dtype, stream);
+  }
+  int rc = mfma ? launch_attn_partial_mfma(ap, a->dtype, stream) : launch_attn_partial(ap, a->dtype, stream);
   if (rc != TKA_OK) return rc;
   CombineParams cp;
   memset(&cp, 0, sizeof cp);

@@ -181,9 +181,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
           o += sh_acc[r][tid] * w;
         }
       }
-      const int64_t slot = (row0 + g) * p.num_splits + split;
-      p.part_acc[slot * kHeadDim + tid] = o;
-      if (tid == 0) { p.part_m[slot] = M; p.part_l[slot] = L; }
+      if (p.out) {
+        // the only split of its row: what the combine would compute from this one partial (weight 2^0)
+        const float r = L > 0.0f ? o / L : 0.0f;
+        uint16_t* out = (uint16_t*)p.out + (int64_t)b * p.out_stride_b + ((int64_t)h * G + g) * kHeadDim;
+        out[tid] = p.out_dtype == TKA_F16 ? Elem<TKA_F16>::narrow(r) : Elem<TKA_BF16>::narrow(r);
+        if (p.out_lse && tid == 0)
+          p.out_lse[row0 + g] = L > 0.0f ? (M + __builtin_log2f(L)) * 0.69314718055994531f : -INFINITY;
+      } else {
+        const int64_t slot = (row0 + g) * p.num_splits + split;
+        p.part_acc[slot * kHeadDim + tid] = o;
+        if (tid == 0) { p.part_m[slot] = M; p.part_l[slot] = L; }
+      }
     }
   }
 }

@@ -111,6 +111,11 @@ struct AttnParams {
   int idx_len;
   int tokens_per_split;     // positions per workgroup
   float scale_log2e;        // scale * log2(e)
+  // One split per row: the VALU kernel normalises and writes the result itself (no combine launch) when out is set.
+  void* out;                // [batch][query heads][128] or nullptr
+  float* out_lse;           // [rows] or nullptr
+  int64_t out_stride_b;
+  int out_dtype;
 };
 int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream);       // VALU path (any group, logits)
 int launch_attn_partial_mfma(const AttnParams& p, int dtype, hipStream_t stream);  // matrix-core path, group >= 2
