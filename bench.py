@@ -9,7 +9,8 @@ The default workload is the one the headline metric is quoted on:
       local tokens -> gathered attention -> LSE combine; bf16 output.
 
 The other workloads time one stage each at the sizes of the remaining configurations (c1 single-head
-GEMV + top-k, c2 centre-only top-k, c3 dense flash-decoding, c5 one-million-token tie stress).
+GEMV + top-k, c2 centre-only top-k, c3 dense flash-decoding, c5 one-million-token tie stress); `ra` times
+the reference's operator at its own test shape (--batch, --topk).
 
 Prints ONE JSON line.  `value` is algorithmic bytes per step / step time (GB/s); `roofline` is the dominant
 kernel timed with HIP events on its launch stream; `cpu_baseline` is the torch-CPU restatement of the same
@@ -200,6 +201,32 @@ class FlashDecode:
         return kv + 2 * 32 * 128 * 2, kv, {}
 
 
+class RetrievalOp:
+    """ra: the reference's operator at its own test shape (test_ra.py:162-172: 32 heads, 8192 keys shared by the
+    batch, 4 chunks of 2048, top-K per chunk), batch entries and K selectable."""
+
+    def __init__(self, torch, dev, batch=4, topk=128):
+        from topk_attn_amd import retrieval_attention_cpp as ra
+        g = torch.Generator(device=dev)
+        g.manual_seed(6)
+        self.B, self.topk = batch, topk
+        self.q = (torch.randn((batch, 32, 128), generator=g, device=dev) * 0.1).half()
+        self.K = (torch.randn((8192, 32, 128), generator=g, device=dev) * 0.1).half()
+        self.V = (torch.randn((8192, 32, 128), generator=g, device=dev) * 0.1).half()
+        self.out = torch.zeros((batch, 32, 128), dtype=torch.float16, device=dev)
+        self.fn = getattr(ra, "retrieval_attention_%d" % topk)
+        self.desc = "ra: retrieval_attention_%d, B=%d, 32 heads, 8192 keys fp16 shared by the batch" % (topk, batch)
+        self.dominant = "gemv_scores_shared" if batch >= 2 else "gemv_topk_fused"
+
+    def step(self):
+        self.fn(self.q, self.K, self.V, self.out)
+
+    def bytes(self):
+        keys = 8192 * 32 * 128 * 2                               # read once for the whole batch
+        rows = self.B * 32 * 4 * self.topk * 128 * 2             # gathered V rows
+        return keys + rows + 2 * self.B * 32 * 128 * 2, keys, {}
+
+
 class PlainCopy:
     """Calibration workload for the HBM traffic counters: a device-to-device copy of known size."""
 
@@ -232,6 +259,8 @@ def build_workload(name, torch, ops, dev, args):
         return CenterTopk(torch, ops, dev, centroids=1024, expand=128, rotate=args.rotate)
     if name == "c3":
         return FlashDecode(torch, ops, dev, args.splits)
+    if name == "ra":
+        return RetrievalOp(torch, dev, batch=args.batch, topk=args.topk)
     if name == "c5":
         return GemvTopk(torch, ops, dev, 1, 8, 8, 1048576, 4096, "bfloat16", 5, "c5", levels=True)
     raise ValueError(name)
@@ -250,7 +279,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c5", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c5", "ra", "copy"])
+    ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
+    ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--splits", type=int, default=0, help="c3, c4: split count of the attention (0 = library default)")
     ap.add_argument("--rotate", type=int, default=0,
                     help="c1, c2, c2-ref: number of key sets taken in turn (working set beyond the Infinity Cache)")
