@@ -185,6 +185,20 @@ def test_retrieval_attention_op_batches(B, topk):
             assert np.abs(got[b, h] - ref).max() < TOL, "b=%d h=%d" % (b, h)
 
 
+def test_harness_ra(capfd):
+    """The harness in the shape of the reference's test_ra.py: PASSED lines per variant, a performance table built
+    from the timing line the op prints on request, exit status 0.  (Parity proper is checked against the oracle in
+    the tests above; the harness's own torch model is held to 5e-3 here, test_ra.py:202 uses 1e-2.)"""
+    from topk_attn_amd import harness_ra
+    announce("harness_ra --batch 2 --topk 32 256")
+    rc = harness_ra.main(["--batch", "2", "--topk", "32", "256", "--tol", "5e-3"])
+    text = capfd.readouterr().out
+    assert rc == 0, text[-2000:]
+    assert text.count("PASSED") == 12 and "FAILED" not in text
+    rows = [ln for ln in text.splitlines() if ln.startswith("| 32 ") or ln.startswith("| 256 ")]
+    assert len(rows) == 12 and all(float(r.split("|")[3]) > 0 for r in rows)
+
+
 def test_retrieval_attention_variants_agree():
     """All six reference variants are one function here: identical bits."""
     from topk_attn_amd import retrieval_attention_cpp as ra
