@@ -298,8 +298,13 @@ void flash_plan(const tka_flash_decode_args* a, int* splits, int* tokens_per_spl
   int64_t want = a->num_splits;
   if (want <= 0) {
     // measured: the dense scan likes about 2048 workgroups, the gathered form about one resident set (3 per CU)
-    want = (a->kv_idx ? 1024 : 2048) / ((int64_t)a->batch * a->num_kv_heads);
+    const int64_t rows = (int64_t)a->batch * a->num_kv_heads;
+    want = (a->kv_idx ? 1024 : 2048) / rows;
     if (want < 1) want = 1;
+    // short lists on the VALU kernel: one workgroup per row writes the result itself, which saves the combine
+    // launch (measured on the operator: quicker up to 512 ids per row, and up to 1024 from 256 rows on)
+    const bool valu = a->group == 1 || a->kv_logit;
+    if (valu && a->kv_idx && (len <= 512 || (len <= 1024 && rows >= 256))) want = 1;
   }
   int64_t tps = (len + want - 1) / want;
   tps = (tps + 127) / 128 * 128;
