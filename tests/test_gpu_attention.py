@@ -168,7 +168,7 @@ def test_retrieval_attention_op(topk):
 @pytest.mark.parametrize("B,topk", [(9, 128), (33, 1024), (2, 32)])
 def test_retrieval_attention_op_batches(B, topk):
     """Batches whose keys are scored several entries per pass (with a ragged last tile), selected one segment per
-    wavefront, and, from 32 entries on, attended by one workgroup per row without a combine launch."""
+    small workgroup, and, from 32 entries on, attended by one workgroup per row without a combine launch."""
     from topk_attn_amd import retrieval_attention_cpp as ra
     announce("retrieval_attention op B=%d topk=%d" % (B, topk))
     rng = np.random.default_rng(B)

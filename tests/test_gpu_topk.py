@@ -109,7 +109,7 @@ def test_short_segments(n, k):
     announce("topk short segments n=%d k=%d" % (n, k))
     rng = np.random.default_rng(n * 7 + k)
     rows = _short_segment_rows(rng, n)
-    rows += [rng.standard_normal(n).astype(np.float32) for _ in range(256)]   # enough segments for the wavefront route
+    rows += [rng.standard_normal(n).astype(np.float32) for _ in range(256)]   # enough segments for the small-workgroup route
     _check(np.stack(rows), k)
 
 

@@ -137,8 +137,8 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
 }
 
-// Short segments in numbers: one wavefront per segment selects (no workgroup barriers; a compute unit works on
-// many segments at a time).
+// Short segments in numbers: a four-wave workgroup per segment selects (a compute unit works on many segments
+// at a time).
 int wave_select_min_segments() {
   static const int v = [] {
     const char* e = getenv("TKA_WAVE_MIN_SEGS");
@@ -198,7 +198,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // Keys shared by the batch are read once for several batch entries.
   const bool shared_keys = a->key_stride_b == 0 && a->batch >= 2 && !cluster_ids;
 
-  // Many short segments: plain scores, then one wavefront per segment selects.
+  // Many short segments: plain scores, then a four-wave workgroup per segment selects.
   if (a->out_idx && !u && wave_select_fits(chunk_len, a->k, segs)) {
     gp.hist = nullptr;
     int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);

@@ -65,7 +65,7 @@ struct SelectParams {
   int segs_per_row;       // chunks per (batch, head): index base = (s % segs_per_row) * seg_len
   int expand;             // cluster_len of the expansion, 0 = none
   int sink, local;        // union mode
-  int unordered;          // wave-per-segment kernel: out_idx / out_val need not be in rank order
+  int unordered;          // select_wave kernel: out_idx / out_val need not be in rank order
 };
 size_t select_workspace_bytes(int num_segments, int64_t seg_len);
 // Carves the workspace; returns how many leading 32-bit words (the histograms) need clearing.
@@ -80,7 +80,7 @@ int launch_select_finalize(const SelectParams& p, hipStream_t stream);
 int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
 int select_cand_max_parts();   // most candidate slices per segment
 int select_cand_capacity();    // most candidates per segment
-// One wavefront per segment: rank-ordered top-k of fp32 scores, segments of up to select_wave_max_len() scores.
+// A four-wave workgroup per segment: rank-ordered top-k of fp32 scores, segments of up to select_wave_max_len() scores.
 int launch_select_wave(const SelectParams& p, hipStream_t stream);
 int select_wave_max_len();
 int select_wave_max_k();

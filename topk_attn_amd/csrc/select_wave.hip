@@ -1,27 +1,33 @@
-// Exact top-k of many short segments: one wavefront per segment, no workgroup barriers.
+// Exact top-k of many short segments: a small workgroup (W = 4 wavefronts) per segment.
 //
 // The operator of the reference selects inside 2048-key chunks, one chunk per (batch entry, head, quarter of
-// the sequence) (retrieval_attention.cu:335-354 sorts each chunk whole), so a call has thousands of short
-// segments.  A 1024-thread workgroup per segment spends its time in barriers; here a segment belongs to one
-// wave, whose 64 lanes hold its 2048 keys in registers (32 each), and a compute unit works on twenty
-// segments at a time.
+// the sequence) (retrieval_attention.cu:335-354 sorts each chunk whole), so a call has hundreds to thousands of
+// short segments.  A 1024-thread workgroup per segment spends its time in barriers and leaves most of the GPU
+// idle.  Here the 2048 keys of a segment sit in the registers of W waves (8 per lane for W = 4), eight segments are
+// in flight per compute unit, and the whole selection is a few hundred instructions per wave with eight barriers.
+// The code is written for any W that divides 8; W = 1 (32 keys per lane, no s_barrier at all) measured the same
+// or slower from 256 to 16384 segments, and what a launch of this kernel costs at a few hundred segments is
+// mostly the first fetch of its instructions, so the short form wins.
 //
 //   1. fp32 scores -> order-preserving keys, relative to the smallest key of the segment and shifted so that the
 //      largest one fills 32 bits;
-//   2. radix select, 11 bits per pass, on (key, 2047 - index): LDS histogram of the wave, suffix scan by DPP,
-//      the bin of the k-th largest; passes end as soon as a bucket is taken whole.  Equal keys are told apart
-//      by the last pass, whose digit is the index: lower index first;
-//   3. the k selected composites are compacted into LDS (the histogram's space) and sorted by the wave with a
-//      bitonic network; rank-ordered ids and scores are written.
+//   2. one 11-bit histogram pass in LDS, suffix scans by DPP, the bin of the k-th largest.  If that bin is taken
+//      whole, or holds at most 64 entries (they are ranked directly, one per lane), the selection is known -
+//      ordinary data.  Otherwise up to three more passes: 11 and 10 more bits of the key, then 2047 - token among
+//      the entries that equal the threshold key: lower index first;
+//   3. the k selected composites are compacted into LDS (the histogram's space) and sorted with the bitonic
+//      network of bitonic.hpp (registers, DPP, and LDS for the strides that cross waves); rank-ordered ids and
+//      scores are written.  A caller that takes any order skips the sort.
 #include "bitonic.hpp"
 #include "kernels.hpp"
 
 namespace tka {
 
 namespace {
+
 constexpr int kWsMaxLen = 2048;             // keys per segment at most
-constexpr int kWsEpl = kWsMaxLen / kWave;   // keys per lane
 constexpr int kWsBins = 2048;
+constexpr int kWsMaxWaves = 4;
 
 __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
   v = min(v, lane_xor<1>(v));
@@ -42,51 +48,85 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
   return v;
 }
 
-// Token of register e of a lane: 256-token groups, four consecutive tokens per lane in each (16-byte loads).
-__device__ __forceinline__ int ws_token(int e, int lane) { return (e >> 2) * 256 + 4 * lane + (e & 3); }
+// Order-preserving key of a score, as score_key() (NaN lowest, -0 == +0).
+__device__ __forceinline__ uint32_t ws_key(float x) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x + 0.0f);
+  const uint32_t key = u ^ ((uint32_t)((int32_t)u >> 31) | 0x80000000u);
+  return x != x ? 0u : key;
+}
 
-// The bin d of the wave's histogram with  count(bins > d) < need <= count(bins >= d);  `above` = count(bins > d),
-// `cnt` = its own count.  The histogram must hold at least `need` entries.  Two levels: lane l sums bins
-// 32l .. 32l+31 and a suffix scan over the lanes finds the lane that owns d; then the first 32 lanes take one
-// bin of that lane each and scan again.
-__device__ __forceinline__ void ws_find_bin(const uint32_t* sh, uint32_t need, int lane, uint32_t& d, uint32_t& above, uint32_t& cnt) {
+// What the W waves of a segment share.  (A one-wave workgroup's __syncthreads() is no s_barrier, only a wait
+// on the LDS counter.)
+template <int W>
+struct WsShared {
+  __align__(16) uint32_t bins[kWsBins];   // the histogram, then the sort buffer (1024 composites)
+  uint64_t cand[kWave];                   // entries of the threshold bucket when there are few
+  uint64_t trash[W * kWave];              // where a thread stores what is not selected
+  uint32_t wave_a[kWsMaxWaves], wave_b[kWsMaxWaves];   // per-wave partial results
+  uint32_t owner[4];                      // find_bin: owning thread, entries above its bins, entries in its bins
+};
+
+// Register e of thread t holds token (e / 4) * (256 W) + 4 t + e % 4: 16-byte loads, consecutive across threads.
+template <int W>
+__device__ __forceinline__ int ws_token(int e, int tid) { return (e >> 2) * (256 * W) + 4 * tid + (e & 3); }
+
+template <int W>
+__device__ __forceinline__ void ws_clear(uint32_t* bins, int tid) {
+#pragma unroll
+  for (int i = 0; i < 8 / W; ++i) *(u32x4*)(bins + (256 * W) * i + 4 * tid) = u32x4{0u, 0u, 0u, 0u};
+}
+
+// The bin d of the histogram with  count(bins > d) < need <= count(bins >= d);  `above` = count(bins > d),
+// `cnt` = its own count.  The histogram must hold at least `need` entries.  Two levels: a thread sums its
+// 32 / W consecutive bins, suffix sums over the threads find the thread that owns d; then the first lanes of every
+// wave take one of that thread's bins each and scan again.  All threads return the same values.
+template <int W>
+__device__ __forceinline__ void ws_find_bin(WsShared<W>& sh, uint32_t need, int tid, uint32_t& d, uint32_t& above, uint32_t& cnt) {
+  constexpr int BPT = 32 / W;   // bins per thread
+  const int lane = tid & 63, wave = tid >> 6;
   uint32_t tot = 0;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const u32x4 v = *(const u32x4*)(sh + 32 * lane + 4 * i);
+  for (int i = 0; i < BPT / 4; ++i) {
+    const u32x4 v = *(const u32x4*)(sh.bins + BPT * tid + 4 * i);
     tot += (v[0] + v[1]) + (v[2] + v[3]);
   }
   const uint32_t inc = wave_inclusive_scan(tot);
-  const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)inc, 63);
-  const uint32_t higher = total - inc;            // entries in the bins of higher lanes
-  const int owner = __builtin_ctzll(__ballot(higher < need && need <= higher + tot));
-  const uint32_t owner_higher = (uint32_t)__builtin_amdgcn_readlane((int)higher, owner);
-  const uint32_t owner_tot = (uint32_t)__builtin_amdgcn_readlane((int)tot, owner);
-  const uint32_t v = lane < 32 ? sh[32 * owner + lane] : 0u;
+  const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)inc, 63);
+  uint32_t higher = wave_total - inc;            // entries in the bins of higher lanes of this wave
+  if constexpr (W > 1) {
+    if (lane == 0) sh.wave_a[wave] = wave_total;
+    __syncthreads();
+#pragma unroll
+    for (int w = 1; w < W; ++w) higher += w > wave ? sh.wave_a[w] : 0u;
+  }
+  if (higher < need && need <= higher + tot) {   // exactly one thread
+    sh.owner[0] = (uint32_t)tid;
+    sh.owner[1] = higher;
+    sh.owner[2] = tot;
+  }
+  __syncthreads();
+  const uint32_t owner = sh.owner[0], owner_higher = sh.owner[1], owner_tot = sh.owner[2];
+  const uint32_t v = lane < BPT ? sh.bins[BPT * owner + lane] : 0u;
   const uint32_t vinc = wave_inclusive_scan(v);
-  const uint32_t vhigher = owner_higher + (owner_tot - vinc);   // entries in bins above bin 32*owner + lane
-  const int bin = __builtin_ctzll(__ballot(lane < 32 && vhigher < need && need <= vhigher + v));
-  d = 32u * (uint32_t)owner + (uint32_t)bin;
+  const uint32_t vhigher = owner_higher + (owner_tot - vinc);   // entries in bins above bin BPT*owner + lane
+  const int bin = __builtin_ctzll(__ballot(lane < BPT && vhigher < need && need <= vhigher + v));
+  d = (uint32_t)BPT * owner + (uint32_t)bin;
   above = (uint32_t)__builtin_amdgcn_readlane((int)vhigher, bin);
   cnt = (uint32_t)__builtin_amdgcn_readlane((int)v, bin);
-}
-
-__device__ __forceinline__ void ws_clear(uint32_t* sh, int lane) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) *(u32x4*)(sh + 256 * i + 4 * lane) = u32x4{0u, 0u, 0u, 0u};
 }
 
 // One radix pass below the first.  PASS 1, 2: the second and third digit of the relative key (11 and 10 bits)
 // among the entries that share the digits found so far; PASS 3: the digit is 2047 - token among the entries
 // whose key equals the threshold key.  `thr` is the threshold so far (digits of later passes zero), `need` how
 // many entries of the current bucket are still to be taken.  Returns true when the bucket found is taken whole.
-template <int PASS>
-__device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[kWsEpl], int lane, uint32_t* sh, uint32_t& thr, uint32_t& need,
+template <int PASS, int W>
+__device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[32 / W], int tid, WsShared<W>& sh, uint32_t& thr, uint32_t& need,
                                         uint32_t& tok_limit) {
-  ws_clear(sh, lane);
+  __syncthreads();              // the previous histogram has been read
+  ws_clear<W>(sh.bins, tid);
   __syncthreads();
 #pragma unroll
-  for (int e = 0; e < kWsEpl; ++e) {
+  for (int e = 0; e < 32 / W; ++e) {
     bool active;
     uint32_t digit;
     if constexpr (PASS == 1) {
@@ -97,14 +137,13 @@ __device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[kWsEpl], int lane,
       digit = rel[e] & 1023u;
     } else {
       active = rel[e] == thr;
-      digit = 2047u - (uint32_t)ws_token(e, lane);
+      digit = 2047u - (uint32_t)ws_token<W>(e, tid);
     }
-    if (active) atomicAdd(&sh[digit], 1u);
+    if (active) atomicAdd(&sh.bins[digit], 1u);
   }
   __syncthreads();
   uint32_t d, above, cnt;
-  ws_find_bin(sh, need, lane, d, above, cnt);
-  __syncthreads();
+  ws_find_bin<W>(sh, need, tid, d, above, cnt);
   need -= above;
   if constexpr (PASS == 1) thr |= d << 10;
   if constexpr (PASS == 2) thr |= d;
@@ -112,31 +151,28 @@ __device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[kWsEpl], int lane,
   return cnt == need;
 }
 
-// Order-preserving key of a score, as score_key() (NaN lowest, -0 == +0).
-__device__ __forceinline__ uint32_t ws_key(float x) {
-  const uint32_t u = __builtin_bit_cast(uint32_t, x + 0.0f);
-  const uint32_t key = u ^ ((uint32_t)((int32_t)u >> 31) | 0x80000000u);
-  return x != x ? 0u : key;
-}
-
-// Compaction of the entries that satisfy PRED into `dst` (order-preserving composites (rel << 32) | ~token, lane
-// after lane).  Straight-line: a count per lane, one scan, and every lane stores all its entries, the ones
-// that do not qualify into its own slot of `trash`.
-template <typename PRED>
-__device__ __forceinline__ void ws_compact(const uint32_t (&rel)[kWsEpl], int lane, uint64_t* dst, uint64_t* trash, PRED pred) {
-  const uint32_t not_t0 = ~(uint32_t)(4 * lane);
+// How many of the thread's entries satisfy PRED.
+template <int W, typename PRED>
+__device__ __forceinline__ uint32_t ws_count(const uint32_t (&rel)[32 / W], int tid, PRED pred) {
+  const uint32_t not_t0 = ~(uint32_t)(4 * tid);
   uint32_t count[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int e = 0; e < kWsEpl; ++e) {
-    const uint32_t not_t = not_t0 - (uint32_t)((e >> 2) * 256 + (e & 3));   // ~token
+  for (int e = 0; e < 32 / W; ++e) {
+    const uint32_t not_t = not_t0 - (uint32_t)((e >> 2) * (256 * W) + (e & 3));   // ~token
     count[e & 3] += pred(rel[e], not_t) ? 1u : 0u;
   }
-  const uint32_t mine = (count[0] + count[1]) + (count[2] + count[3]);
-  uint32_t pos = wave_inclusive_scan(mine) - mine;
-  uint64_t* own = trash + lane;
+  return (count[0] + count[1]) + (count[2] + count[3]);
+}
+
+// Stores the thread's entries that satisfy PRED to dst[pos ...] as order-preserving composites (rel << 32) | ~token.
+// Straight-line: the thread stores all its entries, the ones that do not qualify into its own trash slot.
+template <int W, typename PRED>
+__device__ __forceinline__ void ws_scatter(const uint32_t (&rel)[32 / W], int tid, uint64_t* dst, uint32_t pos, uint64_t* trash, PRED pred) {
+  const uint32_t not_t0 = ~(uint32_t)(4 * tid);
+  uint64_t* own = trash + tid;
 #pragma unroll
-  for (int e = 0; e < kWsEpl; ++e) {
-    const uint32_t not_t = not_t0 - (uint32_t)((e >> 2) * 256 + (e & 3));
+  for (int e = 0; e < 32 / W; ++e) {
+    const uint32_t not_t = not_t0 - (uint32_t)((e >> 2) * (256 * W) + (e & 3));
     const bool take = pred(rel[e], not_t);
     uint64_t* at = take ? dst + pos : own;
     *at = ((uint64_t)rel[e] << 32) | not_t;
@@ -144,25 +180,49 @@ __device__ __forceinline__ void ws_compact(const uint32_t (&rel)[kWsEpl], int la
   }
 }
 
-// The selected composites (sh_sort[0 .. 64*E), zero past the k-th) into rank order.  Lane l takes elements
-// l*E .. l*E+E-1; the bitonic network runs in registers (strides below E) and through DPP / ds_swizzle /
-// ds_bpermute.
-template <int E>
-__device__ __forceinline__ void ws_sort(uint64_t* sh_sort, int lane) {
-  uint64_t v[E];
+// Exclusive prefix of `mine` over the threads of the workgroup (slot: one of the per-wave arrays).
+// W > 1: contains one barrier, every thread must call it.
+template <int W>
+__device__ __forceinline__ uint32_t ws_exclusive(uint32_t mine, int tid, uint32_t* slot) {
+  const int lane = tid & 63, wave = tid >> 6;
+  const uint32_t inc = wave_inclusive_scan(mine);
+  uint32_t pos = inc - mine;
+  if constexpr (W > 1) {
+    if (lane == 63) slot[wave] = inc;
+    __syncthreads();
 #pragma unroll
-  for (int s = 0; s < E; ++s) v[s] = sh_sort[lane * E + s];
-  bitonic_net<64 * E, E, 2, 1>(v, nullptr, lane, true);
-  __syncthreads();
-#pragma unroll
-  for (int s = 0; s < E; ++s) sh_sort[lane * E + s] = v[s];
+    for (int w = 0; w < W - 1; ++w) pos += w < wave ? slot[w] : 0u;
+  }
+  return pos;
 }
 
-__global__ __launch_bounds__(kWave) void select_wave_kernel(SelectParams p, int kpad) {
-  __shared__ __align__(16) uint32_t sh[kWsBins];   // the histogram, then the sort buffer (1024 composites)
-  __shared__ uint64_t sh_cand[kWave];              // entries of the threshold bucket when there are few
-  __shared__ uint64_t sh_trash[kWave];             // where a lane stores what is not selected
-  const int lane = threadIdx.x;
+// The composites sh_sort[0 .. N) (zero past the k-th) into descending order, by the first N / E threads.
+template <int N, int W>
+__device__ __forceinline__ void ws_sort(uint64_t* sh_sort, int tid) {
+  constexpr int T = W * kWave;
+  constexpr int E = N > T ? N / T : 1;
+  constexpr int NT = N / E;
+  uint64_t v[E];
+  const bool active = tid < NT;
+  if (active) {
+#pragma unroll
+    for (int s = 0; s < E; ++s) v[s] = sh_sort[tid * E + s];
+  }
+  bitonic_net<N, E, 2, 1>(v, sh_sort, tid, active);   // (the exchange stages write the buffer only behind a barrier)
+  __syncthreads();
+  if (active) {
+#pragma unroll
+    for (int s = 0; s < E; ++s) sh_sort[tid * E + s] = v[s];
+  }
+}
+
+template <int W>
+__global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, int kpad) {
+  constexpr int T = W * kWave;
+  constexpr int EPT = 32 / W;              // keys per thread
+  __shared__ WsShared<W> sh;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
   const int seg = blockIdx.x;
   const int n = (int)p.seg_len;
   const uint32_t k = (uint32_t)p.k;
@@ -171,14 +231,14 @@ __global__ __launch_bounds__(kWave) void select_wave_kernel(SelectParams p, int 
   // Keys of the segment.  Entries past its end get the smallest relative key (0) and, by their position, lose
   // every tie against a real entry: they sit at the bottom of the order and k <= n keeps them out.
   constexpr uint32_t kPad = ~0u;   // marks them until then (no key is ~0: the largest is that of +inf)
-  uint32_t rel[kWsEpl];
+  uint32_t rel[EPT];
   uint32_t kmin = ~0u, kmax = 0u;
   const bool vec = ((uintptr_t)sc & 15u) == 0;
-  ws_clear(sh, lane);
+  ws_clear<W>(sh.bins, tid);
 #pragma unroll
-  for (int c = 0; c < kWsEpl / 4; ++c) {
-    const int t0 = c * 256 + 4 * lane;
-    if (vec && c * 256 + 256 <= n) {             // a full group: no checks per entry
+  for (int c = 0; c < EPT / 4; ++c) {
+    const int t0 = c * (4 * T) + 4 * tid;
+    if (vec && (c + 1) * (4 * T) <= n) {             // a full group: no checks per entry
       const f32x4 w = *(const f32x4*)(sc + t0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -200,16 +260,25 @@ __global__ __launch_bounds__(kWave) void select_wave_kernel(SelectParams p, int 
   }
   kmin = wave_min_u32(kmin);
   kmax = wave_max_u32(kmax);
+  if constexpr (W > 1) {
+    if (lane == 0) { sh.wave_a[wave] = kmin; sh.wave_b[wave] = kmax; }
+  }
+  __syncthreads();
+  if constexpr (W > 1) {
+#pragma unroll
+    for (int w = 0; w < W; ++w) { kmin = min(kmin, sh.wave_a[w]); kmax = max(kmax, sh.wave_b[w]); }
+  }
   const uint32_t range = kmax - kmin;
   const int bits = range ? 32 - __builtin_clz(range) : 0;
   const int lshift = bits ? 32 - bits : 0;
-  __syncthreads();
   const bool padded = n < kWsMaxLen;
+  if (padded && tid == 0) atomicAdd(&sh.bins[0], (uint32_t)(kWsMaxLen - n));   // the entries past the end, at once
 #pragma unroll
-  for (int e = 0; e < kWsEpl; ++e) {
+  for (int e = 0; e < EPT; ++e) {
     const uint32_t r = (rel[e] - kmin) << lshift;
-    rel[e] = padded && rel[e] == kPad ? 0u : r;
-    atomicAdd(&sh[rel[e] >> 21], 1u);   // first pass: the leading 11 bits
+    const bool pad = padded && rel[e] == kPad;
+    rel[e] = pad ? 0u : r;
+    if (!pad) atomicAdd(&sh.bins[r >> 21], 1u);   // first pass: the leading 11 bits
   }
   __syncthreads();
 
@@ -218,58 +287,72 @@ __global__ __launch_bounds__(kWave) void select_wave_kernel(SelectParams p, int 
   // further passes fix the threshold (thr, tok_limit): selected are the entries with
   // (rel, 2047 - token) >= (thr, 2047 - tok_limit).
   uint32_t d, above, cnt;
-  ws_find_bin(sh, k, lane, d, above, cnt);
-  __syncthreads();
+  ws_find_bin<W>(sh, k, tid, d, above, cnt);
   uint32_t need = k - above;
-  uint64_t* sh_sort = (uint64_t*)sh;
+  uint64_t* sh_sort = (uint64_t*)sh.bins;
   const bool rank_bucket = cnt != need && cnt <= (uint32_t)kWave;
-  if (cnt == need) {
-    ws_compact(rel, lane, sh_sort, sh_trash, [d](uint32_t r, uint32_t) { return (r >> 21) >= d; });
-  } else if (rank_bucket) {
-    ws_compact(rel, lane, sh_sort, sh_trash, [d](uint32_t r, uint32_t) { return (r >> 21) > d; });
-    ws_compact(rel, lane, sh_cand, sh_trash, [d](uint32_t r, uint32_t) { return (r >> 21) == d; });
+  if (cnt == need || rank_bucket) {
+    const uint32_t sel_from = cnt == need ? d : d + 1u;            // first digit of the entries that are in for sure
+    auto in_sel = [sel_from](uint32_t r, uint32_t) { return (r >> 21) >= sel_from; };
+    auto in_bucket = [d](uint32_t r, uint32_t) { return (r >> 21) == d; };
+    const uint32_t n_sel = ws_count<W>(rel, tid, in_sel);
+    const uint32_t n_cand = rank_bucket ? ws_count<W>(rel, tid, in_bucket) : 0u;
+    __syncthreads();                                               // every wave has read the histogram
+    const uint32_t pos = ws_exclusive<W>(n_sel, tid, sh.wave_a);
+    ws_scatter<W>(rel, tid, sh_sort, pos, sh.trash, in_sel);
+    if (rank_bucket) {
+      const uint32_t cpos = ws_exclusive<W>(n_cand, tid, sh.wave_b);
+      ws_scatter<W>(rel, tid, sh.cand, cpos, sh.trash, in_bucket);
+    }
   } else {
     uint32_t thr = d << 21, tok_limit = 2047u;
     bool done = false;
-    if (bits > 11) done = ws_pass<1>(rel, lane, sh, thr, need, tok_limit);
-    if (!done && bits > 22) done = ws_pass<2>(rel, lane, sh, thr, need, tok_limit);
-    if (!done) ws_pass<3>(rel, lane, sh, thr, need, tok_limit);
+    if (bits > 11) done = ws_pass<1, W>(rel, tid, sh, thr, need, tok_limit);
+    if (!done && bits > 22) done = ws_pass<2, W>(rel, tid, sh, thr, need, tok_limit);
+    if (!done) ws_pass<3, W>(rel, tid, sh, thr, need, tok_limit);
     const uint64_t thr43 = ((uint64_t)thr << 11) | (2047u - tok_limit);
-    ws_compact(rel, lane, sh_sort, sh_trash, [thr43](uint32_t r, uint32_t not_t) {
+    auto in_sel = [thr43](uint32_t r, uint32_t not_t) {
       return (((uint64_t)r << 11) | (not_t & 2047u)) >= thr43;   // (~token & 2047 == 2047 - token)
-    });
+    };
+    const uint32_t n_sel = ws_count<W>(rel, tid, in_sel);
+    __syncthreads();
+    const uint32_t pos = ws_exclusive<W>(n_sel, tid, sh.wave_a);
+    ws_scatter<W>(rel, tid, sh_sort, pos, sh.trash, in_sel);
   }
-  for (uint32_t r = k + lane; r < (uint32_t)kpad; r += kWave) sh_sort[r] = 0ull;
+  for (uint32_t r = k + tid; r < (uint32_t)kpad; r += T) sh_sort[r] = 0ull;
   __syncthreads();
   if (rank_bucket) {
-    // `cnt` entries of the threshold bucket, one per lane: an entry beaten by fewer than `need` others is in
-    const uint64_t c = lane < (int)cnt ? sh_cand[lane] : 0ull;
-    uint32_t rank = 0;
-    for (uint32_t j = 0; j < cnt; ++j) {
-      const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)c, (int)j);
-      const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(c >> 32), (int)j);
-      rank += (((uint64_t)hi << 32) | lo) > c ? 1u : 0u;
+    // `cnt` entries of the threshold bucket, one per lane of the first wave: an entry beaten by fewer than
+    // `need` others is in
+    if (wave == 0) {
+      const uint64_t c = lane < (int)cnt ? sh.cand[lane] : 0ull;
+      uint32_t rank = 0;
+      for (uint32_t j = 0; j < cnt; ++j) {
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)c, (int)j);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(c >> 32), (int)j);
+        rank += (((uint64_t)hi << 32) | lo) > c ? 1u : 0u;
+      }
+      if (lane < (int)cnt && rank < need) sh_sort[above + rank] = c;
     }
-    if (lane < (int)cnt && rank < need) sh_sort[above + rank] = c;
     __syncthreads();
   }
 
-  const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
-                                           : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
-  int32_t* oi = p.out_idx + (int64_t)seg * p.out_stride;
-  float* ov = p.out_val ? p.out_val + (int64_t)seg * p.out_stride : nullptr;
   if (!p.unordered) {
     switch (kpad) {
-      case 1024: ws_sort<16>(sh_sort, lane); break;
-      case 512: ws_sort<8>(sh_sort, lane); break;
-      case 256: ws_sort<4>(sh_sort, lane); break;
-      case 128: ws_sort<2>(sh_sort, lane); break;
-      default: ws_sort<1>(sh_sort, lane); break;
+      case 1024: ws_sort<1024, W>(sh_sort, tid); break;
+      case 512: ws_sort<512, W>(sh_sort, tid); break;
+      case 256: ws_sort<256, W>(sh_sort, tid); break;
+      case 128: ws_sort<128, W>(sh_sort, tid); break;
+      default: ws_sort<64, W>(sh_sort, tid); break;
     }
     __syncthreads();
   }
   // out; the composites carry relative keys: key = (rel >> lshift) + kmin
-  for (uint32_t r = lane; r < k; r += kWave) {
+  const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
+                                           : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
+  int32_t* oi = p.out_idx + (int64_t)seg * p.out_stride;
+  float* ov = p.out_val ? p.out_val + (int64_t)seg * p.out_stride : nullptr;
+  for (uint32_t r = tid; r < k; r += T) {
     const uint64_t c = sh_sort[r];
     oi[r] = (int32_t)(~(uint32_t)c + idx_base);
     if (ov) ov[r] = key_score(((uint32_t)(c >> 32) >> lshift) + kmin);
@@ -277,7 +360,7 @@ __global__ __launch_bounds__(kWave) void select_wave_kernel(SelectParams p, int 
   if (p.out_expand) {
     int32_t* oe = p.out_expand + (int64_t)seg * p.k * p.expand;
     const uint32_t total = k * (uint32_t)p.expand;
-    for (uint32_t e = lane; e < total; e += kWave) {
+    for (uint32_t e = tid; e < total; e += T) {
       const uint32_t jj = e / (uint32_t)p.expand, ii = e % (uint32_t)p.expand;
       oe[e] = (int32_t)(~(uint32_t)sh_sort[jj] * (uint32_t)p.expand + ii);
     }
@@ -295,7 +378,7 @@ int launch_select_wave(const SelectParams& p, hipStream_t stream) {
   int kpad = kWave;
   while (kpad < p.k) kpad <<= 1;
   LaunchTimer timer("select_wave", stream);
-  hipLaunchKernelGGL(select_wave_kernel, dim3(p.num_segments), dim3(kWave), 0, stream, p, kpad);
+  hipLaunchKernelGGL(select_wave_kernel<4>, dim3(p.num_segments), dim3(4 * kWave), 0, stream, p, kpad);
   return hip_status(hipGetLastError());
 }
 
