@@ -81,13 +81,13 @@ def test_shared_kv_chunked():
 @pytest.mark.parametrize("B,H", [(2, 32), (3, 22), (5, 13), (8, 8), (9, 8), (17, 4)])
 def test_shared_kv_batch_tiles(B, H):
     """Keys shared by the batch are scored for several batch entries per pass (tiles of 2, 4 or 8 entries, with
-    a ragged last tile) and the 256 or more short segments are selected by a small workgroup each."""
+    a ragged last tile) and the 128 or more short segments are selected by a small workgroup each."""
     announce("gemv_topk shared KV batch tiles B=%d H=%d N=8192 chunks=4 k=128" % (B, H))
     _run_flat(oracle.F16, B, H, 1, 8192, 128, seed=60 + B, shared_kv=True, num_chunks=4, scale=1.0)
 
 
 def test_many_short_segments_routes():
-    """256 or more segments of at most 2048 rows: plain scores + a small workgroup per segment; both dtypes, grouped
+    """128 or more segments of at most 2048 rows: plain scores + a small workgroup per segment; both dtypes, grouped
     queries, odd lengths, ties, keys per sequence and shared."""
     announce("gemv_topk many short segments")
     _run_flat(oracle.BF16, 8, 8, 2, 8000, 500, seed=70, num_chunks=4)                      # per-sequence keys

@@ -142,7 +142,7 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
 int wave_select_min_segments() {
   static const int v = [] {
     const char* e = getenv("TKA_WAVE_MIN_SEGS");
-    return e && *e ? atoi(e) : 256;
+    return e && *e ? atoi(e) : 128;
   }();
   return v;
 }
