@@ -103,9 +103,11 @@ def _short_segment_rows(rng, n):
 
 
 @pytest.mark.parametrize("n,k", [(2048, 128), (2048, 1024), (2048, 2048 // 2 - 1), (2048, 1), (2047, 33), (1024, 64),
-                                 (1280, 512), (777, 777), (64, 5), (3, 2), (1, 1)])
+                                 (1280, 512), (777, 777), (64, 5), (3, 2), (1, 1), (4096, 64), (4096, 1024), (2049, 1000),
+                                 (3000, 7), (4095, 513)])
 def test_short_segments(n, k):
-    """Segments of at most 2048 scores, many per call (the operator's chunks): adversarial rows and random ones."""
+    """Segments of at most 4096 scores, many per call (the operator's chunks, the centroids of a head):
+    adversarial rows and random ones."""
     announce("topk short segments n=%d k=%d" % (n, k))
     rng = np.random.default_rng(n * 7 + k)
     rows = _short_segment_rows(rng, n)

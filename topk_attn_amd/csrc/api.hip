@@ -137,8 +137,9 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
 }
 
-// Short segments in numbers: a four-wave workgroup per segment selects (a compute unit works on many segments
-// at a time).
+// Short segments (up to 4096 scores, k up to 1024): a workgroup of four or eight waves per segment selects from
+// plain scores.  Segments of up to 2048 rows that still have to be scored take this route only in numbers: a few
+// are quicker scored and selected by one workgroup each in one launch.
 int wave_select_min_segments() {
   static const int v = [] {
     const char* e = getenv("TKA_WAVE_MIN_SEGS");
@@ -146,9 +147,7 @@ int wave_select_min_segments() {
   }();
   return v;
 }
-bool wave_select_fits(int64_t seg_len, int k, int64_t segments) {
-  return seg_len <= select_wave_max_len() && k <= select_wave_max_k() && segments >= wave_select_min_segments();
-}
+bool wave_select_fits(int64_t seg_len, int k) { return seg_len <= select_wave_max_len() && k <= select_wave_max_k(); }
 
 struct UnionOut {
   int32_t* idx;
@@ -198,8 +197,9 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // Keys shared by the batch are read once for several batch entries.
   const bool shared_keys = a->key_stride_b == 0 && a->batch >= 2 && !cluster_ids;
 
-  // Many short segments: plain scores, then a four-wave workgroup per segment selects.
-  if (a->out_idx && !u && wave_select_fits(chunk_len, a->k, segs)) {
+  // Short segments: plain scores, then a small workgroup per segment selects.
+  if (a->out_idx && !u && wave_select_fits(chunk_len, a->k) &&
+      (chunk_len > kFusedMaxSegLen || a->out_scores || segs >= wave_select_min_segments())) {
     gp.hist = nullptr;
     int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);
     if (rc != TKA_OK) return rc;
@@ -458,7 +458,7 @@ int tka_topk_f32(const tka_topk_args* a) {
   sp.num_segments = a->num_segments;
   sp.k = a->k;
   sp.segs_per_row = 1;
-  if (wave_select_fits(a->seg_len, a->k, a->num_segments)) return launch_select_wave(sp, stream);
+  if (wave_select_fits(a->seg_len, a->k)) return launch_select_wave(sp, stream);
   if (a->seg_len <= select_cand_capacity()) {   // the segment fits in LDS whole: one launch
     GemvParams none;
     memset(&none, 0, sizeof none);

@@ -1,20 +1,21 @@
-// Exact top-k of many short segments: a small workgroup (W = 4 wavefronts) per segment.
+// Exact top-k of short segments: a small workgroup (W = 4 or 8 wavefronts) per segment.
 //
 // The operator of the reference selects inside 2048-key chunks, one chunk per (batch entry, head, quarter of
 // the sequence) (retrieval_attention.cu:335-354 sorts each chunk whole), so a call has hundreds to thousands of
-// short segments.  A 1024-thread workgroup per segment spends its time in barriers and leaves most of the GPU
-// idle.  Here the 2048 keys of a segment sit in the registers of W waves (8 per lane for W = 4), eight segments are
-// in flight per compute unit, and the whole selection is a few hundred instructions per wave with eight barriers.
-// The code is written for any W that divides 8; W = 1 (32 keys per lane, no s_barrier at all) measured the same
-// or slower from 256 to 16384 segments, and what a launch of this kernel costs at a few hundred segments is
-// mostly the first fetch of its instructions, so the short form wins.
+// short segments; the centre-only selection (center_only_topk/gemv_topk.cu:251-279) has one of 1024 to 4096
+// centroids per head.  A 1024-thread workgroup per segment spends its time in barriers and leaves most of the
+// GPU idle.  Here the keys of a segment sit in the registers of W waves, 8 per lane (2048 keys for W = 4, 4096
+// for W = 8), several segments are in flight per compute unit, and the whole selection is a few hundred
+// instructions per wave with eight barriers.  (A one-wave form, 32 keys per lane and no s_barrier at all, measured
+// the same or slower from 256 to 16384 segments: what a launch of this kernel costs at a few hundred segments is
+// mostly the first fetch of its instructions, so the form with less code per phase wins.)
 //
 //   1. fp32 scores -> order-preserving keys, relative to the smallest key of the segment and shifted so that the
 //      largest one fills 32 bits;
 //   2. one 11-bit histogram pass in LDS, suffix scans by DPP, the bin of the k-th largest.  If that bin is taken
 //      whole, or holds at most 64 entries (they are ranked directly, one per lane), the selection is known -
-//      ordinary data.  Otherwise up to three more passes: 11 and 10 more bits of the key, then 2047 - token among
-//      the entries that equal the threshold key: lower index first;
+//      ordinary data.  Otherwise up to three more passes over the next 11-bit digits of the 44-bit order number
+//      (relative key, then 4095 - token: among equal keys the lower index comes first);
 //   3. the k selected composites are compacted into LDS (the histogram's space) and sorted with the bitonic
 //      network of bitonic.hpp (registers, DPP, and LDS for the strides that cross waves); rank-ordered ids and
 //      scores are written.  A caller that takes any order skips the sort.
@@ -25,9 +26,10 @@ namespace tka {
 
 namespace {
 
-constexpr int kWsMaxLen = 2048;             // keys per segment at most
+constexpr int kWsEpt = 8;                   // keys per thread
 constexpr int kWsBins = 2048;
-constexpr int kWsMaxWaves = 4;
+constexpr int kWsMaxWaves = 8;
+constexpr int kWsMaxLen = kWsMaxWaves * kWave * kWsEpt;   // 4096 keys per segment at most
 
 __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
   v = min(v, lane_xor<1>(v));
@@ -67,22 +69,25 @@ struct WsShared {
 };
 
 // Register e of thread t holds token (e / 4) * (256 W) + 4 t + e % 4: 16-byte loads, consecutive across threads.
-template <int W>
-__device__ __forceinline__ int ws_token(int e, int tid) { return (e >> 2) * (256 * W) + 4 * tid + (e & 3); }
+// The part of it that does not depend on the thread:
+__device__ __forceinline__ constexpr uint32_t ws_token_base(int e, int W) { return (uint32_t)((e >> 2) * (256 * W) + (e & 3)); }
+
+// The order within a segment as one 44-bit number: relative key, then 4095 - token (lower token first).
+__device__ __forceinline__ uint64_t ws_c44(uint32_t rel, uint32_t not_token) { return ((uint64_t)rel << 12) | (not_token & 4095u); }
 
 template <int W>
 __device__ __forceinline__ void ws_clear(uint32_t* bins, int tid) {
 #pragma unroll
-  for (int i = 0; i < 8 / W; ++i) *(u32x4*)(bins + (256 * W) * i + 4 * tid) = u32x4{0u, 0u, 0u, 0u};
+  for (int i = 0; i < kWsBins / (256 * W); ++i) *(u32x4*)(bins + (256 * W) * i + 4 * tid) = u32x4{0u, 0u, 0u, 0u};
 }
 
 // The bin d of the histogram with  count(bins > d) < need <= count(bins >= d);  `above` = count(bins > d),
 // `cnt` = its own count.  The histogram must hold at least `need` entries.  Two levels: a thread sums its
-// 32 / W consecutive bins, suffix sums over the threads find the thread that owns d; then the first lanes of every
+// 2048 / (64 W) consecutive bins, suffix sums over the threads find the thread that owns d; then the first lanes of every
 // wave take one of that thread's bins each and scan again.  All threads return the same values.
 template <int W>
 __device__ __forceinline__ void ws_find_bin(WsShared<W>& sh, uint32_t need, int tid, uint32_t& d, uint32_t& above, uint32_t& cnt) {
-  constexpr int BPT = 32 / W;   // bins per thread
+  constexpr int BPT = kWsBins / (W * kWave);   // bins per thread
   const int lane = tid & 63, wave = tid >> 6;
   uint32_t tot = 0;
 #pragma unroll
@@ -115,29 +120,33 @@ __device__ __forceinline__ void ws_find_bin(WsShared<W>& sh, uint32_t need, int 
   cnt = (uint32_t)__builtin_amdgcn_readlane((int)v, bin);
 }
 
-// One radix pass below the first.  PASS 1, 2: the second and third digit of the relative key (11 and 10 bits)
-// among the entries that share the digits found so far; PASS 3: the digit is 2047 - token among the entries
-// whose key equals the threshold key.  `thr` is the threshold so far (digits of later passes zero), `need` how
-// many entries of the current bucket are still to be taken.  Returns true when the bucket found is taken whole.
+// One radix pass below the first: digit PASS (11 bits, counted from the top) of the 44-bit order number, among
+// the entries that share the digits found so far.  (thr_rel, thr_low) is the threshold so far, relative key and
+// 12-bit token part, digits of later passes zero; `need` is how many entries of the current bucket are still to
+// be taken.  Returns true when the bucket found is taken whole; after pass 3 it always is (the order numbers are
+// distinct).  Digits: 1 = key bits 20..10; 2 = key bits 9..0 and the top bit of the token part; 3 = the rest
+// of the token part.  (32-bit arithmetic: the 64-bit form cost 16 registers more than the rest of the kernel.)
 template <int PASS, int W>
-__device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[32 / W], int tid, WsShared<W>& sh, uint32_t& thr, uint32_t& need,
-                                        uint32_t& tok_limit) {
+__device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[kWsEpt], int tid, WsShared<W>& sh, uint32_t& thr_rel, uint32_t& thr_low,
+                                        uint32_t& need) {
   __syncthreads();              // the previous histogram has been read
   ws_clear<W>(sh.bins, tid);
   __syncthreads();
+  const uint32_t not_t0 = ~(uint32_t)(4 * tid);
 #pragma unroll
-  for (int e = 0; e < 32 / W; ++e) {
+  for (int e = 0; e < kWsEpt; ++e) {
+    const uint32_t low = (not_t0 - ws_token_base(e, W)) & 4095u;   // 4095 - token
     bool active;
     uint32_t digit;
     if constexpr (PASS == 1) {
-      active = (rel[e] >> 21) == (thr >> 21);
+      active = (rel[e] >> 21) == (thr_rel >> 21);
       digit = (rel[e] >> 10) & 2047u;
     } else if constexpr (PASS == 2) {
-      active = (rel[e] >> 10) == (thr >> 10);
-      digit = rel[e] & 1023u;
+      active = (rel[e] >> 10) == (thr_rel >> 10);
+      digit = ((rel[e] & 1023u) << 1) | (low >> 11);
     } else {
-      active = rel[e] == thr;
-      digit = 2047u - (uint32_t)ws_token<W>(e, tid);
+      active = rel[e] == thr_rel && (low >> 11) == (thr_low >> 11);
+      digit = low & 2047u;
     }
     if (active) atomicAdd(&sh.bins[digit], 1u);
   }
@@ -145,20 +154,20 @@ __device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[32 / W], int tid, 
   uint32_t d, above, cnt;
   ws_find_bin<W>(sh, need, tid, d, above, cnt);
   need -= above;
-  if constexpr (PASS == 1) thr |= d << 10;
-  if constexpr (PASS == 2) thr |= d;
-  if constexpr (PASS == 3) tok_limit = 2047u - d;
+  if constexpr (PASS == 1) thr_rel |= d << 10;
+  if constexpr (PASS == 2) { thr_rel |= d >> 1; thr_low |= (d & 1u) << 11; }
+  if constexpr (PASS == 3) thr_low |= d;
   return cnt == need;
 }
 
 // How many of the thread's entries satisfy PRED.
 template <int W, typename PRED>
-__device__ __forceinline__ uint32_t ws_count(const uint32_t (&rel)[32 / W], int tid, PRED pred) {
+__device__ __forceinline__ uint32_t ws_count(const uint32_t (&rel)[kWsEpt], int tid, PRED pred) {
   const uint32_t not_t0 = ~(uint32_t)(4 * tid);
   uint32_t count[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int e = 0; e < 32 / W; ++e) {
-    const uint32_t not_t = not_t0 - (uint32_t)((e >> 2) * (256 * W) + (e & 3));   // ~token
+  for (int e = 0; e < kWsEpt; ++e) {
+    const uint32_t not_t = not_t0 - ws_token_base(e, W);   // ~token
     count[e & 3] += pred(rel[e], not_t) ? 1u : 0u;
   }
   return (count[0] + count[1]) + (count[2] + count[3]);
@@ -167,12 +176,12 @@ __device__ __forceinline__ uint32_t ws_count(const uint32_t (&rel)[32 / W], int 
 // Stores the thread's entries that satisfy PRED to dst[pos ...] as order-preserving composites (rel << 32) | ~token.
 // Straight-line: the thread stores all its entries, the ones that do not qualify into its own trash slot.
 template <int W, typename PRED>
-__device__ __forceinline__ void ws_scatter(const uint32_t (&rel)[32 / W], int tid, uint64_t* dst, uint32_t pos, uint64_t* trash, PRED pred) {
+__device__ __forceinline__ void ws_scatter(const uint32_t (&rel)[kWsEpt], int tid, uint64_t* dst, uint32_t pos, uint64_t* trash, PRED pred) {
   const uint32_t not_t0 = ~(uint32_t)(4 * tid);
   uint64_t* own = trash + tid;
 #pragma unroll
-  for (int e = 0; e < 32 / W; ++e) {
-    const uint32_t not_t = not_t0 - (uint32_t)((e >> 2) * (256 * W) + (e & 3));
+  for (int e = 0; e < kWsEpt; ++e) {
+    const uint32_t not_t = not_t0 - ws_token_base(e, W);
     const bool take = pred(rel[e], not_t);
     uint64_t* at = take ? dst + pos : own;
     *at = ((uint64_t)rel[e] << 32) | not_t;
@@ -219,7 +228,8 @@ __device__ __forceinline__ void ws_sort(uint64_t* sh_sort, int tid) {
 template <int W>
 __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, int kpad) {
   constexpr int T = W * kWave;
-  constexpr int EPT = 32 / W;              // keys per thread
+  constexpr int EPT = kWsEpt;
+  constexpr int kMaxLen = T * EPT;         // 2048 (W = 4) or 4096 (W = 8) keys
   __shared__ WsShared<W> sh;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -271,8 +281,8 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
   const uint32_t range = kmax - kmin;
   const int bits = range ? 32 - __builtin_clz(range) : 0;
   const int lshift = bits ? 32 - bits : 0;
-  const bool padded = n < kWsMaxLen;
-  if (padded && tid == 0) atomicAdd(&sh.bins[0], (uint32_t)(kWsMaxLen - n));   // the entries past the end, at once
+  const bool padded = n < kMaxLen;
+  if (padded && tid == 0) atomicAdd(&sh.bins[0], (uint32_t)(kMaxLen - n));   // the entries past the end, at once
 #pragma unroll
   for (int e = 0; e < EPT; ++e) {
     const uint32_t r = (rel[e] - kmin) << lshift;
@@ -284,8 +294,7 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
 
   // The k-th largest entry in the order (key, lower token first).  One pass is enough when the bucket of the
   // k-th is taken whole, or holds at most 64 entries: those are ranked directly, one per lane.  Otherwise
-  // further passes fix the threshold (thr, tok_limit): selected are the entries with
-  // (rel, 2047 - token) >= (thr, 2047 - tok_limit).
+  // further passes fix the threshold: selected are the entries whose 44-bit order number is >= thr.
   uint32_t d, above, cnt;
   ws_find_bin<W>(sh, k, tid, d, above, cnt);
   uint32_t need = k - above;
@@ -305,15 +314,13 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
       ws_scatter<W>(rel, tid, sh.cand, cpos, sh.trash, in_bucket);
     }
   } else {
-    uint32_t thr = d << 21, tok_limit = 2047u;
+    uint32_t thr_rel = d << 21, thr_low = 0;
     bool done = false;
-    if (bits > 11) done = ws_pass<1, W>(rel, tid, sh, thr, need, tok_limit);
-    if (!done && bits > 22) done = ws_pass<2, W>(rel, tid, sh, thr, need, tok_limit);
-    if (!done) ws_pass<3, W>(rel, tid, sh, thr, need, tok_limit);
-    const uint64_t thr43 = ((uint64_t)thr << 11) | (2047u - tok_limit);
-    auto in_sel = [thr43](uint32_t r, uint32_t not_t) {
-      return (((uint64_t)r << 11) | (not_t & 2047u)) >= thr43;   // (~token & 2047 == 2047 - token)
-    };
+    if (bits > 11) done = ws_pass<1, W>(rel, tid, sh, thr_rel, thr_low, need);    // (bits <= 11: that digit is 0 everywhere)
+    if (!done) done = ws_pass<2, W>(rel, tid, sh, thr_rel, thr_low, need);
+    if (!done) ws_pass<3, W>(rel, tid, sh, thr_rel, thr_low, need);
+    const uint64_t thr = ((uint64_t)thr_rel << 12) | thr_low;
+    auto in_sel = [thr](uint32_t r, uint32_t not_t) { return ws_c44(r, not_t) >= thr; };
     const uint32_t n_sel = ws_count<W>(rel, tid, in_sel);
     __syncthreads();
     const uint32_t pos = ws_exclusive<W>(n_sel, tid, sh.wave_a);
@@ -378,7 +385,10 @@ int launch_select_wave(const SelectParams& p, hipStream_t stream) {
   int kpad = kWave;
   while (kpad < p.k) kpad <<= 1;
   LaunchTimer timer("select_wave", stream);
-  hipLaunchKernelGGL(select_wave_kernel<4>, dim3(p.num_segments), dim3(4 * kWave), 0, stream, p, kpad);
+  if (p.seg_len <= 4 * kWave * kWsEpt)
+    hipLaunchKernelGGL(select_wave_kernel<4>, dim3(p.num_segments), dim3(4 * kWave), 0, stream, p, kpad);
+  else
+    hipLaunchKernelGGL(select_wave_kernel<8>, dim3(p.num_segments), dim3(8 * kWave), 0, stream, p, kpad);
   return hip_status(hipGetLastError());
 }
 
