@@ -115,6 +115,17 @@ def test_short_segments(n, k):
     _check(np.stack(rows), k)
 
 
+@pytest.mark.parametrize("n,k", [(8192, 2048), (5000, 1500), (16384, 100), (12345, 2047), (16384, 2048), (8193, 1), (16383, 999)])
+def test_register_resident_segments(n, k):
+    """Segments of 4097 to 16384 scores (one 1024-thread workgroup holds the keys in registers), k up to 2048:
+    adversarial rows and random ones."""
+    announce("topk register-resident segments n=%d k=%d" % (n, k))
+    rng = np.random.default_rng(n + k)
+    rows = _short_segment_rows(rng, n)
+    rows += [rng.standard_normal(n).astype(np.float32) for _ in range(3)]
+    _check(np.stack(rows), k)
+
+
 def test_short_segments_many():
     """4096 segments in one call (32 batch entries x 32 heads x 4 chunks of the operator)."""
     announce("topk short segments 4096 x 2048, k=128")

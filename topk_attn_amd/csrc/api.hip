@@ -137,9 +137,9 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
 }
 
-// Short segments (up to 4096 scores, k up to 1024): a workgroup of four or eight waves per segment selects from
-// plain scores.  Segments of up to 2048 rows that still have to be scored take this route only in numbers: a few
-// are quicker scored and selected by one workgroup each in one launch.
+// Segments of up to 16384 scores (k up to 1024, 2048 beyond 4096 scores): one workgroup per segment selects from
+// plain scores with the keys in its registers.  Segments of up to 2048 rows that still have to be scored take this
+// route only in numbers: a few are quicker scored and selected by one workgroup each in one launch.
 int wave_select_min_segments() {
   static const int v = [] {
     const char* e = getenv("TKA_WAVE_MIN_SEGS");
@@ -147,7 +147,7 @@ int wave_select_min_segments() {
   }();
   return v;
 }
-bool wave_select_fits(int64_t seg_len, int k) { return seg_len <= select_wave_max_len() && k <= select_wave_max_k(); }
+bool wave_select_fits(int64_t seg_len, int k) { return seg_len <= select_wave_max_len() && k <= select_wave_max_k(seg_len); }
 
 struct UnionOut {
   int32_t* idx;
@@ -197,7 +197,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // Keys shared by the batch are read once for several batch entries.
   const bool shared_keys = a->key_stride_b == 0 && a->batch >= 2 && !cluster_ids;
 
-  // Short segments: plain scores, then a small workgroup per segment selects.
+  // Segments that fit in the registers of a workgroup: plain scores, then one workgroup per segment selects.
   if (a->out_idx && !u && wave_select_fits(chunk_len, a->k) &&
       (chunk_len > kFusedMaxSegLen || a->out_scores || segs >= wave_select_min_segments())) {
     gp.hist = nullptr;

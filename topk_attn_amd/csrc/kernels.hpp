@@ -80,10 +80,11 @@ int launch_select_finalize(const SelectParams& p, hipStream_t stream);
 int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
 int select_cand_max_parts();   // most candidate slices per segment
 int select_cand_capacity();    // most candidates per segment
-// A four-wave workgroup per segment: rank-ordered top-k of fp32 scores, segments of up to select_wave_max_len() scores.
+// One workgroup per segment, keys in registers: rank-ordered top-k of fp32 scores, segments of up to
+// select_wave_max_len() scores, k up to select_wave_max_k(segment length).
 int launch_select_wave(const SelectParams& p, hipStream_t stream);
 int select_wave_max_len();
-int select_wave_max_k();
+int select_wave_max_k(int64_t seg_len);
 
 struct UnionParams {
   const int32_t* idx;     // [num_segments][k]

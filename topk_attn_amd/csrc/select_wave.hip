@@ -1,21 +1,25 @@
-// Exact top-k of short segments: a small workgroup (W = 4 or 8 wavefronts) per segment.
+// Exact top-k of segments whose keys fit in the registers of one workgroup: W wavefronts per segment.
 //
 // The operator of the reference selects inside 2048-key chunks, one chunk per (batch entry, head, quarter of
 // the sequence) (retrieval_attention.cu:335-354 sorts each chunk whole), so a call has hundreds to thousands of
 // short segments; the centre-only selection (center_only_topk/gemv_topk.cu:251-279) has one of 1024 to 4096
-// centroids per head.  A 1024-thread workgroup per segment spends its time in barriers and leaves most of the
-// GPU idle.  Here the keys of a segment sit in the registers of W waves, 8 per lane (2048 keys for W = 4, 4096
-// for W = 8), several segments are in flight per compute unit, and the whole selection is a few hundred
-// instructions per wave with eight barriers.  (A one-wave form, 32 keys per lane and no s_barrier at all, measured
-// the same or slower from 256 to 16384 segments: what a launch of this kernel costs at a few hundred segments is
-// mostly the first fetch of its instructions, so the form with less code per phase wins.)
+// centroids per head.  Here the keys of a segment sit in the registers of W waves, EPT per lane:
+//     W = 4,  EPT = 8        2048 keys     several segments in flight per compute unit
+//     W = 8,  EPT = 8        4096 keys
+//     W = 16, EPT = 8, 16    8192, 16384 keys (k up to 2048)
+// and the whole selection is a few hundred instructions per wave with about eight barriers.  (A one-wave form,
+// 32 keys per lane and no s_barrier at all, measured the same or slower from 256 to 16384 segments of 2048: what
+// a launch of this kernel costs at a few hundred segments is mostly the first fetch of its instructions, so
+// the form with less code per phase wins.  32 keys per lane in 16 waves, for 32768 keys, does not fit the 128
+// registers a 1024-thread workgroup has: it spilled and was slower than the multi-launch path.)
 //
 //   1. fp32 scores -> order-preserving keys, relative to the smallest key of the segment and shifted so that the
 //      largest one fills 32 bits;
 //   2. one 11-bit histogram pass in LDS, suffix scans by DPP, the bin of the k-th largest.  If that bin is taken
 //      whole, or holds at most 64 entries (they are ranked directly, one per lane), the selection is known -
-//      ordinary data.  Otherwise up to three more passes over the next 11-bit digits of the 44-bit order number
-//      (relative key, then 4095 - token: among equal keys the lower index comes first);
+//      ordinary data.  Otherwise up to two more passes over the remaining 11 and 10 bits of the key, and if the
+//      threshold key itself is shared by more entries than are still needed, a scan in token order gives them
+//      their rank among equals: lower index first;
 //   3. the k selected composites are compacted into LDS (the histogram's space) and sorted with the bitonic
 //      network of bitonic.hpp (registers, DPP, and LDS for the strides that cross waves); rank-ordered ids and
 //      scores are written.  A caller that takes any order skips the sort.
@@ -26,10 +30,9 @@ namespace tka {
 
 namespace {
 
-constexpr int kWsEpt = 8;                   // keys per thread
 constexpr int kWsBins = 2048;
-constexpr int kWsMaxWaves = 8;
-constexpr int kWsMaxLen = kWsMaxWaves * kWave * kWsEpt;   // 4096 keys per segment at most
+constexpr int kWsMaxWaves = 16;
+constexpr int kWsMaxLen = kWsMaxWaves * kWave * 16;   // 16384 keys per segment at most
 
 __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
   v = min(v, lane_xor<1>(v));
@@ -57,28 +60,32 @@ __device__ __forceinline__ uint32_t ws_key(float x) {
   return x != x ? 0u : key;
 }
 
-// What the W waves of a segment share.  (A one-wave workgroup's __syncthreads() is no s_barrier, only a wait
-// on the LDS counter.)
+// Most composites the sort buffer holds: 2048 for the 1024-thread form, else 1024 (the histogram's 8 KB).
+constexpr int ws_max_k(int W) { return W >= 16 ? 2048 : 1024; }
+
+// What the W waves of a segment share.
 template <int W>
 struct WsShared {
-  __align__(16) uint32_t bins[kWsBins];   // the histogram, then the sort buffer (1024 composites)
-  uint64_t cand[kWave];                   // entries of the threshold bucket when there are few
-  uint64_t trash[W * kWave];              // where a thread stores what is not selected
+  __align__(16) uint32_t bins[2 * ws_max_k(W)];   // the histogram (2048 bins), then the sort buffer (composites)
+  uint64_t cand[kWave];                           // entries of the threshold bucket when there are few
+  uint64_t trash[W * kWave];                      // where a thread stores what is not selected
   uint32_t wave_a[kWsMaxWaves], wave_b[kWsMaxWaves];   // per-wave partial results
-  uint32_t owner[4];                      // find_bin: owning thread, entries above its bins, entries in its bins
+  uint32_t owner[4];                              // find_bin: owning thread, entries above its bins, entries in its bins
 };
 
 // Register e of thread t holds token (e / 4) * (256 W) + 4 t + e % 4: 16-byte loads, consecutive across threads.
 // The part of it that does not depend on the thread:
 __device__ __forceinline__ constexpr uint32_t ws_token_base(int e, int W) { return (uint32_t)((e >> 2) * (256 * W) + (e & 3)); }
 
-// The order within a segment as one 44-bit number: relative key, then 4095 - token (lower token first).
-__device__ __forceinline__ uint64_t ws_c44(uint32_t rel, uint32_t not_token) { return ((uint64_t)rel << 12) | (not_token & 4095u); }
-
 template <int W>
 __device__ __forceinline__ void ws_clear(uint32_t* bins, int tid) {
+  constexpr int kPer = kWsBins / (W * kWave);   // words per thread
+  if constexpr (kPer >= 4) {
 #pragma unroll
-  for (int i = 0; i < kWsBins / (256 * W); ++i) *(u32x4*)(bins + (256 * W) * i + 4 * tid) = u32x4{0u, 0u, 0u, 0u};
+    for (int i = 0; i < kPer / 4; ++i) *(u32x4*)(bins + (256 * W) * i + 4 * tid) = u32x4{0u, 0u, 0u, 0u};
+  } else {
+    *(u32x2*)(bins + 2 * tid) = u32x2{0u, 0u};
+  }
 }
 
 // The bin d of the histogram with  count(bins > d) < need <= count(bins >= d);  `above` = count(bins > d),
@@ -90,20 +97,23 @@ __device__ __forceinline__ void ws_find_bin(WsShared<W>& sh, uint32_t need, int 
   constexpr int BPT = kWsBins / (W * kWave);   // bins per thread
   const int lane = tid & 63, wave = tid >> 6;
   uint32_t tot = 0;
+  if constexpr (BPT >= 4) {
 #pragma unroll
-  for (int i = 0; i < BPT / 4; ++i) {
-    const u32x4 v = *(const u32x4*)(sh.bins + BPT * tid + 4 * i);
-    tot += (v[0] + v[1]) + (v[2] + v[3]);
+    for (int i = 0; i < BPT / 4; ++i) {
+      const u32x4 v = *(const u32x4*)(sh.bins + BPT * tid + 4 * i);
+      tot += (v[0] + v[1]) + (v[2] + v[3]);
+    }
+  } else {
+    const u32x2 v = *(const u32x2*)(sh.bins + 2 * tid);
+    tot = v[0] + v[1];
   }
   const uint32_t inc = wave_inclusive_scan(tot);
   const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)inc, 63);
   uint32_t higher = wave_total - inc;            // entries in the bins of higher lanes of this wave
-  if constexpr (W > 1) {
-    if (lane == 0) sh.wave_a[wave] = wave_total;
-    __syncthreads();
+  if (lane == 0) sh.wave_a[wave] = wave_total;
+  __syncthreads();
 #pragma unroll
-    for (int w = 1; w < W; ++w) higher += w > wave ? sh.wave_a[w] : 0u;
-  }
+  for (int w = 1; w < W; ++w) higher += w > wave ? sh.wave_a[w] : 0u;
   if (higher < need && need <= higher + tot) {   // exactly one thread
     sh.owner[0] = (uint32_t)tid;
     sh.owner[1] = higher;
@@ -120,33 +130,24 @@ __device__ __forceinline__ void ws_find_bin(WsShared<W>& sh, uint32_t need, int 
   cnt = (uint32_t)__builtin_amdgcn_readlane((int)v, bin);
 }
 
-// One radix pass below the first: digit PASS (11 bits, counted from the top) of the 44-bit order number, among
-// the entries that share the digits found so far.  (thr_rel, thr_low) is the threshold so far, relative key and
-// 12-bit token part, digits of later passes zero; `need` is how many entries of the current bucket are still to
-// be taken.  Returns true when the bucket found is taken whole; after pass 3 it always is (the order numbers are
-// distinct).  Digits: 1 = key bits 20..10; 2 = key bits 9..0 and the top bit of the token part; 3 = the rest
-// of the token part.  (32-bit arithmetic: the 64-bit form cost 16 registers more than the rest of the kernel.)
-template <int PASS, int W>
-__device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[kWsEpt], int tid, WsShared<W>& sh, uint32_t& thr_rel, uint32_t& thr_low,
-                                        uint32_t& need) {
+// One radix pass below the first, among the entries that share the digits found so far: PASS 1 = key bits 20..10,
+// PASS 2 = key bits 9..0.  `thr` is the threshold key so far (digits of later passes zero), `need` how many
+// entries of the current bucket are still to be taken.  Returns true when the bucket found is taken whole.
+template <int PASS, int W, int EPT>
+__device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[EPT], int tid, WsShared<W>& sh, uint32_t& thr, uint32_t& need) {
   __syncthreads();              // the previous histogram has been read
   ws_clear<W>(sh.bins, tid);
   __syncthreads();
-  const uint32_t not_t0 = ~(uint32_t)(4 * tid);
 #pragma unroll
-  for (int e = 0; e < kWsEpt; ++e) {
-    const uint32_t low = (not_t0 - ws_token_base(e, W)) & 4095u;   // 4095 - token
+  for (int e = 0; e < EPT; ++e) {
     bool active;
     uint32_t digit;
     if constexpr (PASS == 1) {
-      active = (rel[e] >> 21) == (thr_rel >> 21);
+      active = (rel[e] >> 21) == (thr >> 21);
       digit = (rel[e] >> 10) & 2047u;
-    } else if constexpr (PASS == 2) {
-      active = (rel[e] >> 10) == (thr_rel >> 10);
-      digit = ((rel[e] & 1023u) << 1) | (low >> 11);
     } else {
-      active = rel[e] == thr_rel && (low >> 11) == (thr_low >> 11);
-      digit = low & 2047u;
+      active = (rel[e] >> 10) == (thr >> 10);
+      digit = rel[e] & 1023u;
     }
     if (active) atomicAdd(&sh.bins[digit], 1u);
   }
@@ -154,55 +155,79 @@ __device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[kWsEpt], int tid, 
   uint32_t d, above, cnt;
   ws_find_bin<W>(sh, need, tid, d, above, cnt);
   need -= above;
-  if constexpr (PASS == 1) thr_rel |= d << 10;
-  if constexpr (PASS == 2) { thr_rel |= d >> 1; thr_low |= (d & 1u) << 11; }
-  if constexpr (PASS == 3) thr_low |= d;
+  thr |= PASS == 1 ? d << 10 : d;
   return cnt == need;
 }
 
-// How many of the thread's entries satisfy PRED.
-template <int W, typename PRED>
-__device__ __forceinline__ uint32_t ws_count(const uint32_t (&rel)[kWsEpt], int tid, PRED pred) {
-  const uint32_t not_t0 = ~(uint32_t)(4 * tid);
+// Exclusive prefix of `mine` over the threads of the workgroup, and the total (slot: one of the per-wave arrays;
+// two calls in a row must use different slots).  Contains one barrier: every thread must call it.
+template <int W>
+__device__ __forceinline__ uint32_t ws_exclusive(uint32_t mine, int tid, uint32_t* slot, uint32_t* total = nullptr) {
+  const int lane = tid & 63, wave = tid >> 6;
+  const uint32_t inc = wave_inclusive_scan(mine);
+  uint32_t pos = inc - mine;
+  if (lane == 63) slot[wave] = inc;
+  __syncthreads();
+  uint32_t all = 0;
+#pragma unroll
+  for (int w = 0; w < W; ++w) {
+    const uint32_t s = slot[w];
+    pos += w < wave ? s : 0u;
+    all += s;
+  }
+  if (total) *total = all;
+  return pos;
+}
+
+// The entries whose key equals the threshold key, when more of them exist than are still needed: the `need`
+// with the lowest tokens are in.  Token order is (register group of four, thread, register in the group), so a
+// scan over the threads per group of four registers ranks them.  Returns the thread's mask of selected equals.
+template <int W, int EPT>
+__device__ __forceinline__ uint32_t ws_rank_equals(const uint32_t (&rel)[EPT], int tid, WsShared<W>& sh, uint32_t thr, uint32_t need) {
+  uint32_t sel_mask = 0, before = 0;
+#pragma unroll
+  for (int c = 0; c < EPT / 4; ++c) {
+    uint32_t eq[4], mine = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      eq[r] = rel[4 * c + r] == thr ? 1u : 0u;
+      mine += eq[r];
+    }
+    uint32_t total;
+    uint32_t rank = before + ws_exclusive<W>(mine, tid, (c & 1) ? sh.wave_b : sh.wave_a, &total);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (eq[r] && rank < need) sel_mask |= 1u << (4 * c + r);
+      rank += eq[r];
+    }
+    before += total;
+  }
+  return sel_mask;
+}
+
+// How many of the thread's entries satisfy PRED(relative key, register index).
+template <int EPT, typename PRED>
+__device__ __forceinline__ uint32_t ws_count(const uint32_t (&rel)[EPT], PRED pred) {
   uint32_t count[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int e = 0; e < kWsEpt; ++e) {
-    const uint32_t not_t = not_t0 - ws_token_base(e, W);   // ~token
-    count[e & 3] += pred(rel[e], not_t) ? 1u : 0u;
-  }
+  for (int e = 0; e < EPT; ++e) count[e & 3] += pred(rel[e], e) ? 1u : 0u;
   return (count[0] + count[1]) + (count[2] + count[3]);
 }
 
 // Stores the thread's entries that satisfy PRED to dst[pos ...] as order-preserving composites (rel << 32) | ~token.
 // Straight-line: the thread stores all its entries, the ones that do not qualify into its own trash slot.
-template <int W, typename PRED>
-__device__ __forceinline__ void ws_scatter(const uint32_t (&rel)[kWsEpt], int tid, uint64_t* dst, uint32_t pos, uint64_t* trash, PRED pred) {
+template <int W, int EPT, typename PRED>
+__device__ __forceinline__ void ws_scatter(const uint32_t (&rel)[EPT], int tid, uint64_t* dst, uint32_t pos, uint64_t* trash, PRED pred) {
   const uint32_t not_t0 = ~(uint32_t)(4 * tid);
   uint64_t* own = trash + tid;
 #pragma unroll
-  for (int e = 0; e < kWsEpt; ++e) {
-    const uint32_t not_t = not_t0 - ws_token_base(e, W);
-    const bool take = pred(rel[e], not_t);
+  for (int e = 0; e < EPT; ++e) {
+    const uint32_t not_t = not_t0 - ws_token_base(e, W);   // ~token
+    const bool take = pred(rel[e], e);
     uint64_t* at = take ? dst + pos : own;
     *at = ((uint64_t)rel[e] << 32) | not_t;
     pos += take ? 1u : 0u;
   }
-}
-
-// Exclusive prefix of `mine` over the threads of the workgroup (slot: one of the per-wave arrays).
-// W > 1: contains one barrier, every thread must call it.
-template <int W>
-__device__ __forceinline__ uint32_t ws_exclusive(uint32_t mine, int tid, uint32_t* slot) {
-  const int lane = tid & 63, wave = tid >> 6;
-  const uint32_t inc = wave_inclusive_scan(mine);
-  uint32_t pos = inc - mine;
-  if constexpr (W > 1) {
-    if (lane == 63) slot[wave] = inc;
-    __syncthreads();
-#pragma unroll
-    for (int w = 0; w < W - 1; ++w) pos += w < wave ? slot[w] : 0u;
-  }
-  return pos;
 }
 
 // The composites sh_sort[0 .. N) (zero past the k-th) into descending order, by the first N / E threads.
@@ -225,11 +250,10 @@ __device__ __forceinline__ void ws_sort(uint64_t* sh_sort, int tid) {
   }
 }
 
-template <int W>
+template <int W, int EPT>
 __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, int kpad) {
   constexpr int T = W * kWave;
-  constexpr int EPT = kWsEpt;
-  constexpr int kMaxLen = T * EPT;         // 2048 (W = 4) or 4096 (W = 8) keys
+  constexpr int kMaxLen = T * EPT;
   __shared__ WsShared<W> sh;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -270,14 +294,10 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
   }
   kmin = wave_min_u32(kmin);
   kmax = wave_max_u32(kmax);
-  if constexpr (W > 1) {
-    if (lane == 0) { sh.wave_a[wave] = kmin; sh.wave_b[wave] = kmax; }
-  }
+  if (lane == 0) { sh.wave_a[wave] = kmin; sh.wave_b[wave] = kmax; }
   __syncthreads();
-  if constexpr (W > 1) {
 #pragma unroll
-    for (int w = 0; w < W; ++w) { kmin = min(kmin, sh.wave_a[w]); kmax = max(kmax, sh.wave_b[w]); }
-  }
+  for (int w = 0; w < W; ++w) { kmin = min(kmin, sh.wave_a[w]); kmax = max(kmax, sh.wave_b[w]); }
   const uint32_t range = kmax - kmin;
   const int bits = range ? 32 - __builtin_clz(range) : 0;
   const int lshift = bits ? 32 - bits : 0;
@@ -294,37 +314,37 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
 
   // The k-th largest entry in the order (key, lower token first).  One pass is enough when the bucket of the
   // k-th is taken whole, or holds at most 64 entries: those are ranked directly, one per lane.  Otherwise
-  // further passes fix the threshold: selected are the entries whose 44-bit order number is >= thr.
+  // further passes fix the threshold key, and a scan the equals that are in.
   uint32_t d, above, cnt;
   ws_find_bin<W>(sh, k, tid, d, above, cnt);
   uint32_t need = k - above;
   uint64_t* sh_sort = (uint64_t*)sh.bins;
-  const bool rank_bucket = cnt != need && cnt <= (uint32_t)kWave;
-  if (cnt == need || rank_bucket) {
-    const uint32_t sel_from = cnt == need ? d : d + 1u;            // first digit of the entries that are in for sure
-    auto in_sel = [sel_from](uint32_t r, uint32_t) { return (r >> 21) >= sel_from; };
-    auto in_bucket = [d](uint32_t r, uint32_t) { return (r >> 21) == d; };
-    const uint32_t n_sel = ws_count<W>(rel, tid, in_sel);
-    const uint32_t n_cand = rank_bucket ? ws_count<W>(rel, tid, in_bucket) : 0u;
-    __syncthreads();                                               // every wave has read the histogram
-    const uint32_t pos = ws_exclusive<W>(n_sel, tid, sh.wave_a);
-    ws_scatter<W>(rel, tid, sh_sort, pos, sh.trash, in_sel);
-    if (rank_bucket) {
-      const uint32_t cpos = ws_exclusive<W>(n_cand, tid, sh.wave_b);
-      ws_scatter<W>(rel, tid, sh.cand, cpos, sh.trash, in_bucket);
-    }
-  } else {
-    uint32_t thr_rel = d << 21, thr_low = 0;
-    bool done = false;
-    if (bits > 11) done = ws_pass<1, W>(rel, tid, sh, thr_rel, thr_low, need);    // (bits <= 11: that digit is 0 everywhere)
-    if (!done) done = ws_pass<2, W>(rel, tid, sh, thr_rel, thr_low, need);
-    if (!done) ws_pass<3, W>(rel, tid, sh, thr_rel, thr_low, need);
-    const uint64_t thr = ((uint64_t)thr_rel << 12) | thr_low;
-    auto in_sel = [thr](uint32_t r, uint32_t not_t) { return ws_c44(r, not_t) >= thr; };
-    const uint32_t n_sel = ws_count<W>(rel, tid, in_sel);
+  // compaction of the entries that satisfy `pred` into dst (in the histogram's space: behind a barrier)
+  auto compact = [&](uint64_t* dst, uint32_t* slot, auto pred) {
+    const uint32_t mine = ws_count<EPT>(rel, pred);
     __syncthreads();
-    const uint32_t pos = ws_exclusive<W>(n_sel, tid, sh.wave_a);
-    ws_scatter<W>(rel, tid, sh_sort, pos, sh.trash, in_sel);
+    const uint32_t pos = ws_exclusive<W>(mine, tid, slot);
+    ws_scatter<W, EPT>(rel, tid, dst, pos, sh.trash, pred);
+  };
+  const bool rank_bucket = cnt != need && cnt <= (uint32_t)kWave;
+  if (cnt == need) {
+    compact(sh_sort, sh.wave_a, [d](uint32_t r, int) { return (r >> 21) >= d; });
+  } else if (rank_bucket) {
+    compact(sh_sort, sh.wave_a, [d](uint32_t r, int) { return (r >> 21) > d; });
+    compact(sh.cand, sh.wave_b, [d](uint32_t r, int) { return (r >> 21) == d; });
+  } else {
+    uint32_t thr = d << 21;
+    bool whole = false;     // the bucket of the threshold is taken whole
+    if (bits > 11) whole = ws_pass<1, W, EPT>(rel, tid, sh, thr, need);      // (bits <= 11: that digit is 0 everywhere)
+    if (!whole && bits > 22) whole = ws_pass<2, W, EPT>(rel, tid, sh, thr, need);
+    if (whole) {
+      compact(sh_sort, sh.wave_a, [thr](uint32_t r, int) { return r >= thr; });
+    } else {
+      // `thr` is now a full key shared by more entries than the `need` still to be taken
+      __syncthreads();                                             // (the per-wave slots of the last pass have been read)
+      const uint32_t eq_sel = ws_rank_equals<W, EPT>(rel, tid, sh, thr, need);
+      compact(sh_sort, (EPT / 4) & 1 ? sh.wave_b : sh.wave_a, [thr, eq_sel](uint32_t r, int e) { return r > thr || ((eq_sel >> e) & 1u); });
+    }
   }
   for (uint32_t r = k + tid; r < (uint32_t)kpad; r += T) sh_sort[r] = 0ull;
   __syncthreads();
@@ -345,12 +365,16 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
   }
 
   if (!p.unordered) {
-    switch (kpad) {
-      case 1024: ws_sort<1024, W>(sh_sort, tid); break;
-      case 512: ws_sort<512, W>(sh_sort, tid); break;
-      case 256: ws_sort<256, W>(sh_sort, tid); break;
-      case 128: ws_sort<128, W>(sh_sort, tid); break;
-      default: ws_sort<64, W>(sh_sort, tid); break;
+    if (ws_max_k(W) >= 2048 && kpad == 2048) {
+      ws_sort<ws_max_k(W) >= 2048 ? 2048 : 1024, W>(sh_sort, tid);
+    } else {
+      switch (kpad) {
+        case 1024: ws_sort<1024, W>(sh_sort, tid); break;
+        case 512: ws_sort<512, W>(sh_sort, tid); break;
+        case 256: ws_sort<256, W>(sh_sort, tid); break;
+        case 128: ws_sort<128, W>(sh_sort, tid); break;
+        default: ws_sort<64, W>(sh_sort, tid); break;
+      }
     }
     __syncthreads();
   }
@@ -377,18 +401,22 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
 }  // namespace
 
 int select_wave_max_len() { return kWsMaxLen; }
-int select_wave_max_k() { return kWsBins / 2; }
+int select_wave_max_k(int64_t seg_len) { return seg_len > 8 * kWave * 8 ? ws_max_k(16) : ws_max_k(4); }
 
 int launch_select_wave(const SelectParams& p, hipStream_t stream) {
-  if (p.seg_len < 1 || p.seg_len > kWsMaxLen || p.k < 1 || p.k > p.seg_len || p.k > kWsBins / 2 || !p.out_idx || !p.scores)
+  if (p.seg_len < 1 || p.seg_len > kWsMaxLen || p.k < 1 || p.k > p.seg_len || p.k > select_wave_max_k(p.seg_len) || !p.out_idx ||
+      !p.scores)
     return TKA_EINVAL;
   int kpad = kWave;
   while (kpad < p.k) kpad <<= 1;
   LaunchTimer timer("select_wave", stream);
-  if (p.seg_len <= 4 * kWave * kWsEpt)
-    hipLaunchKernelGGL(select_wave_kernel<4>, dim3(p.num_segments), dim3(4 * kWave), 0, stream, p, kpad);
-  else
-    hipLaunchKernelGGL(select_wave_kernel<8>, dim3(p.num_segments), dim3(8 * kWave), 0, stream, p, kpad);
+  const dim3 grid(p.num_segments);
+#define TKA_LAUNCH_WS(W, EPT) hipLaunchKernelGGL((select_wave_kernel<W, EPT>), grid, dim3(W * kWave), 0, stream, p, kpad)
+  if (p.seg_len <= 2048) TKA_LAUNCH_WS(4, 8);
+  else if (p.seg_len <= 4096) TKA_LAUNCH_WS(8, 8);
+  else if (p.seg_len <= 8192) TKA_LAUNCH_WS(16, 8);
+  else TKA_LAUNCH_WS(16, 16);
+#undef TKA_LAUNCH_WS
   return hip_status(hipGetLastError());
 }
 
