@@ -348,3 +348,38 @@ def test_sparse_decode_step_graph_replay():
         assert torch.equal(plan.union_count, want_cnt), "replay %d: union counts differ" % it
         assert torch.equal(plan.union_idx, want_idx), "replay %d: union lists differ" % it
         assert torch.equal(plan.out, want_out), "replay %d: outputs differ" % it
+
+
+def test_retrieval_attention_graph_replay():
+    """The operator captured in a HIP graph (the batch path: shared-key scoring, small-workgroup selection,
+    attention that writes the result itself) and replayed with new queries; every replay is compared with the
+    eager result for the same query, with eager work in between."""
+    from topk_attn_amd import retrieval_attention_cpp as ra
+    announce("retrieval_attention_128 captured in a graph, 3 replays with changing queries (B=6)")
+    rng = np.random.default_rng(78)
+    dtype, B = oracle.F16, 6
+    q = to_dev(randn_bits(rng, (B, 32, 128), dtype, 0.1), dtype)
+    K, V = to_dev(randn_bits(rng, (8192, 32, 128), dtype, 0.1), dtype), to_dev(randn_bits(rng, (8192, 32, 128), dtype, 0.1), dtype)
+    out = torch.zeros((B, 32, 128), dtype=torch.float16, device="cuda")
+    ra.retrieval_attention_128(q, K, V, out)     # warm-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        ra.retrieval_attention_128(q, K, V, out)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            ra.retrieval_attention_128(q, K, V, out)
+    torch.cuda.synchronize()
+    for it in range(3):
+        q.copy_(to_dev(randn_bits(rng, (B, 32, 128), dtype, 0.1 * (1 + it)), dtype))
+        ra.retrieval_attention_128(q, K, V, out)
+        torch.cuda.synchronize()
+        want = out.clone()
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), "replay %d: outputs differ" % it
+    ref, _, _ = oracle.retrieval_attention(bits_of(q)[B - 1, 3], bits_of(K)[:, 3], bits_of(V)[:, 3], dtype, 4, 128, 1.0)
+    assert np.abs(f32_of(out)[B - 1, 3] - ref).max() < TOL
