@@ -276,7 +276,10 @@ def test_sparse_decode_step(dtype, out_dt, B, H, G, N, k, sink, local):
     (oracle.BF16, 1, 3, 4, 8000, 8000, 4, 4, "heavy"),
     (oracle.F16, 1, 2, 4, 1500, 300, 8, 8, "heavy"),
     (oracle.BF16, 1, 2, 2, 2048, 2048, 0, 16, "levels"),
-    (oracle.F16, 1, 1, 8, 16384, 4000, 64, 512, "equal")])
+    (oracle.F16, 1, 1, 8, 16384, 4000, 64, 512, "equal"),
+    (oracle.F16, 1, 2, 2, 5000, 700, 3000, 3000, "heavy"),        # sink range and local window overlap
+    (oracle.BF16, 3, 2, 4, 9000, 2048, 1, 8999, "levels"),        # the window covers nearly everything
+    (oracle.F16, 2, 2, 1, 12289, 2048, 5, 7, "equal")])
 def test_sparse_decode_step_union_only(dtype, B, H, G, N, k, sink, local, kind, out_dt=torch.float16):
     """Production form of the step: no rank-ordered output.  The union list must still equal the oracle's bit for
     bit — with heavy hitters, with 16-level keys (large tie buckets), with all keys equal (every token ties) and

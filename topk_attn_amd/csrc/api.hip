@@ -198,7 +198,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   const bool shared_keys = a->key_stride_b == 0 && a->batch >= 2 && !cluster_ids;
 
   // Segments that fit in the registers of a workgroup: plain scores, then one workgroup per segment selects.
-  if (a->out_idx && !u && wave_select_fits(chunk_len, a->k) &&
+  if ((a->out_idx || u) && wave_select_fits(chunk_len, a->k) &&
       (chunk_len > kFusedMaxSegLen || a->out_scores || segs >= wave_select_min_segments())) {
     gp.hist = nullptr;
     int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);

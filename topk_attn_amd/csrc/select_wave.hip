@@ -71,6 +71,7 @@ struct WsShared {
   uint64_t trash[W * kWave];                      // where a thread stores what is not selected
   uint32_t wave_a[kWsMaxWaves], wave_b[kWsMaxWaves];   // per-wave partial results
   uint32_t owner[4];                              // find_bin: owning thread, entries above its bins, entries in its bins
+  uint64_t thr;                                   // the k-th largest composite, when one thread finds it
 };
 
 // Register e of thread t holds token (e / 4) * (256 W) + 4 t + e % 4: 16-byte loads, consecutive across threads.
@@ -159,19 +160,20 @@ __device__ __forceinline__ bool ws_pass(const uint32_t (&rel)[EPT], int tid, WsS
   return cnt == need;
 }
 
-// Exclusive prefix of `mine` over the threads of the workgroup, and the total (slot: one of the per-wave arrays;
-// two calls in a row must use different slots).  Contains one barrier: every thread must call it.
+// Exclusive prefix of `mine` over the threads of the workgroup, and the total.  Two barriers (the first one lets
+// the per-wave slots be reused right after an earlier call): every thread must call it.
 template <int W>
-__device__ __forceinline__ uint32_t ws_exclusive(uint32_t mine, int tid, uint32_t* slot, uint32_t* total = nullptr) {
+__device__ __forceinline__ uint32_t ws_exclusive(uint32_t mine, int tid, WsShared<W>& sh, uint32_t* total = nullptr) {
   const int lane = tid & 63, wave = tid >> 6;
   const uint32_t inc = wave_inclusive_scan(mine);
   uint32_t pos = inc - mine;
-  if (lane == 63) slot[wave] = inc;
+  __syncthreads();
+  if (lane == 63) sh.wave_a[wave] = inc;
   __syncthreads();
   uint32_t all = 0;
 #pragma unroll
   for (int w = 0; w < W; ++w) {
-    const uint32_t s = slot[w];
+    const uint32_t s = sh.wave_a[w];
     pos += w < wave ? s : 0u;
     all += s;
   }
@@ -179,12 +181,18 @@ __device__ __forceinline__ uint32_t ws_exclusive(uint32_t mine, int tid, uint32_
   return pos;
 }
 
+// Order-preserving composite of an entry: (relative key << 32) | ~token.  Larger = earlier in the order
+// (key descending, token ascending); all composites of a segment are distinct.
+__device__ __forceinline__ uint64_t ws_composite(uint32_t rel, uint32_t not_token) { return ((uint64_t)rel << 32) | not_token; }
+
 // The entries whose key equals the threshold key, when more of them exist than are still needed: the `need`
 // with the lowest tokens are in.  Token order is (register group of four, thread, register in the group), so a
-// scan over the threads per group of four registers ranks them.  Returns the thread's mask of selected equals.
+// scan over the threads per group of four registers ranks them; the thread that holds the need-th publishes its
+// composite, which is the k-th largest of the segment, in sh.thr.
 template <int W, int EPT>
-__device__ __forceinline__ uint32_t ws_rank_equals(const uint32_t (&rel)[EPT], int tid, WsShared<W>& sh, uint32_t thr, uint32_t need) {
-  uint32_t sel_mask = 0, before = 0;
+__device__ __forceinline__ void ws_rank_equals(const uint32_t (&rel)[EPT], int tid, WsShared<W>& sh, uint32_t thr, uint32_t need) {
+  const uint32_t not_t0 = ~(uint32_t)(4 * tid);
+  uint32_t before = 0;
 #pragma unroll
   for (int c = 0; c < EPT / 4; ++c) {
     uint32_t eq[4], mine = 0;
@@ -194,28 +202,28 @@ __device__ __forceinline__ uint32_t ws_rank_equals(const uint32_t (&rel)[EPT], i
       mine += eq[r];
     }
     uint32_t total;
-    uint32_t rank = before + ws_exclusive<W>(mine, tid, (c & 1) ? sh.wave_b : sh.wave_a, &total);
+    uint32_t rank = before + ws_exclusive<W>(mine, tid, sh, &total);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      if (eq[r] && rank < need) sel_mask |= 1u << (4 * c + r);
+      if (eq[r] && rank == need - 1u) sh.thr = ws_composite(thr, not_t0 - ws_token_base(4 * c + r, W));
       rank += eq[r];
     }
     before += total;
   }
-  return sel_mask;
 }
 
-// How many of the thread's entries satisfy PRED(relative key, register index).
-template <int EPT, typename PRED>
-__device__ __forceinline__ uint32_t ws_count(const uint32_t (&rel)[EPT], PRED pred) {
+// How many of the thread's entries satisfy PRED(relative key, ~token).
+template <int W, int EPT, typename PRED>
+__device__ __forceinline__ uint32_t ws_count(const uint32_t (&rel)[EPT], int tid, PRED pred) {
+  const uint32_t not_t0 = ~(uint32_t)(4 * tid);
   uint32_t count[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int e = 0; e < EPT; ++e) count[e & 3] += pred(rel[e], e) ? 1u : 0u;
+  for (int e = 0; e < EPT; ++e) count[e & 3] += pred(rel[e], not_t0 - ws_token_base(e, W)) ? 1u : 0u;
   return (count[0] + count[1]) + (count[2] + count[3]);
 }
 
-// Stores the thread's entries that satisfy PRED to dst[pos ...] as order-preserving composites (rel << 32) | ~token.
-// Straight-line: the thread stores all its entries, the ones that do not qualify into its own trash slot.
+// Stores the thread's entries that satisfy PRED to dst[pos ...] as composites.  Straight-line: the thread stores
+// all its entries, the ones that do not qualify into its own trash slot.
 template <int W, int EPT, typename PRED>
 __device__ __forceinline__ void ws_scatter(const uint32_t (&rel)[EPT], int tid, uint64_t* dst, uint32_t pos, uint64_t* trash, PRED pred) {
   const uint32_t not_t0 = ~(uint32_t)(4 * tid);
@@ -223,9 +231,9 @@ __device__ __forceinline__ void ws_scatter(const uint32_t (&rel)[EPT], int tid, 
 #pragma unroll
   for (int e = 0; e < EPT; ++e) {
     const uint32_t not_t = not_t0 - ws_token_base(e, W);   // ~token
-    const bool take = pred(rel[e], e);
+    const bool take = pred(rel[e], not_t);
     uint64_t* at = take ? dst + pos : own;
-    *at = ((uint64_t)rel[e] << 32) | not_t;
+    *at = ws_composite(rel[e], not_t);
     pos += take ? 1u : 0u;
   }
 }
@@ -312,46 +320,27 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
   }
   __syncthreads();
 
-  // The k-th largest entry in the order (key, lower token first).  One pass is enough when the bucket of the
-  // k-th is taken whole, or holds at most 64 entries: those are ranked directly, one per lane.  Otherwise
-  // further passes fix the threshold key, and a scan the equals that are in.
+  // The k-th largest composite T in the order (key, lower token first): selected are the entries >= T.  One pass
+  // is enough when the bucket of the k-th is taken whole, or holds at most 64 entries: those are ranked
+  // directly, one per lane.  Otherwise further passes fix the threshold key, and a scan ranks its equals.
   uint32_t d, above, cnt;
   ws_find_bin<W>(sh, k, tid, d, above, cnt);
   uint32_t need = k - above;
   uint64_t* sh_sort = (uint64_t*)sh.bins;
-  // compaction of the entries that satisfy `pred` into dst (in the histogram's space: behind a barrier)
-  auto compact = [&](uint64_t* dst, uint32_t* slot, auto pred) {
-    const uint32_t mine = ws_count<EPT>(rel, pred);
-    __syncthreads();
-    const uint32_t pos = ws_exclusive<W>(mine, tid, slot);
+  // compaction of the entries that satisfy `pred` into dst
+  auto compact = [&](uint64_t* dst, auto pred) {
+    const uint32_t mine = ws_count<W, EPT>(rel, tid, pred);
+    const uint32_t pos = ws_exclusive<W>(mine, tid, sh);     // (its barriers: every wave has read the histogram)
     ws_scatter<W, EPT>(rel, tid, dst, pos, sh.trash, pred);
   };
-  const bool rank_bucket = cnt != need && cnt <= (uint32_t)kWave;
+  uint64_t thr_c;
   if (cnt == need) {
-    compact(sh_sort, sh.wave_a, [d](uint32_t r, int) { return (r >> 21) >= d; });
-  } else if (rank_bucket) {
-    compact(sh_sort, sh.wave_a, [d](uint32_t r, int) { return (r >> 21) > d; });
-    compact(sh.cand, sh.wave_b, [d](uint32_t r, int) { return (r >> 21) == d; });
-  } else {
-    uint32_t thr = d << 21;
-    bool whole = false;     // the bucket of the threshold is taken whole
-    if (bits > 11) whole = ws_pass<1, W, EPT>(rel, tid, sh, thr, need);      // (bits <= 11: that digit is 0 everywhere)
-    if (!whole && bits > 22) whole = ws_pass<2, W, EPT>(rel, tid, sh, thr, need);
-    if (whole) {
-      compact(sh_sort, sh.wave_a, [thr](uint32_t r, int) { return r >= thr; });
-    } else {
-      // `thr` is now a full key shared by more entries than the `need` still to be taken
-      __syncthreads();                                             // (the per-wave slots of the last pass have been read)
-      const uint32_t eq_sel = ws_rank_equals<W, EPT>(rel, tid, sh, thr, need);
-      compact(sh_sort, (EPT / 4) & 1 ? sh.wave_b : sh.wave_a, [thr, eq_sel](uint32_t r, int e) { return r > thr || ((eq_sel >> e) & 1u); });
-    }
-  }
-  for (uint32_t r = k + tid; r < (uint32_t)kpad; r += T) sh_sort[r] = 0ull;
-  __syncthreads();
-  if (rank_bucket) {
-    // `cnt` entries of the threshold bucket, one per lane of the first wave: an entry beaten by fewer than
-    // `need` others is in
+    thr_c = ws_composite(d << 21, 0u);
+  } else if (cnt <= (uint32_t)kWave) {
+    compact(sh.cand, [d](uint32_t r, uint32_t) { return (r >> 21) == d; });
+    __syncthreads();
     if (wave == 0) {
+      // the bucket's entries, one per lane: the one beaten by exactly need - 1 others is the k-th largest
       const uint64_t c = lane < (int)cnt ? sh.cand[lane] : 0ull;
       uint32_t rank = 0;
       for (uint32_t j = 0; j < cnt; ++j) {
@@ -359,42 +348,98 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
         const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(c >> 32), (int)j);
         rank += (((uint64_t)hi << 32) | lo) > c ? 1u : 0u;
       }
-      if (lane < (int)cnt && rank < need) sh_sort[above + rank] = c;
+      if (lane < (int)cnt && rank == need - 1u) sh.thr = c;
     }
     __syncthreads();
-  }
-
-  if (!p.unordered) {
-    if (ws_max_k(W) >= 2048 && kpad == 2048) {
-      ws_sort<ws_max_k(W) >= 2048 ? 2048 : 1024, W>(sh_sort, tid);
+    thr_c = sh.thr;
+  } else {
+    uint32_t thr = d << 21;
+    bool whole = false;     // the bucket of the threshold is taken whole
+    if (bits > 11) whole = ws_pass<1, W, EPT>(rel, tid, sh, thr, need);      // (bits <= 11: that digit is 0 everywhere)
+    if (!whole && bits > 22) whole = ws_pass<2, W, EPT>(rel, tid, sh, thr, need);
+    if (whole) {
+      thr_c = ws_composite(thr, 0u);
     } else {
-      switch (kpad) {
-        case 1024: ws_sort<1024, W>(sh_sort, tid); break;
-        case 512: ws_sort<512, W>(sh_sort, tid); break;
-        case 256: ws_sort<256, W>(sh_sort, tid); break;
-        case 128: ws_sort<128, W>(sh_sort, tid); break;
-        default: ws_sort<64, W>(sh_sort, tid); break;
+      // `thr` is now a full key shared by more entries than the `need` still to be taken
+      ws_rank_equals<W, EPT>(rel, tid, sh, thr, need);
+      __syncthreads();
+      thr_c = sh.thr;
+    }
+  }
+  const uint32_t thr_hi = (uint32_t)(thr_c >> 32), thr_lo = (uint32_t)thr_c;
+  auto selected = [thr_hi, thr_lo](uint32_t r, uint32_t not_t) { return r > thr_hi || (r == thr_hi && not_t >= thr_lo); };
+
+  if (p.out_idx) {
+    compact(sh_sort, selected);
+    for (uint32_t r = k + tid; r < (uint32_t)kpad; r += T) sh_sort[r] = 0ull;
+    __syncthreads();
+    if (!p.unordered) {
+      if (ws_max_k(W) >= 2048 && kpad == 2048) {
+        ws_sort<ws_max_k(W) >= 2048 ? 2048 : 1024, W>(sh_sort, tid);
+      } else {
+        switch (kpad) {
+          case 1024: ws_sort<1024, W>(sh_sort, tid); break;
+          case 512: ws_sort<512, W>(sh_sort, tid); break;
+          case 256: ws_sort<256, W>(sh_sort, tid); break;
+          case 128: ws_sort<128, W>(sh_sort, tid); break;
+          default: ws_sort<64, W>(sh_sort, tid); break;
+        }
+      }
+      __syncthreads();
+    }
+    // out; the composites carry relative keys: key = (rel >> lshift) + kmin
+    const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
+                                             : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
+    int32_t* oi = p.out_idx + (int64_t)seg * p.out_stride;
+    float* ov = p.out_val ? p.out_val + (int64_t)seg * p.out_stride : nullptr;
+    for (uint32_t r = tid; r < k; r += T) {
+      const uint64_t c = sh_sort[r];
+      oi[r] = (int32_t)(~(uint32_t)c + idx_base);
+      if (ov) ov[r] = key_score(((uint32_t)(c >> 32) >> lshift) + kmin);
+    }
+    if (p.out_expand) {
+      int32_t* oe = p.out_expand + (int64_t)seg * p.k * p.expand;
+      const uint32_t total = k * (uint32_t)p.expand;
+      for (uint32_t e = tid; e < total; e += T) {
+        const uint32_t jj = e / (uint32_t)p.expand, ii = e % (uint32_t)p.expand;
+        oe[e] = (int32_t)(~(uint32_t)sh_sort[jj] * (uint32_t)p.expand + ii);
       }
     }
-    __syncthreads();
   }
-  // out; the composites carry relative keys: key = (rel >> lshift) + kmin
-  const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
-                                           : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
-  int32_t* oi = p.out_idx + (int64_t)seg * p.out_stride;
-  float* ov = p.out_val ? p.out_val + (int64_t)seg * p.out_stride : nullptr;
-  for (uint32_t r = tid; r < k; r += T) {
-    const uint64_t c = sh_sort[r];
-    oi[r] = (int32_t)(~(uint32_t)c + idx_base);
-    if (ov) ov[r] = key_score(((uint32_t)(c >> 32) >> lshift) + kmin);
-  }
-  if (p.out_expand) {
-    int32_t* oe = p.out_expand + (int64_t)seg * p.k * p.expand;
-    const uint32_t total = k * (uint32_t)p.expand;
-    for (uint32_t e = tid; e < total; e += T) {
-      const uint32_t jj = e / (uint32_t)p.expand, ii = e % (uint32_t)p.expand;
-      oe[e] = (int32_t)(~(uint32_t)sh_sort[jj] * (uint32_t)p.expand + ii);
+
+  if (p.union_idx) {
+    // ascending union with the sink range [0, lo) and the local window [hi, n): the selected tokens between them,
+    // in token order (register group, thread, register), then the two ranges, -1 padding and the count
+    const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
+    const uint32_t hi = (uint32_t)(n - p.local > (int)lo ? n - p.local : (int)lo);
+    const int cap = p.k + p.sink + p.local;
+    int32_t* uo = p.union_idx + (int64_t)seg * cap;
+    const uint32_t not_t0 = ~(uint32_t)(4 * tid);
+    uint32_t run_mid = 0;
+#pragma unroll
+    for (int c = 0; c < EPT / 4; ++c) {
+      uint32_t mid[4], mine = 0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const uint32_t not_t = not_t0 - ws_token_base(4 * c + r, W);
+        const uint32_t t = ~not_t;
+        mid[r] = selected(rel[4 * c + r], not_t) && t >= lo && t < hi ? 1u : 0u;
+        mine += mid[r];
+      }
+      uint32_t total;
+      uint32_t at = lo + run_mid + ws_exclusive<W>(mine, tid, sh, &total);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (mid[r]) uo[at++] = (int32_t)(c * (4 * T) + 4 * tid + r);
+      }
+      run_mid += total;
     }
+    for (uint32_t t = tid; t < lo; t += T) uo[t] = (int32_t)t;
+    const uint32_t mid_end = lo + run_mid;
+    for (int t = (int)hi + tid; t < n; t += T) uo[mid_end + (uint32_t)(t - (int)hi)] = t;
+    const uint32_t count = mid_end + (uint32_t)(n - (int)hi);
+    for (int i = (int)count + tid; i < cap; i += T) uo[i] = -1;
+    if (tid == 0) p.union_count[seg] = (int32_t)count;
   }
 }
 
@@ -404,8 +449,8 @@ int select_wave_max_len() { return kWsMaxLen; }
 int select_wave_max_k(int64_t seg_len) { return seg_len > 8 * kWave * 8 ? ws_max_k(16) : ws_max_k(4); }
 
 int launch_select_wave(const SelectParams& p, hipStream_t stream) {
-  if (p.seg_len < 1 || p.seg_len > kWsMaxLen || p.k < 1 || p.k > p.seg_len || p.k > select_wave_max_k(p.seg_len) || !p.out_idx ||
-      !p.scores)
+  if (p.seg_len < 1 || p.seg_len > kWsMaxLen || p.k < 1 || p.k > p.seg_len || p.k > select_wave_max_k(p.seg_len) ||
+      (!p.out_idx && !p.union_idx) || !p.scores)
     return TKA_EINVAL;
   int kpad = kWave;
   while (kpad < p.k) kpad <<= 1;
