@@ -12,10 +12,11 @@
 //   dense      every score is stored and a first-level histogram is flushed (short segments and callers that
 //              want all scores);
 //   candidate  a threshold tau per segment comes from an order statistic of a strided sample of the segment,
-//              chosen so that about 2k tokens pass; only tokens with key >= tau are stored, in index order,
-//              in the workgroup's own slice (the count rides in the first entry: one partial line per
-//              workgroup).  The selection kernel checks that at least k tokens passed and otherwise flags
-//              the segment for the fallback kernel, so the result is exact whatever the data.
+//              chosen so that about 2k tokens pass; only tokens at or above it (key > tau, or key == tau and
+//              token <= a cut that heavy ties make finite) are stored, in index order, in the workgroup's own
+//              slice (the count rides in the first entry: one partial line per workgroup).  The selection
+//              kernel checks that at least k tokens passed and otherwise redoes the segment from the keys, so
+//              the result is exact whatever the data.
 //              The sampling runs inside the same launch: the first workgroups of the grid score the samples,
 //              the last of them to finish publishes the threshold, and the streaming workgroups need it only
 //              when their rows are scored and wait (bounded) for it then.
@@ -236,9 +237,9 @@ __device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) 
 // Sampling workgroup: scores 256 of the segment's p.num_samples sample tokens (one round of
 // loads) and stores their keys in the segment's pool.  The workgroup that arrives last (epoch-valued arrival
 // flags, so that the workspace needs no clearing) takes the p.sample_rank-th largest key of the whole pool and
-// publishes it as the segment's threshold word, (epoch << 32) | key.  The sample is spread evenly over the
-// segment, so about sample_rank/num_samples of the segment's tokens lie at or above that key wherever the
-// large scores sit.
+// publishes it as the segment's threshold word, (epoch << 32) | key (and, in front of it, the token cut among
+// the keys equal to it).  The sample is spread evenly over the segment, so about sample_rank/num_samples of the
+// segment's tokens lie at or above that threshold wherever the large scores sit.
 // Ordering between workgroups: the keys are agent-scope atomic stores, their completion and a barrier precede
 // the workgroup's arrival flag; the last workgroup reads the pool with agent-scope atomic loads after it has
 // seen every flag.
@@ -246,7 +247,7 @@ __device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) 
 template <int DT>
 __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int part, uint32_t* sh) {
   uint32_t* sh_hist = sh;                   // 2048 bins
-  uint32_t* sh_wtot = sh_hist + kHistBins;  // 8 wave totals, then [8] bin, [9] count above it, [10] "last" flag
+  uint32_t* sh_wtot = sh_hist + kHistBins;  // 8 wave totals, then [8] bin, [9] count above it, [10] "last" flag, [11] count in the bin, [12..14] tie scan
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int j = tid & 15, rg = tid >> 4;
@@ -305,9 +306,9 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
     const int i = u * kCandThreads + tid;
     keys[u] = i < p.num_samples ? __hip_atomic_load(pool + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
   }
-  uint32_t need = (uint32_t)p.sample_rank, prefix = 0;
-  for (int pass = 0; pass < 2; ++pass) {
-    const int shift = pass ? 32 - 2 * kHistBits : 32 - kHistBits;
+  // One radix pass over the pooled keys: histogram of digit (key >> shift) & mask among the keys whose bits above the
+  // digit equal `match`; finds the bin of the need-th largest.  sh_wtot[8] = bin, [9] = keys above it, [11] = keys in it.
+  auto radix_pass = [&](int shift, uint32_t mask, int match_shift, uint32_t match, uint32_t need) {
     __syncthreads();
 #pragma unroll
     for (int e = 0; e < kBinsPerThread; ++e) sh_hist[kBinsPerThread * tid + e] = 0;
@@ -315,8 +316,8 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
 #pragma unroll
     for (int u = 0; u < kPerThread; ++u) {
       const uint32_t key = keys[u];
-      if (u * kCandThreads + tid < p.num_samples && (pass == 0 || (key >> (32 - kHistBits)) == prefix))
-        atomicAdd(&sh_hist[(key >> shift) & (kHistBins - 1)], 1u);
+      if (u * kCandThreads + tid < p.num_samples && (match_shift >= 32 || (key >> match_shift) == match))
+        atomicAdd(&sh_hist[(key >> shift) & mask], 1u);
     }
     __syncthreads();
     uint32_t h[kBinsPerThread], mine = 0;
@@ -337,22 +338,80 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
     if (ge >= need && ge - mine < need) {   // the bin sits among this thread's four: walk them from the top
       uint32_t above = ge - mine;
       int bin = 0;
+      uint32_t in_bin = 0;
       bool found = false;
 #pragma unroll
       for (int e = kBinsPerThread - 1; e >= 0; --e) {
-        if (!found && above + h[e] >= need) { bin = kBinsPerThread * tid + e; found = true; }
+        if (!found && above + h[e] >= need) { bin = kBinsPerThread * tid + e; in_bin = h[e]; found = true; }
         if (!found) above += h[e];
       }
       sh_wtot[8] = (uint32_t)bin;
       sh_wtot[9] = above;
+      sh_wtot[11] = in_bin;
     }
     __syncthreads();
-    prefix = (prefix << kHistBits) | sh_wtot[8];
+  };
+  uint32_t need = (uint32_t)p.sample_rank;
+  radix_pass(32 - kHistBits, kHistBins - 1, 32, 0u, need);
+  uint32_t prefix = sh_wtot[8];
+  need -= sh_wtot[9];
+  radix_pass(32 - 2 * kHistBits, kHistBins - 1, 32 - kHistBits, prefix, need);
+  prefix = (prefix << kHistBits) | sh_wtot[8];
+  need -= sh_wtot[9];
+  uint32_t tau = prefix << (32 - 2 * kHistBits);
+  uint32_t cut = 0x7fffffffu;                 // tokens of the threshold key that pass: all
+  // The threshold so far admits every key that shares the 22 leading bits of the order statistic.  When many
+  // samples do (heavy ties: quantised or constant scores), that is far more tokens than planned, so the order
+  // statistic is taken in the full order instead: the key to its last bit, and among the samples that hold that
+  // key the need-th in token order, whose token becomes the cut.  The candidates (key > tau, or key == tau and
+  // token <= cut) are still an upper set of the order (score descending, token ascending): if at least k pass
+  // they contain the top k, whatever the data, and their number again concentrates around n R / S.
+  constexpr uint32_t kTieSlack = 4;           // samples at the threshold beyond the need-th that are let pass as they are
+  if (sh_wtot[11] - need > kTieSlack) {
+    radix_pass(0, (1u << (32 - 2 * kHistBits)) - 1u, 32 - 2 * kHistBits, prefix, need);
+    tau |= sh_wtot[8];
     need -= sh_wtot[9];
+    if (sh_wtot[11] - need > kTieSlack) {
+      // samples with key == tau in sample order (u, thread): counts per (u, wave), one scan, the need-th one
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < kPerThread; ++u) {
+        const bool eq = u * kCandThreads + tid < p.num_samples && keys[u] == tau;
+        const unsigned long long m = __ballot(eq);
+        if (lane == 0) sh_hist[u * kCandWaves + wave] = (uint32_t)__popcll(m);
+      }
+      __syncthreads();
+      if (wave == 0) {
+        constexpr int kCells = kPerThread * kCandWaves;   // 128: two per lane, in order
+        const uint32_t c0 = sh_hist[2 * lane], c1 = sh_hist[2 * lane + 1];
+        const uint32_t inc = wave_inclusive_scan(c0 + c1);
+        const uint32_t before0 = inc - (c0 + c1), before1 = before0 + c0;
+        static_assert(kCells == 2 * kWave, "two cells per lane");
+        if (before0 < need && need <= before0 + c0) { sh_wtot[12] = 2 * lane; sh_wtot[13] = need - before0; }
+        if (before1 < need && need <= before1 + c1) { sh_wtot[12] = 2 * lane + 1; sh_wtot[13] = need - before1; }
+      }
+      __syncthreads();
+      const int cell = (int)sh_wtot[12];
+      const uint32_t nth = sh_wtot[13];              // 1-based position inside the cell's wave
+#pragma unroll
+      for (int u = 0; u < kPerThread; ++u) {
+        if (u == cell / kCandWaves && wave == cell % kCandWaves) {
+          const bool eq = u * kCandThreads + tid < p.num_samples && keys[u] == tau;
+          const unsigned long long m = __ballot(eq);
+          const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+          if (eq && rank + 1u == nth) sh_wtot[14] = (uint32_t)sample_token(seg, u * kCandThreads + tid, stride);
+        }
+      }
+      __syncthreads();
+      cut = sh_wtot[14];
+    }
   }
-  prefix <<= 32 - 2 * kHistBits;
-  if (tid == 0)
-    __hip_atomic_store(p.tau_words + seg, ((uint64_t)p.epoch << 32) | prefix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0) {
+    // the cut first, then, once it has completed, the word the streaming workgroups wait for
+    __hip_atomic_store(p.tau_words + 2 * seg + 1, (uint64_t)cut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __hip_atomic_store(p.tau_words + 2 * seg, ((uint64_t)p.epoch << 32) | tau, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 // Scores of one slice (up to 512 tokens from sbase on) as keys into LDS: lane j < 8 of row group rg writes the
@@ -408,7 +467,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
   }
   uint32_t* sh_key = sh;                               // keys of this workgroup's tokens, slice after slice
   uint32_t* sh_wcnt = sh + kEarlySlices * kCandThreads; // candidates per wave
-  __shared__ uint32_t sh_tau[2];                        // the segment's threshold and whether it has arrived
+  __shared__ uint32_t sh_tau[3];                        // the segment's threshold key, whether it has arrived, its token cut
 
   const int j = tid & 15;            // lane inside the row: dims 8j..8j+7
   const int rg = tid >> 4;           // row group 0..15 inside the workgroup
@@ -446,7 +505,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
   }
   __syncthreads();
 
-  uint32_t tau = 0;
+  uint32_t tau = 0, cut = 0;
   bool tau_ready = false;
   int64_t tau_seg = first_seg, seg = first_seg;
   int wg_in_chunk = first_wg;
@@ -461,7 +520,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
       tau_seg = seg;
       if (s) __syncthreads();   // the previous slice's threshold has been read
       if (tid == 0) {
-        const uint64_t* word = p.tau_words + seg;
+        const uint64_t* word = p.tau_words + 2 * seg;
         uint64_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         for (int spin = 0; (uint32_t)(v >> 32) != p.epoch && spin < kTauSpinLimit; ++spin) {
           __builtin_amdgcn_s_sleep(16);
@@ -469,17 +528,20 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
         }
         sh_tau[0] = (uint32_t)v;
         sh_tau[1] = (uint32_t)(v >> 32) == p.epoch ? 1u : 0u;
+        sh_tau[2] = (uint32_t)__hip_atomic_load(word + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (written before the word)
       }
       __syncthreads();
       tau = sh_tau[0];
       tau_ready = sh_tau[1] != 0u;
+      cut = sh_tau[2];
     }
 
     // thread t owns token t_begin + t: candidates in index order into the slice.
     // Slice format: word = key << 32 | count << 9 | token - first token of the slice; only entry 0 carries
     // the count (0 .. 512), so a workgroup with few candidates writes a single line and nothing else.
     const uint32_t key = sh_key[s * kCandThreads + tid];
-    const bool pass = tau_ready && t_begin + tid < t_end && key >= tau;
+    // at or above the threshold in the order (score descending, token ascending)
+    const bool pass = tau_ready && t_begin + tid < t_end && (key > tau || (key == tau && (uint32_t)(t_begin + tid) <= cut));
     const unsigned long long mask = __ballot(pass);
     if (s) __syncthreads();   // the previous slice's counts have been read
     if (lane == 0) sh_wcnt[wave] = (uint32_t)__popcll(mask);

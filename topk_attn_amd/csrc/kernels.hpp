@@ -12,7 +12,7 @@ struct GemvParams {
   const int32_t* cluster_ids;  // [batch*num_kv_heads*num_chunks] or nullptr: chunk c covers the tokens of that cluster
   uint32_t* hist;       // [batch*num_kv_heads*num_chunks][kHistBins] or nullptr; must be zero on entry
   // candidate mode: only tokens whose key reaches the segment's sampled threshold are stored
-  uint64_t* tau_words;        // [segments] (epoch << 32) | threshold key
+  uint64_t* tau_words;        // [segments][2] (epoch << 32) | threshold key, and the token cut among keys equal to it
   uint32_t* sample_flags;     // [segments][64] epoch of the call in which that sampling workgroup last arrived
   uint32_t* sample_pool;      // [segments][num_samples] keys of the sampled tokens
   uint32_t epoch;             // tells this call's words from older contents of the workspace (never 0)
@@ -41,7 +41,7 @@ struct SelectParams {
   int64_t seg_len;
   int64_t seg_stride;
   uint32_t* hist;         // [num_segments][kHistBins]; nullptr: the lists hold candidates above a sampled threshold
-  uint64_t* tau_words;    // [num_segments] candidate thresholds (workspace); the candidate selection kernel clears them
+  uint64_t* tau_words;    // [num_segments][2] candidate thresholds (workspace); the candidate selection kernel clears them
   uint32_t* sample_flags; // [num_segments][64] arrival flags of the sampling workgroups (workspace)
   uint32_t* sample_pool;  // [num_segments][kGemvMaxSamples] sampled keys (workspace)
   uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment was redone from the keys

@@ -756,7 +756,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     // the threshold and the arrival flags are spent: a replay of the same launches (a captured graph) must not
     // take them for its own
     if (tid >= 64 && tid < 128) p.sample_flags[(int64_t)seg * 64 + (tid - 64)] = 0u;
-    if (tid == 0) p.tau_words[seg] = 0ull;
+    if (tid == 0) p.tau_words[2 * seg] = 0ull;
   }
   if (redo) {
     __syncthreads();
@@ -992,7 +992,7 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   l.list_stride = (seg_len + 16 * kSelThreads - 1) / (16 * kSelThreads) * (16 * kSelThreads);  // whole slices
   l.hist = take((size_t)num_segments * kHistBins * sizeof(uint32_t));
   l.flags = take((size_t)num_segments * sizeof(uint32_t));
-  l.tau = take((size_t)num_segments * sizeof(uint64_t));
+  l.tau = take((size_t)num_segments * 2 * sizeof(uint64_t));
   const size_t cand_segs = seg_len >= kCandMinSegLen ? (size_t)num_segments : 0;   // sampling state: long segments only
   l.ctr = take(cand_segs * 64 * sizeof(uint32_t));
   l.pool = take(cand_segs * kGemvMaxSamples * sizeof(uint32_t));
