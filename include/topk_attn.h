@@ -101,6 +101,13 @@ int tka_gemv_topk(const tka_gemv_topk_args* args);
  * Counterpart of gemv_phase_kernel, gemv_profile_split.cu:69-252. */
 int tka_gemv_scores(const tka_gemv_topk_args* args);
 
+/* Diagnostic (no counterpart in the reference): after a tka_gemv_topk call with the same arguments, *count =
+ * how many of its segments were redone from the keys by the selection kernel (segments of 65536 tokens and more
+ * are selected from candidates above a sampled threshold; a segment whose candidates turn out fewer than k, or
+ * more than fit, is redone - exact, but about a millisecond per 131072 tokens).  0 for calls that do not take
+ * that path.  Waits for the stream. */
+int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* args, int32_t* count);
+
 /* ------------------------------------------------------------------------------------------------
  * Stage 1b — selection phase alone on caller-supplied fp32 scores.
  * Counterpart of the sort-only kernel of gemv_profile_split.cu:255-323 and of every

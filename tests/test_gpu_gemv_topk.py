@@ -179,11 +179,14 @@ def _sampled_positions(seg, n, samples=2048):
     return [i * stride + _mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) % stride for i in range(samples)]
 
 
-def _check_long(K, q, dtype, G, k, scale=SCALE):
+def _check_long(K, q, dtype, G, k, scale=SCALE, redone=None):
+    """`redone`: how many segments the selection kernel is expected to redo from the keys (None: not checked)."""
     from topk_attn_amd import ops
-    idx, val = ops.gemv_topk(to_dev(q, dtype), to_dev(K, dtype), k, group=G, scale=scale)
+    plan = ops.GemvTopkPlan(to_dev(q, dtype), to_dev(K, dtype), k, group=G, scale=scale).run()
     torch.cuda.synchronize()
-    idx, val = idx.cpu().numpy(), val.cpu().numpy()
+    if redone is not None:
+        assert plan.redone_segments() == redone
+    idx, val = plan.idx.cpu().numpy(), plan.val.cpu().numpy()
     B, N, H = K.shape[:3]
     for b in range(B):
         for h in range(H):
@@ -198,15 +201,15 @@ def test_long_segment_candidates():
     rng = np.random.default_rng(31)
     K = randn_bits(rng, (1, 131072, 2, 128), oracle.F16)
     K[0, rng.permutation(131072)[:1300]] = oracle.to_bits(rng.standard_normal((1300, 2, 128)) * 4.0, oracle.F16)
-    _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 2048)
+    _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 2048, redone=0)
 
 
-def test_long_segment_all_equal_falls_back():
-    """Every key equal: every token passes the sampled threshold, the segment is redone from the keys."""
-    announce("gemv_topk long segment all keys equal (fallback: too many candidates)")
+def test_long_segment_all_equal():
+    """Every key equal: the sampled threshold is a (key, token) pair, so only the first tokens pass."""
+    announce("gemv_topk long segment all keys equal")
     rng = np.random.default_rng(32)
     K = np.broadcast_to(randn_bits(rng, (1, 1, 1, 128), oracle.BF16), (1, 70001, 2, 128)).copy()
-    _check_long(K, randn_bits(rng, (1, 2, 128), oracle.BF16), oracle.BF16, 1, 1000)
+    _check_long(K, randn_bits(rng, (1, 2, 128), oracle.BF16), oracle.BF16, 1, 1000, redone=0)
 
 
 def test_long_segment_sample_hits_only_heavy_tokens_falls_back():
@@ -227,6 +230,34 @@ def test_long_segment_bf16_levels_group8():
     rng = np.random.default_rng(34)
     K = oracle.to_bits(np.linspace(-2, 2, 16)[rng.integers(0, 16, (1, 262144, 1, 128))], oracle.BF16)
     _check_long(K, randn_bits(rng, (1, 8, 128), oracle.BF16), oracle.BF16, 8, 4096)
+
+
+@pytest.mark.parametrize("layout", ["spread", "tail", "head", "two_buckets"])
+def test_long_segment_heavy_ties(layout):
+    """Scores that take three values on a long segment, with the k-th largest inside a bucket of tens of
+    thousands of equal scores (a unit query makes the score one key column): the sampled threshold must cut the
+    bucket by token, wherever its tokens sit, and the result must be the lowest tokens of the bucket."""
+    announce("gemv_topk long segment heavy ties (%s)" % layout)
+    rng = np.random.default_rng(37)
+    dtype, N, k = oracle.F16, 131072, 2048
+    col = np.full(N, -1.0)
+    if layout == "spread":
+        col[rng.permutation(N)[:60000]] = 0.5
+    elif layout == "tail":
+        col[N - 60000:] = 0.5
+    elif layout == "head":
+        col[:60000] = 0.5
+    else:
+        col[rng.permutation(N)[:40000]] = 0.5                 # the bucket of the k-th
+        col[rng.permutation(N)[:30000]] = 0.25                # a second large bucket right below (and over part of it)
+    top = rng.permutation(N)[:1000]
+    col[top] = 2.0 + rng.random(1000)                         # 1000 distinct scores above the bucket
+    Kf = rng.standard_normal((1, N, 2, 128)) * 0.01
+    Kf[0, :, 0, 0] = col
+    Kf[0, :, 1, 0] = col[::-1]                                # second head: the mirrored layout
+    qv = np.zeros((1, 2, 128))
+    qv[0, :, 0] = 1.0
+    _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qv, dtype), dtype, 1, k, scale=1.0, redone=0)
 
 
 def test_long_segment_chunked_shared_kv():
@@ -309,4 +340,4 @@ def test_long_segment_forced_redo(monkeypatch):
     rng = np.random.default_rng(39)
     K = randn_bits(rng, (1, 70001, 2, 128), oracle.F16)
     K[0, rng.permutation(70001)[:700]] = oracle.to_bits(rng.standard_normal((700, 2, 128)) * 4.0, oracle.F16)
-    _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 3000)
+    _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 3000, redone=2)

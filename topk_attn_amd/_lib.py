@@ -87,6 +87,7 @@ PROTOTYPES = {
     "tka_gemv_topk_workspace_bytes": (_sz, [C.POINTER(GemvTopkArgs)]),
     "tka_gemv_topk": (C.c_int, [C.POINTER(GemvTopkArgs)]),
     "tka_gemv_scores": (C.c_int, [C.POINTER(GemvTopkArgs)]),
+    "tka_gemv_topk_redone_segments": (C.c_int, [C.POINTER(GemvTopkArgs), C.POINTER(C.c_int32)]),
     "tka_topk_workspace_bytes": (_sz, [C.POINTER(TopkArgs)]),
     "tka_topk_f32": (C.c_int, [C.POINTER(TopkArgs)]),
     "tka_center_topk_expand_workspace_bytes": (_sz, [C.POINTER(CenterTopkArgs)]),

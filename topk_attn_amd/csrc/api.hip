@@ -149,6 +149,17 @@ int wave_select_min_segments() {
 }
 bool wave_select_fits(int64_t seg_len, int k) { return seg_len <= select_wave_max_len() && k <= select_wave_max_k(seg_len); }
 
+// Samples per segment and rank of the threshold statistic when the call takes the candidate route (long segments,
+// k a small share of them), else 0.
+void candidate_plan(const tka_gemv_topk_args* a, int* num_samples, int* sample_rank) {
+  *num_samples = *sample_rank = 0;
+  const int64_t chunk_len = a->seq_len / a->num_chunks;
+  const int64_t cand_slices = (chunk_len + kGemvCandTokensPerWg - 1) / kGemvCandTokensPerWg;
+  // (the candidate kernel addresses the rows of a slice with 32-bit byte offsets)
+  if (!a->out_scores && cand_slices <= select_cand_max_parts() && a->key_stride_n < (int64_t)1 << 21)
+    gemv_candidate_plan(chunk_len, a->k, select_cand_capacity(), num_samples, sample_rank);
+}
+
 struct UnionOut {
   int32_t* idx;
   int32_t* count;
@@ -228,9 +239,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
 
   int num_samples = 0, sample_rank = 0;
   const int64_t cand_slices = (chunk_len + kGemvCandTokensPerWg - 1) / kGemvCandTokensPerWg;
-  // (the candidate kernel addresses the rows of a slice with 32-bit byte offsets)
-  if (!a->out_scores && cand_slices <= select_cand_max_parts() && a->key_stride_n < (int64_t)1 << 21)
-    gemv_candidate_plan(chunk_len, a->k, select_cand_capacity(), &num_samples, &sample_rank);
+  candidate_plan(a, &num_samples, &sample_rank);
   if (num_samples == 0) {
     // dense: clear histograms, GEMV with histogram, filter, finalize
     int rc = launch_zero_u32(sp.hist, zero_words, stream);
@@ -416,6 +425,26 @@ int tka_gemv_topk(const tka_gemv_topk_args* a) {
   if (rc != TKA_OK) return rc;
   if (!a->workspace || a->workspace_bytes < tka_gemv_topk_workspace_bytes(a)) return TKA_EWORKSPACE;
   return run_gemv_topk(a, nullptr, 0);
+}
+
+int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* a, int32_t* count) {
+  if (!count) return TKA_EINVAL;
+  *count = 0;
+  int rc = check_gemv(a, true);
+  if (rc != TKA_OK) return rc;
+  if (!a->workspace || a->workspace_bytes < tka_gemv_topk_workspace_bytes(a)) return TKA_EWORKSPACE;
+  int num_samples = 0, sample_rank = 0;
+  candidate_plan(a, &num_samples, &sample_rank);
+  if (num_samples == 0) return TKA_OK;
+  const int segs = a->batch * a->num_kv_heads * a->num_chunks;
+  SelectParams sp;
+  memset(&sp, 0, sizeof sp);
+  select_carve((unsigned char*)a->workspace + gemv_scores_bytes(a), segs, a->seq_len / a->num_chunks, &sp);
+  std::vector<uint32_t> flags((size_t)segs);
+  if (hipStreamSynchronize((hipStream_t)a->stream) != hipSuccess) return TKA_EHIP;
+  if (hipMemcpy(flags.data(), sp.seg_flags, flags.size() * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return TKA_EHIP;
+  for (uint32_t f : flags) *count += f ? 1 : 0;
+  return TKA_OK;
 }
 
 int tka_gemv_scores(const tka_gemv_topk_args* a) {

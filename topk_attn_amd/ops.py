@@ -93,6 +93,12 @@ class GemvTopkPlan:
         L.check(self._fn(C.byref(self.args)), "tka_gemv_topk")
         return self
 
+    def redone_segments(self):
+        """Diagnostic: segments of the last run() that the selection kernel had to redo from the keys."""
+        n = C.c_int32(0)
+        L.check(L.lib().tka_gemv_topk_redone_segments(C.byref(self.args), C.byref(n)), "tka_gemv_topk_redone_segments")
+        return n.value
+
 
 def gemv_topk(q, keys, k, group=1, scale=1.0, num_chunks=1, return_scores=False):
     """Fused GEMV + top-k.  Returns (idx int32 [B,Hkv,num_chunks*k], val fp32 same shape[, scores fp32 [B,Hkv,N]])."""
