@@ -204,6 +204,15 @@ def test_long_segment_candidates():
     _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 2048, redone=0)
 
 
+def test_mid_segments_large_call_candidates():
+    """Segments between 32768 and 65536 tokens take the sampled-threshold path when the call is large (a million
+    rows): 4 x 8 segments of 40000 tokens, ragged slices, none redone."""
+    announce("gemv_topk mid segments B=4 H=8 N=40000 k=1500 (candidate lists)")
+    rng = np.random.default_rng(41)
+    K = randn_bits(rng, (4, 40000, 8, 128), oracle.F16)
+    _check_long(K, randn_bits(rng, (4, 8, 128), oracle.F16), oracle.F16, 1, 1500, redone=0)
+
+
 def test_long_segment_all_equal():
     """Every key equal: the sampled threshold is a (key, token) pair, so only the first tokens pass."""
     announce("gemv_topk long segment all keys equal")

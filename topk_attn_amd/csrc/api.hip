@@ -157,7 +157,7 @@ void candidate_plan(const tka_gemv_topk_args* a, int* num_samples, int* sample_r
   const int64_t cand_slices = (chunk_len + kGemvCandTokensPerWg - 1) / kGemvCandTokensPerWg;
   // (the candidate kernel addresses the rows of a slice with 32-bit byte offsets)
   if (!a->out_scores && cand_slices <= select_cand_max_parts() && a->key_stride_n < (int64_t)1 << 21)
-    gemv_candidate_plan(chunk_len, a->k, select_cand_capacity(), num_samples, sample_rank);
+    gemv_candidate_plan(chunk_len, (int64_t)a->batch * a->num_kv_heads * a->seq_len, a->k, select_cand_capacity(), num_samples, sample_rank);
 }
 
 struct UnionOut {
