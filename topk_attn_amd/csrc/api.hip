@@ -310,10 +310,13 @@ void flash_plan(const tka_flash_decode_args* a, int* splits, int* tokens_per_spl
     const int64_t rows = (int64_t)a->batch * a->num_kv_heads;
     want = (a->kv_idx ? 1024 : 2048) / rows;
     if (want < 1) want = 1;
-    // short lists on the VALU kernel: one workgroup per row writes the result itself, which saves the combine
-    // launch (measured on the operator: quicker up to 512 ids per row, and up to 1024 from 256 rows on)
+    // id lists on the VALU kernel: from 512 rows on (256 with up to 2048 ids per row), or up to 512 ids per row, one
+    // workgroup per row, which writes the result itself and saves the combine launch; below that about 512
+    // workgroups (measured on the operator: 16 x 32 rows of 4096 ids 54 instead of 69 us, 4 x 32 rows 24.6 instead
+    // of 25.4)
     const bool valu = a->group == 1 || a->kv_logit;
-    if (valu && a->kv_idx && (len <= 512 || (len <= 1024 && rows >= 256))) want = 1;
+    if (valu && a->kv_idx) want = (rows >= 512 || len <= 512 || (rows >= 256 && len <= 2048)) ? 1 : 512 / rows;
+    if (want < 1) want = 1;
   }
   int64_t tps = (len + want - 1) / want;
   tps = (tps + 127) / 128 * 128;
