@@ -126,6 +126,44 @@ def test_register_resident_segments(n, k):
     _check(np.stack(rows), k)
 
 
+def test_random_shapes_and_distributions():
+    """Eighty seeded (segment length, k, segment count, distribution) draws up to 16384 scores per segment, checked
+    against numpy's lexsort on the order-preserving keys (oracle.score_keys is pinned against the C oracle)."""
+    from topk_attn_amd import ops
+    announce("topk 80 random shapes and distributions")
+    rng = np.random.default_rng(2024)
+    for it in range(80):
+        n = int(rng.choice([rng.integers(1, 65), rng.integers(1, 2049), rng.integers(2049, 4097), rng.integers(4097, 16385)]))
+        kmax = min(n, 1024 if n <= 4096 else 2048)
+        k = int(rng.choice([1, kmax, rng.integers(1, kmax + 1)]))
+        S = int(rng.choice([1, 3, rng.integers(1, 300)]))
+        S = max(1, min(S, 2_000_000 // n))
+        kind = it % 6
+        if kind == 0:
+            x = rng.standard_normal((S, n))
+        elif kind == 1:
+            x = np.linspace(-2, 2, 16)[rng.integers(0, 16, (S, n))]
+        elif kind == 2:
+            x = 1.0 + rng.integers(0, 1 << int(rng.integers(1, 20)), (S, n)) * 2.0 ** -23
+        elif kind == 3:
+            x = rng.standard_normal((S, n))
+            m = rng.random((S, n))
+            x[m < 0.1], x[(m >= 0.1) & (m < 0.2)], x[(m >= 0.2) & (m < 0.22)] = 0.0, -0.0, np.inf
+            x[(m >= 0.22) & (m < 0.24)], x[(m >= 0.24) & (m < 0.3)] = -np.inf, np.nan
+        elif kind == 4:
+            x = np.round(rng.standard_normal((S, n)) * int(rng.integers(1, 6)))
+        else:
+            x = np.full((S, n), float(rng.standard_normal()))
+        x = x.astype(np.float32)
+        idx, val = ops.topk(torch.from_numpy(x).cuda(), k)
+        torch.cuda.synchronize()
+        keys = oracle.score_keys(x).astype(np.int64)
+        order = np.lexsort((np.broadcast_to(np.arange(n), x.shape), -keys), axis=1)[:, :k]
+        case = "draw %d: n=%d k=%d S=%d kind=%d" % (it, n, k, S, kind)
+        assert np.array_equal(idx.cpu().numpy(), order.astype(np.int32)), case
+        assert np.array_equal(oracle.score_keys(val.cpu().numpy()), np.take_along_axis(oracle.score_keys(x), order, axis=1)), case
+
+
 def test_short_segments_many():
     """4096 segments in one call (32 batch entries x 32 heads x 4 chunks of the operator)."""
     announce("topk short segments 4096 x 2048, k=128")
