@@ -205,21 +205,27 @@ class RetrievalOp:
     """ra: the reference's operator at its own test shape (test_ra.py:162-172: 32 heads, 8192 keys shared by the
     batch, 4 chunks of 2048, top-K per chunk), batch entries and K selectable."""
 
-    def __init__(self, torch, dev, batch=4, topk=128):
+    def __init__(self, torch, dev, batch=4, topk=128, rotate=0):
         from topk_attn_amd import retrieval_attention_cpp as ra
         g = torch.Generator(device=dev)
         g.manual_seed(6)
         self.B, self.topk = batch, topk
         self.q = (torch.randn((batch, 32, 128), generator=g, device=dev) * 0.1).half()
-        self.K = (torch.randn((8192, 32, 128), generator=g, device=dev) * 0.1).half()
-        self.V = (torch.randn((8192, 32, 128), generator=g, device=dev) * 0.1).half()
+        K = (torch.randn((8192, 32, 128), generator=g, device=dev) * 0.1).half()
+        V = (torch.randn((8192, 32, 128), generator=g, device=dev) * 0.1).half()
+        # rotate > 1: that many copies of the caches taken in turn, so that they come from HBM, not the Infinity Cache
+        self.kv = [(K, V)] + [(K.clone(), V.clone()) for _ in range(max(rotate - 1, 0))]
+        self.turn = 0
         self.out = torch.zeros((batch, 32, 128), dtype=torch.float16, device=dev)
         self.fn = getattr(ra, "retrieval_attention_%d" % topk)
-        self.desc = "ra: retrieval_attention_%d, B=%d, 32 heads, 8192 keys fp16 shared by the batch" % (topk, batch)
-        self.dominant = "gemv_scores_shared" if batch >= 2 else "gemv_topk_fused"
+        self.desc = "ra: retrieval_attention_%d, B=%d, 32 heads, 8192 keys fp16 shared by the batch%s" % (
+            topk, batch, ", %d rotating cache copies" % rotate if rotate > 1 else "")
+        self.dominant = "gemv_scores_shared" if batch >= 2 else "gemv_scores"
 
     def step(self):
-        self.fn(self.q, self.K, self.V, self.out)
+        K, V = self.kv[self.turn % len(self.kv)]
+        self.turn += 1
+        self.fn(self.q, K, V, self.out)
 
     def bytes(self):
         keys = 8192 * 32 * 128 * 2                               # read once for the whole batch
@@ -260,7 +266,7 @@ def build_workload(name, torch, ops, dev, args):
     if name == "c3":
         return FlashDecode(torch, ops, dev, args.splits)
     if name == "ra":
-        return RetrievalOp(torch, dev, batch=args.batch, topk=args.topk)
+        return RetrievalOp(torch, dev, batch=args.batch, topk=args.topk, rotate=args.rotate)
     if name == "c5":
         return GemvTopk(torch, ops, dev, 1, 8, 8, 1048576, 4096, "bfloat16", 5, "c5", levels=True)
     raise ValueError(name)
@@ -284,7 +290,7 @@ def main():
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--splits", type=int, default=0, help="c3, c4: split count of the attention (0 = library default)")
     ap.add_argument("--rotate", type=int, default=0,
-                    help="c1, c2, c2-ref: number of key sets taken in turn (working set beyond the Infinity Cache)")
+                    help="c1, c2, c2-ref, ra: number of key sets taken in turn (working set beyond the Infinity Cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-runs", type=int, default=3)
     args = ap.parse_args()
