@@ -83,6 +83,14 @@ def test_strided_segments():
     for r in range(5):
         ei, _ = oracle.topk_stable(full[r, :7000], 300)
         assert np.array_equal(idx[r].cpu().numpy(), ei)
+    # rows that start 4 bytes off a 16-byte boundary (no vector loads), long and short
+    for lo, hi, k in ((1, 7001, 300), (3, 1500, 64), (1, 4000, 1000)):
+        idx, val = ops.topk(s[:, lo:hi], k)
+        torch.cuda.synchronize()
+        for r in range(5):
+            ei, ev = oracle.topk_stable(full[r, lo:hi], k)
+            assert np.array_equal(idx[r].cpu().numpy(), ei)
+            assert np.array_equal(val[r].cpu().numpy().view(np.uint32), ev.view(np.uint32))
 
 
 def _short_segment_rows(rng, n):
