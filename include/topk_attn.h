@@ -274,6 +274,9 @@ int tka_lse_combine(const tka_lse_combine_args* args);
  * One call = chunked GEMV + per-chunk top-k + softmax over the num_chunks*k survivors + gathered
  * P.V, i.e. retrieval_topk_kernel + retrieval_reduce_kernel (retrieval_attention.cu:1162-1339).
  * The reference's six hand-off variants compute the same function and map onto this one path.
+ * The caches are shared by the batch (retrieval_attention.cu:681-683); where the reference pipelines the batch
+ * entries through one cluster (retrieval_attention.cu:654-896), this call reads the keys once per tile of up to
+ * eight entries.
  * ---------------------------------------------------------------------------------------------- */
 typedef struct tka_ra_args {
   const void* q;          /* device [batch][num_heads][128]                                   */
