@@ -98,6 +98,21 @@ def _valid_gemv():
     return a
 
 
+def test_redone_segments_validation():
+    """The diagnostic validates like the call it reports on, and a call that cannot take the long-segment path
+    reports zero without touching the device."""
+    lib = L.lib()
+    n = C.c_int32(-1)
+    a = _valid_gemv()
+    assert lib.tka_gemv_topk_redone_segments(C.byref(a), None) == L.TKA_EINVAL
+    assert lib.tka_gemv_topk_redone_segments(None, C.byref(n)) == L.TKA_EINVAL
+    assert lib.tka_gemv_topk_redone_segments(C.byref(a), C.byref(n)) == L.TKA_EWORKSPACE
+    a.workspace, a.workspace_bytes = 0x10000, lib.tka_gemv_topk_workspace_bytes(C.byref(a))
+    assert lib.tka_gemv_topk_redone_segments(C.byref(a), C.byref(n)) == L.TKA_OK and n.value == 0   # 4096-token segments
+    a.k = 0
+    assert lib.tka_gemv_topk_redone_segments(C.byref(a), C.byref(n)) == L.TKA_EINVAL
+
+
 def test_gemv_topk_validation():
     lib = L.lib()
     a = _valid_gemv()
