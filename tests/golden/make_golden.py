@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/sparse_decode_small.npz: seeded inputs (bit patterns) and the oracle's outputs for one
-small end-to-end case per element type.  The reference repository holds no vectors of its own (all its data is
-generated at run time), so these fixtures freeze the oracle instead: a change in tka_oracle.c that alters any
-result fails tests/test_golden.py.  Run from the repository root:  python tests/golden/make_golden.py"""
+"""Writes tests/golden/sparse_decode_small.npz and tests/golden/retrieval_op_small.npz: seeded inputs (bit patterns)
+and the oracle's outputs for one small end-to-end case (resp. one small call of the operator) per element type.
+The reference repository holds no vectors of its own (all its data is generated at run time), so these fixtures
+freeze the oracle instead: a change in tka_oracle.c that alters any result fails tests/test_golden.py.
+Run from the repository root:  python tests/golden/make_golden.py"""
 import os
 import sys
 
@@ -35,6 +36,27 @@ def main():
                     tag + "_topk_val": np.stack(tval), tag + "_union": np.stack(unis), tag + "_union_count": np.array(cnts)})
     out["params"] = np.array([128, 2, 4, 24, 4, 8], np.int64)
     np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "sparse_decode_small.npz"), **out)
+
+    # The operator (test_ra.py:88-160 in small): caches shared by a batch of 16, 2 heads, 4 chunks of 64 keys,
+    # 8 survivors per chunk, raw-exp softmax, no scale.  128 segments: enough for the batch route of the library.
+    op = {}
+    B, N, H, chunks, topk = 16, 256, 2, 4, 8
+    for tag, dtype, seed in (("f16", oracle.F16, 21), ("bf16", oracle.BF16, 22)):
+        rng = np.random.default_rng(seed)
+        q = oracle.to_bits(rng.standard_normal((B, H, 128)) * 0.1, dtype)
+        Kf = rng.standard_normal((N, H, 128)) * 0.1
+        Kf[100:140] = Kf[100]                                    # forty equal keys: ties inside and across chunks
+        K = oracle.to_bits(Kf, dtype)
+        V = oracle.to_bits(rng.standard_normal((N, H, 128)) * 0.1, dtype)
+        outs = np.empty((B, H, 128))
+        idx = np.empty((B, H, chunks * topk), np.int32)
+        val = np.empty((B, H, chunks * topk), np.float32)
+        for b in range(B):
+            for h in range(H):
+                outs[b, h], idx[b, h], val[b, h] = oracle.retrieval_attention(q[b, h], K[:, h], V[:, h], dtype, chunks, topk, 1.0)
+        op.update({tag + "_q": q, tag + "_K": K, tag + "_V": V, tag + "_out": outs, tag + "_idx": idx, tag + "_val": val})
+    op["params"] = np.array([B, N, H, chunks, topk], np.int64)
+    np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "retrieval_op_small.npz"), **op)
 
 
 if __name__ == "__main__":

@@ -42,3 +42,37 @@ def test_gpu_matches_fixture(tag, dtype):
     for h in range(H):
         assert np.array_equal(uidx[0, h, :cnt[h]].cpu().numpy(), FIX[tag + "_union"][h][:cnt[h]])
     assert np.abs(f32_of(out)[0] - FIX[tag + "_out"].reshape(H * G, 128)).max() < 2e-3
+
+
+OP = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "retrieval_op_small.npz"))
+OP_B, OP_N, OP_H, OP_CHUNKS, OP_TOPK = (int(x) for x in OP["params"])
+
+
+@pytest.mark.parametrize("tag,dtype", CASES)
+def test_oracle_reproduces_operator_fixture(tag, dtype):
+    q, K, V = OP[tag + "_q"], OP[tag + "_K"], OP[tag + "_V"]
+    for b in range(OP_B):
+        for h in range(OP_H):
+            o, i, v = oracle.retrieval_attention(q[b, h], K[:, h], V[:, h], dtype, OP_CHUNKS, OP_TOPK, 1.0)
+            assert np.array_equal(i, OP[tag + "_idx"][b, h])
+            assert np.array_equal(v.view(np.uint32), OP[tag + "_val"][b, h].view(np.uint32))
+            assert np.abs(o - OP[tag + "_out"][b, h]).max() < 1e-12
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,dtype", CASES)
+def test_gpu_matches_operator_fixture(tag, dtype):
+    """The operator and its selection stage on the fixture: 128 short segments over caches shared by 16 batch entries."""
+    import torch
+    from tests.util import TORCH_DT, announce, f32_of, to_dev
+    from topk_attn_amd import ops
+    announce("golden operator fixture %s" % tag)
+    q, K, V = to_dev(OP[tag + "_q"], dtype), to_dev(OP[tag + "_K"], dtype), to_dev(OP[tag + "_V"], dtype)
+    out = torch.zeros((OP_B, OP_H, 128), dtype=TORCH_DT[dtype], device="cuda")
+    ops.retrieval_attention(q, K, V, out, OP_TOPK, OP_CHUNKS, 1.0)
+    idx, val = ops.gemv_topk(q, K, OP_TOPK, group=1, scale=1.0, num_chunks=OP_CHUNKS)
+    torch.cuda.synchronize()
+    assert np.array_equal(idx.cpu().numpy(), OP[tag + "_idx"])
+    assert np.array_equal(val.cpu().numpy().view(np.uint32), OP[tag + "_val"].view(np.uint32))
+    tol = 2e-3 if dtype == oracle.F16 else 2e-3 + np.abs(OP[tag + "_out"]).max() * 2.0 ** -8   # (bf16 output: its own rounding)
+    assert np.abs(f32_of(out) - OP[tag + "_out"]).max() < tol
