@@ -405,8 +405,37 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
     __syncthreads();
     for (int i = tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite
   }
+  if (want_rank && !want_union) {
+    // The sort that follows takes the composites in any order: every wave reserves room for its selected
+    // entries with one add, no walk in index order.
+    if (tid == 0) sh_res[3] = 0u;
+    __syncthreads();
+    const int lane = tid & 63;
+    uint32_t mine = 0;
+#pragma unroll
+    for (int i = 0; i < kEntryCache; ++i)
+      mine += ((uint32_t)i * kSelThreads + tid < n_entries && cache[i] >= threshold) ? 1u : 0u;
+    for (uint32_t v = kEntryCache * kSelThreads + tid; v < n_entries; v += kSelThreads) mine += entry(v) >= threshold ? 1u : 0u;
+    const uint32_t inc = wave_inclusive_scan(mine);
+    uint32_t first = 0;
+    if (lane == 63) first = atomicAdd(&sh_res[3], inc);
+    uint32_t pos = (uint32_t)__builtin_amdgcn_readlane((int)first, 63) + inc - mine;
+#pragma unroll
+    for (int i = 0; i < kEntryCache; ++i)
+      if ((uint32_t)i * kSelThreads + tid < n_entries && cache[i] >= threshold) {
+        if (pos < k) sh_sort[pos] = cache[i];
+        ++pos;
+      }
+    for (uint32_t v = kEntryCache * kSelThreads + tid; v < n_entries; v += kSelThreads) {
+      const uint64_t c = entry(v);
+      if (c >= threshold) {
+        if (pos < k) sh_sort[pos] = c;
+        ++pos;
+      }
+    }
+  }
   uint32_t run_sel = 0, run_mid = 0;
-  for (uint32_t base = 0, step = 0; base < n_entries; base += kSelThreads, ++step) {
+  for (uint32_t base = 0, step = 0; base < n_entries && want_union; base += kSelThreads, ++step) {
     const uint32_t v = base + tid;
     uint64_t c = 0;
     if (step < kEntryCache) {
