@@ -218,6 +218,17 @@ __global__ __launch_bounds__(kCombineThreads) void lse_combine_kernel(CombinePar
   const float* pl = p.part_l + (int64_t)row * S;
   const f32x4* pa = (const f32x4*)(p.part_acc + (int64_t)row * S * kHeadDim);
 
+  // accumulators: group g takes splits g, g+32, ...; the first four of them are requested before anything else,
+  // so that their round trip to memory runs beside that of the maxima and sums
+  const int g = tid / kCombineLanes, dl = tid % kCombineLanes;
+  const f32x4 zero4 = (f32x4){0.f, 0.f, 0.f, 0.f};
+  f32x4 a0[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int s = g + u * kCombineGroups;
+    a0[u] = s < S ? pa[(int64_t)s * kCombineLanes + dl] : zero4;
+  }
+
   // M = max over non-empty splits
   float ms = -INFINITY, ls = 0.0f;
   if (tid < S) {
@@ -247,22 +258,27 @@ __global__ __launch_bounds__(kCombineThreads) void lse_combine_kernel(CombinePar
     sh_stat[0] = M;
     sh_stat[1] = L;
   }
-  // accumulators: group g takes splits g, g+32, ...
-  const int g = tid / kCombineLanes, dl = tid % kCombineLanes;
-  f32x4 o = (f32x4){0.f, 0.f, 0.f, 0.f};
-  // four splits per trip, loads first: a load behind the weight test would make every trip a memory round trip
-  for (int s0 = g; s0 < S; s0 += 4 * kCombineGroups) {
+  f32x4 o = zero4;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int s = g + u * kCombineGroups;
+    const float w = s < S ? sh_w[s] : 0.0f;
+    if (w != 0.0f) o += a0[u] * w;   // the accumulator of an empty split is never looked at
+  }
+  // beyond 128 splits: four per trip, loads first (a load behind the weight test would make every trip a memory
+  // round trip)
+  for (int s0 = g + 4 * kCombineGroups; s0 < S; s0 += 4 * kCombineGroups) {
     f32x4 a[4];
     float w[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int s = s0 + u * kCombineGroups;
       w[u] = s < S ? sh_w[s] : 0.0f;
-      a[u] = pa[(int64_t)(s < S ? s : g) * kCombineLanes + dl];
+      a[u] = s < S ? pa[(int64_t)s * kCombineLanes + dl] : zero4;
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u)
-      if (w[u] != 0.0f) o += a[u] * w[u];   // the accumulator of an empty split is never looked at
+      if (w[u] != 0.0f) o += a[u] * w[u];
   }
   sh_o[g][dl] = o;
   __syncthreads();
