@@ -47,11 +47,23 @@ def randn16(torch, shape, dt, g, dev, chunk_dim0=True):
     return out
 
 
+def levels16(torch, shape, dt, g, dev):
+    """[B, N, H, 128] tensor whose entries take 16 uniform levels in [-2, 2], generated in slices of 131072 tokens."""
+    out = torch.empty(shape, device=dev, dtype=dt)
+    lv = torch.linspace(-2.0, 2.0, 16, device=dev)
+    for b in range(shape[0]):
+        for t0 in range(0, shape[1], 131072):
+            t1 = min(shape[1], t0 + 131072)
+            ids = torch.randint(0, 16, (t1 - t0,) + tuple(shape[2:]), generator=g, device=dev)
+            out[b, t0:t1] = lv[ids].to(dt)
+    return out
+
+
 class SparseDecode:
     """c4 (and a small variant): the end-to-end step."""
 
     def __init__(self, torch, ops, dev, batch=8, hkv=8, group=4, seq_len=131072, k=2048, sink=64, local=512,
-                 dtype="float16", out_dtype="bfloat16", heavy=0.01, seed=4, name="c4", num_splits=0):
+                 dtype="float16", out_dtype="bfloat16", heavy=0.01, seed=4, name="c4", num_splits=0, levels=False):
         self.torch, self.name = torch, name
         g = torch.Generator(device=dev)
         g.manual_seed(seed)
@@ -59,7 +71,10 @@ class SparseDecode:
         B, H, G, N = batch, hkv, group, seq_len
         self.B, self.H, self.G, self.N, self.k, self.sink, self.local = B, H, G, N, k, sink, local
         self.q = randn16(torch, (B, H * G, 128), dt, g, dev, chunk_dim0=False)
-        self.K = randn16(torch, (B, N, H, 128), dt, g, dev)
+        if levels:  # 16 uniform levels in [-2, 2]: many exact score ties
+            self.K = levels16(torch, (B, N, H, 128), dt, g, dev)
+        else:
+            self.K = randn16(torch, (B, N, H, 128), dt, g, dev)
         self.V = randn16(torch, (B, N, H, 128), dt, g, dev)
         n_heavy = int(N * heavy)
         for b in range(B):
@@ -123,13 +138,7 @@ class GemvTopk:
         self.B, self.H, self.G, self.N, self.k = batch, hkv, group, seq_len, k
         self.q = randn16(torch, (batch, hkv * group, 128), dt, g, dev, chunk_dim0=False)
         if levels:  # 16 uniform levels in [-2, 2]: many exact score ties
-            self.K = torch.empty((batch, seq_len, hkv, 128), device=dev, dtype=dt)
-            lv = torch.linspace(-2.0, 2.0, 16, device=dev)
-            for b in range(batch):
-                for t0 in range(0, seq_len, 131072):
-                    t1 = min(seq_len, t0 + 131072)
-                    ids = torch.randint(0, 16, (t1 - t0, hkv, 128), generator=g, device=dev)
-                    self.K[b, t0:t1] = lv[ids].to(dt)
+            self.K = levels16(torch, (batch, seq_len, hkv, 128), dt, g, dev)
         else:
             self.K = randn16(torch, (batch, seq_len, hkv, 128), dt, g, dev)
         # rotate > 0: that many copies of the keys, one plan each, taken in turn, so that a key set much smaller
@@ -267,8 +276,11 @@ def build_workload(name, torch, ops, dev, args):
         return FlashDecode(torch, ops, dev, args.splits)
     if name == "ra":
         return RetrievalOp(torch, dev, batch=args.batch, topk=args.topk, rotate=args.rotate)
-    if name == "c5":
-        return GemvTopk(torch, ops, dev, 1, 8, 8, 1048576, 4096, "bfloat16", 5, "c5", levels=True)
+    if name == "c5":       # the tie-stress step: selection under exact ties at 1M tokens, attention over the selected tokens
+        return SparseDecode(torch, ops, dev, batch=1, hkv=8, group=8, seq_len=1048576, k=4096, sink=0, local=0,
+                            dtype="bfloat16", heavy=0.0, seed=5, name="c5", levels=True)
+    if name == "c5-topk":  # its selection stage alone, rank-ordered output
+        return GemvTopk(torch, ops, dev, 1, 8, 8, 1048576, 4096, "bfloat16", 5, "c5-topk", levels=True)
     raise ValueError(name)
 
 
@@ -285,7 +297,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c5", "ra", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c5", "c5-topk", "ra", "copy"])
     ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--splits", type=int, default=0, help="c3, c4: split count of the attention (0 = library default)")

@@ -1,0 +1,147 @@
+"""The configurations the throughput figures are quoted on, at their full sizes, through properties that need no CPU
+pass over gigabytes of keys:
+
+* selection: the fused GEMV + top-k (candidate lists, sampled thresholds) must return exactly the first k entries of a
+  STABLE descending sort of the plain score vector of the same keys (stable = ties keep the lower index first).  The
+  score vector comes from the library's GEMV-only entry point, whose values are pinned bit for bit against the CPU
+  oracle in test_gpu_gemv_topk.py at sizes the oracle finishes; the sort is torch's, an independent selection.
+* union: ascending, duplicate-free, sink range + selected middle + local window, count = size of that set.
+* attention: against a torch fp32 softmax over the union rows of each KV head, within the 2e-3 of the end-to-end
+  tests (plus the half-ulp of a bf16 output).
+* dense flash-decoding: against torch fp32 attention over all 131 072 tokens, and invariant under the split count.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import announce
+
+pytestmark = pytest.mark.gpu
+
+SCALE = float(np.float32(1.0 / np.sqrt(128.0)))
+
+
+def _randn16(shape, dt, gen, rows_per_chunk=1 << 16):
+    """Normal 16-bit tensor [B, N, H, 128] filled chunk by chunk (no fp32 copy of the whole cache)."""
+    out = torch.empty(shape, dtype=dt, device="cuda")
+    flat = out.view(-1, shape[-2] * shape[-1])
+    for r0 in range(0, flat.shape[0], rows_per_chunk):
+        r1 = min(r0 + rows_per_chunk, flat.shape[0])
+        flat[r0:r1] = torch.randn((r1 - r0, flat.shape[1]), generator=gen, device="cuda").to(dt)
+    return out
+
+
+def _check_selection(scores, idx, val, k):
+    """idx/val [B,H,k] against the stable descending sort of scores [B,H,N]; bit-exact."""
+    B, H, _ = scores.shape
+    for b in range(B):
+        sv, si = torch.sort(scores[b], dim=-1, descending=True, stable=True)
+        assert torch.equal(idx[b].long(), si[:, :k]), "top-k indices differ from the stable sort (batch entry %d)" % b
+        assert torch.equal(val[b].view(torch.int32), sv[:, :k].contiguous().view(torch.int32)), "top-k values differ"
+
+
+def test_c4_end_to_end_full_size():
+    """B=8, 8 KV heads x GQA 4, N=131072 fp16, k=2048, sink 64, local 512, bf16 output; 1% heavy-hitter keys."""
+    from topk_attn_amd import ops
+    B, H, G, N, k, sink, local = 8, 8, 4, 131072, 2048, 64, 512
+    announce("full size c4: B=%d Hkv=%d G=%d N=%d k=%d" % (B, H, G, N, k))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(404)
+    q = torch.randn((B, H * G, 128), generator=gen, device="cuda").to(torch.float16)
+    K = _randn16((B, N, H, 128), torch.float16, gen)
+    V = _randn16((B, N, H, 128), torch.float16, gen)
+    for b in range(B):
+        for h in range(H):
+            hh = torch.randperm(N, generator=gen, device="cuda")[:N // 100]
+            K[b, hh, h] = (K[b, hh, h].float() * 4.0).to(torch.float16)
+    out, tidx, tval, uidx, ucnt = ops.sparse_decode_step(q, K, V, k, sink, local, SCALE, G, out_dtype=torch.bfloat16)
+    scores = ops.gemv_scores(q, K, group=G, scale=SCALE)
+    torch.cuda.synchronize()
+    _check_selection(scores, tidx, tval, k)
+
+    lo, hi = sink, N - local
+    edge = torch.cat([torch.arange(lo, device="cuda"), torch.arange(hi, N, device="cuda")])
+    worst = 0.0
+    for b in range(B):
+        for h in range(H):
+            sel = tidx[b, h].long()
+            want = torch.unique(torch.cat([edge, sel]))          # sorted ascending, duplicate-free
+            n = int(ucnt[b, h])
+            assert n == want.numel(), "union count"
+            assert torch.equal(uidx[b, h, :n].long(), want), "union list"
+            ks, vs = K[b, want, h].float(), V[b, want, h].float()
+            logits = (q[b, h * G:(h + 1) * G].float() @ ks.T) * SCALE
+            ref = torch.softmax(logits, dim=-1) @ vs
+            got = out[b, h * G:(h + 1) * G].float()
+            tol = 2e-3 + ref.abs() * 2.0 ** -8                   # bf16 output: its own rounding on top
+            assert bool(((got - ref).abs() < tol).all()), "attention output (b=%d, h=%d)" % (b, h)
+            worst = max(worst, float((got - ref).abs().max()))
+    print("c4 full size: worst attention error %.2e" % worst, flush=True)
+
+
+def _levels16(shape, dt, gen):
+    levels = torch.linspace(-2, 2, 16, device="cuda")
+    out = torch.empty(shape, dtype=dt, device="cuda")
+    flat = out.view(-1, shape[-2] * shape[-1])
+    for r0 in range(0, flat.shape[0], 1 << 16):
+        r1 = min(r0 + (1 << 16), flat.shape[0])
+        flat[r0:r1] = levels[torch.randint(0, 16, (r1 - r0, flat.shape[1]), generator=gen, device="cuda")].to(dt)
+    return out
+
+
+@pytest.mark.parametrize("pool", [0, 4096])
+def test_c5_tie_stress_full_size(pool):
+    """8 KV heads x GQA 8, N=1048576 bf16 keys on 16 levels, k=4096, attention over the selected tokens.
+    pool=0: every key row drawn independently (exact ties between scores wherever the level sums coincide).
+    pool=4096: the rows are drawn from 4096 distinct ones, so every score is shared by about 256 tokens and the cut
+    at rank k falls inside a run of equal scores on every head: the lower token index must win throughout."""
+    from topk_attn_amd import ops
+    H, G, N, k = 8, 8, 1 << 20, 4096
+    announce("full size c5: Hkv=%d G=%d N=%d k=%d bf16 levels, row pool %d" % (H, G, N, k, pool))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(505 + pool)
+    if pool:
+        rows = _levels16((1, pool, H, 128), torch.bfloat16, gen)[0]
+        K = rows[torch.randint(0, pool, (N,), generator=gen, device="cuda")].unsqueeze(0).contiguous()
+    else:
+        K = _levels16((1, N, H, 128), torch.bfloat16, gen)
+    V = _randn16((1, N, H, 128), torch.bfloat16, gen)
+    q = torch.randn((1, H * G, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    plan = ops.SparseDecodePlan(q, K, V, k, 0, 0, SCALE, G, out_dtype=torch.bfloat16)
+    out = plan.step()
+    scores = ops.gemv_scores(q, K, group=G, scale=SCALE)
+    torch.cuda.synchronize()
+    _check_selection(scores, plan.topk_idx, plan.topk_val, k)
+    kth = plan.topk_val[0, :, k - 1]
+    ties = (scores[0] == kth[:, None]).sum(dim=1)
+    print("c5 full size (pool %d): tokens sharing the k-th score per head: %s" % (pool, ties.tolist()), flush=True)
+    if pool:
+        assert bool((ties >= 2).all()), "the cut does not fall inside a run of equal scores"
+    for h in range(H):
+        want = torch.sort(plan.topk_idx[0, h].long()).values
+        assert int(plan.union_count[0, h]) == k and torch.equal(plan.union_idx[0, h, :k].long(), want), "union list"
+        logits = (q[0, h * G:(h + 1) * G].float() @ K[0, want, h].float().T) * SCALE
+        ref = torch.softmax(logits, dim=-1) @ V[0, want, h].float()
+        got = out[0, h * G:(h + 1) * G].float()
+        assert bool(((got - ref).abs() < 2e-3 + ref.abs() * 2.0 ** -8).all()), "attention output (h=%d)" % h
+
+
+def test_c3_dense_flash_decode_full_size():
+    """32 query heads over 8 KV heads, N=131072 fp16: against torch fp32 attention, and across split counts."""
+    from topk_attn_amd import ops
+    B, H, G, N = 1, 8, 4, 131072
+    announce("full size c3: Hq=%d Hkv=%d N=%d dense flash-decoding" % (H * G, H, N))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(303)
+    q = torch.randn((B, H * G, 128), generator=gen, device="cuda").to(torch.float16)
+    K = _randn16((B, N, H, 128), torch.float16, gen)
+    V = _randn16((B, N, H, 128), torch.float16, gen)
+    out = ops.flash_decode(q, K, V, SCALE, group=G)
+    out_1 = ops.flash_decode(q, K, V, SCALE, group=G, num_splits=1)
+    out_37 = ops.flash_decode(q, K, V, SCALE, group=G, num_splits=37)
+    torch.cuda.synchronize()
+    for h in range(H):
+        logits = (q[0, h * G:(h + 1) * G].float() @ K[0, :, h].float().T) * SCALE
+        ref = torch.softmax(logits, dim=-1) @ V[0, :, h].float()
+        for o in (out, out_1, out_37):
+            assert float((o[0, h * G:(h + 1) * G].float() - ref).abs().max()) < 2e-3
