@@ -12,6 +12,14 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """What is built is used as it is; only when the library or the command-line program is missing are they made."""
+    lib = os.path.join(ROOT, "topk_attn_amd", "lib")
+    if not all(os.path.exists(os.path.join(lib, f)) for f in ("libtka.so", "tka_standalone")):
+        import topk_attn_amd
+        topk_attn_amd.build(force=False)
+
+
 def pytest_collection_modifyitems(config, items):
     try:
         import torch
