@@ -138,18 +138,24 @@ def test_center_only_config2_shape():
         assert np.array_equal(out[h].reshape(top_c, clen), cids[h][:, None] * clen + np.arange(clen)[None])
 
 
-def test_two_level_cluster_reference_shape():
-    """Reference constants of gemv_topk.cu:21-28 scaled down in heads: 32 centroids, clusters of 1280 tokens,
-    top-5 clusters, top-512 inside each."""
+@pytest.mark.parametrize("H,tied_centres", [(4, False), (32, False), (32, True)])
+def test_two_level_cluster_reference_shape(H, tied_centres):
+    """Reference constants of gemv_topk.cu:21-28: 32 centroids, clusters of 1280 tokens, top-5 clusters, top-512
+    inside each.  With all 32 heads (160 segments) the centre stage runs inside the GEMV launch of the token stage;
+    with 4 heads it is a launch of its own.  tied_centres: three identical centroids per head, aligned with the
+    query so that they take ranks 0-2: equal scores, the lower centroid id must come first."""
     from topk_attn_amd import ops
-    announce("cluster_gemv_topk CSZ=32 CLEN=1280 TOPC=5 k=512")
+    announce("cluster_gemv_topk CSZ=32 CLEN=1280 TOPC=5 k=512 H=%d tied_centres=%s" % (H, tied_centres))
     rng = np.random.default_rng(12345)
-    H, CSZ, CLEN, TOPC, K = 4, 32, 1280, 5, 512
+    CSZ, CLEN, TOPC, K = 32, 1280, 5, 512
     cen = rng.uniform(-0.5, 0.5, (H, CSZ, 128))
+    qf = rng.uniform(-0.5, 0.5, (H, 128))
+    if tied_centres:
+        cen[:, [20, 3, 7]] = 0.9 * qf[:, None, :]
     keys = cen.transpose(1, 0, 2)[:, None, :, :] + 0.05 * rng.standard_normal((CSZ, CLEN, H, 128))
     keys = keys.reshape(CSZ * CLEN, H, 128)
     cen_b, keys_b = oracle.to_bits(cen, oracle.F16), oracle.to_bits(keys, oracle.F16)
-    q_b = oracle.to_bits(rng.uniform(-0.5, 0.5, (H, 128)), oracle.F16)
+    q_b = oracle.to_bits(qf, oracle.F16)
     out = ops.cluster_gemv_topk(to_dev(q_b, oracle.F16), to_dev(cen_b, oracle.F16), to_dev(keys_b, oracle.F16),
                                 TOPC, CLEN, K, 1.0)
     torch.cuda.synchronize()
@@ -157,6 +163,8 @@ def test_two_level_cluster_reference_shape():
     for h in range(H):
         want = oracle.cluster_topk(q_b[h], cen_b[h], keys_b[:, h, :], oracle.F16, TOPC, CLEN, K, 1.0)
         assert np.array_equal(out[h], want)
+        if tied_centres:
+            assert [int(want[r * K]) // CLEN for r in range(3)] == [3, 7, 20]
         # the reference's own check (gemv_topk.cu:138-170): set equality per (head, rank) slice
         for r in range(TOPC):
             assert set(out[h, r * K:(r + 1) * K]) == set(want[r * K:(r + 1) * K])

@@ -115,6 +115,9 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->scores = scores;
   g->hist = hist;
   g->cluster_ids = nullptr;
+  g->centers = nullptr;
+  g->cluster_ids_out = nullptr;
+  g->num_centers = 0;
   g->chunk_len = a->seq_len / a->num_chunks;
   g->q_stride_b = a->q_stride_b;
   g->key_stride_b = a->key_stride_b;
@@ -169,8 +172,23 @@ struct UnionOut {
 // Runs clear + GEMV (+histogram) + select.  `ws` holds [scores][select workspace].
 // a->out_idx == nullptr skips the rank-order sort (then `u` must ask for the union list).
 // `any_order`: the caller does not need out_idx / out_val in rank order (a route may still deliver it).
+// Centre stage of a two-level selection done inside the GEMV launch of the token stage (see wave_route).
+struct InlineCentres {
+  const void* centers;   // [num_kv_heads][num_centers][128]
+  int num_centers;
+  int32_t* ids_out;      // [num_kv_heads*num_chunks] chosen cluster per (head, rank)
+};
+
+// Segments that fit in the registers of a workgroup: plain scores, then one workgroup per segment selects.
+bool wave_route(const tka_gemv_topk_args* a, bool want_union) {
+  const int segs = a->batch * a->num_kv_heads * a->num_chunks;
+  const int64_t chunk_len = a->seq_len / a->num_chunks;
+  return (a->out_idx || want_union) && wave_select_fits(chunk_len, a->k) &&
+         (chunk_len > kFusedMaxSegLen || a->out_scores || segs >= wave_select_min_segments());
+}
+
 int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, const int32_t* cluster_ids = nullptr,
-                  const UnionOut* u = nullptr, bool any_order = false) {
+                  const UnionOut* u = nullptr, bool any_order = false, const InlineCentres* ic = nullptr) {
   hipStream_t stream = (hipStream_t)a->stream;
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
@@ -208,16 +226,21 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // Keys shared by the batch are read once for several batch entries.
   const bool shared_keys = a->key_stride_b == 0 && a->batch >= 2 && !cluster_ids;
 
-  // Segments that fit in the registers of a workgroup: plain scores, then one workgroup per segment selects.
-  if ((a->out_idx || u) && wave_select_fits(chunk_len, a->k) &&
-      (chunk_len > kFusedMaxSegLen || a->out_scores || segs >= wave_select_min_segments())) {
+  if (wave_route(a, u != nullptr)) {
     gp.hist = nullptr;
-    int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);
-    if (rc != TKA_OK) return rc;
     SelectParams sw = sp;
     sw.unordered = any_order ? 1 : 0;
+    if (ic) {   // the GEMV launch ranks the centroids itself and leaves the chosen ids for the selection
+      gp.centers = ic->centers;
+      gp.num_centers = ic->num_centers;
+      gp.cluster_ids_out = ic->ids_out;
+      sw.seg_base_ids = ic->ids_out;
+    }
+    int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);
+    if (rc != TKA_OK) return rc;
     return launch_select_wave(sw, stream);
   }
+  if (ic) return TKA_EINVAL;   // (callers ask wave_route first)
 
   // Short segments: one launch, each workgroup scores and selects its own segment.  One CU pulls about
   // 55 GB/s, so beyond 2048 rows (0.5 MB) the separate GEMV launch with many workgroups per segment wins.
@@ -626,6 +649,13 @@ int tka_cluster_gemv_topk(const tka_cluster_topk_args* a) {
   unsigned char* ws = (unsigned char*)a->workspace;
   int32_t* centre_ids = (int32_t*)ws;
   ws += align_up((size_t)a->num_heads * a->top_c * sizeof(int32_t), 256);
+  if (a->num_centers <= kGemvInlineCentres && wave_route(&t, false)) {
+    // few centroids, clusters that a workgroup selects from registers: two launches instead of three
+    const InlineCentres ic = {a->centers, a->num_centers, centre_ids};
+    t.workspace = ws + tka_gemv_topk_workspace_bytes(&c);
+    t.workspace_bytes = tka_gemv_topk_workspace_bytes(&t);
+    return run_gemv_topk(&t, nullptr, 0, nullptr, nullptr, false, &ic);
+  }
   c.out_idx = centre_ids;
   c.workspace = ws;
   c.workspace_bytes = tka_gemv_topk_workspace_bytes(&c);

@@ -22,6 +22,7 @@ constexpr int kHistBins = 1 << kHistBits;  // first-level selection histogram: t
 constexpr int kGemvDenseTokensPerWg = 256; // tokens per workgroup of the dense GEMV on large problems
 constexpr int kGemvCandTokensPerWg = 512;  // tokens (and threads) per streaming workgroup of the candidate GEMV = slice length
 constexpr int64_t kFusedMaxSegLen = 2048;   // segments up to this length are scored and selected by one workgroup in one launch
+constexpr int kGemvInlineCentres = 256;     // centroids per head that the GEMV launch of a two-level selection ranks itself
 constexpr int64_t kCandMinSegLen = 32768;   // shorter segments never take the candidate mode
 constexpr int64_t kCandMinRows = 1 << 20;   // ... nor do segments below 65536 tokens unless the call has this many rows
 constexpr int kGemvMaxSamples = 8192;      // most samples per segment of the candidate-mode threshold estimate

@@ -47,9 +47,6 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
   const int chunk = blockIdx.x / p.wgs_per_chunk;
   const int wg_in_chunk = blockIdx.x % p.wgs_per_chunk;
   const int64_t seg = ((int64_t)b * p.num_kv_heads + h) * p.num_chunks + chunk;
-  // tokens are counted inside the chunk; the chunk starts at chunk*chunk_len, or at the start of the
-  // cluster chosen for this (head, rank) in two-level selection
-  const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
   const int64_t t_begin = (int64_t)wg_in_chunk * p.tokens_per_wg;
   int64_t t_end = t_begin + p.tokens_per_wg;
   if (t_end > p.chunk_len) t_end = p.chunk_len;
@@ -62,6 +59,50 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
 
   float qf[8];
   load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+
+  // tokens are counted inside the chunk; the chunk starts at chunk*chunk_len, or at the start of the
+  // cluster chosen for this (head, rank) in two-level selection
+  int64_t chunk_base;
+  if (p.centers) {
+    // Centre stage inline: every workgroup scores the (few) centroids of its head in the same order as any
+    // other row, ranks them by (key descending, id ascending) and takes the one of rank `chunk`.  It costs a
+    // round trip to memory at the head of the workgroup and saves a launch.
+    __shared__ uint32_t sh_ckey[kGemvInlineCentres];
+    __shared__ int sh_cid;
+    const uint16_t* cbase = (const uint16_t*)p.centers + ((int64_t)b * p.num_kv_heads + h) * p.num_centers * kHeadDim + 8 * j;
+    for (int c0 = 0; c0 < p.num_centers; c0 += kGemvRowsPerIter) {
+      u32x4 cv[kGemvUnroll];
+#pragma unroll
+      for (int u = 0; u < kGemvUnroll; ++u) {
+        const int c = c0 + rg * kGemvUnroll + u;
+        cv[u] = *(const u32x4*)(cbase + (int64_t)(c < p.num_centers ? c : p.num_centers - 1) * kHeadDim);
+      }
+      float mine = 0.0f;
+#pragma unroll
+      for (int u = 0; u < kGemvUnroll; ++u) {
+        const float s = row_score<DT>(qf, cv[u], p.scale);
+        if (j == u) mine = s;
+      }
+      const int c = c0 + rg * kGemvUnroll + j;
+      if (j < kGemvUnroll && c < p.num_centers) sh_ckey[c] = score_key(mine);
+    }
+    __syncthreads();
+    if (tid < p.num_centers) {
+      const uint32_t my = sh_ckey[tid];
+      int ahead = 0;
+      for (int i = 0; i < p.num_centers; ++i) {
+        const uint32_t other = sh_ckey[i];
+        ahead += (other > my || (other == my && i < tid)) ? 1 : 0;
+      }
+      if (ahead == chunk) sh_cid = tid;
+    }
+    __syncthreads();
+    const int cid = sh_cid;
+    if (wg_in_chunk == 0 && tid == 0) p.cluster_ids_out[seg] = cid;
+    chunk_base = (int64_t)cid * p.chunk_len;
+  } else {
+    chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
+  }
 
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
                           chunk_base * p.key_stride_n + 8 * j;

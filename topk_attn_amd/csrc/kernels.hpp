@@ -10,6 +10,11 @@ struct GemvParams {
   const void* keys;
   float* scores;        // [batch][num_kv_heads][num_chunks][chunk_len]; selection kernels also read them
   const int32_t* cluster_ids;  // [batch*num_kv_heads*num_chunks] or nullptr: chunk c covers the tokens of that cluster
+  // two-level selection with the centre stage inside the GEMV launch (gemv_scores_kernel only): chunk c of head h
+  // covers the cluster whose centroid has rank c among centers[h], and the id is also written to cluster_ids_out
+  const void* centers;         // [num_kv_heads][num_centers][128] or nullptr
+  int32_t* cluster_ids_out;    // [num_kv_heads*num_chunks]
+  int num_centers;             // <= kGemvInlineCentres
   uint32_t* hist;       // [batch*num_kv_heads*num_chunks][kHistBins] or nullptr; must be zero on entry
   // candidate mode: only tokens whose key reaches the segment's sampled threshold are stored
   uint64_t* tau_words;        // [segments][2] (epoch << 32) | threshold key, and the token cut among keys equal to it
