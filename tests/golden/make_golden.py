@@ -1,6 +1,7 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/sparse_decode_small.npz and tests/golden/retrieval_op_small.npz: seeded inputs (bit patterns)
-and the oracle's outputs for one small end-to-end case (resp. one small call of the operator) per element type.
+"""Writes tests/golden/sparse_decode_small.npz, retrieval_op_small.npz and cluster_small.npz: seeded inputs (bit patterns)
+and the oracle's outputs for one small end-to-end case, one small call of the operator, and one small two-level /
+centre-only selection per element type.
 The reference repository holds no vectors of its own (all its data is generated at run time), so these fixtures
 freeze the oracle instead: a change in tka_oracle.c that alters any result fails tests/test_golden.py.
 Run from the repository root:  python tests/golden/make_golden.py"""
@@ -57,6 +58,30 @@ def main():
         op.update({tag + "_q": q, tag + "_K": K, tag + "_V": V, tag + "_out": outs, tag + "_idx": idx, tag + "_val": val})
     op["params"] = np.array([B, N, H, chunks, topk], np.int64)
     np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "retrieval_op_small.npz"), **op)
+
+    # Two-level and centre-only selection (gemv_topk.cu:75-135, center_only_topk/gemv_topk.cu:82-119 in small):
+    # 12 centroids, clusters of 16 tokens, top 8 clusters, top 6 tokens of each.  fp16 with 16 heads (128 segments:
+    # the library ranks the centroids inside the token launch), bf16 with 2 heads (a launch of its own).  Three
+    # centroids per head are identical and aligned with the query, so ranks 0-2 are a tie that the lower id must
+    # win, and every cluster holds four equal rows.
+    cl = {}
+    CSZ, CLEN, TOPC, KC = 12, 16, 8, 6
+    for tag, dtype, seed, Hc in (("f16", oracle.F16, 31, 16), ("bf16", oracle.BF16, 32, 2)):
+        rng = np.random.default_rng(seed)
+        cen = rng.uniform(-0.5, 0.5, (Hc, CSZ, 128))
+        qf = rng.uniform(-0.5, 0.5, (Hc, 128))
+        cen[:, [9, 3, 7]] = 0.9 * qf[:, None, :]
+        keys = cen.transpose(1, 0, 2)[:, None, :, :] + 0.05 * rng.standard_normal((CSZ, CLEN, Hc, 128))
+        keys[:, 4:8] = keys[:, 4:5]
+        keys = keys.reshape(CSZ * CLEN, Hc, 128)
+        q, cen_b, keys_b = oracle.to_bits(qf, dtype), oracle.to_bits(cen, dtype), oracle.to_bits(keys, dtype)
+        two = np.stack([oracle.cluster_topk(q[h], cen_b[h], keys_b[:, h, :], dtype, TOPC, CLEN, KC, 1.0) for h in range(Hc)])
+        exp = [oracle.center_topk_expand(q[h], cen_b[h], dtype, TOPC, CLEN, 1.0) for h in range(Hc)]
+        cl.update({tag + "_q": q, tag + "_centers": cen_b, tag + "_keys": keys_b, tag + "_two_level": two,
+                   tag + "_expand": np.stack([e[0] for e in exp]), tag + "_center_ids": np.stack([e[1] for e in exp]),
+                   tag + "_center_val": np.stack([e[2] for e in exp])})
+    cl["params"] = np.array([CSZ, CLEN, TOPC, KC], np.int64)
+    np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "cluster_small.npz"), **cl)
 
 
 if __name__ == "__main__":

@@ -1,5 +1,6 @@
-"""Committed fixtures (tests/golden/, written by make_golden.py): the oracle must still reproduce them, and on a
-GPU the library must match them through the C ABI."""
+"""Committed fixtures (tests/golden/, written by make_golden.py: an end-to-end step, a call of the operator, a
+two-level / centre-only selection): the oracle must still reproduce them, and on a GPU the library must match them
+through the C ABI."""
 import os
 
 import numpy as np
@@ -76,3 +77,37 @@ def test_gpu_matches_operator_fixture(tag, dtype):
     assert np.array_equal(val.cpu().numpy().view(np.uint32), OP[tag + "_val"].view(np.uint32))
     tol = 2e-3 if dtype == oracle.F16 else 2e-3 + np.abs(OP[tag + "_out"]).max() * 2.0 ** -8   # (bf16 output: its own rounding)
     assert np.abs(f32_of(out) - OP[tag + "_out"]).max() < tol
+
+
+CL = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cluster_small.npz"))
+CL_CSZ, CL_CLEN, CL_TOPC, CL_K = (int(x) for x in CL["params"])
+
+
+@pytest.mark.parametrize("tag,dtype", CASES)
+def test_oracle_reproduces_cluster_fixture(tag, dtype):
+    q, cen, keys = CL[tag + "_q"], CL[tag + "_centers"], CL[tag + "_keys"]
+    for h in range(q.shape[0]):
+        two = oracle.cluster_topk(q[h], cen[h], keys[:, h, :], dtype, CL_TOPC, CL_CLEN, CL_K, 1.0)
+        assert np.array_equal(two, CL[tag + "_two_level"][h])
+        out, ids, val = oracle.center_topk_expand(q[h], cen[h], dtype, CL_TOPC, CL_CLEN, 1.0)
+        assert np.array_equal(out, CL[tag + "_expand"][h]) and np.array_equal(ids, CL[tag + "_center_ids"][h])
+        assert np.array_equal(val.view(np.uint32), CL[tag + "_center_val"][h].view(np.uint32))
+        assert list(ids[:3]) == [3, 7, 9]          # the three tied centroids, lower id first
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,dtype", CASES)
+def test_gpu_matches_cluster_fixture(tag, dtype):
+    """Two-level and centre-only selection on the fixture (fp16: 128 segments, centre stage inside the token launch;
+    bf16: 16 segments, centre stage as its own launch)."""
+    import torch
+    from tests.util import announce, to_dev
+    from topk_attn_amd import ops
+    announce("golden cluster fixture %s" % tag)
+    q, cen, keys = to_dev(CL[tag + "_q"], dtype), to_dev(CL[tag + "_centers"], dtype), to_dev(CL[tag + "_keys"], dtype)
+    two = ops.cluster_gemv_topk(q, cen, keys, CL_TOPC, CL_CLEN, CL_K, 1.0)
+    exp = ops.center_topk_expand(q, cen, CL_TOPC, CL_CLEN, 1.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(two.cpu().numpy(), CL[tag + "_two_level"])
+    exp = exp[0] if isinstance(exp, (tuple, list)) else exp
+    assert np.array_equal(exp.cpu().numpy(), CL[tag + "_expand"])
