@@ -13,9 +13,9 @@ def pytest_configure(config):
 
 
 def pytest_sessionstart(session):
-    """What is built is used as it is; only when the library or the command-line program is missing are they made."""
+    """What is built is used as it is; only when the library, the command-line program or the PyTorch extension is missing are they made."""
     lib = os.path.join(ROOT, "topk_attn_amd", "lib")
-    if not all(os.path.exists(os.path.join(lib, f)) for f in ("libtka.so", "tka_standalone")):
+    if not all(os.path.exists(os.path.join(lib, f)) for f in ("libtka.so", "tka_standalone", "retrieval_attention_cpp.so")):
         import topk_attn_amd
         topk_attn_amd.build(force=False)
 

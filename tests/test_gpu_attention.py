@@ -185,13 +185,15 @@ def test_retrieval_attention_op_batches(B, topk):
             assert np.abs(got[b, h] - ref).max() < TOL, "b=%d h=%d" % (b, h)
 
 
-def test_harness_ra(capfd):
+@pytest.mark.parametrize("binding", ["ctypes", "extension"])
+def test_harness_ra(capfd, binding):
     """The harness in the shape of the reference's test_ra.py: PASSED lines per variant, a performance table built
-    from the timing line the op prints on request, exit status 0.  (Parity proper is checked against the oracle in
-    the tests above; the harness's own torch model is held to 5e-3 here, test_ra.py:202 uses 1e-2.)"""
+    from the timing line the op prints on request, exit status 0; through the ctypes binding and through the compiled
+    PyTorch extension module.  (Parity proper is checked against the oracle in the tests above; the harness's own
+    torch model is held to 5e-3 here, test_ra.py:202 uses 1e-2.)"""
     from topk_attn_amd import harness_ra
-    announce("harness_ra --batch 2 --topk 32 256")
-    rc = harness_ra.main(["--batch", "2", "--topk", "32", "256", "--tol", "5e-3"])
+    announce("harness_ra --batch 2 --topk 32 256 --binding %s" % binding)
+    rc = harness_ra.main(["--batch", "2", "--topk", "32", "256", "--tol", "5e-3", "--binding", binding])
     text = capfd.readouterr().out
     assert rc == 0, text[-2000:]
     assert text.count("PASSED") == 12 and "FAILED" not in text

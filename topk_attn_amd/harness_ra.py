@@ -3,7 +3,10 @@ every variant name it runs the op, checks the output against a torch model of th
 PASSED / FAILED per variant and, at the end, the performance table built from the timing line the op prints
 (retrieval_attention.cu:1586-1612 prints that line on every call; here the op is silent unless asked to).
 
-    python -m topk_attn_amd.harness_ra [--batch 4] [--topk 32 128 ...] [--tol 1e-2]
+    python -m topk_attn_amd.harness_ra [--batch 4] [--topk 32 128 ...] [--tol 1e-2] [--binding ctypes|extension]
+
+--binding extension calls the ops of the compiled PyTorch extension module (csrc/torch_ext.cpp, the counterpart of the
+module that test_ra.py:80-85 loads) instead of the ctypes binding; both end in the same C entry point.
 
 The model (test_ra.py:88-160 restated): per head and per 2048-key chunk the K largest q.k (no 1/sqrt(d)),
 softmax over the 4K survivors with raw exp, weighted sum of their V rows.  It runs in fp32 on the GPU with
@@ -70,7 +73,7 @@ def model(q, k, v, topk, num_chunks=ra.NUM_CHUNKS):
     return out
 
 
-def run(topk, batch, tol, results):
+def run(topk, batch, tol, results, mod=ra):
     print("\nTesting with TOPK=%d, BATCH_SIZE=%d..." % (topk, batch))
     torch.manual_seed(0)
     dev = torch.device("cuda")
@@ -85,7 +88,7 @@ def run(topk, batch, tol, results):
         torch.cuda.nvtx.range_push("retrieval_attention%s_%d" % (variant, topk))    # (roctx ranges on ROCm)
         print("Running %s Kernel..." % label)
         with CaptureStdout() as cap:
-            getattr(ra, "retrieval_attention%s_%d" % (variant, topk))(q, k, v, out)
+            getattr(mod, "retrieval_attention%s_%d" % (variant, topk))(q, k, v, out)
             torch.cuda.synchronize()
         torch.cuda.nvtx.range_pop()
         m = re.search(r"Avg time:\s+([\d\.]+)\s+ms,\s+Throughput:\s+([\d\.]+)\s+iter/s", cap.text)
@@ -105,7 +108,12 @@ def main(argv=None):
     ap.add_argument("--batch", type=int, default=4)
     ap.add_argument("--topk", type=int, nargs="*", default=list(L.RA_TOPKS))
     ap.add_argument("--tol", type=float, default=1e-2, help="max-abs tolerance (test_ra.py:202 uses 1e-2)")
+    ap.add_argument("--binding", choices=["ctypes", "extension"], default="ctypes")
     args = ap.parse_args(argv)
+    mod = ra
+    if args.binding == "extension":
+        from . import load_torch_extension
+        mod = load_torch_extension()
     if not torch.cuda.is_available():
         print("harness_ra: no GPU visible", file=sys.stderr)
         return 2
@@ -114,7 +122,7 @@ def main(argv=None):
     os.environ["TKA_BENCH_PRINT"] = "1"          # the named ops then time themselves and print the reference's line
     try:
         for topk in args.topk:
-            ok = run(topk, args.batch, args.tol, results) and ok
+            ok = run(topk, args.batch, args.tol, results, mod) and ok
     finally:
         if before is None:
             del os.environ["TKA_BENCH_PRINT"]
