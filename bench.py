@@ -105,11 +105,11 @@ class SparseDecode:
         # bounded sample: batch entry 0 (1/B of the step); the step is B independent copies of it
         qc, Kc, Vc = self.q[0].cpu(), self.K[0].cpu(), self.V[0].cpu()
         times = []
-        for r in range(runs + 1):
+        for r in range(runs + 2):   # two warm-ups, then the timed runs
             c0 = time.perf_counter()
             ref_out, ref_top = sparse_decode_cpu(qc, Kc, Vc, self.k, self.sink, self.local, SCALE, self.G)
             c1 = time.perf_counter()
-            if r > 0:
+            if r >= 2:
                 times.append(c1 - c0)
         times.sort()
         cpu_s = times[len(times) // 2] * self.B
@@ -304,7 +304,7 @@ def main():
     ap.add_argument("--rotate", type=int, default=0,
                     help="c1, c2, c2-ref, ra: number of key sets taken in turn (working set beyond the Infinity Cache)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-runs", type=int, default=3)
+    ap.add_argument("--cpu-runs", type=int, default=5)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no sharding, no collectives); run with --gpus 1",
