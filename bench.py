@@ -47,6 +47,17 @@ def randn16(torch, shape, dt, g, dev, chunk_dim0=True):
     return out
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def levels16(torch, shape, dt, g, dev):
     """[B, N, H, 128] tensor whose entries take 16 uniform levels in [-2, 2], generated in slices of 131072 tokens."""
     out = torch.empty(shape, device=dev, dtype=dt)
@@ -122,7 +133,7 @@ class SparseDecode:
             got = self.plan.union_idx[0, h, :int(self.plan.union_count[0, h])].tolist()
             same_sets = same_sets and got == sorted(want)
         max_err = (self.plan.out[0].float().cpu() - ref_out).abs().max().item()
-        return cpu_s, {"cores": torch.get_num_threads(), "host_cpus": os.cpu_count(), "kind": "port",
+        return cpu_s, {"cores": torch.get_num_threads(), "host_cpus": os.cpu_count(), "cpu_model": cpu_model(), "kind": "port",
                        "sample": "batch entry 0 of %d (all %d KV heads, full N=%d), median of %d runs, scaled x%d" % (
                            self.B, H, N, runs, self.B),
                        "union_sets_equal_gpu": bool(same_sets), "out_max_abs_diff_vs_gpu": round(max_err, 5)}
