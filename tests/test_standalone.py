@@ -1,5 +1,5 @@
 """tka_standalone, the command-line counterpart of the reference's stand-alone programs (gemv_topk.cu,
-center_only_topk/gemv_topk.cu, baseline_1.cu, flash_decoding.cu mains): argument handling without a GPU, and on a GPU
+center_only_topk/gemv_topk.cu, baseline_1.cu, flash_decoding.cu, retrieval_attention.cu mains): argument handling without a GPU, and on a GPU
 every subcommand with --verify, whose CPU check is computed inside the program."""
 import os
 import subprocess
@@ -30,6 +30,9 @@ def test_usage_and_bad_arguments():
                                        "gemv_topk + flash decode latency:", "✓ GPU indices match", "✓ attention output"]),
     (["flash_decoding", "--verify", "2"], ["flash decode latency:", "✓ attention output"]),
     (["flash_decoding", "--dense", "--verify", "1"], ["flash decode latency:", "✓ attention output"]),
+    (["retrieval_attention", "--batch", "3", "--verify", "2"],
+     ["Baseline Attention - Avg time:", "=== Running Retrieval Attention (Global Memory, TOPK=1024 per block) ===",
+      "Retrieval Attention - Avg time:", "✓ output vs CPU", "Sample output values (head 0, first 8 dims):", "Done!"]),
 ])
 def test_subcommands_verify(args, lines):
     from tests.util import announce

@@ -11,6 +11,9 @@
 //                   baseline_1.cu:613-723
 //   flash_decoding  flash-decoding over a random index list of 2560 tokens per head, flash_decoding.cu:390-480;
 //                   --dense attends to all 40 960 tokens instead
+//   retrieval_attention   the operator's own program, retrieval_attention.cu:2351-2445: dense attention over the 8192
+//                   shared keys as the baseline, then the op for K = 32 ... 1024 per chunk through the
+//                   reference-named launchers (default and _global variant), 100 timed launches each; --batch N
 //
 // The CPU check scores in the library's documented order (16 partial fma chains over 8 dims each, pairwise tree with
 // partner distances 8, 4, 2, 1), so selections are compared for equal order, not only as sets as the reference's
@@ -30,6 +33,7 @@
 #include <vector>
 
 #include "topk_attn.h"
+#include "topk_attn_ra_launchers.h"
 
 namespace {
 
@@ -58,6 +62,7 @@ struct Options {
   int verify_heads = kHeads;
   bool dense = false;
   int centroids = 1024, cluster_len = 128, topc = 64;
+  int batch = 1;
   int warmup = 10, iters = 50;
 };
 
@@ -456,10 +461,115 @@ int run_flash_decoding(const Options& o) {
   return 0;
 }
 
+// ---- retrieval_attention: the operator ------------------------------------------------------------------------
+
+typedef void (*RaLauncher)(const void*, const void*, const void*, void*, int);
+
+// softmax(exp of the 4K surviving scores) . V for one (batch entry, head), in double; survivors = per chunk of 2048
+// keys the K largest scores (library order, no scale, ties to the lower index)
+void operator_on_cpu(const uint16_t* q, const std::vector<uint16_t>& keys, const std::vector<uint16_t>& values, int h, int topk,
+                     double* out) {
+  constexpr int kSeq = 8192, kChunks = 4, kChunk = kSeq / kChunks;
+  std::vector<float> sc(kChunk);
+  std::vector<double> w;
+  std::vector<int> ids;
+  for (int c = 0; c < kChunks; ++c) {
+    for (int t = 0; t < kChunk; ++t) sc[t] = score_in_order(q, &keys[((size_t)(c * kChunk + t) * kHeads + h) * kDim], 1.0f);
+    for (int i : stable_topk(sc, topk)) {
+      ids.push_back(c * kChunk + i);
+      w.push_back(std::exp((double)sc[i]));
+    }
+  }
+  double l = 0.0;
+  for (double x : w) l += x;
+  for (int d = 0; d < kDim; ++d) {
+    double acc = 0.0;
+    for (size_t i = 0; i < ids.size(); ++i) acc += w[i] * (double)half_value(values[((size_t)ids[i] * kHeads + h) * kDim + d]);
+    out[d] = acc / l;
+  }
+}
+
+int run_retrieval_attention(const Options& o) {
+  constexpr int kSeq = 8192;
+  const int B = o.batch;
+  std::printf("Retrieval attention: batch=%d heads=%d dim=%d keys=%d (shared by the batch), 4 chunks of 2048\n", B, kHeads, kDim, kSeq);
+  std::mt19937 rng(2025);
+  std::uniform_real_distribution<float> small(0.0f, 0.1f);   // the value range of retrieval_attention.cu:2286-2296
+  std::vector<uint16_t> q((size_t)B * kHeads * kDim), k((size_t)kSeq * kHeads * kDim), v(k.size());
+  for (auto& x : q) x = half_bits(small(rng));
+  for (size_t i = 0; i < k.size(); ++i) {
+    k[i] = half_bits(small(rng));
+    v[i] = half_bits(small(rng));
+  }
+  uint16_t* d_q = to_device(q);
+  uint16_t* d_k = to_device(k);
+  uint16_t* d_v = to_device(v);
+  uint16_t* d_out = device_buffer<uint16_t>(q.size());
+  Options t = o;
+  t.iters = o.iters == 50 ? 100 : o.iters;   // this program times 100 launches (retrieval_attention.cu:2303)
+  bool ok = true;
+
+  std::printf("\n=== Running Baseline Attention ===\n");
+  {
+    tka_flash_decode_args a{};
+    a.q = d_q; a.keys = d_k; a.values = d_v; a.out = d_out;
+    a.dtype = a.out_dtype = TKA_F16;
+    a.batch = B; a.num_kv_heads = kHeads; a.group = 1; a.head_dim = kDim;
+    a.softmax_mode = TKA_SOFTMAX_SCALED;
+    a.seq_len = kSeq;
+    a.q_stride_b = a.out_stride_b = (int64_t)kHeads * kDim;
+    a.kv_stride_b = 0;
+    a.kv_stride_n = (int64_t)kHeads * kDim;
+    a.kv_stride_h = kDim;
+    a.scale = 1.0f;   // the reference's dense kernel applies no 1/sqrt(d)
+    a.workspace_bytes = tka_flash_decode_workspace_bytes(&a);
+    a.workspace = device_buffer<unsigned char>(a.workspace_bytes);
+    const double us = time_launches(t, [&] { TKA_CALL(tka_flash_decode(&a)); });
+    std::printf("Baseline Attention - Avg time: %.3f ms, Throughput: %.2f iter/s\n", us / 1000.0, 1e6 / us);
+    release(a.workspace);
+  }
+
+  static const struct { int topk; RaLauncher plain, global; } kOps[] = {
+      {32, launch_retrieval_attention_32, launch_retrieval_attention_global_32},
+      {128, launch_retrieval_attention_128, launch_retrieval_attention_global_128},
+      {256, launch_retrieval_attention_256, launch_retrieval_attention_global_256},
+      {512, launch_retrieval_attention_512, launch_retrieval_attention_global_512},
+      {1024, launch_retrieval_attention_1024, launch_retrieval_attention_global_1024}};
+  std::vector<uint16_t> out(q.size());
+  std::vector<double> want(kDim);
+  for (const auto& op : kOps) {
+    for (int variant = 0; variant < 2; ++variant) {
+      std::printf("\n=== Running Retrieval Attention (%sTOPK=%d per block) ===\n", variant ? "Global Memory, " : "", op.topk);
+      const RaLauncher launch = variant ? op.global : op.plain;
+      const double us = time_launches(t, [&] { launch(d_q, d_k, d_v, d_out, B); });
+      std::printf("Retrieval Attention - Avg time: %.3f ms, Throughput: %.2f iter/s\n", us / 1000.0, 1e6 / us);
+      if (o.verify) {
+        HIP_OK(hipMemcpy(out.data(), d_out, out.size() * 2, hipMemcpyDeviceToHost));
+        double worst = 0.0;
+        for (int b = 0; b < B; b += (B > 1 ? B - 1 : 1))          // first and last batch entry
+          for (int h = 0; h < o.verify_heads; ++h) {
+            operator_on_cpu(&q[((size_t)b * kHeads + h) * kDim], k, v, h, op.topk, want.data());
+            for (int d = 0; d < kDim; ++d)
+              worst = std::max(worst, std::fabs(want[d] - (double)half_value(out[((size_t)b * kHeads + h) * kDim + d])));
+          }
+        const bool good = worst < 2e-3;
+        std::printf("%s output vs CPU (double) over %d head(s): max abs diff %.3e (bound 2e-3)\n", good ? "✓" : "✗", o.verify_heads, worst);
+        ok = ok && good;
+      }
+    }
+  }
+  HIP_OK(hipMemcpy(out.data(), d_out, out.size() * 2, hipMemcpyDeviceToHost));
+  std::printf("\nSample output values (head 0, first 8 dims): ");
+  for (int i = 0; i < 8; ++i) std::printf("%.4f ", half_value(out[i]));
+  std::printf("\n\nDone!\n");
+  release(d_out); release(d_v); release(d_k); release(d_q);
+  return ok ? 0 : 1;
+}
+
 void usage() {
   std::fprintf(stderr,
-               "usage: tka_standalone <gemv_topk|center_only|baseline_1|flash_decoding> [--verify [heads]] [--iters N] [--warmup N]\n"
-               "       center_only: [--centroids N] [--cluster-len N] [--topc N]    flash_decoding: [--dense]\n");
+               "usage: tka_standalone <gemv_topk|center_only|baseline_1|flash_decoding|retrieval_attention> [--verify [heads]] [--iters N] [--warmup N]\n"
+               "       center_only: [--centroids N] [--cluster-len N] [--topc N]    flash_decoding: [--dense]    retrieval_attention: [--batch N]\n");
 }
 
 }  // namespace
@@ -491,6 +601,8 @@ int main(int argc, char** argv) {
       ok = int_after(i, 1, 100000, &o.iters);
     } else if (a == "--warmup") {
       ok = int_after(i, 0, 100000, &o.warmup);
+    } else if (a == "--batch") {
+      ok = int_after(i, 1, 4096, &o.batch);
     } else if (a == "--centroids") {
       ok = int_after(i, 1, 1 << 20, &o.centroids);
     } else if (a == "--cluster-len") {
@@ -510,6 +622,7 @@ int main(int argc, char** argv) {
   if (cmd == "center_only") return run_center_only(o);
   if (cmd == "baseline_1") return run_baseline_1(o);
   if (cmd == "flash_decoding") return run_flash_decoding(o);
+  if (cmd == "retrieval_attention") return run_retrieval_attention(o);
   usage();
   return 64;
 }
