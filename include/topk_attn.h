@@ -102,11 +102,30 @@ int tka_gemv_topk(const tka_gemv_topk_args* args);
 int tka_gemv_scores(const tka_gemv_topk_args* args);
 
 /* Diagnostic (no counterpart in the reference): after a tka_gemv_topk call with the same arguments, *count =
- * how many of its segments were redone from the keys by the selection kernel (segments of 65536 tokens and more
- * are selected from candidates above a sampled threshold; a segment whose candidates turn out fewer than k, or
- * more than fit, is redone - exact, but about a millisecond per 131072 tokens).  0 for calls that do not take
- * that path.  Waits for the stream. */
+ * how many of its segments were redone from the keys by the selection kernel.  Long segments are selected from
+ * candidates above a threshold sampled inside the GEMV launch; a segment whose candidates turn out fewer than k,
+ * or more than fit, or one of whose streaming workgroups ran out of its bounded wait for the threshold, is
+ * redone - exact, but about a millisecond per 131072 tokens.  0 for calls that do not take that path.
+ * Waits for the stream. */
 int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* args, int32_t* count);
+/* Same protocol: *count = candidate slices (512 tokens each) of that call whose workgroup gave up waiting. */
+int tka_gemv_topk_gave_up_slices(const tka_gemv_topk_args* args, int32_t* count);
+
+/* Testing hooks (no counterpart in the reference).  Process-wide; read once at the start of every call; they
+ * change how the candidate route of stage 1 gets to its result, never the result.  NULL restores the defaults
+ * (all zero).  Every kernel still runs to its end under any setting: the waits involved are bounded. */
+typedef struct tka_test_hooks {
+  int32_t force_segment_redo;  /* 1: the selection accepts no candidate count, every long segment is redone
+                                  from the keys                                                         */
+  int32_t tau_spin_limit;      /* > 0: polls of a streaming workgroup for its segment's threshold before
+                                  it gives up (default 65536)                                           */
+  int32_t tau_withhold_mod;    /* > 0: the threshold of segments s with s % mod == rem is withheld ...   */
+  int32_t tau_withhold_rem;
+  int32_t tau_withhold_mode;   /* ... 0: for good (every slice of the segment gives up); 1: until the
+                                  first slice of the segment has given up (the later ones see it)       */
+  int32_t reserved0;
+} tka_test_hooks;
+int tka_set_test_hooks(const tka_test_hooks* hooks);
 
 /* ------------------------------------------------------------------------------------------------
  * Stage 1b — selection phase alone on caller-supplied fp32 scores.
@@ -342,6 +361,9 @@ typedef struct tka_sparse_decode_args {
 
 size_t tka_sparse_decode_workspace_bytes(const tka_sparse_decode_args* args);
 int tka_sparse_decode_step(const tka_sparse_decode_args* args);
+/* Diagnostic, as tka_gemv_topk_redone_segments: segments of the last step with these arguments (same workspace)
+ * that the selection kernel redid from the keys.  Waits for the stream. */
+int tka_sparse_decode_redone_segments(const tka_sparse_decode_args* args, int32_t* count);
 
 /* ------------------------------------------------------------------------------------------------
  * Per-kernel timing.  When enabled, every kernel launch made by this library is bracketed by a pair

@@ -13,11 +13,11 @@ def pytest_configure(config):
 
 
 def pytest_sessionstart(session):
-    """What is built is used as it is; only when the library, the command-line program or the PyTorch extension is missing are they made."""
-    lib = os.path.join(ROOT, "topk_attn_amd", "lib")
-    if not all(os.path.exists(os.path.join(lib, f)) for f in ("libtka.so", "tka_standalone", "retrieval_attention_cpp.so")):
-        import topk_attn_amd
-        topk_attn_amd.build(force=False)
+    """What is built is used as it is when it was built from the sources as they are now (a digest of the sources
+    is recorded beside the artefacts); otherwise everything is made again, and a compile error ends the session."""
+    import topk_attn_amd
+    if not topk_attn_amd.is_built():
+        topk_attn_amd.build(force=True)
 
 
 def pytest_collection_modifyitems(config, items):

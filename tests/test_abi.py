@@ -35,7 +35,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = L.lib()
     declared = _declared_symbols()
-    assert len(declared) == 23 + 30
+    assert len(declared) == 26 + 30
     for name in sorted(declared):
         assert hasattr(lib, name), "libtka.so does not export %s" % name
     assert declared == set(L.PROTOTYPES), "ctypes prototypes and headers disagree"
@@ -52,10 +52,26 @@ def test_reference_launcher_names_match_bind_cpp():
         assert callable(getattr(ra, name.replace("launch_", "")))
 
 
+def test_bind_cpp_style_caller_links_unchanged():
+    """The reference's extension declares the thirty launchers with C++ linkage and `half` pointers
+    (bind.cpp:5-243).  libtka.so exports exactly those manglings, and a caller written that way (csrc/bind_link_check.cpp,
+    compiled by g++ with no header of this library) links against it and resolves all thirty."""
+    lib_dir = os.path.join(ROOT, "topk_attn_amd", "lib")
+    syms = subprocess.run(["nm", "-D", "--defined-only", os.path.join(lib_dir, "libtka.so")], capture_output=True, text=True, check=True).stdout
+    for v in L.RA_VARIANTS:
+        for k in L.RA_TOPKS:
+            name = "launch_retrieval_attention%s_%d" % (v, k)
+            mangled = "_Z%d%sPK6__halfS1_S1_PS_i" % (len(name), name)
+            assert re.search(r" T %s$" % re.escape(mangled), syms, flags=re.M), "missing C++ symbol for " + name
+            assert re.search(r" T %s$" % re.escape(name), syms, flags=re.M), "missing C symbol " + name
+    r = subprocess.run([os.path.join(lib_dir, "tka_bind_link_check")], capture_output=True, text=True)
+    assert r.returncode == 0 and "linked 30 launchers declared as in bind.cpp" in r.stdout
+
+
 STRUCTS = {"tka_gemv_topk_args": L.GemvTopkArgs, "tka_topk_args": L.TopkArgs, "tka_center_topk_args": L.CenterTopkArgs,
            "tka_cluster_topk_args": L.ClusterTopkArgs, "tka_index_union_args": L.IndexUnionArgs,
            "tka_flash_decode_args": L.FlashDecodeArgs, "tka_lse_combine_args": L.LseCombineArgs, "tka_ra_args": L.RaArgs,
-           "tka_sparse_decode_args": L.SparseDecodeArgs}
+           "tka_sparse_decode_args": L.SparseDecodeArgs, "tka_test_hooks": L.TestHooks}
 
 
 def test_ctypes_structs_match_the_c_layout():
@@ -193,6 +209,46 @@ def test_other_entry_points_reject_nulls():
     assert lib.tka_retrieval_attention(C.byref(a)) == L.TKA_EWORKSPACE
     a.topk_per_chunk = 4096                                             # more than a chunk holds
     assert lib.tka_retrieval_attention(C.byref(a)) == L.TKA_EINVAL
+
+
+def test_lse_combine_bounds():
+    """The combine kernel keeps one weight per split in LDS: more splits than TKA_MAX_SPLITS are refused before launch."""
+    lib = L.lib()
+    a = L.LseCombineArgs()
+    a.part_m, a.part_l, a.part_acc, a.out = 0x1000, 0x2000, 0x3000, 0x4000
+    a.rows, a.num_splits, a.out_dtype = 4, L.TKA_MAX_SPLITS + 1, L.TKA_F16
+    assert lib.tka_lse_combine(C.byref(a)) == L.TKA_EUNSUPPORTED
+    a.num_splits = 0
+    assert lib.tka_lse_combine(C.byref(a)) == L.TKA_EINVAL
+    a.rows, a.num_splits = 1 << 30, 4
+    assert lib.tka_lse_combine(C.byref(a)) == L.TKA_EUNSUPPORTED
+
+
+def test_sparse_decode_rejects_values_without_indices():
+    lib = L.lib()
+    a = L.SparseDecodeArgs()
+    a.q, a.keys, a.values, a.out = 0x1000, 0x2000, 0x3000, 0x4000
+    a.dtype, a.out_dtype, a.batch, a.num_kv_heads, a.group, a.head_dim = L.TKA_F16, L.TKA_BF16, 1, 8, 4, 128
+    a.k, a.sink, a.local, a.seq_len = 64, 4, 16, 4096
+    a.q_stride_b = a.out_stride_b = 32 * 128
+    a.kv_stride_b, a.kv_stride_n, a.kv_stride_h, a.scale = 4096 * 1024, 1024, 128, 0.088
+    assert lib.tka_sparse_decode_workspace_bytes(C.byref(a)) > 0
+    assert lib.tka_sparse_decode_step(C.byref(a)) == L.TKA_EWORKSPACE     # valid arguments, no workspace
+    a.out_topk_val = 0x5000                                              # values without the rank-ordered ids
+    assert lib.tka_sparse_decode_step(C.byref(a)) == L.TKA_EINVAL
+    n = C.c_int32(-1)
+    a.out_topk_val = None
+    assert lib.tka_sparse_decode_redone_segments(C.byref(a), C.byref(n)) == L.TKA_EWORKSPACE
+    assert lib.tka_sparse_decode_redone_segments(C.byref(a), None) == L.TKA_EINVAL
+
+
+def test_test_hooks_validation():
+    lib = L.lib()
+    assert lib.tka_set_test_hooks(None) == L.TKA_OK
+    assert lib.tka_set_test_hooks(C.byref(L.TestHooks(1, 64, 2, 1, 1, 0))) == L.TKA_OK
+    assert lib.tka_set_test_hooks(C.byref(L.TestHooks(0, -1, 0, 0, 0, 0))) == L.TKA_EINVAL
+    assert lib.tka_set_test_hooks(C.byref(L.TestHooks(0, 0, 0, 0, 2, 0))) == L.TKA_EINVAL
+    assert lib.tka_set_test_hooks(None) == L.TKA_OK
 
 
 def test_profile_interface_without_gpu():

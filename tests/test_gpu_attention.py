@@ -106,6 +106,40 @@ def test_flash_decode_indexed(dtype, G):
             assert (np.abs(out[b, hq] - ref) < out_tol(ref, dtype == oracle.BF16)).all()
 
 
+@pytest.mark.parametrize("dtype,G,logits", [(oracle.F16, 1, False), (oracle.F16, 4, False), (oracle.BF16, 8, False), (oracle.F16, 1, True)])
+def test_flash_decode_indexed_skips_ids_outside_the_cache(dtype, G, logits):
+    """Ids below 0 or at/after seq_len in the MIDDLE of a list are skipped (retrieval_attention.cu:1325); the
+    kernels load row 0 in their place, so row 0 of K and V is filled with infinities here: nothing of it may
+    reach the output (0 * inf).  Token 0 itself is not in the list."""
+    from topk_attn_amd import _lib as L
+    from topk_attn_amd import ops
+    announce("flash_decode indexed with ids outside the cache, dtype=%d G=%d logits=%s" % (dtype, G, logits))
+    rng = np.random.default_rng(170 + G)
+    B, H, N, Lmax = 1, 2, 3000, 600
+    q, K, V = randn_bits(rng, (B, H * G, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype)
+    inf_bits = oracle.to_bits(np.array([np.inf]), dtype)[0]
+    K[:, 0], V[:, 0] = inf_bits, inf_bits
+    idx = np.empty((B, H, Lmax), np.int32)
+    for h in range(H):
+        idx[0, h] = np.sort(rng.choice(np.arange(1, N), Lmax, replace=False))
+    bad = [3, 40, 41, 100, 257, 258, 511]
+    idx[0, 0, bad] = [-1, N, N + 7, -5, 2 ** 31 - 1, -2 ** 31, N]
+    idx[0, 1, 300] = -1
+    lg = (rng.standard_normal((B, H, Lmax)) * 2).astype(np.float32) if logits else None
+    out = ops.flash_decode(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), 1.0 if logits else SCALE, group=G,
+                           kv_idx=torch.from_numpy(idx).cuda(), kv_logit=torch.from_numpy(lg).cuda() if logits else None,
+                           softmax_mode=L.TKA_SOFTMAX_SCALED)
+    torch.cuda.synchronize()
+    out = f32_of(out)
+    assert np.isfinite(out).all()
+    for hq in range(H * G):
+        h = hq // G
+        keep = (idx[0, h] >= 0) & (idx[0, h] < N)
+        ref, _ = oracle.attention_f64(q[0, hq], K[0, :, h], V[0, :, h], dtype, idx=idx[0, h][keep],
+                                      logit=lg[0, h][keep] if logits else None, scale=SCALE)
+        assert (np.abs(out[0, hq] - ref) < out_tol(ref, dtype == oracle.BF16)).all()
+
+
 def test_lse_combine_matches_unsplit():
     from topk_attn_amd import ops
     announce("lse_combine")
@@ -218,6 +252,18 @@ def test_retrieval_attention_variants_agree():
         assert np.array_equal(o, outs[0])
 
 
+def test_bind_cpp_style_caller_runs():
+    """The caller that declares the launchers as the reference's bind.cpp does (C++ linkage, `half` pointers, built
+    by g++ alone) calls one of them on the GPU; the output equals the C symbol's bit for bit."""
+    import os
+    import subprocess
+    announce("tka_bind_link_check run")
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "topk_attn_amd", "lib", "tka_bind_link_check")
+    r = subprocess.run([exe, "run"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "outputs identical" in r.stdout
+
+
 def test_reference_named_launchers():
     """The C-linkage launchers with the reference's names (bind.cpp:5-243), called on the default stream."""
     import ctypes as C
@@ -310,10 +356,41 @@ def test_sparse_decode_step_union_only(dtype, B, H, G, N, k, sink, local, kind, 
             assert (np.abs(out[b, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
 
 
-def test_sparse_decode_step_forced_redo(monkeypatch):
-    """Union mode of the path that redoes a segment from the keys (TKA_FORCE_SEGMENT_REDO), 16-level keys."""
-    monkeypatch.setenv("TKA_FORCE_SEGMENT_REDO", "1")
+@pytest.fixture
+def hooks():
+    """Testing hooks of the candidate route, restored to their defaults afterwards."""
+    from topk_attn_amd import ops
+    yield ops.set_test_hooks
+    ops.set_test_hooks()
+
+
+def test_sparse_decode_step_forced_redo(hooks):
+    """Union mode of the path that redoes a segment from the keys (force_segment_redo hook), 16-level keys."""
+    hooks(force_segment_redo=1)
     test_sparse_decode_step_union_only(oracle.BF16, 1, 2, 4, 66001, 1500, 32, 100, "levels")
+
+
+def test_sparse_decode_step_threshold_never_published(hooks):
+    """Union mode when the streaming workgroups of one segment run out of their wait for the threshold: that segment
+    is redone from the keys, the other keeps the candidate route, union lists and outputs as the oracle's."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step, threshold of segment 0 withheld for good (N=70000 k=1024 G=4)")
+    hooks(tau_spin_limit=64, tau_withhold_mod=2, tau_withhold_rem=0, tau_withhold_mode=0)
+    rng = np.random.default_rng(78)
+    dtype, B, H, G, N, k, sink, local = oracle.F16, 1, 2, 4, 70000, 1024, 16, 128
+    Kf = rng.standard_normal((B, N, H, 128))
+    Kf[:, rng.permutation(N)[:N // 100]] *= 4.0
+    q, K, V = randn_bits(rng, (B, H * G, 128), dtype), oracle.to_bits(Kf, dtype), randn_bits(rng, (B, N, H, 128), dtype)
+    plan = ops.SparseDecodePlan(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), k, sink, local, SCALE, G,
+                                out_dtype=torch.float16, want_topk=False)
+    plan.step()
+    torch.cuda.synchronize()
+    assert plan.redone_segments() == 1
+    out, uidx, ucnt = f32_of(plan.out), plan.union_idx.cpu().numpy(), plan.union_count.cpu().numpy()
+    for h in range(H):
+        ro, ri, rv, ru = oracle.sparse_decode_step(q[0, h * G:(h + 1) * G], K[0, :, h], V[0, :, h], dtype, G, k, sink, local, SCALE)
+        assert ucnt[0, h] == len(ru) and np.array_equal(uidx[0, h, :len(ru)], ru), "union differs (h=%d)" % h
+        assert (np.abs(out[0, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
 
 
 def test_sparse_decode_step_graph_replay():

@@ -126,6 +126,39 @@ def test_c5_tie_stress_full_size(pool):
         assert bool(((got - ref).abs() < 2e-3 + ref.abs() * 2.0 ** -8).all()), "attention output (h=%d)" % h
 
 
+def test_threshold_published_late_some_slices_give_up():
+    """Four segments of a million tokens (2048 candidate slices each, twice what the GPU holds at once).  The
+    threshold of segment 2 is withheld until the first of its streaming workgroups has run out of its (shortened)
+    wait: the first slices of the segment are marked as given up, the later ones see the threshold and store
+    their candidates - more than k of them, which the selection kernel used to accept.  The marked slices force
+    the segment to be redone from the keys; the other three segments keep the candidate route; the result is the
+    stable sort's for every segment, and every kernel runs to its end."""
+    from topk_attn_amd import ops
+    H, N, k = 4, 1 << 20, 4096
+    announce("full size: threshold of one of %d segments of %d tokens published late (k=%d)" % (H, N, k))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(606)
+    K = _randn16((1, N, H, 128), torch.float16, gen)
+    q = torch.randn((1, H, 128), generator=gen, device="cuda").to(torch.float16)
+    ops.set_test_hooks(tau_spin_limit=64, tau_withhold_mod=4, tau_withhold_rem=2, tau_withhold_mode=1)
+    try:
+        plan = ops.GemvTopkPlan(q, K, k, group=1, scale=SCALE).run()
+        torch.cuda.synchronize()
+        redone, gave_up = plan.redone_segments(), plan.gave_up_slices()
+    finally:
+        ops.set_test_hooks()
+    print("late threshold: %d segment(s) redone, %d of 2048 slices gave up" % (redone, gave_up), flush=True)
+    scores = ops.gemv_scores(q, K, group=1, scale=SCALE)
+    torch.cuda.synchronize()
+    _check_selection(scores, plan.idx, plan.val, k)
+    assert redone == 1
+    assert 0 < gave_up < 2048, "the case meant here is a segment with SOME slices given up"
+    plan.run()                                     # the same plan with the hooks off again: nothing is redone
+    torch.cuda.synchronize()
+    assert plan.redone_segments() == 0 and plan.gave_up_slices() == 0
+    _check_selection(scores, plan.idx, plan.val, k)
+
+
 def test_c3_dense_flash_decode_full_size():
     """32 query heads over 8 KV heads, N=131072 fp16: against torch fp32 attention, and across split counts."""
     from topk_attn_amd import ops

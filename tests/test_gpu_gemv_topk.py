@@ -187,13 +187,16 @@ def _sampled_positions(seg, n, samples=2048):
     return [i * stride + _mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) % stride for i in range(samples)]
 
 
-def _check_long(K, q, dtype, G, k, scale=SCALE, redone=None):
-    """`redone`: how many segments the selection kernel is expected to redo from the keys (None: not checked)."""
+def _check_long(K, q, dtype, G, k, scale=SCALE, redone=None, gave_up=None):
+    """`redone`: how many segments the selection kernel is expected to redo from the keys (None: not checked);
+    `gave_up`: how many candidate slices are expected to come from workgroups whose wait for the threshold ran out."""
     from topk_attn_amd import ops
     plan = ops.GemvTopkPlan(to_dev(q, dtype), to_dev(K, dtype), k, group=G, scale=scale).run()
     torch.cuda.synchronize()
     if redone is not None:
         assert plan.redone_segments() == redone
+    if gave_up is not None:
+        assert plan.gave_up_slices() == gave_up
     idx, val = plan.idx.cpu().numpy(), plan.val.cpu().numpy()
     B, N, H = K.shape[:3]
     for b in range(B):
@@ -349,12 +352,36 @@ def test_long_segment_plan_reuse():
         assert np.array_equal(plan.val[0, 0].cpu().numpy().view(np.uint32), ev.view(np.uint32))
 
 
-def test_long_segment_forced_redo(monkeypatch):
-    """TKA_FORCE_SEGMENT_REDO sends every long segment through the path that redoes it from the keys — here on
+@pytest.fixture
+def hooks():
+    """Testing hooks of the candidate route, restored to their defaults afterwards."""
+    from topk_attn_amd import ops
+    yield ops.set_test_hooks
+    ops.set_test_hooks()
+
+
+def test_long_segment_forced_redo(hooks):
+    """The force_segment_redo hook sends every long segment through the path that redoes it from the keys — here on
     ordinary data with heavy hitters, in rank mode, with a ragged length."""
     announce("gemv_topk long segment, every segment redone from the keys (N=70001 k=3000 G=4)")
-    monkeypatch.setenv("TKA_FORCE_SEGMENT_REDO", "1")
+    hooks(force_segment_redo=1)
     rng = np.random.default_rng(39)
     K = randn_bits(rng, (1, 70001, 2, 128), oracle.F16)
     K[0, rng.permutation(70001)[:700]] = oracle.to_bits(rng.standard_normal((700, 2, 128)) * 4.0, oracle.F16)
     _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 3000, redone=2)
+
+
+@pytest.mark.parametrize("withheld", [(2, 1), (1, 0)])
+def test_long_segment_threshold_never_published(hooks, withheld):
+    """The bounded wait of the streaming workgroups runs out: the threshold of one of the two segments (then of
+    both) is never published, the spin limit is lowered so that the wait is short, every slice of such a segment
+    is marked as given up, and the selection kernel redoes exactly those segments from the keys.  The segment
+    that did get its threshold keeps the candidate route.  Every kernel runs to its end."""
+    mod, rem = withheld
+    announce("gemv_topk long segments, threshold of segments s %% %d == %d withheld for good (N=131072 k=2048)" % (mod, rem))
+    hooks(tau_spin_limit=64, tau_withhold_mod=mod, tau_withhold_rem=rem, tau_withhold_mode=0)
+    rng = np.random.default_rng(43)
+    K = randn_bits(rng, (1, 131072, 2, 128), oracle.F16)
+    K[0, rng.permutation(131072)[:1300]] = oracle.to_bits(rng.standard_normal((1300, 2, 128)) * 4.0, oracle.F16)
+    affected = 2 // mod
+    _check_long(K, randn_bits(rng, (1, 2, 128), oracle.F16), oracle.F16, 1, 2048, redone=affected, gave_up=affected * 256)

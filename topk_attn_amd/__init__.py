@@ -10,14 +10,47 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 TORCH_EXT_PATH = os.path.join(_HERE, "lib", "retrieval_attention_cpp.so")
 
 
+STAMP_PATH = os.path.join(_HERE, "lib", "BUILD_STAMP")
+ARTEFACTS = ("libtka.so", "tka_standalone", "tka_bind_link_check", "retrieval_attention_cpp.so")
+
+
+def source_digest():
+    """SHA-256 over the names and contents of everything the built artefacts are made from."""
+    import hashlib
+    h = hashlib.sha256()
+    roots = [os.path.join(_HERE, "csrc"), os.path.join(_HERE, "..", "include")]
+    for root in roots:
+        for name in sorted(os.listdir(root)):
+            path = os.path.join(root, name)
+            if os.path.isfile(path):
+                h.update(name.encode() + b"\0")
+                with open(path, "rb") as f:
+                    h.update(f.read())
+    return h.hexdigest()
+
+
+def is_built():
+    """True when every artefact exists and was built from the sources as they are now (by content, not by time)."""
+    lib = os.path.join(_HERE, "lib")
+    if not all(os.path.exists(os.path.join(lib, f)) for f in ARTEFACTS) or not os.path.exists(STAMP_PATH):
+        return False
+    with open(STAMP_PATH) as f:
+        return f.read().strip() == source_digest()
+
+
 def build(force=True, jobs=8):
-    """Compile libtka.so for gfx950 and tka_standalone with hipcc, and the PyTorch extension module
-    retrieval_attention_cpp with g++ (no GPU needed).  force=False makes only what is missing or out of date."""
+    """Compile libtka.so for gfx950, tka_standalone and tka_bind_link_check with hipcc, and the PyTorch extension
+    module retrieval_attention_cpp with g++ (no GPU needed).  force=False makes only what is missing or out of date.
+    Raises when any compile fails; on success records the digest of the sources next to the artefacts."""
+    if os.path.exists(STAMP_PATH):
+        os.remove(STAMP_PATH)
     cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j%d" % jobs]
     if force:
         cmd.append("-B")
     subprocess.check_call(cmd)
     build_torch_extension(force)
+    with open(STAMP_PATH, "w") as f:
+        f.write(source_digest() + "\n")
     return os.path.join(_HERE, "lib", "libtka.so")
 
 

@@ -77,6 +77,11 @@ class SparseDecodeArgs(C.Structure):
                 ("stream", _p)]
 
 
+class TestHooks(C.Structure):
+    _fields_ = [("force_segment_redo", _i32), ("tau_spin_limit", _i32), ("tau_withhold_mod", _i32),
+                ("tau_withhold_rem", _i32), ("tau_withhold_mode", _i32), ("reserved0", _i32)]
+
+
 RA_VARIANTS = ("", "_global", "_pipelined", "_pipelined_global", "_two_kernels", "_gather_baseline")
 RA_TOPKS = (32, 128, 256, 512, 1024)
 
@@ -88,6 +93,8 @@ PROTOTYPES = {
     "tka_gemv_topk": (C.c_int, [C.POINTER(GemvTopkArgs)]),
     "tka_gemv_scores": (C.c_int, [C.POINTER(GemvTopkArgs)]),
     "tka_gemv_topk_redone_segments": (C.c_int, [C.POINTER(GemvTopkArgs), C.POINTER(C.c_int32)]),
+    "tka_gemv_topk_gave_up_slices": (C.c_int, [C.POINTER(GemvTopkArgs), C.POINTER(C.c_int32)]),
+    "tka_set_test_hooks": (C.c_int, [C.POINTER(TestHooks)]),
     "tka_topk_workspace_bytes": (_sz, [C.POINTER(TopkArgs)]),
     "tka_topk_f32": (C.c_int, [C.POINTER(TopkArgs)]),
     "tka_center_topk_expand_workspace_bytes": (_sz, [C.POINTER(CenterTopkArgs)]),
@@ -102,6 +109,7 @@ PROTOTYPES = {
     "tka_retrieval_attention": (C.c_int, [C.POINTER(RaArgs)]),
     "tka_sparse_decode_workspace_bytes": (_sz, [C.POINTER(SparseDecodeArgs)]),
     "tka_sparse_decode_step": (C.c_int, [C.POINTER(SparseDecodeArgs)]),
+    "tka_sparse_decode_redone_segments": (C.c_int, [C.POINTER(SparseDecodeArgs), C.POINTER(C.c_int32)]),
     "tka_profile_enable": (C.c_int, [C.c_int]),
     "tka_profile_reset": (C.c_int, []),
     "tka_profile_read": (C.c_int, [C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.POINTER(_i64), C.c_int]),

@@ -79,6 +79,14 @@ LaunchTimer::~LaunchTimer() {
 
 namespace {
 
+// Testing hooks (tka_set_test_hooks): process-wide, read once per call.
+std::mutex g_hooks_mutex;
+tka_test_hooks g_hooks = {0, 0, 0, 0, 0, 0};
+tka_test_hooks current_hooks() {
+  std::lock_guard<std::mutex> lock(g_hooks_mutex);
+  return g_hooks;
+}
+
 bool dtype_ok(int d) { return d == TKA_F16 || d == TKA_BF16; }
 bool group_ok(int g) { return g == 1 || g == 2 || g == 4 || g == 8; }
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
@@ -132,6 +140,9 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->sample_flags = nullptr;
   g->sample_pool = nullptr;
   g->epoch = 0;
+  g->seg_flags = nullptr;
+  g->tau_spin_limit = kTauSpinLimit;
+  g->withhold_mod = g->withhold_rem = g->withhold_mode = 0;
   g->num_samples = g->sample_rank = g->sample_wgs = g->early_wgs = 0;
   g->cand = nullptr;
   g->cand_seg_stride = 0;
@@ -284,6 +295,12 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   cp.sample_flags = sp.sample_flags;
   cp.sample_pool = sp.sample_pool;
   cp.epoch = call_counter.fetch_add(1, std::memory_order_relaxed) | 0x80000000u;   // never 0, the cleared state
+  const tka_test_hooks hooks = current_hooks();
+  cp.seg_flags = sp.seg_flags;
+  if (hooks.tau_spin_limit > 0) cp.tau_spin_limit = hooks.tau_spin_limit;
+  cp.withhold_mod = hooks.tau_withhold_mod > 0 ? hooks.tau_withhold_mod : 0;
+  cp.withhold_rem = hooks.tau_withhold_rem;
+  cp.withhold_mode = hooks.tau_withhold_mode;
   cp.num_samples = num_samples;
   cp.sample_rank = sample_rank;
   cp.cand = sp.list;
@@ -295,8 +312,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   sc.parts = cp.wgs_per_chunk;
   sc.part_len = cp.tokens_per_wg;
   sc.list_stride = sp.list_stride;
-  // TKA_FORCE_SEGMENT_REDO (testing): no candidate count is acceptable, every segment is redone from the keys
-  sc.max_entries = getenv("TKA_FORCE_SEGMENT_REDO") ? 0 : select_cand_capacity();
+  // testing hook: no candidate count is acceptable, every segment is redone from the keys
+  sc.max_entries = hooks.force_segment_redo ? 0 : select_cand_capacity();
   sc.scores = scores;
   return launch_select_finalize_cand(gp, sc, a->dtype, stream);
 }
@@ -453,9 +470,10 @@ int tka_gemv_topk(const tka_gemv_topk_args* a) {
   return run_gemv_topk(a, nullptr, 0);
 }
 
-int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* a, int32_t* count) {
-  if (!count) return TKA_EINVAL;
-  *count = 0;
+// Per-segment flag words of the last candidate-route call with these arguments (bit 0: redone from the keys,
+// bits 8..: slices whose workgroup gave up waiting for the threshold); empty for calls that take another route.
+static int read_segment_flags(const tka_gemv_topk_args* a, std::vector<uint32_t>* flags) {
+  flags->clear();
   int rc = check_gemv(a, true);
   if (rc != TKA_OK) return rc;
   if (!a->workspace || a->workspace_bytes < tka_gemv_topk_workspace_bytes(a)) return TKA_EWORKSPACE;
@@ -466,10 +484,37 @@ int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* a, int32_t* count) {
   SelectParams sp;
   memset(&sp, 0, sizeof sp);
   select_carve((unsigned char*)a->workspace + gemv_scores_bytes(a), segs, a->seq_len / a->num_chunks, &sp);
-  std::vector<uint32_t> flags((size_t)segs);
+  flags->resize((size_t)segs);
   if (hipStreamSynchronize((hipStream_t)a->stream) != hipSuccess) return TKA_EHIP;
-  if (hipMemcpy(flags.data(), sp.seg_flags, flags.size() * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return TKA_EHIP;
-  for (uint32_t f : flags) *count += f ? 1 : 0;
+  if (hipMemcpy(flags->data(), sp.seg_flags, flags->size() * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return TKA_EHIP;
+  return TKA_OK;
+}
+
+int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* a, int32_t* count) {
+  if (!count) return TKA_EINVAL;
+  *count = 0;
+  std::vector<uint32_t> flags;
+  const int rc = read_segment_flags(a, &flags);
+  for (uint32_t f : flags) *count += (int32_t)(f & 1u);
+  return rc;
+}
+
+int tka_gemv_topk_gave_up_slices(const tka_gemv_topk_args* a, int32_t* count) {
+  if (!count) return TKA_EINVAL;
+  *count = 0;
+  std::vector<uint32_t> flags;
+  const int rc = read_segment_flags(a, &flags);
+  for (uint32_t f : flags) *count += (int32_t)(f >> 8);
+  return rc;
+}
+
+int tka_set_test_hooks(const tka_test_hooks* hooks) {
+  if (hooks && (hooks->tau_spin_limit < 0 || hooks->tau_withhold_mod < 0 || hooks->tau_withhold_rem < 0 ||
+                (hooks->tau_withhold_mode != 0 && hooks->tau_withhold_mode != 1)))
+    return TKA_EINVAL;
+  std::lock_guard<std::mutex> lock(g_hooks_mutex);
+  if (hooks) g_hooks = *hooks;
+  else g_hooks = tka_test_hooks{0, 0, 0, 0, 0, 0};
   return TKA_OK;
 }
 
@@ -703,6 +748,8 @@ int tka_lse_combine(const tka_lse_combine_args* a) {
   if (!a || !a->part_m || !a->part_l || !a->part_acc || !a->out) return TKA_EINVAL;
   if (a->rows < 1 || a->num_splits < 1) return TKA_EINVAL;
   if (!dtype_ok(a->out_dtype)) return TKA_EUNSUPPORTED;
+  // the kernel keeps one weight per split in LDS; one workgroup per row on a 1-D grid
+  if (a->num_splits > TKA_MAX_SPLITS || (int64_t)a->rows * a->num_splits > 0x7fffffffLL) return TKA_EUNSUPPORTED;
   CombineParams cp;
   memset(&cp, 0, sizeof cp);
   cp.part_m = a->part_m;
@@ -921,11 +968,32 @@ size_t tka_sparse_decode_workspace_bytes(const tka_sparse_decode_args* a) {
          tka_gemv_topk_workspace_bytes(&g) + flash_bytes(&f);
 }
 
+// Offset of the stage-1 workspace inside the workspace of the step.
+static size_t sd_gemv_ws_offset(const tka_sparse_decode_args* a, const tka_flash_decode_args& f) {
+  const size_t segs = (size_t)a->batch * a->num_kv_heads;
+  return align_up(segs * a->k * sizeof(int32_t), 256) + align_up(segs * a->k * sizeof(float), 256) +
+         align_up(segs * (size_t)f.idx_len * sizeof(int32_t), 256) + align_up(segs * sizeof(int32_t), 256);
+}
+
+int tka_sparse_decode_redone_segments(const tka_sparse_decode_args* a, int32_t* count) {
+  if (!count) return TKA_EINVAL;
+  *count = 0;
+  tka_gemv_topk_args g;
+  tka_flash_decode_args f;
+  int rc = sd_check(a, &g, &f);
+  if (rc != TKA_OK) return rc;
+  if (!a->workspace || a->workspace_bytes < tka_sparse_decode_workspace_bytes(a)) return TKA_EWORKSPACE;
+  g.workspace = (unsigned char*)a->workspace + sd_gemv_ws_offset(a, f);
+  g.workspace_bytes = tka_gemv_topk_workspace_bytes(&g);
+  return tka_gemv_topk_redone_segments(&g, count);
+}
+
 int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
   tka_gemv_topk_args g;
   tka_flash_decode_args f;
   int rc = sd_check(a, &g, &f);
   if (rc != TKA_OK) return rc;
+  if (a->out_topk_val && !a->out_topk_idx) return TKA_EINVAL;   // values come with the rank-ordered ids only
   const size_t need = tka_sparse_decode_workspace_bytes(a);
   if (!a->workspace || a->workspace_bytes < need) return TKA_EWORKSPACE;
   const size_t segs = (size_t)a->batch * a->num_kv_heads;

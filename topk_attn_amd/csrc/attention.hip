@@ -121,6 +121,19 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
       vv[u] = MODE == MODE_DENSE ? __builtin_nontemporal_load(vsrc) : *vsrc;
     }
     if (MODE != MODE_DENSE) fetch_ids(base + kStep);
+    if (MODE != MODE_DENSE) {
+      // A skipped id had row 0 loaded in its place (and a position past the end of the list the last row): its
+      // weight is 0, but 0 * inf would still poison the sum, so such a V row is cleared.  Wave-uniform test:
+      // steps made of valid ids only pay one ballot.
+      bool skipped = false;
+#pragma unroll
+      for (int u = 0; u < U; ++u) skipped |= !valid[u];
+      if (__ballot(skipped) != 0ull) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (!valid[u]) vv[u] = (u32x4){0u, 0u, 0u, 0u};
+      }
+    }
     float x[G][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {

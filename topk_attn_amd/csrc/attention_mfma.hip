@@ -111,13 +111,14 @@ __global__ __launch_bounds__(kThreads) void attn_mfma_kernel(AttnParams p) {
     }
     int64_t tv[8];
     bool okv[8];
+    bool skipped = false;   // an id outside the cache among this lane's slots
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int64_t pos = tile + slot_token(j, s);
       okv[s] = pos < end;
       const int64_t pc = okv[s] ? pos : end - 1;
       int64_t t = INDEXED ? (int64_t)idx[pc] : pc;
-      if (INDEXED && (t < 0 || t >= p.seq_len)) { okv[s] = false; t = 0; }
+      if (INDEXED && (t < 0 || t >= p.seq_len)) { okv[s] = false; t = 0; skipped = true; }
       tv[s] = t;
     }
     // ---- loads: 8 x 16 B of K (2 tiles x 4 k-blocks), 8 x 16 B of V (8 rows).  A K request covers half a line
@@ -179,8 +180,9 @@ __global__ __launch_bounds__(kThreads) void attn_mfma_kernel(AttnParams p) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[c][i] *= ah[i];
 
-    // ---- V rows of masked tokens must not reach the product (0 * inf)
-    if (tile + kTile > end) {
+    // ---- V rows of masked tokens (past the end of the list, or ids outside the cache, whose slot loaded row 0
+    // instead) must not reach the product (0 * inf).  Wave-uniform test: full tiles of valid ids skip the selects.
+    if (tile + kTile > end || (INDEXED && __ballot(skipped) != 0ull)) {
 #pragma unroll
       for (int s = 0; s < 8; ++s)
         if (!okv[s]) vr[s] = (u32x4){0u, 0u, 0u, 0u};

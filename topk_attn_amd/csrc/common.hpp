@@ -26,6 +26,10 @@ constexpr int kGemvInlineCentres = 256;     // centroids per head that the GEMV 
 constexpr int64_t kCandMinSegLen = 32768;   // shorter segments never take the candidate mode
 constexpr int64_t kCandMinRows = 1 << 20;   // ... nor do segments below 65536 tokens unless the call has this many rows
 constexpr int kGemvMaxSamples = 8192;      // most samples per segment of the candidate-mode threshold estimate
+constexpr int kTauSpinLimit = 1 << 16;     // polls of a streaming workgroup for its threshold before it gives up
+// Count field (10 bits) of a candidate slice whose workgroup never saw its threshold: no real slice holds more than
+// 512 candidates, so the selection kernel cannot take it for a count, and it redoes the segment from the keys.
+constexpr uint32_t kSliceGaveUp = 1023u;
 
 // ---- lane exchanges ---------------------------------------------------------------------------
 

@@ -29,7 +29,6 @@ namespace {
 constexpr int kGemvThreads = 256;
 constexpr int kGemvUnroll = 8;                                         // loads in flight per lane
 constexpr int kGemvRowsPerIter = (kGemvThreads / 16) * kGemvUnroll;    // 128 tokens per WG iteration
-constexpr int kTauSpinLimit = 1 << 16; // polls of a streaming workgroup for its threshold before it gives up
 constexpr int kEarlySlices = 3;        // slices of a streaming workgroup that starts before the threshold is published
 constexpr int kCandThreads = kGemvCandTokensPerWg;                     // candidate kernel: one thread per token of the slice
 constexpr int kCandWaves = kCandThreads / kWave;
@@ -447,6 +446,17 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
       cut = sh_wtot[14];
     }
   }
+  if (p.withhold_mod > 0 && seg % p.withhold_mod == p.withhold_rem) {
+    // testing: this segment's threshold is withheld, so that streaming workgroups run into the end of their
+    // bounded wait.  Mode 0: for good.  Mode 1: until one of them has given up (it leaves the call's epoch in the
+    // segment's flag word), or this wait, bounded like theirs, runs out.
+    if (p.withhold_mode == 0) return;
+    if (tid == 0) {
+      const uint32_t* flag = p.seg_flags + seg;
+      for (int spin = 0; spin < kTauSpinLimit && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != p.epoch; ++spin)
+        __builtin_amdgcn_s_sleep(16);
+    }
+  }
   if (tid == 0) {
     // the cut first, then, once it has completed, the word the streaming workgroups wait for
     __hip_atomic_store(p.tau_words + 2 * seg + 1, (uint64_t)cut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -556,14 +566,15 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
     if (t_end > p.chunk_len) t_end = p.chunk_len;
     // Threshold of the slice's segment: one lane fetches the word and hands it on through LDS (every wave
     // asking for itself makes a hot spot of the few words).  A bounded wait: a workgroup that never sees its
-    // threshold stores no candidates, and the selection kernel then redoes the segment from the keys.
+    // threshold stores no candidates and marks its slice (kSliceGaveUp in the count field); the selection kernel
+    // redoes a segment that holds such a slice from the keys, however many candidates the other slices hold.
     if (s == 0 || seg != tau_seg) {
       tau_seg = seg;
       if (s) __syncthreads();   // the previous slice's threshold has been read
       if (tid == 0) {
         const uint64_t* word = p.tau_words + 2 * seg;
         uint64_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (int spin = 0; (uint32_t)(v >> 32) != p.epoch && spin < kTauSpinLimit; ++spin) {
+        for (int spin = 0; (uint32_t)(v >> 32) != p.epoch && spin < p.tau_spin_limit; ++spin) {
           __builtin_amdgcn_s_sleep(16);
           v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -599,7 +610,8 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
       const uint32_t pos = before + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
       slice[pos] = ((uint64_t)key << 32) | (pos == 0 ? total << 9 : 0u) | (uint32_t)tid;
     }
-    if (tid == 0 && total == 0) slice[0] = 0ull;
+    if (tid == 0 && total == 0) slice[0] = tau_ready ? 0ull : (uint64_t)(kSliceGaveUp << 9);
+    if (tid == 0 && !tau_ready) __hip_atomic_store(p.seg_flags + seg, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (++wg_in_chunk == p.wgs_per_chunk) { wg_in_chunk = 0; ++seg; }
   }
 }

@@ -21,6 +21,11 @@ struct GemvParams {
   uint32_t* sample_flags;     // [segments][64] epoch of the call in which that sampling workgroup last arrived
   uint32_t* sample_pool;      // [segments][num_samples] keys of the sampled tokens
   uint32_t epoch;             // tells this call's words from older contents of the workspace (never 0)
+  uint32_t* seg_flags;        // [segments] a streaming workgroup whose wait for the threshold expired stores the epoch here
+  int tau_spin_limit;         // polls of a streaming workgroup for its threshold before it gives up
+  // testing (tka_test_hooks): the threshold of segments with seg % withhold_mod == withhold_rem is never published
+  // (mode 0) or published only once a slice of the segment has given up, after a bounded wait (mode 1); 0 = off
+  int withhold_mod, withhold_rem, withhold_mode;
   int num_samples, sample_rank;   // per segment
   int sample_wgs;             // sampling workgroups at the front of the candidate grid (set by the launcher)
   int early_wgs;              // streaming workgroups behind them that take several slices each (set by the launcher)
@@ -49,7 +54,8 @@ struct SelectParams {
   uint64_t* tau_words;    // [num_segments][2] candidate thresholds (workspace); the candidate selection kernel clears them
   uint32_t* sample_flags; // [num_segments][64] arrival flags of the sampling workgroups (workspace)
   uint32_t* sample_pool;  // [num_segments][kGemvMaxSamples] sampled keys (workspace)
-  uint32_t* seg_flags;    // [num_segments] candidate mode writes 1 when a segment was redone from the keys
+  uint32_t* seg_flags;    // [num_segments] candidate mode: bit 0 = the segment was redone from the keys, bits 8.. = how many
+                          // of its slices came from workgroups whose wait for the threshold had expired
   int max_entries;        // candidate mode: a segment with more candidates than this is also redone from the keys
   int from_keys;          // candidate selection kernel: no slices, the workgroup scores its (short) segment itself
   int from_scores;        // candidate selection kernel: no slices, the entries are all scores of the segment (<= 16384)

@@ -619,7 +619,8 @@ constexpr int kSmallBucket = 64;   // a threshold bucket of this many entries or
 // index inside and across slices (format: GemvParams::cand).  One workgroup per segment copies them into LDS
 // as composites (entry v of the segment at position v), finds the k-th largest composite by radix passes that start below the common prefix of
 // the smallest and largest candidate, and walks the entries once in index order.
-// A segment with fewer than k candidates, or more than fit, is redone by fallback_segment (and flagged in
+// A segment with fewer than k candidates, or more than fit, or with a slice whose workgroup gave up waiting for
+// the threshold (such a slice holds none of its candidates), is redone by fallback_segment (and flagged in
 // seg_flags, for the curious).
 // Dynamic LDS: kCandCap composites; rank mode reuses them as sort and exchange buffers.
 template <int DT>
@@ -637,11 +638,14 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   __shared__ uint64_t sh_mm[3];
   __shared__ uint64_t sh_small[kSmallBucket];
   __shared__ uint32_t sh_small_cnt;
+  __shared__ uint32_t sh_gave_up;   // slices of this segment whose workgroup never saw the threshold
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
+  if (tid == 0) sh_gave_up = 0u;
+  __syncthreads();
 
   // Copy the slices into LDS.  Up to kRound slices: 32 lanes per slice load its first 32 entries (entry 0 carries
   // the slice's count; entries beyond the count are stale memory and ignored), the counts are scanned into
@@ -706,6 +710,10 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
         cnt[u] = ((uint32_t)__shfl((int)(uint32_t)first[u], lane & ~(kSliceLanes - 1), 64) >> 9) & 0x3ffu;
+        if (cnt[u] == kSliceGaveUp) {
+          cnt[u] = 0u;
+          if (sub == 0) atomicAdd(&sh_gave_up, 1u);
+        }
         if (sub == 0) sh_cnt[u * kGroups + grp] = cnt[u];
       }
       __syncthreads();
@@ -735,6 +743,10 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     for (int q = 0; q < 4; ++q) {
       const int sl = 4 * tid + q;
       c4[q] = sl < p.parts ? ((uint32_t)lists[(int64_t)sl * p.part_len] >> 9) & 0x3ffu : 0u;
+      if (c4[q] == kSliceGaveUp) {
+        c4[q] = 0u;
+        atomicAdd(&sh_gave_up, 1u);
+      }
       sum += c4[q];
     }
     uint32_t total;
@@ -774,14 +786,16 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     }
   }
   const bool whole = p.from_keys || p.from_scores;   // the entries are the whole segment, not candidate slices
-  const bool redo = !whole && (n_entries < k || n_entries > cap);
+  // (every add to sh_gave_up lies in front of a barrier of the copy)
+  const uint32_t n_gave_up = sh_gave_up;
+  const bool redo = !whole && (n_entries < k || n_entries > cap || n_gave_up != 0u);
   if (tid == 0) {
     sh_small_cnt = 0;
     sh_kminmax[0] = ~0u;
     sh_kminmax[1] = 0u;
   }
   if (!whole) {
-    if (tid == 0) p.seg_flags[seg] = redo ? 1u : 0u;
+    if (tid == 0) p.seg_flags[seg] = (redo ? 1u : 0u) | (n_gave_up << 8);
     // the threshold and the arrival flags are spent: a replay of the same launches (a captured graph) must not
     // take them for its own
     if (tid >= 64 && tid < 128) p.sample_flags[(int64_t)seg * 64 + (tid - 64)] = 0u;

@@ -24,13 +24,23 @@ def _stream():
 
 
 def _workspace(nbytes, device):
-    """One growing byte buffer per (device, stream); calls on one stream are ordered, so they may share it."""
+    """Workspace of the one-shot wrappers: one growing byte buffer per (device, stream), looked up by the stream the
+    call is about to be launched on; calls on one stream are ordered, so they may share it.  Never grown during a
+    graph capture (the allocation would belong to the capture's pool and be handed to later eager calls)."""
     key = (device.index, torch.cuda.current_stream().cuda_stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("the workspace of this stream must exist before a graph capture: call once eagerly, "
+                               "or use a plan object (it owns its workspace)")
         buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
+
+
+def _own_workspace(nbytes, device):
+    """Workspace of a plan object: its own buffer, so that plans run on different streams never share one."""
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
 def _need_cuda(*tensors):
@@ -83,7 +93,7 @@ class GemvTopkPlan:
         a.out_idx, a.out_val = self.idx.data_ptr(), self.val.data_ptr()
         a.out_scores = self.scores.data_ptr() if self.scores is not None else None
         need = L.lib().tka_gemv_topk_workspace_bytes(C.byref(a))
-        self.ws = _workspace(need, q.device)
+        self.ws = _own_workspace(need, q.device)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
         self.args = a
         self._fn = L.lib().tka_gemv_topk
@@ -97,6 +107,12 @@ class GemvTopkPlan:
         """Diagnostic: segments of the last run() that the selection kernel had to redo from the keys."""
         n = C.c_int32(0)
         L.check(L.lib().tka_gemv_topk_redone_segments(C.byref(self.args), C.byref(n)), "tka_gemv_topk_redone_segments")
+        return n.value
+
+    def gave_up_slices(self):
+        """Diagnostic: candidate slices of the last run() whose workgroup ran out of its wait for the threshold."""
+        n = C.c_int32(0)
+        L.check(L.lib().tka_gemv_topk_gave_up_slices(C.byref(self.args), C.byref(n)), "tka_gemv_topk_gave_up_slices")
         return n.value
 
 
@@ -164,7 +180,7 @@ class CenterTopkPlan:
         a.scale = scale
         a.out_idx, a.out_centers, a.out_center_val = self.out.data_ptr(), self.cen.data_ptr(), self.val.data_ptr()
         need = L.lib().tka_center_topk_expand_workspace_bytes(C.byref(a))
-        self.ws = _workspace(need, q.device)
+        self.ws = _own_workspace(need, q.device)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
 
     def run(self):
@@ -247,7 +263,7 @@ class FlashDecodePlan:
                 a.kv_logit = self.kv_logit.data_ptr()
         a.out_lse = self.lse.data_ptr() if self.lse is not None else None
         need = L.lib().tka_flash_decode_workspace_bytes(C.byref(a))
-        self.ws = _workspace(need, q.device)
+        self.ws = _own_workspace(need, q.device)
         a.workspace, a.workspace_bytes = self.ws.data_ptr(), self.ws.numel()
         self.args = a
         self._fn = L.lib().tka_flash_decode
@@ -352,6 +368,12 @@ class SparseDecodePlan:
             L.check(rc, "tka_sparse_decode_step")
         return self.out
 
+    def redone_segments(self):
+        """Diagnostic: segments of the last step() that the selection kernel had to redo from the keys."""
+        n = C.c_int32(0)
+        L.check(L.lib().tka_sparse_decode_redone_segments(C.byref(self.args), C.byref(n)), "tka_sparse_decode_redone_segments")
+        return n.value
+
 
 def sparse_decode_step(q, keys, values, k, sink, local, scale, group, out_dtype=None, num_splits=0, want_topk=True):
     """End-to-end decode step.  Returns (out, topk_idx, topk_val, union_idx, union_count); without want_topk the
@@ -359,6 +381,12 @@ def sparse_decode_step(q, keys, values, k, sink, local, scale, group, out_dtype=
     plan = SparseDecodePlan(q, keys, values, k, sink, local, scale, group, out_dtype, num_splits, want_topk=want_topk)
     plan.step()
     return plan.out, plan.topk_idx, plan.topk_val, plan.union_idx, plan.union_count
+
+
+def set_test_hooks(force_segment_redo=0, tau_spin_limit=0, tau_withhold_mod=0, tau_withhold_rem=0, tau_withhold_mode=0):
+    """Testing hooks of the candidate route (see tka_test_hooks in include/topk_attn.h); no arguments = defaults."""
+    h = L.TestHooks(force_segment_redo, tau_spin_limit, tau_withhold_mod, tau_withhold_rem, tau_withhold_mode, 0)
+    L.check(L.lib().tka_set_test_hooks(C.byref(h)), "tka_set_test_hooks")
 
 
 def profile_enable(on=True):
