@@ -39,13 +39,16 @@ extern "C" {
 #define TKA_MAX_TOPK 8192      /* largest k of one selection                                   */
 #define TKA_MAX_GROUP 8        /* query heads sharing one KV head: 1, 2, 4 or 8               */
 #define TKA_MAX_SPLITS 1024    /* largest split count of flash-decoding / retrieval attention */
+#define TKA_NOALLOC_SCRATCH_BYTES (128u << 20) /* built-in scratch of tka_sparse_decode_step_noalloc, per GPU */
 
 typedef enum tka_status {
   TKA_OK = 0,
   TKA_EINVAL = 1,        /* null pointer, non-positive size, k > seq_len, ...          */
   TKA_EUNSUPPORTED = 2,  /* head_dim != 128, unknown dtype, group too large, ...       */
   TKA_EHIP = 3,          /* a HIP runtime call failed (launch error, bad stream)       */
-  TKA_EWORKSPACE = 4     /* workspace missing or smaller than *_workspace_bytes()      */
+  TKA_EWORKSPACE = 4,    /* workspace missing or smaller than *_workspace_bytes()      */
+  TKA_ESCRATCH = 5       /* tka_sparse_decode_step_noalloc: the call needs more than
+                            TKA_NOALLOC_SCRATCH_BYTES of scratch memory                */
 } tka_status;
 
 typedef enum tka_dtype { TKA_F16 = 0, TKA_BF16 = 1 } tka_dtype;
@@ -361,6 +364,18 @@ typedef struct tka_sparse_decode_args {
 
 size_t tka_sparse_decode_workspace_bytes(const tka_sparse_decode_args* args);
 int tka_sparse_decode_step(const tka_sparse_decode_args* args);
+/* The same step for callers that cannot allocate device memory and bring no workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * launchers allocate and free their scratch inside every call (retrieval_attention.cu:1658-1659,1978-1979).
+ * `workspace` and `workspace_bytes` are ignored: the temporaries live in a buffer of TKA_NOALLOC_SCRATCH_BYTES
+ * (128 MiB) that is part of the library's device code - every GPU the library runs on holds one from load to
+ * process exit - and the call itself allocates nothing.  A call whose tka_sparse_decode_workspace_bytes() is
+ * larger returns TKA_ESCRATCH before anything is launched (batch 8 x 8 KV heads x 131072 tokens, k = 2048 needs
+ * 102 MiB; 8 heads x 1048576 tokens, k = 4096 needs 98 MiB).  Outputs are identical to tka_sparse_decode_step's.
+ * All calls on one GPU share that one buffer: two calls may only overlap in time if they run on different
+ * GPUs; on one GPU they must be ordered (one stream, or events between streams), otherwise they race. */
+int tka_sparse_decode_step_noalloc(const tka_sparse_decode_args* args);
+
 /* Diagnostic, as tka_gemv_topk_redone_segments: segments of the last step with these arguments (same workspace)
  * that the selection kernel redid from the keys.  Waits for the stream. */
 int tka_sparse_decode_redone_segments(const tka_sparse_decode_args* args, int32_t* count);

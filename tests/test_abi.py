@@ -35,7 +35,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = L.lib()
     declared = _declared_symbols()
-    assert len(declared) == 26 + 30
+    assert len(declared) == 27 + 30
     for name in sorted(declared):
         assert hasattr(lib, name), "libtka.so does not export %s" % name
     assert declared == set(L.PROTOTYPES), "ctypes prototypes and headers disagree"

@@ -5,7 +5,8 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libtka.so")
 
-TKA_OK, TKA_EINVAL, TKA_EUNSUPPORTED, TKA_EHIP, TKA_EWORKSPACE = 0, 1, 2, 3, 4
+TKA_OK, TKA_EINVAL, TKA_EUNSUPPORTED, TKA_EHIP, TKA_EWORKSPACE, TKA_ESCRATCH = 0, 1, 2, 3, 4, 5
+TKA_NOALLOC_SCRATCH_BYTES = 128 << 20
 TKA_F16, TKA_BF16 = 0, 1
 TKA_SOFTMAX_SCALED, TKA_SOFTMAX_RAW_EXP = 0, 1
 TKA_MAX_TOPK = 8192
@@ -109,6 +110,7 @@ PROTOTYPES = {
     "tka_retrieval_attention": (C.c_int, [C.POINTER(RaArgs)]),
     "tka_sparse_decode_workspace_bytes": (_sz, [C.POINTER(SparseDecodeArgs)]),
     "tka_sparse_decode_step": (C.c_int, [C.POINTER(SparseDecodeArgs)]),
+    "tka_sparse_decode_step_noalloc": (C.c_int, [C.POINTER(SparseDecodeArgs)]),
     "tka_sparse_decode_redone_segments": (C.c_int, [C.POINTER(SparseDecodeArgs), C.POINTER(C.c_int32)]),
     "tka_profile_enable": (C.c_int, [C.c_int]),
     "tka_profile_reset": (C.c_int, []),

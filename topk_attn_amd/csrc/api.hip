@@ -9,6 +9,11 @@
 
 #include "kernels.hpp"
 
+// Scratch of tka_sparse_decode_step_noalloc: device memory that belongs to the loaded code object, one copy per
+// GPU, there from the moment the library is loaded on that GPU until the process ends.  In host code this name is
+// only a handle for hipGetSymbolAddress (noalloc_scratch below); kernels get the address it returns.
+static __device__ __align__(256) unsigned char scratch[TKA_NOALLOC_SCRATCH_BYTES];
+
 namespace tka {
 
 // ---- per-kernel timing ------------------------------------------------------------------------
@@ -449,6 +454,7 @@ const char* tka_status_string(int status) {
     case TKA_EUNSUPPORTED: return "unsupported configuration";
     case TKA_EHIP: return "HIP runtime error";
     case TKA_EWORKSPACE: return "workspace missing or too small";
+    case TKA_ESCRATCH: return "the call needs more scratch memory than the library's built-in buffer holds";
     default: return "unknown status";
   }
 }
@@ -1022,6 +1028,52 @@ int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
   f.kv_idx = uidx;
   f.kv_count = ucnt;
   return run_flash(&f, ws + gemv_ws);
+}
+
+// ---- the step for callers that cannot allocate ------------------------------------------------
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};   // address of `scratch` on each device, looked up once with that device current
+std::mutex g_scratch_mutex;
+
+// Device address of the built-in scratch array on the current device.
+int noalloc_scratch(void** ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TKA_EHIP;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return TKA_EHIP;
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return TKA_OK;
+}
+}  // namespace
+
+int tka_sparse_decode_step_noalloc(const tka_sparse_decode_args* a) {
+  tka_gemv_topk_args g;
+  tka_flash_decode_args f;
+  int rc = sd_check(a, &g, &f);
+  if (rc != TKA_OK) return rc;
+  const size_t need = tka_sparse_decode_workspace_bytes(a);
+  if (need == 0) return TKA_EINVAL;
+  if (need > (size_t)TKA_NOALLOC_SCRATCH_BYTES) return TKA_ESCRATCH;
+  void* ptr = nullptr;
+  if ((rc = noalloc_scratch(&ptr)) != TKA_OK) return rc;
+  // The array keeps what the last call left, laid out for that call's shapes.  The words by which the
+  // candidate route tells this call's sampling state from older contents (thresholds, arrival flags, segment
+  // flags) are cleared for this call's layout, with a fill kernel; the histograms are cleared by the route
+  // that uses them; everything else is written before it is read.
+  uint32_t* words = nullptr;
+  const size_t n_words = select_epoch_words((unsigned char*)ptr + sd_gemv_ws_offset(a, f) + gemv_scores_bytes(&g),
+                                            a->batch * a->num_kv_heads, a->seq_len, &words);
+  if ((rc = launch_zero_u32(words, n_words, (hipStream_t)a->stream)) != TKA_OK) return rc;
+  tka_sparse_decode_args b = *a;
+  b.workspace = ptr;
+  b.workspace_bytes = (size_t)TKA_NOALLOC_SCRATCH_BYTES;
+  return tka_sparse_decode_step(&b);
 }
 
 // ---- per-kernel timing ------------------------------------------------------------------------

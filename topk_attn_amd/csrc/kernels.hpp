@@ -81,6 +81,7 @@ struct SelectParams {
 size_t select_workspace_bytes(int num_segments, int64_t seg_len);
 // Carves the workspace; returns how many leading 32-bit words (the histograms) need clearing.
 size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p);
+size_t select_epoch_words(void* ws, int num_segments, int64_t seg_len, uint32_t** words);
 void select_plan(int64_t seg_len, int num_segments, SelectParams* p);
 int launch_zero_u32(uint32_t* ptr, size_t count, hipStream_t stream);
 int launch_select_hist(const SelectParams& p, hipStream_t stream);

@@ -1063,6 +1063,14 @@ size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p
   return (size_t)num_segments * kHistBins;  // the flags follow the histograms; candidate mode writes them itself
 }
 
+// The words of a carved workspace that tell a call's sampling state from older contents (segment flags, thresholds,
+// arrival flags: contiguous): *words = their start, returns how many 32-bit words they are.
+size_t select_epoch_words(void* ws, int num_segments, int64_t seg_len, uint32_t** words) {
+  const SelectLayout l = select_layout(num_segments, seg_len);
+  *words = (uint32_t*)((unsigned char*)ws + l.flags);
+  return (l.pool - l.flags) / sizeof(uint32_t);
+}
+
 // Slice per workgroup: 16384 scores (16 per thread) when that still gives every CU work, else 4096.
 void select_plan(int64_t seg_len, int num_segments, SelectParams* p) {
   const int64_t big = 16 * kSelThreads;
