@@ -103,6 +103,9 @@ class SparseDecode:
     def step(self):
         self.plan.step()
 
+    def redone_segments(self):
+        return self.plan.redone_segments()
+
     def bytes(self):
         sel = int(self.plan.union_count.sum().item())
         gemv = self.B * self.N * self.H * 128 * 2
@@ -165,6 +168,9 @@ class GemvTopk:
     def step(self):
         self.plans[self.turn % len(self.plans)].run()
         self.turn += 1
+
+    def redone_segments(self):
+        return self.plans[(self.turn - 1) % len(self.plans)].redone_segments()
 
     def bytes(self):
         gemv = self.B * self.N * self.H * 128 * 2
@@ -296,11 +302,33 @@ def build_workload(name, torch, ops, dev, args):
 
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 counter runs of this file's default configurations
-# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors a plain copy of known size gives on this part);
-# the counters cannot be read from inside the process, so the figures are recorded here with their source.
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors a plain copy of known size gives on this part).
+# The counters cannot be read from inside the process, so the figures are recorded here with the file that holds
+# the counter run and the digest of the kernel's source at the time of that run: a figure is only reported
+# while the source still has that digest.
 RECORDED_TRAFFIC = {
-    ("c4", "gemv_candidates"): 2186209587,   # profiles/gemv_candidates_c4.md: 2 x 1066011.8 KiB + 2946.7 KiB
+    ("c4", "gemv_candidates"): {"bytes": 2186209587,   # 2 x 1066011.8 KiB + 2946.7 KiB
+                                "source": "profiles/gemv_candidates_c4.md",
+                                "kernel_source": "topk_attn_amd/csrc/gemv_scores.hip",
+                                "kernel_source_sha16": "RECORD_ME"},
 }
+
+
+def recorded_traffic(workload, kernel):
+    """(bytes or None, note) for roofline.traffic / roofline.traffic_source."""
+    import hashlib
+    rec = RECORDED_TRAFFIC.get((workload, kernel))
+    if rec is None:
+        return None, None
+    try:
+        with open(os.path.join(ROOT, rec["kernel_source"]), "rb") as f:
+            sha = hashlib.sha256(f.read()).hexdigest()[:16]
+    except OSError:
+        sha = None
+    if sha != rec["kernel_source_sha16"]:
+        return None, "%s is older than the kernel's source (recorded for %s, now %s): not reported" % (
+            rec["source"], rec["kernel_source_sha16"], sha)
+    return rec["bytes"], "%s (rocprofv3 counter runs, recorded; kernel source %s)" % (rec["source"], sha)
 
 
 def main():
@@ -345,12 +373,28 @@ def main():
     step_bytes, dom_bytes, extra = w.bytes()
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    # every step once more between its own pair of HIP events, recorded on the stream the library launches on
+    # (torch's current stream): median and minimum, next to the mean of the back-to-back loop above
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for e0, e1 in pairs:
+        e0.record()
+        w.step()
+        e1.record()
+    torch.cuda.synchronize()
+    per_step_us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in pairs)
+    us_median, us_min = per_step_us[len(per_step_us) // 2], per_step_us[0]
+
     # per-kernel times from HIP events recorded by the library on the launch stream (second timed loop: the
     # event pairs add a few microseconds per kernel, so they stay out of the loop that `value` comes from)
+    # the same loop also asks after every step how many segments the selection had to redo from the keys (a
+    # redone segment costs about a millisecond: a run that hit one must say so)
     ops.profile_reset()
     ops.profile_enable(True)
+    redone = 0 if hasattr(w, "redone_segments") else None
     for _ in range(args.steps):
         w.step()
+        if redone is not None:
+            redone += w.redone_segments()
     torch.cuda.synchronize()
     prof = ops.profile_read()
     ops.profile_enable(False)
@@ -360,18 +404,20 @@ def main():
         dominant = "gemv_candidates"                    # long segments run the candidate-mode GEMV
     dom_us = kern.get(dominant, ms_per_step * 1e3)     # a workload with one foreign kernel: the step itself
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
-    traffic = RECORDED_TRAFFIC.get((args.workload, dominant)) if not args.splits else None
+    traffic, traffic_source = recorded_traffic(args.workload, dominant) if not args.splits else (None, None)
 
     out = {
         "metric": "us/decode-step + achieved HBM GB/s (% of peak), GEMV+top-k+sparse attn @128k",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "us_per_step": round(ms_per_step * 1e3, 2),
+        "us_per_step_median": round(us_median, 2), "us_per_step_min": round(us_min, 2),
+        "redone_segments": redone,
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (seeded torch generator on the GPU)",
         "config": dict({"workload": w.desc, "algorithmic_bytes_per_step": step_bytes}, **extra),
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 2)},
         "kernels_us": {k_: round(v, 2) for k_, v in sorted(kern.items())},
     }

@@ -1,6 +1,7 @@
 // C ABI of the library: argument validation (before any HIP call), workspace carving, launch sequence.
 #include <atomic>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <mutex>
@@ -151,6 +152,7 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->num_samples = g->sample_rank = g->sample_wgs = g->early_wgs = 0;
   g->cand = nullptr;
   g->cand_seg_stride = 0;
+  g->cand_head = nullptr;
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   g->tokens_per_wg = gemv_tokens_per_wg(rows, g->chunk_len);
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
@@ -299,7 +301,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   cp.tau_words = sp.tau_words;
   cp.sample_flags = sp.sample_flags;
   cp.sample_pool = sp.sample_pool;
-  cp.epoch = call_counter.fetch_add(1, std::memory_order_relaxed) | 0x80000000u;   // never 0, the cleared state
+  // never 0, the cleared state; bit 30 stays free for the "has a cut" mark of the threshold words
+  cp.epoch = (call_counter.fetch_add(1, std::memory_order_relaxed) & ~kTauHasCut) | 0x80000000u;
   const tka_test_hooks hooks = current_hooks();
   cp.seg_flags = sp.seg_flags;
   if (hooks.tau_spin_limit > 0) cp.tau_spin_limit = hooks.tau_spin_limit;
@@ -310,6 +313,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   cp.sample_rank = sample_rank;
   cp.cand = sp.list;
   cp.cand_seg_stride = sp.list_stride;
+  cp.cand_head = const_cast<uint64_t*>(sp.cand_head);
   int rc = launch_gemv_candidates(cp, a->dtype, stream);
   if (rc != TKA_OK) return rc;
   SelectParams sc = sp;

@@ -25,7 +25,9 @@ constexpr int64_t kFusedMaxSegLen = 2048;   // segments up to this length are sc
 constexpr int kGemvInlineCentres = 256;     // centroids per head that the GEMV launch of a two-level selection ranks itself
 constexpr int64_t kCandMinSegLen = 32768;   // shorter segments never take the candidate mode
 constexpr int64_t kCandMinRows = 1 << 20;   // ... nor do segments below 65536 tokens unless the call has this many rows
+constexpr int kCandHead = 32;               // first candidates of a slice, kept in a compact array of their own (see GemvParams::cand_head)
 constexpr int kGemvMaxSamples = 8192;      // most samples per segment of the candidate-mode threshold estimate
+constexpr uint32_t kTauHasCut = 0x40000000u; // bit of the epoch half of a threshold word: a token cut among equal keys goes with it
 constexpr int kTauSpinLimit = 1 << 16;     // polls of a streaming workgroup for its threshold before it gives up
 // Count field (10 bits) of a candidate slice whose workgroup never saw its threshold: no real slice holds more than
 // 512 candidates, so the selection kernel cannot take it for a count, and it redoes the segment from the keys.

@@ -458,10 +458,15 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
     }
   }
   if (tid == 0) {
-    // the cut first, then, once it has completed, the word the streaming workgroups wait for
-    __hip_atomic_store(p.tau_words + 2 * seg + 1, (uint64_t)cut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __hip_atomic_store(p.tau_words + 2 * seg, ((uint64_t)p.epoch << 32) | tau, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // A cut (rare: heavy ties) goes out first, and once it has completed, the word the streaming workgroups wait
+    // for; bit 30 of the word's epoch half says that there is a cut to fetch.
+    const bool has_cut = cut != 0x7fffffffu;
+    if (has_cut) {
+      __hip_atomic_store(p.tau_words + 2 * seg + 1, (uint64_t)cut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __hip_atomic_store(p.tau_words + 2 * seg, ((uint64_t)(p.epoch | (has_cut ? kTauHasCut : 0u)) << 32) | tau, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -530,6 +535,12 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
   const int64_t first_seg = first_slice / p.wgs_per_chunk;
   const int first_wg = (int)(first_slice % p.wgs_per_chunk);
 
+  // A workgroup that starts after the first wave of them finds its threshold published: it asks for the word
+  // now, so that the answer travels beside the rows instead of costing a round trip of its own behind them
+  // (a request issued at the end queues behind the loads of the other workgroups of the CU).
+  uint64_t early_word = 0;
+  if (num_slices == 1 && tid == 0) early_word = __hip_atomic_load(p.tau_words + 2 * first_seg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
   const uint32_t row_bytes = (uint32_t)p.key_stride_n * 2u;
   {
     int64_t seg = first_seg;
@@ -573,14 +584,17 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
       if (s) __syncthreads();   // the previous slice's threshold has been read
       if (tid == 0) {
         const uint64_t* word = p.tau_words + 2 * seg;
-        uint64_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (int spin = 0; (uint32_t)(v >> 32) != p.epoch && spin < p.tau_spin_limit; ++spin) {
-          __builtin_amdgcn_s_sleep(16);
+        uint64_t v = early_word;
+        for (int spin = 0; ((uint32_t)(v >> 32) & ~kTauHasCut) != p.epoch && spin < p.tau_spin_limit; ++spin) {
+          if (spin) __builtin_amdgcn_s_sleep(16);
           v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        early_word = 0;
+        const uint32_t ep = (uint32_t)(v >> 32);
         sh_tau[0] = (uint32_t)v;
-        sh_tau[1] = (uint32_t)(v >> 32) == p.epoch ? 1u : 0u;
-        sh_tau[2] = (uint32_t)__hip_atomic_load(word + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (written before the word)
+        sh_tau[1] = (ep & ~kTauHasCut) == p.epoch ? 1u : 0u;
+        // (a cut was written, and had completed, before the word that announces it)
+        sh_tau[2] = (ep & kTauHasCut) ? (uint32_t)__hip_atomic_load(word + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0x7fffffffu;
       }
       __syncthreads();
       tau = sh_tau[0];
@@ -590,7 +604,9 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
 
     // thread t owns token t_begin + t: candidates in index order into the slice.
     // Slice format: word = key << 32 | count << 9 | token - first token of the slice; only entry 0 carries
-    // the count (0 .. 512), so a workgroup with few candidates writes a single line and nothing else.
+    // the count (0 .. 512).  Entries 0 .. 31 go to the slice's 256 bytes of the dense head array, further
+    // ones (rare) to the slice's place in the wide array: the stores of a launch then touch a few megabytes
+    // of whole lines, which stay in the L2 until the kernel ends, instead of one partial line per 4 KB.
     const uint32_t key = sh_key[s * kCandThreads + tid];
     // at or above the threshold in the order (score descending, token ascending)
     const bool pass = tau_ready && t_begin + tid < t_end && (key > tau || (key == tau && (uint32_t)(t_begin + tid) <= cut));
@@ -606,11 +622,12 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
       total += c;
     }
     uint64_t* slice = p.cand + seg * p.cand_seg_stride + (int64_t)wg_in_chunk * kCandThreads;
+    uint64_t* head = p.cand_head + (seg * p.wgs_per_chunk + wg_in_chunk) * kCandHead;
     if (pass) {
       const uint32_t pos = before + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-      slice[pos] = ((uint64_t)key << 32) | (pos == 0 ? total << 9 : 0u) | (uint32_t)tid;
+      (pos < (uint32_t)kCandHead ? head : slice)[pos] = ((uint64_t)key << 32) | (pos == 0 ? total << 9 : 0u) | (uint32_t)tid;
     }
-    if (tid == 0 && total == 0) slice[0] = tau_ready ? 0ull : (uint64_t)(kSliceGaveUp << 9);
+    if (tid == 0 && total == 0) head[0] = tau_ready ? 0ull : (uint64_t)(kSliceGaveUp << 9);
     if (tid == 0 && !tau_ready) __hip_atomic_store(p.seg_flags + seg, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (++wg_in_chunk == p.wgs_per_chunk) { wg_in_chunk = 0; ++seg; }
   }

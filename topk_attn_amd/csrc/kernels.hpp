@@ -32,6 +32,9 @@ struct GemvParams {
   uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] one slice per workgroup, ascending index:
                               // key << 32 | count << 9 | token offset in the slice (count in entry 0 only)
   int64_t cand_seg_stride;    // entries between the slice arrays of consecutive segments
+  uint64_t* cand_head;        // [segments][wgs_per_chunk][kCandHead] entries 0 .. kCandHead-1 of every slice, densely packed:
+                              // an ordinary slice (about 18 candidates) lies here whole, two full lines that stay in the
+                              // L2 until the kernel ends; `cand` only takes what goes beyond (heavy ties)
   int64_t chunk_len;    // tokens per chunk
   int64_t q_stride_b, key_stride_b, key_stride_n, key_stride_h;
   int batch, num_kv_heads, group, num_chunks;
@@ -61,6 +64,7 @@ struct SelectParams {
   int from_scores;        // candidate selection kernel: no slices, the entries are all scores of the segment (<= 16384)
   uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)
   uint64_t* list;         // [num_segments][list_stride] composites with bin >= threshold bin, slice p at p*part_len
+  const uint64_t* cand_head;  // candidate mode: [num_segments][parts][kCandHead] the first entries of every slice
   int64_t list_stride;
   int32_t* out_idx;       // [num_segments][out_stride] rank order, or nullptr (no sort)
   float* out_val;         // same shape or nullptr

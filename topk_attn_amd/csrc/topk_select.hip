@@ -652,6 +652,8 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   // start positions, and the entries go to their place: one memory round trip.
   const uint32_t cap = (uint32_t)(p.max_entries < kCandCap ? p.max_entries : kCandCap);
   const uint64_t* lists = p.list + (int64_t)seg * p.list_stride;   // (not read when the entries come from keys or scores)
+  const uint64_t* heads = p.cand_head + (int64_t)seg * p.parts * kCandHead;   // entries 0 .. 31 of every slice
+  static_assert(kSliceLanes == kCandHead, "one lane per head entry");
   const int sub = tid & (kSliceLanes - 1), grp = tid / kSliceLanes;
   uint32_t n_entries = 0;
   if (p.from_keys) {
@@ -705,7 +707,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
         const int sl = s0 + u * kGroups + grp;
-        first[u] = sl < p.parts ? lists[(int64_t)sl * p.part_len + sub] : 0ull;
+        first[u] = sl < p.parts ? heads[(int64_t)sl * kCandHead + sub] : 0ull;
       }
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
@@ -742,7 +744,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int sl = 4 * tid + q;
-      c4[q] = sl < p.parts ? ((uint32_t)lists[(int64_t)sl * p.part_len] >> 9) & 0x3ffu : 0u;
+      c4[q] = sl < p.parts ? ((uint32_t)heads[(int64_t)sl * kCandHead] >> 9) & 0x3ffu : 0u;
       if (c4[q] == kSliceGaveUp) {
         c4[q] = 0u;
         atomicAdd(&sh_gave_up, 1u);
@@ -770,7 +772,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
         const int sl = s0 + u * kGroups2 + grp2;
         start[u] = sl < p.parts ? sh_pos[sl] : 0u;
         cnt[u] = sl < p.parts ? sh_pos[sl + 1] - start[u] : 0u;
-        w[u] = (uint32_t)sub2 < cnt[u] ? lists[(int64_t)sl * p.part_len + sub2] : 0ull;
+        w[u] = (uint32_t)sub2 < cnt[u] ? heads[(int64_t)sl * kCandHead + sub2] : 0ull;
       }
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
@@ -779,7 +781,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
         if ((uint32_t)sub2 < cnt[u] && start[u] + sub2 < cap)
           sh_ent[start[u] + sub2] = (w[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w[u] & 0x1ffu));
         for (uint32_t j = kLanes2 + sub2; j < cnt[u] && start[u] + j < cap; j += kLanes2) {
-          const uint64_t x = lists[(int64_t)sl * p.part_len + j];
+          const uint64_t x = j < (uint32_t)kCandHead ? heads[(int64_t)sl * kCandHead + j] : lists[(int64_t)sl * p.part_len + j];
           sh_ent[start[u] + j] = (x & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)x & 0x1ffu));
         }
       }
@@ -1020,11 +1022,12 @@ int kpad_for(int k) {
 }  // namespace
 
 // Workspace layout (each part 256-byte aligned):
-//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S] u64 | arrival flags [S][64] u32 | sample pool [S][8192] u32 | list_cnt [S][slices] u32 |
+//   hist [S][2048] u32 (cleared per call) | flags [S] u32 | tau [S] u64 | arrival flags [S][64] u32 | sample pool [S][8192] u32 |
+//   candidate heads [S][slices][32] u64 | list_cnt [S][slices] u32 |
 //   list [S][slices*slice_len] u64      (slices: dense 4096/16384 scores, candidate mode one per GEMV workgroup)
 namespace {
 struct SelectLayout {
-  size_t hist, flags, tau, ctr, pool, list_cnt, list, total;
+  size_t hist, flags, tau, ctr, pool, head, list_cnt, list, total;
   int64_t list_stride;
 };
 SelectLayout select_layout(int num_segments, int64_t seg_len) {
@@ -1039,6 +1042,7 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   const size_t cand_segs = seg_len >= kCandMinSegLen ? (size_t)num_segments : 0;   // sampling state: long segments only
   l.ctr = take(cand_segs * 64 * sizeof(uint32_t));
   l.pool = take(cand_segs * kGemvMaxSamples * sizeof(uint32_t));
+  l.head = take(cand_segs * (size_t)(seg_len / kGemvCandTokensPerWg + 1) * kCandHead * sizeof(uint64_t));
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
   l.total = off;
@@ -1057,6 +1061,7 @@ size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p
   p->tau_words = (uint64_t*)(c + l.tau);
   p->sample_flags = (uint32_t*)(c + l.ctr);
   p->sample_pool = (uint32_t*)(c + l.pool);
+  p->cand_head = (const uint64_t*)(c + l.head);
   p->list_cnt = (uint32_t*)(c + l.list_cnt);
   p->list = (uint64_t*)(c + l.list);
   p->list_stride = l.list_stride;
