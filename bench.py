@@ -231,7 +231,7 @@ class RetrievalOp:
     """ra: the reference's operator at its own test shape (test_ra.py:162-172: 32 heads, 8192 keys shared by the
     batch, 4 chunks of 2048, top-K per chunk), batch entries and K selectable."""
 
-    def __init__(self, torch, dev, batch=4, topk=128, rotate=0):
+    def __init__(self, torch, dev, batch=4, topk=128, rotate=0, score_mode=0):
         from topk_attn_amd import retrieval_attention_cpp as ra
         g = torch.Generator(device=dev)
         g.manual_seed(6)
@@ -243,10 +243,12 @@ class RetrievalOp:
         self.kv = [(K, V)] + [(K.clone(), V.clone()) for _ in range(max(rotate - 1, 0))]
         self.turn = 0
         self.out = torch.zeros((batch, 32, 128), dtype=torch.float16, device=dev)
-        self.fn = getattr(ra, "retrieval_attention_%d" % topk)
-        self.desc = "ra: retrieval_attention_%d, B=%d, 32 heads, 8192 keys fp16 shared by the batch%s" % (
-            topk, batch, ", %d rotating cache copies" % rotate if rotate > 1 else "")
-        self.dominant = "gemv_scores_shared" if batch >= 2 else "gemv_scores"
+        self.score_mode = score_mode
+        self.fn = lambda q, K, V, out: ra.retrieval_attention(q, K, V, out, topk, score_mode=score_mode)
+        self.desc = "ra: retrieval_attention_%d, B=%d, 32 heads, 8192 keys fp16 shared by the batch%s%s" % (
+            topk, batch, ", %d rotating cache copies" % rotate if rotate > 1 else "",
+            ", scores on the matrix cores" if score_mode else "")
+        self.dominant = ("gemv_scores_mfma" if score_mode else "gemv_scores_shared") if batch >= 2 else "gemv_scores"
 
     def step(self):
         K, V = self.kv[self.turn % len(self.kv)]
@@ -292,7 +294,7 @@ def build_workload(name, torch, ops, dev, args):
     if name == "c3":
         return FlashDecode(torch, ops, dev, args.splits)
     if name == "ra":
-        return RetrievalOp(torch, dev, batch=args.batch, topk=args.topk, rotate=args.rotate)
+        return RetrievalOp(torch, dev, batch=args.batch, topk=args.topk, rotate=args.rotate, score_mode=args.score_mode)
     if name == "c5":       # the tie-stress step: selection under exact ties at 1M tokens, attention over the selected tokens
         return SparseDecode(torch, ops, dev, batch=1, hkv=8, group=8, seq_len=1048576, k=4096, sink=0, local=0,
                             dtype="bfloat16", heavy=0.0, seed=5, name="c5", levels=True)
@@ -339,6 +341,8 @@ def main():
     ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c5", "c5-topk", "ra", "copy"])
     ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
+    ap.add_argument("--score-mode", type=int, default=0, choices=[0, 1],
+                    help="ra: 1 = scores on the matrix cores (tka_score_mode), 0 = the canonical order")
     ap.add_argument("--splits", type=int, default=0, help="c3, c4: split count of the attention (0 = library default)")
     ap.add_argument("--rotate", type=int, default=0,
                     help="c1, c2, c2-ref, ra: number of key sets taken in turn (working set beyond the Infinity Cache)")

@@ -59,6 +59,16 @@ typedef enum tka_softmax_mode {
                              evaluated max-subtracted in fp32, which is the same function               */
 } tka_softmax_mode;
 
+/* How stage 1 adds up the 128 products of a score.
+ * TKA_SCORE_CANONICAL: the 16-lane order defined above; scores are bit-identical to the reference order on any route.
+ * TKA_SCORE_MATRIX: where keys are shared by a batch of at least two entries (key_stride_b == 0, group == 1) the
+ *   scores come from the matrix cores (v_mfma_f32_16x16x32, fp32 accumulation in the unit's own order): within a
+ *   few units in the last place of the canonical ones (1e-5 of the exact dot product), not bit-identical to them.
+ *   The selection is exact on the scores the call computed: out_idx / out_val are the first k of a stable
+ *   descending sort of what out_scores would hold.  Calls it does not apply to run as TKA_SCORE_CANONICAL.
+ *   (The batch pipeline of retrieval_attention.cu:654-896 as a skinny GEMM; about 4x quicker at batch 32.) */
+typedef enum tka_score_mode { TKA_SCORE_CANONICAL = 0, TKA_SCORE_MATRIX = 1 } tka_score_mode;
+
 const char* tka_status_string(int status);
 /* Library version as major*10000 + minor*100 + patch. */
 int tka_version(void);
@@ -81,7 +91,7 @@ typedef struct tka_gemv_topk_args {
   int32_t head_dim;       /* must be 128                                                      */
   int32_t k;              /* selected per chunk                                               */
   int32_t num_chunks;     /* >= 1; seq_len must be a multiple                                 */
-  int32_t reserved0;
+  int32_t score_mode;     /* tka_score_mode; 0 = the canonical order of the header            */
   int64_t seq_len;
   int64_t q_stride_b;     /* elements between batch entries of q                              */
   int64_t key_stride_b;   /* 0 = keys shared by all batch entries (retrieval_attention.cu:681-683) */
@@ -316,7 +326,7 @@ typedef struct tka_ra_args {
                              (retrieval_attention.cu:1610) after a blocking timed rerun       */
   int64_t seq_len;        /* reference: 8192                                                  */
   float scale;            /* reference: 1.0f                                                  */
-  int32_t reserved0;
+  int32_t score_mode;     /* tka_score_mode of the scoring stage; 0 = canonical               */
   void* workspace;
   size_t workspace_bytes;
   void* stream;

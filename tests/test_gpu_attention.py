@@ -199,6 +199,28 @@ def test_retrieval_attention_op(topk):
             assert np.abs(got[b, h] - ref).max() < TOL
 
 
+@pytest.mark.parametrize("B,topk", [(4, 128), (32, 256)])
+def test_retrieval_attention_op_matrix_core_scores(B, topk):
+    """The operator with score_mode = TKA_SCORE_MATRIX (its scoring stage on the matrix cores): same tolerance against
+    the fp64 oracle as the canonical form (a token at the very edge of a chunk's top K may change places with its
+    neighbour in score; its weight is about 1/(4K))."""
+    from topk_attn_amd import _lib as L
+    from topk_attn_amd import retrieval_attention_cpp as ra
+    announce("retrieval_attention op on the matrix cores B=%d topk=%d" % (B, topk))
+    rng = np.random.default_rng(5)
+    dtype = oracle.F16
+    H, N = 32, 8192
+    q, K, V = randn_bits(rng, (B, H, 128), dtype, 0.1), randn_bits(rng, (N, H, 128), dtype, 0.1), randn_bits(rng, (N, H, 128), dtype, 0.1)
+    out = torch.zeros((B, H, 128), dtype=torch.float16, device="cuda")
+    ra.retrieval_attention(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), out, topk, score_mode=L.TKA_SCORE_MATRIX)
+    torch.cuda.synchronize()
+    got = f32_of(out)
+    for b in range(0, B, 7):
+        for h in range(0, H, 5):
+            ref, _, _ = oracle.retrieval_attention(q[b, h], K[:, h], V[:, h], dtype, 4, topk, 1.0)
+            assert np.abs(got[b, h] - ref).max() < TOL
+
+
 @pytest.mark.parametrize("B,topk", [(9, 128), (33, 1024), (2, 32)])
 def test_retrieval_attention_op_batches(B, topk):
     """Batches whose keys are scored several entries per pass (with a ragged last tile), selected one segment per

@@ -86,6 +86,40 @@ def test_shared_kv_batch_tiles(B, H):
     _run_flat(oracle.F16, B, H, 1, 8192, 128, seed=60 + B, shared_kv=True, num_chunks=4, scale=1.0)
 
 
+@pytest.mark.parametrize("dtype,B,H,N,chunks,k", [(oracle.F16, 2, 3, 4096, 2, 128), (oracle.F16, 17, 2, 4100, 1, 300),
+                                                  (oracle.BF16, 32, 2, 8192, 4, 128), (oracle.F16, 33, 1, 4099, 1, 64),
+                                                  (oracle.BF16, 9, 4, 2048, 1, 2048)])
+def test_matrix_core_scores_shared_kv(dtype, B, H, N, chunks, k):
+    """score_mode = TKA_SCORE_MATRIX on a key cache shared by the batch: the scores come from the matrix cores, whose
+    order of addition is not the canonical one, so they are held to 1e-5 of the exact dot product (the stated rule
+    for fp32 scores), and the selection must be exact ON THOSE SCORES: indices and values are the first k of a
+    stable descending sort of the score vector the call returned, chunk by chunk."""
+    from topk_attn_amd import _lib as L
+    from topk_attn_amd import ops
+    announce("gemv_topk on the matrix cores dtype=%d B=%d H=%d N=%d chunks=%d k=%d" % (dtype, B, H, N, chunks, k))
+    rng = np.random.default_rng(1000 + B)
+    q, K = randn_bits(rng, (B, H, 128), dtype), randn_bits(rng, (N, H, 128), dtype)
+    idx, val, scores = ops.gemv_topk(to_dev(q, dtype), to_dev(K, dtype), k, group=1, scale=SCALE, num_chunks=chunks,
+                                     return_scores=True, score_mode=L.TKA_SCORE_MATRIX)
+    plain = ops.gemv_scores(to_dev(q, dtype), to_dev(K, dtype), group=1, scale=SCALE, score_mode=L.TKA_SCORE_MATRIX)
+    torch.cuda.synchronize()
+    idx, val, scores, plain = idx.cpu().numpy(), val.cpu().numpy(), scores.cpu().numpy(), plain.cpu().numpy()
+    assert np.array_equal(scores.view(np.uint32), plain.view(np.uint32))      # the GEMV-only entry point runs the same kernel
+    chunk = N // chunks
+    differs = 0
+    for b in range(B):
+        for h in range(H):
+            truth = oracle.scores_f64(K[:, h, :], dtype, q[b, h:h + 1], SCALE)
+            assert np.abs(scores[b, h].astype(np.float64) - truth).max() < 1e-5 * max(1.0, np.abs(truth).max() / 4)
+            canon = oracle.scores_canonical(K[:, h, :], dtype, oracle.group_query(q[b, h:h + 1], dtype, 1), SCALE)
+            differs += int((canon.view(np.uint32) != scores[b, h].view(np.uint32)).sum())
+            for c in range(chunks):
+                ei, ev = oracle.topk_stable(scores[b, h, c * chunk:(c + 1) * chunk], k)   # (pinned against lexsort / stable sort)
+                assert np.array_equal(idx[b, h, c * k:(c + 1) * k], ei + c * chunk), "indices differ (b=%d h=%d c=%d)" % (b, h, c)
+                assert np.array_equal(val[b, h, c * k:(c + 1) * k].view(np.uint32), ev.view(np.uint32))
+    print("matrix-core scores that differ from the canonical ones in their last bits: %d of %d" % (differs, B * H * N), flush=True)
+
+
 def test_many_short_segments_routes():
     """128 or more segments of at most 2048 rows: plain scores + a small workgroup per segment; both dtypes, grouped
     queries, odd lengths, ties, keys per sequence and shared."""

@@ -9,6 +9,7 @@ TKA_OK, TKA_EINVAL, TKA_EUNSUPPORTED, TKA_EHIP, TKA_EWORKSPACE, TKA_ESCRATCH = 0
 TKA_NOALLOC_SCRATCH_BYTES = 128 << 20
 TKA_F16, TKA_BF16 = 0, 1
 TKA_SOFTMAX_SCALED, TKA_SOFTMAX_RAW_EXP = 0, 1
+TKA_SCORE_CANONICAL, TKA_SCORE_MATRIX = 0, 1
 TKA_MAX_TOPK = 8192
 TKA_MAX_SPLITS = 1024
 
@@ -17,7 +18,7 @@ _p, _i32, _i64, _f, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_size_
 
 class GemvTopkArgs(C.Structure):
     _fields_ = [("q", _p), ("keys", _p), ("dtype", _i32), ("batch", _i32), ("num_kv_heads", _i32), ("group", _i32),
-                ("head_dim", _i32), ("k", _i32), ("num_chunks", _i32), ("reserved0", _i32), ("seq_len", _i64),
+                ("head_dim", _i32), ("k", _i32), ("num_chunks", _i32), ("score_mode", _i32), ("seq_len", _i64),
                 ("q_stride_b", _i64), ("key_stride_b", _i64), ("key_stride_n", _i64), ("key_stride_h", _i64),
                 ("scale", _f), ("reserved1", _i32), ("out_idx", _p), ("out_val", _p), ("out_scores", _p),
                 ("workspace", _p), ("workspace_bytes", _sz), ("stream", _p)]
@@ -65,7 +66,7 @@ class RaArgs(C.Structure):
     _fields_ = [("q", _p), ("keys", _p), ("values", _p), ("out", _p), ("dtype", _i32), ("batch", _i32),
                 ("num_heads", _i32), ("head_dim", _i32), ("topk_per_chunk", _i32), ("num_chunks", _i32),
                 ("softmax_mode", _i32), ("bench_print", _i32), ("seq_len", _i64), ("scale", _f),
-                ("reserved0", _i32), ("workspace", _p), ("workspace_bytes", _sz), ("stream", _p)]
+                ("score_mode", _i32), ("workspace", _p), ("workspace_bytes", _sz), ("stream", _p)]
 
 
 class SparseDecodeArgs(C.Structure):

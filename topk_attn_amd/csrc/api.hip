@@ -102,6 +102,7 @@ int check_gemv(const tka_gemv_topk_args* a, bool need_topk) {
   if (!a->q || !a->keys) return TKA_EINVAL;
   if (a->head_dim != TKA_HEAD_DIM || !dtype_ok(a->dtype) || !group_ok(a->group)) return TKA_EUNSUPPORTED;
   if (a->batch < 1 || a->num_kv_heads < 1 || a->seq_len < 1 || a->num_chunks < 1) return TKA_EINVAL;
+  if (a->score_mode != TKA_SCORE_CANONICAL && a->score_mode != TKA_SCORE_MATRIX) return TKA_EUNSUPPORTED;
   if (a->batch > 65535 || a->num_kv_heads > 65535) return TKA_EUNSUPPORTED;
   if (a->seq_len > 0x7fffffffLL) return TKA_EUNSUPPORTED;  // token ids are int32
   if (a->seq_len % a->num_chunks != 0) return TKA_EINVAL;
@@ -197,6 +198,12 @@ struct InlineCentres {
   int32_t* ids_out;      // [num_kv_heads*num_chunks] chosen cluster per (head, rank)
 };
 
+// Plain scores of a batch over one key cache: the matrix cores when the caller opted in, else the canonical order.
+int launch_shared_scores(const tka_gemv_topk_args* a, const GemvParams& gp, hipStream_t stream) {
+  if (a->score_mode == TKA_SCORE_MATRIX && a->group == 1) return launch_gemv_scores_mfma(gp, a->dtype, stream);
+  return launch_gemv_scores_shared(gp, a->dtype, stream);
+}
+
 // Segments that fit in the registers of a workgroup: plain scores, then one workgroup per segment selects.
 bool wave_route(const tka_gemv_topk_args* a, bool want_union) {
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
@@ -254,7 +261,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
       gp.cluster_ids_out = ic->ids_out;
       sw.seg_base_ids = ic->ids_out;
     }
-    int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);
+    int rc = shared_keys ? launch_shared_scores(a, gp, stream) : launch_gemv_scores(gp, a->dtype, stream);
     if (rc != TKA_OK) return rc;
     return launch_select_wave(sw, stream);
   }
@@ -271,7 +278,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // Segments that fit in LDS whole: GEMV that stores plain scores (no histogram), then one selection launch.
   if (chunk_len <= select_cand_capacity()) {
     gp.hist = nullptr;
-    int rc = shared_keys ? launch_gemv_scores_shared(gp, a->dtype, stream) : launch_gemv_scores(gp, a->dtype, stream);
+    int rc = shared_keys ? launch_shared_scores(a, gp, stream) : launch_gemv_scores(gp, a->dtype, stream);
     if (rc != TKA_OK) return rc;
     SelectParams sw = sp;
     sw.from_scores = 1;
@@ -533,7 +540,7 @@ int tka_gemv_scores(const tka_gemv_topk_args* a) {
   if (rc != TKA_OK) return rc;
   GemvParams gp;
   fill_gemv_params(a, a->out_scores, nullptr, &gp);
-  if (a->key_stride_b == 0 && a->batch >= 2) return launch_gemv_scores_shared(gp, a->dtype, (hipStream_t)a->stream);
+  if (a->key_stride_b == 0 && a->batch >= 2) return launch_shared_scores(a, gp, (hipStream_t)a->stream);
   return launch_gemv_scores(gp, a->dtype, (hipStream_t)a->stream);
 }
 
@@ -797,6 +804,7 @@ static int ra_parts(const tka_ra_args* a, tka_gemv_topk_args* g, tka_flash_decod
   g->key_stride_n = (int64_t)a->num_heads * TKA_HEAD_DIM;
   g->key_stride_h = TKA_HEAD_DIM;
   g->scale = a->scale;
+  g->score_mode = a->score_mode;
   g->stream = a->stream;
   memset(f, 0, sizeof *f);
   f->q = a->q;

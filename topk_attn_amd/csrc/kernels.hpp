@@ -44,6 +44,8 @@ struct GemvParams {
 int launch_gemv_scores(const GemvParams& p, int dtype, hipStream_t stream);
 // Keys shared by the batch (key_stride_b == 0): one pass over the keys scores several batch entries; plain scores only.
 int launch_gemv_scores_shared(const GemvParams& p, int dtype, hipStream_t stream);
+// The same on the matrix cores (one query head per KV head): scores to a few units in the last place of the canonical ones.
+int launch_gemv_scores_mfma(const GemvParams& p, int dtype, hipStream_t stream);
 int launch_gemv_candidates(const GemvParams& p, int dtype, hipStream_t stream);   // thresholds + candidate slices
 void gemv_candidate_plan(int64_t chunk_len, int64_t total_rows, int k, int max_candidates, int* num_samples, int* sample_rank);
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);

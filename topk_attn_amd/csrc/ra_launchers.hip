@@ -38,6 +38,11 @@ void run(const void* q, const void* k, const void* v, void* out, int batch, int 
   a.softmax_mode = TKA_SOFTMAX_RAW_EXP;
   const char* env = getenv("TKA_BENCH_PRINT");
   a.bench_print = env && env[0] == '1';
+  static const bool matrix_scores = [] {   // TKA_RA_SCORE_MODE=1, read once: scoring on the matrix cores
+    const char* e = getenv("TKA_RA_SCORE_MODE");
+    return e && e[0] == '1' && e[1] == 0;
+  }();
+  a.score_mode = matrix_scores ? TKA_SCORE_MATRIX : TKA_SCORE_CANONICAL;
   a.seq_len = kRaSeqLen;
   a.scale = 1.0f;
   a.stream = nullptr;  // the reference launches on the default stream

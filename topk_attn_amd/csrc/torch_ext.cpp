@@ -21,7 +21,7 @@ namespace {
 constexpr int64_t kHeads = 32, kDim = 128, kSeqLen = 8192, kChunks = 4;   // retrieval_attention.cu:30-34
 
 void run(const torch::Tensor& query, const torch::Tensor& key_cache, const torch::Tensor& value_cache, torch::Tensor& output,
-         int64_t topk, int64_t num_chunks, double scale, bool fixed_shape) {
+         int64_t topk, int64_t num_chunks, double scale, bool fixed_shape, int64_t score_mode) {
   for (const torch::Tensor* t : {&query, &key_cache, &value_cache, (const torch::Tensor*)&output}) {
     TORCH_CHECK(t->is_cuda(), "retrieval_attention: tensors must live on the GPU");
     TORCH_CHECK(t->scalar_type() == at::kHalf || (!fixed_shape && t->scalar_type() == at::kBFloat16),
@@ -55,6 +55,7 @@ void run(const torch::Tensor& query, const torch::Tensor& key_cache, const torch
   a.bench_print = print && print[0] == '1' && print[1] == 0;   // the timing line that test_ra.py:63-75 parses
   a.seq_len = key_cache.size(0);
   a.scale = (float)scale;
+  a.score_mode = (int32_t)score_mode;
   const size_t need = tka_retrieval_attention_workspace_bytes(&a);
   TORCH_CHECK(need != 0, "retrieval_attention: unsupported arguments (top-k ", topk, ", chunks ", num_chunks, ")");
   torch::Tensor workspace = torch::empty({(int64_t)need}, query.options().dtype(torch::kUInt8));
@@ -65,12 +66,21 @@ void run(const torch::Tensor& query, const torch::Tensor& key_cache, const torch
   TORCH_CHECK(rc == TKA_OK, "tka_retrieval_attention: ", tka_status_string(rc), " (status ", rc, ")");
 }
 
+// TKA_RA_SCORE_MODE=1 (read once): the fixed-shape ops score on the matrix cores (tka_score_mode in topk_attn.h)
+int64_t env_score_mode() {
+  static const int64_t mode = [] {
+    const char* e = std::getenv("TKA_RA_SCORE_MODE");
+    return (int64_t)(e && e[0] == '1' && e[1] == 0 ? TKA_SCORE_MATRIX : TKA_SCORE_CANONICAL);
+  }();
+  return mode;
+}
+
 }  // namespace
 
 #define RA_OP(variant, K, title)                                                                             \
   m.def("retrieval_attention" variant "_" #K,                                                                \
         [](torch::Tensor query, torch::Tensor key_cache, torch::Tensor value_cache, torch::Tensor output) {  \
-          run(query, key_cache, value_cache, output, K, kChunks, 1.0, true);                                 \
+          run(query, key_cache, value_cache, output, K, kChunks, 1.0, true, env_score_mode());               \
         },                                                                                                   \
         title " (TopK=" #K ")");
 #define RA_OPS(variant, title) \
@@ -85,8 +95,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   RA_OPS("_gather_baseline", "Retrieval Attention Gather Baseline")      // bind.cpp:752-756
   m.def("retrieval_attention",
         [](torch::Tensor query, torch::Tensor key_cache, torch::Tensor value_cache, torch::Tensor output, int64_t topk,
-           int64_t num_chunks, double scale) { run(query, key_cache, value_cache, output, topk, num_chunks, scale, false); },
-        "Retrieval attention with the top-k per chunk, the chunk count and the score scale as arguments (fp16 or bf16)",
+           int64_t num_chunks, double scale, int64_t score_mode) {
+          run(query, key_cache, value_cache, output, topk, num_chunks, scale, false, score_mode);
+        },
+        "Retrieval attention with the top-k per chunk, the chunk count and the score scale as arguments (fp16 or bf16); "
+        "score_mode 1 computes the scores on the matrix cores",
         py::arg("query"), py::arg("key_cache"), py::arg("value_cache"), py::arg("output"), py::arg("topk"),
-        py::arg("num_chunks") = 4, py::arg("scale") = 1.0);
+        py::arg("num_chunks") = 4, py::arg("scale") = 1.0, py::arg("score_mode") = 0);
 }

@@ -73,7 +73,7 @@ def _q3(q):
 class GemvTopkPlan:
     """Argument block, outputs and workspace of one fused GEMV + top-k configuration; run() is one C call."""
 
-    def __init__(self, q, keys, k, group=1, scale=1.0, num_chunks=1, return_scores=False):
+    def __init__(self, q, keys, k, group=1, scale=1.0, num_chunks=1, return_scores=False, score_mode=L.TKA_SCORE_CANONICAL):
         _need_cuda(q, keys)
         q = _q3(q)
         B = q.shape[0]
@@ -87,7 +87,7 @@ class GemvTopkPlan:
         a = L.GemvTopkArgs()
         a.q, a.keys = q.data_ptr(), keys.data_ptr()
         a.dtype, a.batch, a.num_kv_heads, a.group, a.head_dim = _dtype_code(keys), B, H, group, 128
-        a.k, a.num_chunks, a.seq_len = k, num_chunks, N
+        a.k, a.num_chunks, a.seq_len, a.score_mode = k, num_chunks, N, score_mode
         a.q_stride_b, a.key_stride_b, a.key_stride_n, a.key_stride_h = q.stride(0), sb, sn, sh
         a.scale = scale
         a.out_idx, a.out_val = self.idx.data_ptr(), self.val.data_ptr()
@@ -116,13 +116,13 @@ class GemvTopkPlan:
         return n.value
 
 
-def gemv_topk(q, keys, k, group=1, scale=1.0, num_chunks=1, return_scores=False):
+def gemv_topk(q, keys, k, group=1, scale=1.0, num_chunks=1, return_scores=False, score_mode=L.TKA_SCORE_CANONICAL):
     """Fused GEMV + top-k.  Returns (idx int32 [B,Hkv,num_chunks*k], val fp32 same shape[, scores fp32 [B,Hkv,N]])."""
-    plan = GemvTopkPlan(q, keys, k, group, scale, num_chunks, return_scores).run()
+    plan = GemvTopkPlan(q, keys, k, group, scale, num_chunks, return_scores, score_mode).run()
     return (plan.idx, plan.val, plan.scores) if return_scores else (plan.idx, plan.val)
 
 
-def gemv_scores(q, keys, group=1, scale=1.0):
+def gemv_scores(q, keys, group=1, scale=1.0, score_mode=L.TKA_SCORE_CANONICAL):
     """GEMV phase alone: fp32 scores [B,Hkv,N]."""
     _need_cuda(q, keys)
     q = _q3(q)
@@ -132,7 +132,7 @@ def gemv_scores(q, keys, group=1, scale=1.0):
     a = L.GemvTopkArgs()
     a.q, a.keys = q.data_ptr(), keys.data_ptr()
     a.dtype, a.batch, a.num_kv_heads, a.group, a.head_dim = _dtype_code(keys), B, H, group, 128
-    a.k, a.num_chunks, a.seq_len = 1, 1, N
+    a.k, a.num_chunks, a.seq_len, a.score_mode = 1, 1, N, score_mode
     a.q_stride_b, a.key_stride_b, a.key_stride_n, a.key_stride_h = q.stride(0), sb, sn, sh
     a.scale = scale
     a.out_scores = scores.data_ptr()
@@ -300,7 +300,7 @@ def lse_combine(part_m, part_l, part_acc, out_dtype=torch.float16, return_lse=Fa
 
 
 def retrieval_attention(q, k, v, out, topk, num_chunks=4, scale=1.0, softmax_mode=L.TKA_SOFTMAX_RAW_EXP,
-                        bench_print=False):
+                        bench_print=False, score_mode=L.TKA_SCORE_CANONICAL):
     """The reference op, general form: q [B,H,128], k/v [N,H,128] contiguous, writes out [B,H,128] in place."""
     _need_cuda(q, k, v, out)
     for t in (q, k, v, out):
@@ -313,7 +313,7 @@ def retrieval_attention(q, k, v, out, topk, num_chunks=4, scale=1.0, softmax_mod
     a.q, a.keys, a.values, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     a.dtype, a.batch, a.num_heads, a.head_dim = _dtype_code(q), B, H, 128
     a.topk_per_chunk, a.num_chunks, a.softmax_mode, a.bench_print = topk, num_chunks, softmax_mode, int(bench_print)
-    a.seq_len, a.scale = k.shape[0], scale
+    a.seq_len, a.scale, a.score_mode = k.shape[0], scale, score_mode
     need = L.lib().tka_retrieval_attention_workspace_bytes(C.byref(a))
     ws = _workspace(need, q.device)
     a.workspace, a.workspace_bytes, a.stream = ws.data_ptr(), ws.numel(), _stream()

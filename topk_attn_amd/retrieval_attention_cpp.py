@@ -13,10 +13,16 @@ from . import ops
 NUM_HEADS, HEAD_DIM, SEQ_LEN, NUM_CHUNKS = 32, 128, 8192, 4  # retrieval_attention.cu:30-34
 
 
+def _env_score_mode():
+    """TKA_RA_SCORE_MODE=1: the fixed-shape ops score on the matrix cores (see tka_score_mode in include/topk_attn.h)."""
+    import os
+    return L.TKA_SCORE_MATRIX if os.environ.get("TKA_RA_SCORE_MODE") == "1" else L.TKA_SCORE_CANONICAL
+
+
 def retrieval_attention(query, key_cache, value_cache, output, topk, num_chunks=NUM_CHUNKS, scale=1.0,
-                        bench_print=False):
+                        bench_print=False, score_mode=L.TKA_SCORE_CANONICAL):
     return ops.retrieval_attention(query, key_cache, value_cache, output, topk, num_chunks, scale,
-                                   L.TKA_SOFTMAX_RAW_EXP, bench_print)
+                                   L.TKA_SOFTMAX_RAW_EXP, bench_print, score_mode)
 
 
 def _make(variant, topk):
@@ -29,7 +35,7 @@ def _make(variant, topk):
             raise ValueError("expected query/output [B,32,128] and key/value cache [8192,32,128]")
         import os
         ops.retrieval_attention(query, key_cache, value_cache, output, topk, NUM_CHUNKS, 1.0, L.TKA_SOFTMAX_RAW_EXP,
-                                os.environ.get("TKA_BENCH_PRINT") == "1")
+                                os.environ.get("TKA_BENCH_PRINT") == "1", _env_score_mode())
 
     op.__name__ = "retrieval_attention%s_%d" % (variant, topk)
     op.__doc__ = "Retrieval Attention%s (TopK=%d)" % (variant.replace("_", " ").title(), topk)
