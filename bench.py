@@ -312,7 +312,7 @@ RECORDED_TRAFFIC = {
     ("c4", "gemv_candidates"): {"bytes": 2186529279,   # 2 x 1066171.7 KiB + 2939.1 KiB
                                 "source": "profiles/gemv_candidates_c4.md",
                                 "kernel_source": "topk_attn_amd/csrc/gemv_scores.hip",
-                                "kernel_source_sha16": "1c1dfdd9762fdd7e"},
+                                "kernel_source_sha16": "77c6c150e0fb0ef9"},
 }
 
 

@@ -676,6 +676,17 @@ int launch_gemv_scores_shared(const GemvParams& p0, int dtype, hipStream_t strea
   return hip_status(hipGetLastError());
 }
 
+// Streaming workgroups of the candidate kernel that the current device holds at once: 8 waves per SIMD, 4 SIMDs per
+// CU, 8 waves per workgroup = 4 per CU (1024 on the 256 CUs of MI355X).  Asked for once.
+static int64_t resident_streaming_wgs() {
+  static const int64_t n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+    return (int64_t)4 * cus;
+  }();
+  return n;
+}
+
 // Candidate mode: sampling workgroups (256 samples each) at the front of the grid, then the streaming ones.
 int launch_gemv_candidates(const GemvParams& p0, int dtype, hipStream_t stream) {
   GemvParams p = p0;
@@ -684,9 +695,9 @@ int launch_gemv_candidates(const GemvParams& p0, int dtype, hipStream_t stream) 
       p.num_samples > kGemvMaxSamples || p.sample_rank < 1 || p.sample_rank > p.num_samples)
     return TKA_EINVAL;
   p.sample_wgs = (int)(segs * (p.num_samples / kCandRowsPerIter));
-  // early workgroups: as many as the GPU holds at once (256 CUs x 4 workgroups of 8 waves)
+  // early workgroups: as many as the GPU holds at once
   const int64_t slices = segs * p.wgs_per_chunk;
-  int64_t early = 1024;
+  int64_t early = resident_streaming_wgs();
   if (early > slices / (2 * kEarlySlices)) early = slices / (2 * kEarlySlices);
   p.early_wgs = (int)early;
   const int64_t wgs = p.sample_wgs + early + (slices - early * kEarlySlices);
