@@ -154,6 +154,8 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->cand = nullptr;
   g->cand_seg_stride = 0;
   g->cand_head = nullptr;
+  g->cand_count = nullptr;
+  g->cut_splits = nullptr;
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   g->tokens_per_wg = gemv_tokens_per_wg(rows, g->chunk_len);
   g->wgs_per_chunk = (int)((g->chunk_len + g->tokens_per_wg - 1) / g->tokens_per_wg);
@@ -180,6 +182,26 @@ void candidate_plan(const tka_gemv_topk_args* a, int* num_samples, int* sample_r
   // (the candidate kernel addresses the rows of a slice with 32-bit byte offsets)
   if (!a->out_scores && cand_slices <= select_cand_max_parts() && a->key_stride_n < (int64_t)1 << 21)
     gemv_candidate_plan(chunk_len, (int64_t)a->batch * a->num_kv_heads * a->seq_len, a->k, select_cand_capacity(), num_samples, sample_rank);
+}
+
+// Samples per segment and rank of the cut when the call takes the common-cut route (a few segments of middling
+// length, rank-ordered output), else 0.  Shorter segments are selected from the registers of one workgroup, longer
+// ones (or many of them) by the sampling workgroups of the candidate route.
+int64_t cut_route_min_len() {
+  static const int64_t v = [] {
+    const char* e = getenv("TKA_CUT_MIN_LEN");
+    return e && *e ? (int64_t)atoll(e) : (int64_t)select_cand_capacity() + 1;
+  }();
+  return v;
+}
+void cut_plan(const tka_gemv_topk_args* a, bool want_union, int* num_samples, int* sample_rank) {
+  *num_samples = *sample_rank = 0;
+  const int64_t chunk_len = a->seq_len / a->num_chunks;
+  if (!a->out_idx || want_union || a->out_scores || chunk_len < cut_route_min_len()) return;
+  int cs = 0, cr = 0;
+  candidate_plan(a, &cs, &cr);
+  if (cs != 0) return;
+  gemv_cut_plan(chunk_len, a->k, num_samples, sample_rank);
 }
 
 struct UnionOut {
@@ -250,6 +272,34 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
 
   // Keys shared by the batch are read once for several batch entries.
   const bool shared_keys = a->key_stride_b == 0 && a->batch >= 2 && !cluster_ids;
+
+  // A few segments of middling length: every GEMV workgroup derives the segment's cut from common sample rows and
+  // stores its candidates, one workgroup per segment ranks them.
+  int cut_samples = 0, cut_rank = 0;
+  cut_plan(a, u != nullptr, &cut_samples, &cut_rank);
+  if (cut_samples != 0 && !ic) {
+    GemvParams cp = gp;
+    cp.hist = nullptr;
+    cp.tokens_per_wg = kCutTokensPerWg;
+    cp.wgs_per_chunk = (int)((chunk_len + kCutTokensPerWg - 1) / kCutTokensPerWg);
+    cp.num_samples = cut_samples;
+    cp.sample_rank = cut_rank;
+    cp.cand = sp.list;
+    cp.cand_seg_stride = sp.list_stride;
+    cp.cand_head = const_cast<uint64_t*>(sp.cand_head);
+    cp.cand_count = sp.list_cnt;
+    cp.cut_splits = (uint64_t*)sp.hist;   // (the histograms of the dense path: 8 KB per segment, free on this route)
+    int rc = launch_gemv_cut(cp, a->dtype, stream);
+    if (rc != TKA_OK) return rc;
+    SelectParams sc = sp;
+    sc.hist = nullptr;
+    sc.parts = cp.wgs_per_chunk;
+    sc.part_len = kCutTokensPerWg;
+    sc.max_entries = current_hooks().force_segment_redo ? 0 : kCutMaxCandidates;
+    sc.scores = scores;
+    sc.cut_splits = cp.cut_splits;
+    return launch_select_rank(gp, sc, a->dtype, stream);
+  }
 
   if (wave_route(a, u != nullptr)) {
     gp.hist = nullptr;
@@ -496,6 +546,7 @@ static int read_segment_flags(const tka_gemv_topk_args* a, std::vector<uint32_t>
   if (!a->workspace || a->workspace_bytes < tka_gemv_topk_workspace_bytes(a)) return TKA_EWORKSPACE;
   int num_samples = 0, sample_rank = 0;
   candidate_plan(a, &num_samples, &sample_rank);
+  if (num_samples == 0) cut_plan(a, false, &num_samples, &sample_rank);
   if (num_samples == 0) return TKA_OK;
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
   SelectParams sp;

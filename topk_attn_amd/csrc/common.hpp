@@ -33,6 +33,15 @@ constexpr int kTauSpinLimit = 1 << 16;     // polls of a streaming workgroup for
 // 512 candidates, so the selection kernel cannot take it for a count, and it redoes the segment from the keys.
 constexpr uint32_t kSliceGaveUp = 1023u;
 
+// Common-cut route (a few segments of middling length: gemv_cut_kernel + select_rank_kernel)
+constexpr int kCutTokensPerWg = 256;       // tokens (and threads) per workgroup of the GEMV = slice length
+constexpr int kCutHead = 64;               // entries of a slice that the ranking kernel reads in its first round trip
+constexpr int kCutMaxSlices = 128;         // slices per segment: segments of up to 32768 tokens
+constexpr int kCutMaxK = 2048;             // largest k
+constexpr int kCutMaxCandidates = 8192;    // candidates of one segment that the ranking kernel holds
+constexpr int kCutMaxExtras = 2048;        // of them, entries beyond the first kCutHead of their slices
+constexpr int kCutParts = 8;               // ranking workgroups per segment, each with its own range of the order
+
 // ---- lane exchanges ---------------------------------------------------------------------------
 
 // DPP move: returns the value of the lane selected by CTRL inside the 16-lane row.
@@ -173,6 +182,19 @@ __device__ __forceinline__ float key_score(uint32_t key) {
 }
 // 64-bit composite: all elements distinct, larger = earlier in (score desc, index asc) order.
 __device__ __forceinline__ uint64_t composite(uint32_t key, uint32_t idx) { return ((uint64_t)key << 32) | (uint32_t)~idx; }
+
+// ---- sampled thresholds -------------------------------------------------------------------------
+
+__device__ __forceinline__ uint32_t mix32(uint32_t x) {  // integer hash for the sample jitter
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return x;
+}
+
+// Token of sample i of a segment: one per stride, at a hashed offset inside the stride so that periodic data
+// cannot alias with the sampling.
+__device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) {
+  return (int64_t)i * stride + (int64_t)(mix32((uint32_t)seg * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
+}
 
 // ---- block-wide threshold search (1024 threads, 2048 bins) --------------------------------------
 

@@ -1,0 +1,198 @@
+// Stage 1, GEMV phase for a FEW segments of middling length (a single head of 32768 keys): problems that no launch
+// fills for long, so that what counts is the number of launches and of dependent round trips to memory, not bytes.
+//
+// Every workgroup scores its own slice of 256 tokens AND the same 256 sample tokens of its segment (spread evenly
+// over the segment, at hashed offsets; after the first workgroup they come from the L2), all loads in flight
+// together.  From the sample it takes the R-th largest element in the full order (score descending, token
+// ascending): the segment's cut.  All workgroups of a segment compute the same cut from the same rows, so nobody
+// waits for anybody.  Tokens at or above the cut are stored as the slice's candidates, as composites in token
+// order.  The candidates are an upper set of the order, so whenever at least k of them exist they contain the top
+// k; the ranking kernel (select_rank_kernel) checks that and otherwise redoes the segment from the keys.  About
+// n R / 256 candidates per segment, see gemv_cut_plan.
+//
+// The scores are the canonical ones (gemv_topk.cu:303-332 of the reference: fma chain over the lane's 8 dims,
+// xor butterfly over 16 lanes, one multiply).
+#include <math.h>
+
+#include "kernels.hpp"
+
+namespace tka {
+
+namespace {
+
+constexpr int kCutThreads = 1024;
+constexpr int kCutUnroll = 8;                                        // rows per lane
+constexpr int kCutRows = (kCutThreads / 16) * kCutUnroll;            // rows per workgroup: 512
+constexpr int kCutSamples = kCutRows - kCutTokensPerWg;              // 256
+static_assert(kCutSamples == 256 && kCutTokensPerWg == 256, "half of the row groups score the slice, half the sample");
+
+// Sixteen waves and a short program: row groups 0 .. 31 score the 256 tokens of the slice, row groups 32 .. 63 the
+// 256 sample tokens, one round of eight loads per lane.  (Few workgroups run at a time on these problems, so a wave
+// pays the first fetch of every line of code itself: the same work as four waves with four rounds each took twice
+// as long.)
+template <int DT>
+__global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
+  __shared__ __attribute__((aligned(16))) uint32_t sh_key[kCutRows];   // [0, 256) the slice, [256, 512) the sample
+  __shared__ uint32_t sh_wcnt[kCutTokensPerWg / kWave];
+  __shared__ uint32_t sh_cut[2];
+  __shared__ uint32_t sh_rank[kCutSamples];
+  __shared__ __attribute__((aligned(16))) uint32_t sh_rkey[kCutSamples];   // ranking keys of the samples
+
+  const int tid = threadIdx.x;
+  const int j = tid & 15, rg = tid >> 4;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int slice = (int)(blockIdx.x % (uint32_t)p.wgs_per_chunk);
+  const int seg = (int)(blockIdx.x / (uint32_t)p.wgs_per_chunk);
+  const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
+  const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
+  const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
+  const int n = (int)p.chunk_len;
+  const int t_begin = slice * kCutTokensPerWg;
+  const int n_local = n - t_begin < kCutTokensPerWg ? n - t_begin : kCutTokensPerWg;
+  const int64_t stride = n / kCutSamples;
+
+#ifdef TKA_PHASE_STAMPS
+  uint64_t st[8]; int ns = 0;
+#define STAMP() do { if (tid == 0) st[ns] = __builtin_amdgcn_s_memtime(); ++ns; } while (0)
+#else
+#define STAMP() do {} while (0)
+#endif
+  STAMP();
+  float qf[8];
+  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
+                          chunk_base * p.key_stride_n + 8 * j;
+  const bool sampler = rg >= kCutTokensPerWg / kCutUnroll;
+  u32x4 kv[kCutUnroll];
+#pragma unroll
+  for (int u = 0; u < kCutUnroll; ++u) {
+    const int row = rg * kCutUnroll + u;   // 0 .. 255 the slice, 256 .. 511 the sample
+    const int64_t t = sampler ? sample_token(seg, row - kCutTokensPerWg, stride) : (int64_t)(t_begin + (row < n_local ? row : n_local - 1));
+    kv[u] = *(const u32x4*)(kbase + t * p.key_stride_n);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  STAMP();
+  float mine = 0.0f;
+#pragma unroll
+  for (int u = 0; u < kCutUnroll; ++u) {
+    const float sc = row_score<DT>(qf, kv[u], p.scale);
+    if (j == u) mine = sc;
+  }
+  STAMP();
+  if (j < kCutUnroll) {
+    const int row = rg * kCutUnroll + j;
+    const uint32_t key = score_key(mine);
+    sh_key[row] = key;
+    if (sampler) sh_rkey[row - kCutTokensPerWg] = (key & ~0xffu) | (uint32_t)(kCutSamples - 1 - (row - kCutTokensPerWg));
+  }
+  if (tid < kCutSamples) sh_rank[tid] = 0;
+  __syncthreads();
+  STAMP();
+
+  // Rank of every sample by counting: thread (s, q) counts the samples of block q (64 of them, broadcast reads) that
+  // come before sample s, four threads per sample add up in LDS.  The order is that of the ranking keys (the key with
+  // its last 8 bits replaced by 255 - sample number): all different, so one compare decides, exactly one sample holds
+  // rank R - 1, and samples that share a key (heavy ties) come in token order, as in the full order (key descending,
+  // token ascending).  Keys that differ in their last 8 bits only may change places; any sample will do as the cut, it
+  // is its rank among the samples that makes the number of candidates what was planned.
+  // The samples of ranks R g / 8 - 1 split the candidates into eight parts of about equal size for the ranking
+  // kernel's eight workgroups per segment.
+  {
+    const int s = tid & (kCutSamples - 1), q = tid >> 8;   // q is the same for a whole wave
+    const uint32_t ks = sh_rkey[s];
+    const u32x4* blk = (const u32x4*)(sh_rkey + q * kWave);
+    uint32_t ahead = 0;
+#pragma unroll
+    for (int i = 0; i < kWave / 4; ++i) {
+      const u32x4 kj = blk[i];
+      ahead += (kj[0] > ks ? 1u : 0u) + (kj[1] > ks ? 1u : 0u) + (kj[2] > ks ? 1u : 0u) + (kj[3] > ks ? 1u : 0u);
+    }
+    atomicAdd(&sh_rank[s], ahead);
+  }
+  __syncthreads();
+  if (tid < kCutSamples) {
+    const uint32_t r = sh_rank[tid] + 1u, rank = (uint32_t)p.sample_rank;   // 1-based
+    uint32_t part = 0;   // 1 .. 8 when this sample ends part `part` of the candidates (8: the cut itself)
+#pragma unroll
+    for (uint32_t gq = 1; gq <= (uint32_t)kCutParts; ++gq) part = r == rank * gq / (uint32_t)kCutParts ? gq : part;
+    if (part != 0) {   // (R >= 8: every part has a sample of its own)
+      const uint32_t token = (uint32_t)sample_token(seg, tid, stride);
+      if (part == (uint32_t)kCutParts) { sh_cut[0] = sh_key[kCutTokensPerWg + tid]; sh_cut[1] = token; }
+      if (slice == 0) p.cut_splits[(int64_t)seg * kCutParts + (part - 1)] = composite(sh_key[kCutTokensPerWg + tid], token);
+    }
+  }
+  __syncthreads();
+  STAMP();
+  if (tid >= kCutTokensPerWg) return;
+
+  // thread t owns token t_begin + t.  Entries are composites (key << 32 | ~token, token counted inside the segment),
+  // ascending in token; the first kCutHead of a slice go to its place in the dense head array, which is always
+  // written whole (zeros behind the last candidate: no composite is zero), the rest to the slice's place in the wide
+  // array; the slice's count goes to its own word.
+  const uint32_t tau = sh_cut[0], cut = sh_cut[1];
+  const uint32_t key = sh_key[tid];
+  const uint32_t token = (uint32_t)(t_begin + tid);
+  const bool pass = tid < n_local && (key > tau || (key == tau && token <= cut));
+  const unsigned long long mask = __ballot(pass);
+  if (lane == 0) sh_wcnt[wave] = (uint32_t)__popcll(mask);
+  __syncthreads();   // (the waves that have ended no longer count)
+  uint32_t ahead = 0, total = 0;
+#pragma unroll
+  for (int v = 0; v < kCutTokensPerWg / kWave; ++v) {
+    const uint32_t c = sh_wcnt[v];
+    ahead += v < wave ? c : 0u;
+    total += c;
+  }
+  const int64_t slice_id = (int64_t)seg * p.wgs_per_chunk + slice;
+  uint64_t* head = p.cand_head + slice_id * kCutHead;
+  uint64_t* wide = p.cand + (int64_t)seg * p.cand_seg_stride + (int64_t)slice * kCutTokensPerWg;
+  if (pass) {
+    const uint32_t pos = ahead + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+    (pos < (uint32_t)kCutHead ? head : wide)[pos] = composite(key, token);
+  }
+  if ((uint32_t)tid >= total && tid < kCutHead) head[tid] = 0ull;
+  if (tid == 0) p.cand_count[slice_id] = total;
+  STAMP();
+#ifdef TKA_PHASE_STAMPS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  STAMP();
+  if (tid == 0) for (int i = 0; i < ns; ++i) ((uint64_t*)p.scores)[blockIdx.x * 8 + i] = st[i];
+#endif
+}
+
+}  // namespace
+
+int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
+  const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
+  if (p.tokens_per_wg != kCutTokensPerWg || p.num_samples != kCutSamples || p.chunk_len < kCutSamples || p.sample_rank < 1 ||
+      p.sample_rank > kCutSamples || !p.cand || !p.cand_head || !p.cand_count || !p.cut_splits || segs * p.wgs_per_chunk > 0x7fffffffLL)
+    return TKA_EINVAL;
+  const unsigned wgs = (unsigned)(segs * p.wgs_per_chunk);
+  LaunchTimer timer("gemv_cut", stream);
+  if (dtype == TKA_F16)
+    gemv_cut_kernel<TKA_F16><<<wgs, kCutThreads, 0, stream>>>(p);
+  else
+    gemv_cut_kernel<TKA_BF16><<<wgs, kCutThreads, 0, stream>>>(p);
+  return hip_status(hipGetLastError());
+}
+
+// Samples per segment and rank of the cut for a segment of chunk_len tokens and k, or 0 samples when this route
+// does not serve the shape.  With S = 256 samples spread evenly and m = k S / n of them expected inside the top k, the
+// rank is R = m + 5.5 sqrt(m) + 2: "fewer than k tokens pass" (the segment is then redone from the keys, still
+// exact) needs R of the samples inside the top k, more than five deviations out; about n R / S candidates are
+// stored.  Limits: a slice of 256 tokens should stay within the kCutHead entries that the ranking kernel reads
+// in its first round trip (40 expected at most), and a segment within what it ranks in one go.
+void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank) {
+  *num_samples = *sample_rank = 0;
+  if (chunk_len < 2048 || chunk_len > (int64_t)kCutMaxSlices * kCutTokensPerWg || k > kCutMaxK || (int64_t)k * 8 > chunk_len) return;
+  const int s = kCutSamples;
+  const double m = (double)k * s / (double)chunk_len;
+  int r = (int)ceil(m + 5.5 * sqrt(m) + 2.0);
+  if (r < kCutParts) r = kCutParts;   // every part of the candidates ends with a sample of its own
+  const double per_slice = (double)kCutTokensPerWg * r / s, per_segment = (double)chunk_len * r / s;
+  if (r * 2 > s || per_slice > 40.0 || per_segment * 1.25 > (double)kCutMaxCandidates) return;
+  *num_samples = s;
+  *sample_rank = r;
+}
+
+}  // namespace tka

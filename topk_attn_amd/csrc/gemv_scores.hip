@@ -263,17 +263,6 @@ __global__ __launch_bounds__(kGemvThreads) __attribute__((amdgpu_waves_per_eu(4,
 
 // ---- candidate mode -----------------------------------------------------------------------------
 
-__device__ __forceinline__ uint32_t mix32(uint32_t x) {  // integer hash for the sample jitter
-  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
-  return x;
-}
-
-// Token of sample i of a segment: one per stride, at a hashed offset inside the stride so that periodic data
-// cannot alias with the sampling.
-__device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) {
-  return (int64_t)i * stride + (int64_t)(mix32((uint32_t)seg * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
-}
-
 // Sampling workgroup: scores 256 of the segment's p.num_samples sample tokens (one round of
 // loads) and stores their keys in the segment's pool.  The workgroup that arrives last (epoch-valued arrival
 // flags, so that the workspace needs no clearing) takes the p.sample_rank-th largest key of the whole pool and

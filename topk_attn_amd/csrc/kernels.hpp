@@ -35,6 +35,9 @@ struct GemvParams {
   uint64_t* cand_head;        // [segments][wgs_per_chunk][kCandHead] entries 0 .. kCandHead-1 of every slice, densely packed:
                               // an ordinary slice (about 18 candidates) lies here whole, two full lines that stay in the
                               // L2 until the kernel ends; `cand` only takes what goes beyond (heavy ties)
+  uint32_t* cand_count;       // common-cut route: [segments][wgs_per_chunk] candidates of every slice
+  uint64_t* cut_splits;       // common-cut route: [segments][kCutParts] composites of the samples that end the parts of the
+                              // candidates in rank order; the last one is the cut itself
   int64_t chunk_len;    // tokens per chunk
   int64_t q_stride_b, key_stride_b, key_stride_n, key_stride_h;
   int batch, num_kv_heads, group, num_chunks;
@@ -49,6 +52,11 @@ int launch_gemv_scores_mfma(const GemvParams& p, int dtype, hipStream_t stream);
 int launch_gemv_candidates(const GemvParams& p, int dtype, hipStream_t stream);   // thresholds + candidate slices
 void gemv_candidate_plan(int64_t chunk_len, int64_t total_rows, int k, int max_candidates, int* num_samples, int* sample_rank);
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);
+// Common-cut route: every workgroup derives the segment's cut from the same sample rows and stores its slice's candidates
+// (p.cand_head: the first kCutHead of a slice as composites, zeros behind; p.cand: the rest; p.cand_count; p.num_samples /
+// p.sample_rank from gemv_cut_plan).
+int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream);
+void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank);
 
 // ---- stage 1: selection -----------------------------------------------------------------------
 struct SelectParams {
@@ -67,6 +75,7 @@ struct SelectParams {
   uint32_t* list_cnt;     // [num_segments][parts] entries in each slice list (finalize turns them into offsets)
   uint64_t* list;         // [num_segments][list_stride] composites with bin >= threshold bin, slice p at p*part_len
   const uint64_t* cand_head;  // candidate mode: [num_segments][parts][kCandHead] the first entries of every slice
+  const uint64_t* cut_splits; // common-cut route: [num_segments][kCutParts], see GemvParams
   int64_t list_stride;
   int32_t* out_idx;       // [num_segments][out_stride] rank order, or nullptr (no sort)
   float* out_val;         // same shape or nullptr
@@ -97,6 +106,9 @@ int launch_select_finalize(const SelectParams& p, hipStream_t stream);
 // Candidate slices -> outputs; a segment whose slices cannot be used is redone from the keys by its workgroup.
 int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
 int select_cand_max_parts();   // most candidate slices per segment
+// Common-cut route: ranks the candidates of a segment by counting and writes the top k in rank order (and the expansion);
+// p.list / p.list_stride / p.parts describe the slices written by launch_gemv_cut.
+int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
 int select_cand_capacity();    // most candidates per segment
 // One workgroup per segment, keys in registers: rank-ordered top-k of fp32 scores, segments of up to
 // select_wave_max_len() scores, k up to select_wave_max_k(segment length).

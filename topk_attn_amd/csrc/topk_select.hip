@@ -948,6 +948,234 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   write_rank_outputs(sh_sort, p, seg);
 }
 
+// ---- ranking of the common-cut route ---------------------------------------------------------------
+
+constexpr uint32_t kCutBucketMax = 192;   // a bucket with more members than this sends the part to the sorting network
+
+// Rank-ordered outputs of one candidate: index, value and expansion at position `rank` of segment `seg`.
+__device__ __forceinline__ void write_ranked(const SelectParams& p, int seg, uint32_t idx_base, uint32_t rank, uint64_t c) {
+  const uint32_t id = ~(uint32_t)c + idx_base;
+  p.out_idx[(int64_t)seg * p.out_stride + rank] = (int32_t)id;
+  if (p.out_val) p.out_val[(int64_t)seg * p.out_stride + rank] = key_score((uint32_t)(c >> 32));
+  if (p.out_expand) {
+    int32_t* oe = p.out_expand + ((int64_t)seg * p.k + rank) * p.expand;
+    for (int i = 0; i < p.expand; ++i) oe[i] = (int32_t)(~(uint32_t)c * (uint32_t)p.expand + (uint32_t)i);
+  }
+}
+
+// Common-cut route: the slices (256 tokens each, written by gemv_cut_kernel) hold every token at or above the
+// segment's cut, as composites, and kCutParts sample composites split the order into parts of about equal size.
+// kCutParts workgroups per segment (one CU executes 64 lane-operations per cycle, and this is a kernel of a few
+// workgroups: what one workgroup would spend on all candidates is the kernel's duration).  Each reads the head
+// entries of ALL slices (a dense array, zeros behind a slice's last candidate) and the slice counts in one round
+// trip (the rare slice with more than kCutHead candidates costs a second trip), counts the candidates above its
+// part, and ranks the candidates of its part by counting instead of selecting and then sorting: composite minus the
+// part's lower end, cut to its 11 leading bits, gives 2048 buckets in rank order; a histogram and one suffix scan
+// give every bucket its first rank, the composites are scattered to their bucket, and each one counts the larger
+// members of its own bucket.  rank < k: selected, and the rank is the output position.  Heavy ties that fill a bucket
+// send the part to the bitonic network; a segment with fewer than k candidates (the sample misjudged it) or more than
+// fit is redone from the keys by its first workgroup (fallback_segment).
+// Dynamic LDS: kCutMaxCandidates composites (the part, as found), then as many again (the part in bucket order;
+// before that, entries from beyond the heads); the tie path and the fallback reuse both.
+template <int DT>
+__global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, SelectParams p, int kpad) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint64_t* sh_own = (uint64_t*)smem;
+  uint64_t* sh_x = sh_own + kCutMaxCandidates;
+  uint64_t* sh_extra = sh_x;
+  __shared__ uint32_t sh_hist[kHistBins], sh_off[kHistBins], sh_cur[kHistBins];
+  __shared__ uint32_t sh_wtot[kSelWaves];
+  __shared__ uint32_t sh_res[4];
+  __shared__ uint64_t sh_mm[3];
+  __shared__ uint64_t sh_split[kCutParts + 1];
+  __shared__ uint32_t sh_ovf[kCutMaxSlices];
+  __shared__ uint32_t sh_n[8];   // [0] slices with more than kCutHead entries, [1] entries beyond the heads, [2] candidates,
+                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key
+
+  typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+  constexpr int kPairs = kCutMaxSlices * kCutHead / 2 / kSelThreads;   // pairs of head entries per thread: 4
+  constexpr int kMine = 2 * kPairs + kCutMaxExtras / kSelThreads;       // composites per thread: 10
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int seg = blockIdx.x / kCutParts, part = blockIdx.x % kCutParts;
+  const uint32_t k = (uint32_t)p.k;
+  const u64x2* heads = (const u64x2*)(p.cand_head + (int64_t)seg * p.parts * kCutHead);
+  const int n_pairs = p.parts * (kCutHead / 2);
+
+#ifdef TKA_PHASE_STAMPS
+  uint64_t st[12]; int ns = 0;
+#define STAMP() do { if (tid == 0) st[ns] = __builtin_amdgcn_s_memtime(); ++ns; } while (0)
+#else
+#define STAMP() do {} while (0)
+#endif
+  STAMP();
+  u64x2 w[kPairs];
+#pragma unroll
+  for (int e = 0; e < kPairs; ++e) {
+    const int q = e * kSelThreads + tid;
+    w[e] = q < n_pairs ? heads[q] : (u64x2){0ull, 0ull};
+  }
+  const uint32_t slice_cnt = tid < p.parts ? p.list_cnt[(int64_t)seg * p.parts + tid] : 0u;
+  // ends of the parts, in descending order: [part] above this workgroup's part, [part + 1] its lower end
+  // (as a running minimum: the samples were ranked by keys whose last bits were replaced, so two of them may come
+  // in the other order here)
+  if (tid == 0) {
+    uint64_t sp[kCutParts];
+#pragma unroll
+    for (int i = 0; i < kCutParts; ++i) sp[i] = p.cut_splits[(int64_t)seg * kCutParts + i];
+    uint64_t low = ~0ull;
+    sh_split[0] = low;
+#pragma unroll
+    for (int i = 0; i < kCutParts; ++i) {
+      low = sp[i] < low ? sp[i] : low;
+      sh_split[i + 1] = low;
+    }
+  }
+  sh_hist[2 * tid] = 0;
+  sh_hist[2 * tid + 1] = 0;
+  if (tid < 8) sh_n[tid] = 0;
+  __syncthreads();
+  STAMP();
+  if (slice_cnt > (uint32_t)kCutHead) sh_ovf[atomicAdd(&sh_n[0], 1u)] = (uint32_t)tid | (slice_cnt << 16);
+  __syncthreads();
+  const uint32_t n_ovf = sh_n[0];
+  if (n_ovf) {   // rare: slices whose candidates go beyond the head entries (scores that cluster in one place)
+    const uint64_t* wide = p.list + (int64_t)seg * p.list_stride;
+    for (uint32_t i = 0; i < n_ovf; ++i) {
+      const uint32_t sl = sh_ovf[i] & 0xffffu, cnt = sh_ovf[i] >> 16;
+      const uint32_t j = (uint32_t)kCutHead + (uint32_t)tid;
+      if (j < cnt) {
+        const uint64_t x = wide[(int64_t)sl * kCutTokensPerWg + j];
+        const uint32_t pos = atomicAdd(&sh_n[1], 1u);
+        if (pos < (uint32_t)kCutMaxExtras) sh_extra[pos] = x;
+      }
+    }
+    __syncthreads();
+  }
+  const uint32_t n_extra = sh_n[1];
+  uint64_t c[kMine];
+#pragma unroll
+  for (int e = 0; e < kPairs; ++e) {
+    c[2 * e] = w[e][0];
+    c[2 * e + 1] = w[e][1];
+  }
+#pragma unroll
+  for (int e = 0; e < kCutMaxExtras / kSelThreads; ++e) {
+    const uint32_t i = (uint32_t)e * kSelThreads + tid;
+    c[2 * kPairs + e] = (n_ovf && i < n_extra && i < (uint32_t)kCutMaxExtras) ? sh_extra[i] : 0ull;
+  }
+  if (n_ovf) __syncthreads();   // the extras are in registers: their place becomes the bucket-ordered part
+
+  // all candidates, those above this part, those of the part (collected in LDS), the part's largest key
+  const uint64_t t_hi = sh_split[part], t_lo = sh_split[part + 1];
+  {
+    uint32_t n_all = 0, n_above = 0, kmax = 0;
+#pragma unroll
+    for (int i = 0; i < kMine; ++i) {
+      const bool nz = c[i] != 0ull;
+      const bool above = part != 0 && c[i] >= t_hi;
+      const bool own = nz && !above && c[i] >= t_lo;
+      n_all += nz ? 1u : 0u;
+      n_above += above ? 1u : 0u;
+      if (own) {
+        sh_own[atomicAdd(&sh_n[5], 1u)] = c[i];
+        kmax = max(kmax, (uint32_t)(c[i] >> 32));
+      }
+    }
+    const uint32_t inc = wave_inclusive_scan((n_all << 16) | n_above);   // (at most 10 x 64 per wave each)
+    kmax = max(kmax, lane_xor<1>(kmax));
+    kmax = max(kmax, lane_xor<2>(kmax));
+    kmax = max(kmax, lane_xor<4>(kmax));
+    kmax = max(kmax, lane_xor<8>(kmax));
+    kmax = max(kmax, lane_xor<16>(kmax));
+    kmax = max(kmax, lane_xor<32>(kmax));
+    if (lane == 63) {
+      atomicAdd(&sh_n[2], inc >> 16);
+      atomicAdd(&sh_n[4], inc & 0xffffu);
+      atomicMax(&sh_n[6], kmax);
+    }
+  }
+  __syncthreads();
+  STAMP();
+  const uint32_t n_cand = sh_n[2], n_above = sh_n[4], n_own = sh_n[5];
+  const uint32_t cap = (uint32_t)(p.max_entries < kCutMaxCandidates ? p.max_entries : kCutMaxCandidates);
+  const bool redo = n_cand < k || n_cand > cap || n_extra > (uint32_t)kCutMaxExtras;
+  if (tid == 0 && part == 0) p.seg_flags[seg] = redo ? 1u : 0u;
+  if (redo) {   // every workgroup of the segment sees the same counts: the first one redoes it, the others leave
+    if (part != 0) return;
+    __syncthreads();
+    fallback_segment<DT>(g, p, seg, kpad, sh_own, sh_hist, sh_off, sh_wtot, sh_res, sh_mm);
+    return;
+  }
+  if (n_above >= k || n_own == 0u) return;   // nothing of this part is selected
+
+  // buckets: linear in the composite between the ends of the part (the first part ends at its largest key)
+  const uint64_t base = t_lo;
+  const uint64_t span = (part == 0 ? (((uint64_t)sh_n[6] << 32) | 0xffffffffull) : t_hi) - base;
+  const int fixed = __builtin_clzll(span | 1ull);
+  const int shift = 64 - fixed > kHistBits ? 64 - fixed - kHistBits : 0;
+#pragma unroll 1
+  for (uint32_t i = tid; i < n_own; i += kSelThreads) atomicAdd(&sh_hist[(uint32_t)((sh_own[i] - base) >> shift)], 1u);
+  __syncthreads();
+  STAMP();
+  // first rank of every bucket: number of composites in higher buckets (thread t owns buckets 2t, 2t+1)
+  {
+    const int wave = tid >> 6;
+    const uint32_t h0 = sh_hist[2 * tid], h1 = sh_hist[2 * tid + 1];
+    const uint32_t mine = h0 + h1;
+    const uint32_t inc = wave_inclusive_scan(mine);
+    const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)inc, 63);
+    const uint32_t ge = wave_total - inc + mine;   // this wave's composites in buckets >= 2t
+    if (lane == 0) sh_wtot[wave] = ge;
+    if (h0 > kCutBucketMax || h1 > kCutBucketMax) sh_n[3] = 1u;
+    __syncthreads();
+    uint32_t above = 0;
+    for (int v = wave + 1; v < kSelWaves; ++v) above += sh_wtot[v];
+    sh_off[2 * tid + 1] = sh_cur[2 * tid + 1] = above + ge - mine;   // buckets > 2t+1
+    sh_off[2 * tid] = sh_cur[2 * tid] = above + ge - h0;             // buckets > 2t
+  }
+  __syncthreads();
+  STAMP();
+  const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len) : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
+  if (sh_n[3] != 0u) {
+    // heavy ties: sort the part and take it in order
+    uint32_t npad = 64;
+    while (npad < n_own) npad <<= 1;
+    for (uint32_t i = n_own + tid; i < npad; i += kSelThreads) sh_own[i] = 0;   // pad: below every real composite
+    __syncthreads();
+    sort_lds_desc(sh_own, sh_x, (int)npad);
+    for (uint32_t i = tid; i < n_own; i += kSelThreads)
+      if (n_above + i < k) write_ranked(p, seg, idx_base, n_above + i, sh_own[i]);
+    return;
+  }
+#pragma unroll 1
+  for (uint32_t i = tid; i < n_own; i += kSelThreads) {
+    const uint64_t x = sh_own[i];
+    sh_x[atomicAdd(&sh_cur[(uint32_t)((x - base) >> shift)], 1u)] = x;
+  }
+  __syncthreads();
+  STAMP();
+  // every candidate of the part: its rank is the candidates above the part, plus the first rank of its bucket, plus the
+  // larger members of the bucket
+#pragma unroll 1
+  for (uint32_t i = tid; i < n_own; i += kSelThreads) {
+    const uint64_t x = sh_x[i];
+    const uint32_t bin = (uint32_t)((x - base) >> shift);
+    const uint32_t start = sh_off[bin], cnt = sh_hist[bin];
+    uint32_t larger = 0;
+    for (uint32_t j = 0; j < cnt; ++j) larger += sh_x[start + j] > x ? 1u : 0u;
+    const uint32_t rank = n_above + start + larger;
+    if (rank < k) write_ranked(p, seg, idx_base, rank, x);
+  }
+  STAMP();
+#ifdef TKA_PHASE_STAMPS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  STAMP();
+  if (tid == 0) for (int i = 0; i < ns; ++i) ((uint64_t*)g.scores)[2048 + blockIdx.x * 16 + i] = st[i];
+#endif
+}
+
 // Ascending duplicate-free union of the selected ids with [0,sink) and [n-local,n).
 // One workgroup per segment; the middle part is sorted ascending with the same bitonic network
 // (ids complemented so that "descending" composites are ascending ids).
@@ -1042,7 +1270,11 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   const size_t cand_segs = seg_len >= kCandMinSegLen ? (size_t)num_segments : 0;   // sampling state: long segments only
   l.ctr = take(cand_segs * 64 * sizeof(uint32_t));
   l.pool = take(cand_segs * kGemvMaxSamples * sizeof(uint32_t));
-  l.head = take(cand_segs * (size_t)(seg_len / kGemvCandTokensPerWg + 1) * kCandHead * sizeof(uint64_t));
+  // head entries of the slices: the candidate route (32 per slice of 512 tokens) or the common-cut route (64 per slice of 256)
+  const size_t cut_segs = seg_len <= (int64_t)kCutMaxSlices * kCutTokensPerWg ? (size_t)num_segments : 0;
+  const size_t head_cand = cand_segs * (size_t)(seg_len / kGemvCandTokensPerWg + 1) * kCandHead * sizeof(uint64_t);
+  const size_t head_cut = cut_segs * (size_t)(seg_len / kCutTokensPerWg + 1) * kCutHead * sizeof(uint64_t);
+  l.head = take(head_cand > head_cut ? head_cand : head_cut);
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
   l.total = off;
@@ -1165,6 +1397,22 @@ int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int 
     select_finalize_cand_kernel<TKA_F16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
   else
     select_finalize_cand_kernel<TKA_BF16><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
+  return hip_status(hipGetLastError());
+}
+
+int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
+  if (p.parts < 1 || p.parts > kCutMaxSlices || p.part_len != kCutTokensPerWg || p.k > kCutMaxK || !p.out_idx || p.union_idx || !p.cand_head ||
+      !p.list_cnt || !p.cut_splits)
+    return TKA_EINVAL;
+  const int lds = 2 * kCutMaxCandidates * (int)sizeof(uint64_t);
+  if (allow_dynamic_lds((const void*)select_rank_kernel<TKA_F16>, lds) != TKA_OK ||
+      allow_dynamic_lds((const void*)select_rank_kernel<TKA_BF16>, lds) != TKA_OK)
+    return TKA_EHIP;
+  LaunchTimer timer("select_rank", stream);
+  if (dtype == TKA_F16)
+    select_rank_kernel<TKA_F16><<<(unsigned)p.num_segments * kCutParts, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
+  else
+    select_rank_kernel<TKA_BF16><<<(unsigned)p.num_segments * kCutParts, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
   return hip_status(hipGetLastError());
 }
 
