@@ -218,7 +218,7 @@ def _sampled_positions(seg, n, samples=2048):
     """Token positions the threshold estimate of a long segment looks at: one per stride of n/samples tokens, at a
     hashed offset inside the stride (2048 samples for segments below 512K tokens)."""
     stride = n // samples
-    return [i * stride + _mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) % stride for i in range(samples)]
+    return [i * stride + ((_mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) * stride) >> 32) for i in range(samples)]
 
 
 def _check_long(K, q, dtype, G, k, scale=SCALE, redone=None, gave_up=None):
@@ -276,7 +276,7 @@ def test_long_segment_sample_hits_only_heavy_tokens_falls_back():
     qf = rng.standard_normal((1, 2, 128))
     pos = _sampled_positions(0, N)                       # segment 0 = (batch 0, head 0)
     Kf[0, pos, 0, :] = qf[0, 0] * rng.uniform(0.5, 1.5, (len(pos), 1))   # large positive scores, all distinct
-    _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k)
+    _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k, redone=1)
 
 
 def test_long_segment_bf16_levels_group8():
@@ -419,3 +419,96 @@ def test_long_segment_threshold_never_published(hooks, withheld):
     K[0, rng.permutation(131072)[:1300]] = oracle.to_bits(rng.standard_normal((1300, 2, 128)) * 4.0, oracle.F16)
     affected = 2 // mod
     _check_long(K, randn_bits(rng, (1, 2, 128), oracle.F16), oracle.F16, 1, 2048, redone=affected, gave_up=affected * 256)
+
+
+# ---- a few segments of middling length: a cut from common sample rows, candidates ranked by counting ----
+
+@pytest.mark.parametrize("dtype,B,H,G,N,k", [(oracle.F16, 1, 1, 1, 32768, 2048), (oracle.BF16, 1, 2, 4, 20011, 1000),
+                                             (oracle.F16, 2, 2, 1, 65536, 2048), (oracle.F16, 1, 1, 8, 40000, 1),
+                                             (oracle.BF16, 1, 3, 2, 16385, 2048)])
+def test_common_cut_route(dtype, B, H, G, N, k):
+    """Calls of up to 262144 rows with segments of 16385 .. 65536 tokens and no score output: every GEMV workgroup
+    derives the same cut from 256 sample rows, eight ranking workgroups per segment rank the candidates.  Ordinary
+    data with heavy hitters; no segment is redone from the keys."""
+    announce("gemv_topk common-cut route dtype=%d B=%d H=%d G=%d N=%d k=%d" % (dtype, B, H, G, N, k))
+    rng = np.random.default_rng(51)
+    K = randn_bits(rng, (B, N, H, 128), dtype)
+    K[:, rng.permutation(N)[:N // 100]] = oracle.to_bits(rng.standard_normal((B, N // 100, H, 128)) * 4.0, dtype)
+    _check_long(K, randn_bits(rng, (B, H * G, 128), dtype), dtype, G, k, redone=0)
+
+
+@pytest.mark.parametrize("kind", ["levels", "all_equal", "two_buckets", "ramp", "tail_block"])
+def test_common_cut_route_ties_and_clusters(kind):
+    """Ties (16-level keys, constant keys, three-valued scores with the k-th inside a bucket of thousands of equal
+    scores) and top scores that sit in one place (a ramp over the tokens; all of the top k in the last tokens, so
+    that their slices hold more candidates than the ranking kernel reads in its first round trip)."""
+    announce("gemv_topk common-cut route, %s" % kind)
+    rng = np.random.default_rng(52)
+    dtype, N, k = oracle.F16, 32768, 2048
+    q = randn_bits(rng, (1, 1, 128), dtype)
+    if kind == "levels":
+        K = oracle.to_bits(np.linspace(-2, 2, 16)[rng.integers(0, 16, (1, N, 1, 128))], dtype)
+    elif kind == "all_equal":
+        K = np.broadcast_to(randn_bits(rng, (1, 1, 1, 128), dtype), (1, N, 1, 128)).copy()
+    else:
+        col = np.full(N, -1.0)
+        if kind == "two_buckets":
+            col[rng.permutation(N)[:9000]] = 0.5
+            col[rng.permutation(N)[:700]] = 2.0
+        elif kind == "ramp":
+            col = np.linspace(-1.0, 1.0, N) + rng.standard_normal(N) * 0.01
+        else:
+            col = rng.standard_normal(N) * 0.1
+            col[N - 2300:] += 3.0
+        Kf = np.zeros((1, N, 1, 128))
+        Kf[0, :, 0, 5] = col
+        qf = np.zeros((1, 1, 128))
+        qf[0, 0, 5] = 1.0            # unit query: the score is one key column
+        K, q = oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype)
+    _check_long(K, q, dtype, 1, k, scale=1.0, redone=0)
+
+
+def _cut_sample_positions(seg, n):
+    """Token positions of the 256 sample rows of a segment on the common-cut route."""
+    stride = n // 256
+    return [i * stride + ((_mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) * stride) >> 32) for i in range(256)]
+
+
+def test_common_cut_route_adversarial_sample_falls_back():
+    """Heavy tokens exactly where the cut is sampled: the cut lands among them, fewer than k tokens pass, and the
+    segment is redone from the keys by its first ranking workgroup; the other head keeps the route."""
+    announce("gemv_topk common-cut route, adversarial sample (fallback)")
+    rng = np.random.default_rng(53)
+    N, k, dtype = 32768, 2048, oracle.F16
+    Kf = rng.standard_normal((1, N, 2, 128)) * 0.05
+    qf = rng.standard_normal((1, 2, 128))
+    pos = _cut_sample_positions(0, N)
+    Kf[0, pos, 0, :] = qf[0, 0] * rng.uniform(0.5, 1.5, (len(pos), 1))
+    _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k, redone=1)
+
+
+def test_common_cut_route_forced_redo(hooks):
+    announce("gemv_topk common-cut route, every segment redone from the keys")
+    hooks(force_segment_redo=1)
+    rng = np.random.default_rng(54)
+    K = randn_bits(rng, (1, 30001, 2, 128), oracle.BF16)
+    _check_long(K, randn_bits(rng, (1, 4, 128), oracle.BF16), oracle.BF16, 2, 1500, redone=2)
+
+
+def test_common_cut_route_chunked():
+    """Two chunks of 32768 tokens per head: per-chunk top-k with indices counted over the whole sequence."""
+    announce("gemv_topk common-cut route, 2 chunks x 32768")
+    from topk_attn_amd import ops
+    rng = np.random.default_rng(55)
+    dtype, N, k = oracle.F16, 65536, 1024
+    K = randn_bits(rng, (1, N, 2, 128), dtype)
+    q = randn_bits(rng, (1, 2, 128), dtype)
+    idx, val = ops.gemv_topk(to_dev(q, dtype), to_dev(K, dtype), k, scale=SCALE, num_chunks=2)
+    torch.cuda.synchronize()
+    idx, val = idx.cpu().numpy(), val.cpu().numpy()
+    for h in range(2):
+        ref = oracle.scores_canonical(K[0, :, h, :], dtype, oracle.group_query(q[0, h:h + 1], dtype, 1), SCALE)
+        for c in range(2):
+            ei, ev = oracle.topk_stable(ref[c * 32768:(c + 1) * 32768], k)
+            assert np.array_equal(idx[0, h, c * k:(c + 1) * k], ei + c * 32768)
+            assert np.array_equal(val[0, h, c * k:(c + 1) * k].view(np.uint32), ev.view(np.uint32))

@@ -36,10 +36,11 @@ constexpr uint32_t kSliceGaveUp = 1023u;
 // Common-cut route (a few segments of middling length: gemv_cut_kernel + select_rank_kernel)
 constexpr int kCutTokensPerWg = 256;       // tokens (and threads) per workgroup of the GEMV = slice length
 constexpr int kCutHead = 64;               // entries of a slice that the ranking kernel reads in its first round trip
-constexpr int kCutMaxSlices = 128;         // slices per segment: segments of up to 32768 tokens
+constexpr int kCutMaxSlices = 256;         // slices per segment: segments of up to 65536 tokens
 constexpr int kCutMaxK = 2048;             // largest k
 constexpr int kCutMaxCandidates = 8192;    // candidates of one segment that the ranking kernel holds
-constexpr int kCutMaxExtras = 2048;        // of them, entries beyond the first kCutHead of their slices
+constexpr int kCutMaxExtras = 6144;        // of them, entries beyond the first kCutHead of their slices
+constexpr int64_t kCutMaxRows = 262144;    // rows of a call (all segments) up to which the route is taken
 constexpr int kCutParts = 8;               // ranking workgroups per segment, each with its own range of the order
 
 // ---- lane exchanges ---------------------------------------------------------------------------
@@ -146,17 +147,29 @@ struct Elem<TKA_BF16> {
 // ---- canonical row score (gemv_topk.cu:303-332) ------------------------------------------------
 
 // Group query of this lane in fp32: ((q0 + q1) + q2) + ... in ascending head order, dims 8j..8j+7.
-template <int DT>
+// Groups are 1, 2, 4 or 8 heads; up to PAR heads of a group are asked for together (one round trip, not one per head;
+// PAR bounds the registers in flight for kernels that have few).
+template <int DT, int G, int PAR>
+__device__ __forceinline__ void sum_group_query(const uint16_t* qb, float (&qf)[8]) {
+  constexpr int P = G < PAR ? G : PAR;
+#pragma unroll
+  for (int g0 = 0; g0 < G; g0 += P) {
+    u32x4 w[P];
+#pragma unroll
+    for (int g = 0; g < P; ++g) w[g] = *(const u32x4*)(qb + (int64_t)(g0 + g) * kHeadDim);
+#pragma unroll
+    for (int g = 0; g < P; ++g)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[i] = (g0 + g == 0) ? Elem<DT>::get(w[g], i) : qf[i] + Elem<DT>::get(w[g], i);
+  }
+}
+template <int DT, int PAR = 8>
 __device__ __forceinline__ void load_group_query(const void* q, int64_t q_stride_b, int b, int h, int group, int j, float (&qf)[8]) {
   const uint16_t* qb = (const uint16_t*)q + (int64_t)b * q_stride_b + (int64_t)h * group * kHeadDim + 8 * j;
-  u32x4 v = *(const u32x4*)qb;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) qf[i] = Elem<DT>::get(v, i);
-  for (int g = 1; g < group; ++g) {
-    u32x4 w = *(const u32x4*)(qb + (int64_t)g * kHeadDim);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) qf[i] = qf[i] + Elem<DT>::get(w, i);
-  }
+  if (group == 1) sum_group_query<DT, 1, PAR>(qb, qf);
+  else if (group == 2) sum_group_query<DT, 2, PAR>(qb, qf);
+  else if (group == 4) sum_group_query<DT, 4, PAR>(qb, qf);
+  else sum_group_query<DT, 8, PAR>(qb, qf);
 }
 
 // Canonical score of the row in `kv` for the lane's 8 dims: fma chain, DPP butterfly, one multiply.
@@ -193,7 +206,8 @@ __device__ __forceinline__ uint32_t mix32(uint32_t x) {  // integer hash for the
 // Token of sample i of a segment: one per stride, at a hashed offset inside the stride so that periodic data
 // cannot alias with the sampling.
 __device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) {
-  return (int64_t)i * stride + (int64_t)(mix32((uint32_t)seg * 0x9e3779b9u + (uint32_t)i) % (uint32_t)stride);
+  // (hash scaled to [0, stride) by a multiply-high: the hardware has no integer division)
+  return (int64_t)i * stride + (int64_t)__umulhi(mix32((uint32_t)seg * 0x9e3779b9u + (uint32_t)i), (uint32_t)stride);
 }
 
 // ---- block-wide threshold search (1024 threads, 2048 bins) --------------------------------------

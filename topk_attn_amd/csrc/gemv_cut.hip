@@ -58,8 +58,8 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
 #define STAMP() do {} while (0)
 #endif
   STAMP();
-  float qf[8];
-  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  // the rows are asked for first and the query behind them: its conversion waits for it, and that wait would
+  // otherwise stand in front of the row loads (one more round trip to memory in a kernel made of a few)
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
                           chunk_base * p.key_stride_n + 8 * j;
   const bool sampler = rg >= kCutTokensPerWg / kCutUnroll;
@@ -67,9 +67,13 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
 #pragma unroll
   for (int u = 0; u < kCutUnroll; ++u) {
     const int row = rg * kCutUnroll + u;   // 0 .. 255 the slice, 256 .. 511 the sample
-    const int64_t t = sampler ? sample_token(seg, row - kCutTokensPerWg, stride) : (int64_t)(t_begin + (row < n_local ? row : n_local - 1));
-    kv[u] = *(const u32x4*)(kbase + t * p.key_stride_n);
+    const int64_t ts = sample_token(seg, row & (kCutSamples - 1), stride);
+    const int64_t to = (int64_t)(t_begin + (row < n_local ? row : n_local - 1));
+    kv[u] = *(const u32x4*)(kbase + (sampler ? ts : to) * p.key_stride_n);
   }
+  __builtin_amdgcn_sched_barrier(0);
+  float qf[8];
+  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
   __builtin_amdgcn_sched_barrier(0);
   STAMP();
   float mine = 0.0f;
@@ -190,7 +194,7 @@ void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank)
   int r = (int)ceil(m + 5.5 * sqrt(m) + 2.0);
   if (r < kCutParts) r = kCutParts;   // every part of the candidates ends with a sample of its own
   const double per_slice = (double)kCutTokensPerWg * r / s, per_segment = (double)chunk_len * r / s;
-  if (r * 2 > s || per_slice > 40.0 || per_segment * 1.25 > (double)kCutMaxCandidates) return;
+  if (r * 2 > s || per_slice > 40.0 || per_segment * 1.2 > (double)kCutMaxCandidates) return;
   *num_samples = s;
   *sample_rank = r;
 }

@@ -56,8 +56,9 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
   }
   __syncthreads();
 
+  // (without a centre stage the query is asked for behind the first rows, see below)
   float qf[8];
-  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  if (p.centers) load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
 
   // tokens are counted inside the chunk; the chunk starts at chunk*chunk_len, or at the start of the
   // cluster chosen for this (head, rank) in two-level selection
@@ -107,14 +108,26 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_scores_kernel(GemvParams p)
                           chunk_base * p.key_stride_n + 8 * j;
   float* sc_out = p.scores + seg * p.chunk_len;
 
-  for (int64_t base = t_begin; base < t_end; base += kGemvRowsPerIter) {
-    // row group rg owns 8 consecutive tokens per iteration: load u brings token base + rg*8 + u
-    u32x4 kv[kGemvUnroll];
+  // row group rg owns 8 consecutive tokens per iteration: load u brings token base + rg*8 + u.  The first rows are
+  // asked for before the query: its conversion waits for it, and that wait would otherwise stand in front of the
+  // row loads (a round trip to memory that short launches feel).
+  u32x4 kv[kGemvUnroll];
 #pragma unroll
-    for (int u = 0; u < kGemvUnroll; ++u) {
-      int64_t t = base + rg * kGemvUnroll + u;
-      int64_t tc = t < t_end ? t : t_end - 1;
-      kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + tc * p.key_stride_n));
+  for (int u = 0; u < kGemvUnroll; ++u) {
+    int64_t t = t_begin + rg * kGemvUnroll + u;
+    int64_t tc = t < t_end ? t : t_end - 1;
+    kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + tc * p.key_stride_n));
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  if (!p.centers) load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  for (int64_t base = t_begin; base < t_end; base += kGemvRowsPerIter) {
+    if (base != t_begin) {
+#pragma unroll
+      for (int u = 0; u < kGemvUnroll; ++u) {
+        int64_t t = base + rg * kGemvUnroll + u;
+        int64_t tc = t < t_end ? t : t_end - 1;
+        kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + tc * p.key_stride_n));
+      }
     }
     float mine = 0.0f;
 #pragma unroll
@@ -284,7 +297,7 @@ __device__ __forceinline__ void sample_role(const GemvParams& p, int seg, int pa
   const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
   float qf[8];
-  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  load_group_query<DT, 1>(p.q, p.q_stride_b, b, h, p.group, j, qf);
   const int64_t stride = p.chunk_len / p.num_samples;
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
                           chunk_base * p.key_stride_n + 8 * j;
@@ -542,7 +555,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
       const int64_t t_begin = (int64_t)wg_in_chunk * kCandThreads;
       const int n_local = (int)(p.chunk_len - t_begin < kCandThreads ? p.chunk_len - t_begin : kCandThreads);
       float qf[8];
-      load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+      load_group_query<DT, 1>(p.q, p.q_stride_b, b, h, p.group, j, qf);   // (one head at a time: the kernel has 64 registers per lane, and its workgroups overlap each other's waits)
       // uniform base of the slice + 32-bit lane offsets: one address register per load
       const unsigned char* sbase = (const unsigned char*)p.keys +
                                    2 * ((int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h + (chunk_base + t_begin) * p.key_stride_n);

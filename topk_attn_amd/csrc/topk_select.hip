@@ -977,7 +977,8 @@ __device__ __forceinline__ void write_ranked(const SelectParams& p, int seg, uin
 // fit is redone from the keys by its first workgroup (fallback_segment).
 // Dynamic LDS: kCutMaxCandidates composites (the part, as found), then as many again (the part in bucket order;
 // before that, entries from beyond the heads); the tie path and the fallback reuse both.
-template <int DT>
+// PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256).
+template <int DT, int PAIRS>
 __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, SelectParams p, int kpad) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint64_t* sh_own = (uint64_t*)smem;
@@ -993,8 +994,9 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
                                  // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key
 
   typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
-  constexpr int kPairs = kCutMaxSlices * kCutHead / 2 / kSelThreads;   // pairs of head entries per thread: 4
-  constexpr int kMine = 2 * kPairs + kCutMaxExtras / kSelThreads;       // composites per thread: 10
+  constexpr int kPairs = PAIRS;
+  constexpr int kHeadMine = 2 * kPairs;                                  // head entries per thread
+  constexpr int kMine = kHeadMine + kCutMaxExtras / kSelThreads;        // composites per thread, with those from beyond the heads
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1071,19 +1073,24 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   const uint64_t t_hi = sh_split[part], t_lo = sh_split[part + 1];
   {
     uint32_t n_all = 0, n_above = 0, kmax = 0;
-#pragma unroll
-    for (int i = 0; i < kMine; ++i) {
-      const bool nz = c[i] != 0ull;
-      const bool above = part != 0 && c[i] >= t_hi;
-      const bool own = nz && !above && c[i] >= t_lo;
+    auto take = [&](uint64_t x) {
+      const bool nz = x != 0ull;
+      const bool above = part != 0 && x >= t_hi;
+      const bool own = nz && !above && x >= t_lo;
       n_all += nz ? 1u : 0u;
       n_above += above ? 1u : 0u;
       if (own) {
-        sh_own[atomicAdd(&sh_n[5], 1u)] = c[i];
-        kmax = max(kmax, (uint32_t)(c[i] >> 32));
+        sh_own[atomicAdd(&sh_n[5], 1u)] = x;
+        kmax = max(kmax, (uint32_t)(x >> 32));
       }
+    };
+#pragma unroll
+    for (int i = 0; i < kHeadMine; ++i) take(c[i]);
+    if (n_ovf) {
+#pragma unroll
+      for (int i = kHeadMine; i < kMine; ++i) take(c[i]);
     }
-    const uint32_t inc = wave_inclusive_scan((n_all << 16) | n_above);   // (at most 10 x 64 per wave each)
+    const uint32_t inc = wave_inclusive_scan((n_all << 16) | n_above);   // (at most 18 x 64 per wave each)
     kmax = max(kmax, lane_xor<1>(kmax));
     kmax = max(kmax, lane_xor<2>(kmax));
     kmax = max(kmax, lane_xor<4>(kmax));
@@ -1405,14 +1412,21 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
       !p.list_cnt || !p.cut_splits)
     return TKA_EINVAL;
   const int lds = 2 * kCutMaxCandidates * (int)sizeof(uint64_t);
-  if (allow_dynamic_lds((const void*)select_rank_kernel<TKA_F16>, lds) != TKA_OK ||
-      allow_dynamic_lds((const void*)select_rank_kernel<TKA_BF16>, lds) != TKA_OK)
-    return TKA_EHIP;
+  const void* kernels[4] = {(const void*)select_rank_kernel<TKA_F16, 4>, (const void*)select_rank_kernel<TKA_F16, 8>,
+                            (const void*)select_rank_kernel<TKA_BF16, 4>, (const void*)select_rank_kernel<TKA_BF16, 8>};
+  for (const void* kn : kernels)
+    if (allow_dynamic_lds(kn, lds) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("select_rank", stream);
-  if (dtype == TKA_F16)
-    select_rank_kernel<TKA_F16><<<(unsigned)p.num_segments * kCutParts, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
-  else
-    select_rank_kernel<TKA_BF16><<<(unsigned)p.num_segments * kCutParts, kSelThreads, lds, stream>>>(g, p, kpad_for(p.k));
+  const unsigned wgs = (unsigned)p.num_segments * kCutParts;
+  const int kpad = kpad_for(p.k);
+  const bool wide = p.parts * kCutHead > 8 * kSelThreads;   // more head entries than 8 per thread
+  if (dtype == TKA_F16) {
+    if (wide) select_rank_kernel<TKA_F16, 8><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
+    else select_rank_kernel<TKA_F16, 4><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
+  } else {
+    if (wide) select_rank_kernel<TKA_BF16, 8><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
+    else select_rank_kernel<TKA_BF16, 4><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
+  }
   return hip_status(hipGetLastError());
 }
 
