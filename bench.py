@@ -406,6 +406,8 @@ def main():
     dominant = w.dominant
     if dominant == "gemv_scores" and "gemv_candidates" in kern:
         dominant = "gemv_candidates"                    # long segments run the candidate-mode GEMV
+    if dominant == "gemv_scores" and "gemv_cut" in kern:
+        dominant = "gemv_cut"                           # a few segments of middling length: the common-cut GEMV
     dom_us = kern.get(dominant, ms_per_step * 1e3)     # a workload with one foreign kernel: the step itself
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     traffic, traffic_source = recorded_traffic(args.workload, dominant) if not args.splits else (None, None)

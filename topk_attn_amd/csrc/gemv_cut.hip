@@ -22,17 +22,17 @@ namespace {
 
 constexpr int kCutThreads = 1024;
 constexpr int kCutUnroll = 8;                                        // rows per lane
-constexpr int kCutRows = (kCutThreads / 16) * kCutUnroll;            // rows per workgroup: 512
-constexpr int kCutSamples = kCutRows - kCutTokensPerWg;              // 256
-static_assert(kCutSamples == 256 && kCutTokensPerWg == 256, "half of the row groups score the slice, half the sample");
 
-// Sixteen waves and a short program: row groups 0 .. 31 score the 256 tokens of the slice, row groups 32 .. 63 the
-// 256 sample tokens, one round of eight loads per lane.  (Few workgroups run at a time on these problems, so a wave
-// pays the first fetch of every line of code itself: the same work as four waves with four rounds each took twice
-// as long.)
-template <int DT>
+// Row groups 0 .. 31 score the 256 tokens of the slice, the row groups behind them the S sample tokens (S = 256:
+// sixteen waves), one round of eight loads per lane.
+// Many waves and a short program: few workgroups run at a time on these problems, so a wave pays the first fetch
+// of every line of code itself (the same work as four waves with four rounds each took twice as long).
+template <int DT, int S>
 __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
-  __shared__ __attribute__((aligned(16))) uint32_t sh_key[kCutRows];   // [0, 256) the slice, [256, 512) the sample
+  constexpr int kCutSamples = S;
+  constexpr int kCutRows = kCutTokensPerWg + S;
+  static_assert(S == 64 || S == 256, "samples per segment (a power of two, 4 S threads rank them)");
+  __shared__ __attribute__((aligned(16))) uint32_t sh_key[kCutRows];   // [0, 256) the slice, then the sample
   __shared__ uint32_t sh_wcnt[kCutTokensPerWg / kWave];
   __shared__ uint32_t sh_cut[2];
   __shared__ uint32_t sh_rank[kCutSamples];
@@ -51,13 +51,6 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   const int n_local = n - t_begin < kCutTokensPerWg ? n - t_begin : kCutTokensPerWg;
   const int64_t stride = n / kCutSamples;
 
-#ifdef TKA_PHASE_STAMPS
-  uint64_t st[8]; int ns = 0;
-#define STAMP() do { if (tid == 0) st[ns] = __builtin_amdgcn_s_memtime(); ++ns; } while (0)
-#else
-#define STAMP() do {} while (0)
-#endif
-  STAMP();
   // the rows are asked for first and the query behind them: its conversion waits for it, and that wait would
   // otherwise stand in front of the row loads (one more round trip to memory in a kernel made of a few)
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
@@ -66,7 +59,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   u32x4 kv[kCutUnroll];
 #pragma unroll
   for (int u = 0; u < kCutUnroll; ++u) {
-    const int row = rg * kCutUnroll + u;   // 0 .. 255 the slice, 256 .. 511 the sample
+    const int row = rg * kCutUnroll + u;   // 0 .. 255 the slice, from 256 on the sample
     const int64_t ts = sample_token(seg, row & (kCutSamples - 1), stride);
     const int64_t to = (int64_t)(t_begin + (row < n_local ? row : n_local - 1));
     kv[u] = *(const u32x4*)(kbase + (sampler ? ts : to) * p.key_stride_n);
@@ -75,14 +68,12 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   float qf[8];
   load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
   __builtin_amdgcn_sched_barrier(0);
-  STAMP();
   float mine = 0.0f;
 #pragma unroll
   for (int u = 0; u < kCutUnroll; ++u) {
     const float sc = row_score<DT>(qf, kv[u], p.scale);
     if (j == u) mine = sc;
   }
-  STAMP();
   if (j < kCutUnroll) {
     const int row = rg * kCutUnroll + j;
     const uint32_t key = score_key(mine);
@@ -91,23 +82,22 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   }
   if (tid < kCutSamples) sh_rank[tid] = 0;
   __syncthreads();
-  STAMP();
 
-  // Rank of every sample by counting: thread (s, q) counts the samples of block q (64 of them, broadcast reads) that
+  // Rank of every sample by counting: thread (s, q) counts the samples of block q (a quarter of them, broadcast reads) that
   // come before sample s, four threads per sample add up in LDS.  The order is that of the ranking keys (the key with
-  // its last 8 bits replaced by 255 - sample number): all different, so one compare decides, exactly one sample holds
+  // its last 8 bits replaced by S - 1 - sample number): all different, so one compare decides, exactly one sample holds
   // rank R - 1, and samples that share a key (heavy ties) come in token order, as in the full order (key descending,
   // token ascending).  Keys that differ in their last 8 bits only may change places; any sample will do as the cut, it
   // is its rank among the samples that makes the number of candidates what was planned.
   // The samples of ranks R g / 8 - 1 split the candidates into eight parts of about equal size for the ranking
   // kernel's eight workgroups per segment.
-  {
-    const int s = tid & (kCutSamples - 1), q = tid >> 8;   // q is the same for a whole wave
+  if (tid < 4 * kCutSamples) {
+    const int s = tid & (kCutSamples - 1), q = tid / kCutSamples;   // q is the same for a whole wave
     const uint32_t ks = sh_rkey[s];
-    const u32x4* blk = (const u32x4*)(sh_rkey + q * kWave);
+    const u32x4* blk = (const u32x4*)(sh_rkey + q * (kCutSamples / 4));
     uint32_t ahead = 0;
 #pragma unroll
-    for (int i = 0; i < kWave / 4; ++i) {
+    for (int i = 0; i < kCutSamples / 16; ++i) {
       const u32x4 kj = blk[i];
       ahead += (kj[0] > ks ? 1u : 0u) + (kj[1] > ks ? 1u : 0u) + (kj[2] > ks ? 1u : 0u) + (kj[3] > ks ? 1u : 0u);
     }
@@ -126,7 +116,6 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
     }
   }
   __syncthreads();
-  STAMP();
   if (tid >= kCutTokensPerWg) return;
 
   // thread t owns token t_begin + t.  Entries are composites (key << 32 | ~token, token counted inside the segment),
@@ -156,43 +145,42 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   }
   if ((uint32_t)tid >= total && tid < kCutHead) head[tid] = 0ull;
   if (tid == 0) p.cand_count[slice_id] = total;
-  STAMP();
-#ifdef TKA_PHASE_STAMPS
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  STAMP();
-  if (tid == 0) for (int i = 0; i < ns; ++i) ((uint64_t*)p.scores)[blockIdx.x * 8 + i] = st[i];
-#endif
 }
 
 }  // namespace
 
 int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  if (p.tokens_per_wg != kCutTokensPerWg || p.num_samples != kCutSamples || p.chunk_len < kCutSamples || p.sample_rank < 1 ||
-      p.sample_rank > kCutSamples || !p.cand || !p.cand_head || !p.cand_count || !p.cut_splits || segs * p.wgs_per_chunk > 0x7fffffffLL)
+  if (p.tokens_per_wg != kCutTokensPerWg || p.num_samples != 256 || p.chunk_len < p.num_samples ||
+      p.sample_rank < kCutParts || p.sample_rank > p.num_samples || !p.cand || !p.cand_head || !p.cand_count || !p.cut_splits ||
+      segs * p.wgs_per_chunk > 0x7fffffffLL)
     return TKA_EINVAL;
   const unsigned wgs = (unsigned)(segs * p.wgs_per_chunk);
+  const unsigned threads = (unsigned)(kCutTokensPerWg + p.num_samples) / kCutUnroll * 16;   // 16 lanes per row, 8 rows each
   LaunchTimer timer("gemv_cut", stream);
   if (dtype == TKA_F16)
-    gemv_cut_kernel<TKA_F16><<<wgs, kCutThreads, 0, stream>>>(p);
+    gemv_cut_kernel<TKA_F16, 256><<<wgs, threads, 0, stream>>>(p);
   else
-    gemv_cut_kernel<TKA_BF16><<<wgs, kCutThreads, 0, stream>>>(p);
+    gemv_cut_kernel<TKA_BF16, 256><<<wgs, threads, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 
 // Samples per segment and rank of the cut for a segment of chunk_len tokens and k, or 0 samples when this route
-// does not serve the shape.  With S = 256 samples spread evenly and m = k S / n of them expected inside the top k, the
-// rank is R = m + 5.5 sqrt(m) + 2: "fewer than k tokens pass" (the segment is then redone from the keys, still
-// exact) needs R of the samples inside the top k, more than five deviations out; about n R / S candidates are
-// stored.  Limits: a slice of 256 tokens should stay within the kCutHead entries that the ranking kernel reads
-// in its first round trip (40 expected at most), and a segment within what it ranks in one go.
+// does not serve the shape.  With S = 256 samples spread evenly and m = k S / n of them expected inside the top k,
+// the rank is R = m + 5.5 sqrt(m) + 2 (at least 8: every part of the candidates ends with a sample of its own):
+// "fewer than k tokens pass" (the segment is then redone from the keys, still exact) needs R of the samples inside
+// the top k, more than five deviations out; about n R / S candidates are stored.  Limits: a slice of 256 tokens
+// should stay within the kCutHead entries that the ranking kernel reads in its first round trip (40 expected at
+// most), and a segment within what it ranks in one go.
+// (With 64 samples - enough for a small k on segments of a few thousand rows - the route was measured too: 32 x 4096
+// rows, k = 64: 19.5 us against 13.3 on the route that selects in the registers of one workgroup per segment.)
 void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank) {
   *num_samples = *sample_rank = 0;
   if (chunk_len < 2048 || chunk_len > (int64_t)kCutMaxSlices * kCutTokensPerWg || k > kCutMaxK || (int64_t)k * 8 > chunk_len) return;
-  const int s = kCutSamples;
+  const int s = 256;
   const double m = (double)k * s / (double)chunk_len;
   int r = (int)ceil(m + 5.5 * sqrt(m) + 2.0);
-  if (r < kCutParts) r = kCutParts;   // every part of the candidates ends with a sample of its own
+  if (r < kCutParts) r = kCutParts;
   const double per_slice = (double)kCutTokensPerWg * r / s, per_segment = (double)chunk_len * r / s;
   if (r * 2 > s || per_slice > 40.0 || per_segment * 1.2 > (double)kCutMaxCandidates) return;
   *num_samples = s;

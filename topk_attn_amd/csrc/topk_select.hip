@@ -1005,13 +1005,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   const u64x2* heads = (const u64x2*)(p.cand_head + (int64_t)seg * p.parts * kCutHead);
   const int n_pairs = p.parts * (kCutHead / 2);
 
-#ifdef TKA_PHASE_STAMPS
-  uint64_t st[12]; int ns = 0;
-#define STAMP() do { if (tid == 0) st[ns] = __builtin_amdgcn_s_memtime(); ++ns; } while (0)
-#else
-#define STAMP() do {} while (0)
-#endif
-  STAMP();
   u64x2 w[kPairs];
 #pragma unroll
   for (int e = 0; e < kPairs; ++e) {
@@ -1038,7 +1031,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   sh_hist[2 * tid + 1] = 0;
   if (tid < 8) sh_n[tid] = 0;
   __syncthreads();
-  STAMP();
   if (slice_cnt > (uint32_t)kCutHead) sh_ovf[atomicAdd(&sh_n[0], 1u)] = (uint32_t)tid | (slice_cnt << 16);
   __syncthreads();
   const uint32_t n_ovf = sh_n[0];
@@ -1104,7 +1096,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     }
   }
   __syncthreads();
-  STAMP();
   const uint32_t n_cand = sh_n[2], n_above = sh_n[4], n_own = sh_n[5];
   const uint32_t cap = (uint32_t)(p.max_entries < kCutMaxCandidates ? p.max_entries : kCutMaxCandidates);
   const bool redo = n_cand < k || n_cand > cap || n_extra > (uint32_t)kCutMaxExtras;
@@ -1125,7 +1116,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
 #pragma unroll 1
   for (uint32_t i = tid; i < n_own; i += kSelThreads) atomicAdd(&sh_hist[(uint32_t)((sh_own[i] - base) >> shift)], 1u);
   __syncthreads();
-  STAMP();
   // first rank of every bucket: number of composites in higher buckets (thread t owns buckets 2t, 2t+1)
   {
     const int wave = tid >> 6;
@@ -1143,7 +1133,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     sh_off[2 * tid] = sh_cur[2 * tid] = above + ge - h0;             // buckets > 2t
   }
   __syncthreads();
-  STAMP();
   const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len) : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
   if (sh_n[3] != 0u) {
     // heavy ties: sort the part and take it in order
@@ -1162,7 +1151,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     sh_x[atomicAdd(&sh_cur[(uint32_t)((x - base) >> shift)], 1u)] = x;
   }
   __syncthreads();
-  STAMP();
   // every candidate of the part: its rank is the candidates above the part, plus the first rank of its bucket, plus the
   // larger members of the bucket
 #pragma unroll 1
@@ -1175,12 +1163,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     const uint32_t rank = n_above + start + larger;
     if (rank < k) write_ranked(p, seg, idx_base, rank, x);
   }
-  STAMP();
-#ifdef TKA_PHASE_STAMPS
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  STAMP();
-  if (tid == 0) for (int i = 0; i < ns; ++i) ((uint64_t*)g.scores)[2048 + blockIdx.x * 16 + i] = st[i];
-#endif
 }
 
 // Ascending duplicate-free union of the selected ids with [0,sink) and [n-local,n).
