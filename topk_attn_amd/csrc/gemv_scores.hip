@@ -530,12 +530,14 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
   const int j = tid & 15;            // lane inside the row: dims 8j..8j+7
   const int rg = tid >> 4;           // row group 0..15 inside the workgroup
   const int lane = tid & 63, wave = tid >> 6;
-  const int64_t w = (int64_t)blockIdx.x - p.sample_wgs;
-  const int num_slices = w < p.early_wgs ? kEarlySlices : 1;
-  const int64_t first_slice = w < p.early_wgs ? w * kEarlySlices : (int64_t)p.early_wgs * kEarlySlices + (w - p.early_wgs);
+  // (slices and segments are counted in 32 bits - the launcher checks that the grid fits - because a 64-bit division is
+  // a hundred scalar instructions, and a workgroup asks for its first row only behind them)
+  const uint32_t w = blockIdx.x - (uint32_t)p.sample_wgs;
+  const int num_slices = w < (uint32_t)p.early_wgs ? kEarlySlices : 1;
+  const uint32_t first_slice = w < (uint32_t)p.early_wgs ? w * kEarlySlices : (uint32_t)p.early_wgs * kEarlySlices + (w - (uint32_t)p.early_wgs);
 
-  const int64_t first_seg = first_slice / p.wgs_per_chunk;
-  const int first_wg = (int)(first_slice % p.wgs_per_chunk);
+  const int64_t first_seg = (int64_t)(first_slice / (uint32_t)p.wgs_per_chunk);
+  const int first_wg = (int)(first_slice % (uint32_t)p.wgs_per_chunk);
 
   // A workgroup that starts after the first wave of them finds its threshold published: it asks for the word
   // now, so that the answer travels beside the rows instead of costing a round trip of its own behind them
@@ -548,9 +550,8 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
     int64_t seg = first_seg;
     int wg_in_chunk = first_wg;
     for (int s = 0; s < num_slices; ++s) {
-      const int chunk = (int)(seg % p.num_chunks);
-      const int64_t bh = seg / p.num_chunks;
-      const int h = (int)(bh % p.num_kv_heads), b = (int)(bh / p.num_kv_heads);
+      const uint32_t chunk = (uint32_t)seg % (uint32_t)p.num_chunks, bh = (uint32_t)seg / (uint32_t)p.num_chunks;
+      const int h = (int)(bh % (uint32_t)p.num_kv_heads), b = (int)(bh / (uint32_t)p.num_kv_heads);
       const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
       const int64_t t_begin = (int64_t)wg_in_chunk * kCandThreads;
       const int n_local = (int)(p.chunk_len - t_begin < kCandThreads ? p.chunk_len - t_begin : kCandThreads);
@@ -702,6 +703,7 @@ int launch_gemv_candidates(const GemvParams& p0, int dtype, hipStream_t stream) 
   int64_t early = resident_streaming_wgs();
   if (early > slices / (2 * kEarlySlices)) early = slices / (2 * kEarlySlices);
   p.early_wgs = (int)early;
+  if (slices > 0x7fffffffLL) return TKA_EUNSUPPORTED;
   const int64_t wgs = p.sample_wgs + early + (slices - early * kEarlySlices);
   if (wgs > 0x7fffffffLL) return TKA_EUNSUPPORTED;
   LaunchTimer timer("gemv_candidates", stream);
