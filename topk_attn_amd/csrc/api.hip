@@ -171,6 +171,16 @@ int wave_select_min_segments() {
   }();
   return v;
 }
+int small_select_max_segments() {
+  static const int v = [] {
+    const char* e = getenv("TKA_SMALL_MAX_SEGS");
+    return e && *e ? atoi(e) : 64;
+  }();
+  return v;
+}
+bool small_select_fits(int64_t seg_len, int k, int segs) {
+  return seg_len > kFusedMaxSegLen && seg_len <= select_small_max_len() && k <= select_small_max_k() && segs <= small_select_max_segments();
+}
 bool wave_select_fits(int64_t seg_len, int k) { return seg_len <= select_wave_max_len() && k <= select_wave_max_k(seg_len); }
 
 // Samples per segment and rank of the threshold statistic when the call takes the candidate route (long segments,
@@ -318,6 +328,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     }
     int rc = shared_keys ? launch_shared_scores(a, gp, stream) : launch_gemv_scores(gp, a->dtype, stream);
     if (rc != TKA_OK) return rc;
+    // a small k out of a few thousand scores on a call of a few segments: the short program of one big workgroup
+    if (small_select_fits(chunk_len, a->k, segs) && a->out_idx && !u) return launch_select_small(sw, stream);
     return launch_select_wave(sw, stream);
   }
   if (ic) return TKA_EINVAL;   // (callers ask wave_route first)

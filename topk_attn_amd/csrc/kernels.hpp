@@ -116,6 +116,12 @@ int launch_select_wave(const SelectParams& p, hipStream_t stream);
 int select_wave_max_len();
 int select_wave_max_k(int64_t seg_len);
 
+// One workgroup per segment of up to select_small_max_len() scores, k up to select_small_max_k(), rank order: a short
+// program for calls of a few segments.
+int launch_select_small(const SelectParams& p, hipStream_t stream);
+int select_small_max_len();
+int select_small_max_k();
+
 struct UnionParams {
   const int32_t* idx;     // [num_segments][k]
   int32_t* out_idx;       // [num_segments][k+sink+local]

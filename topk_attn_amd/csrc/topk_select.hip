@@ -183,11 +183,12 @@ __device__ __forceinline__ void write_rank_outputs(const uint64_t* sh_sort, cons
     if (ov) ov[r] = key_score((uint32_t)(c >> 32));
   }
   if (p.out_expand) {
+    // a wave per selected id, a lane per member of its cluster (no division by the cluster length)
     int32_t* oe = p.out_expand + (int64_t)seg * p.k * p.expand;
-    const uint32_t total = k * (uint32_t)p.expand;
-    for (uint32_t e = tid; e < total; e += kSelThreads) {
-      uint32_t jj = e / (uint32_t)p.expand, ii = e % (uint32_t)p.expand;
-      oe[e] = (int32_t)(~(uint32_t)sh_sort[jj] * (uint32_t)p.expand + ii);
+    const uint32_t lane = (uint32_t)tid & 63u, expand = (uint32_t)p.expand;
+    for (uint32_t jj = (uint32_t)tid >> 6; jj < k; jj += kSelThreads / kWave) {
+      const uint32_t first = ~(uint32_t)sh_sort[jj] * expand;
+      for (uint32_t ii = lane; ii < expand; ii += kWave) oe[jj * expand + ii] = (int32_t)(first + ii);
     }
   }
 }
@@ -1165,6 +1166,113 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   }
 }
 
+// ---- a small k out of a few thousand scores, few segments -------------------------------------------------
+
+constexpr int kSmallMaxLen = 4096;    // scores per segment: four per thread
+constexpr int kSmallMaxK = 256;
+constexpr int kSmallMaxCand = 1024;   // entries of the threshold bucket and above that are ranked by counting
+
+// Rank-ordered top k of a segment of up to 4096 scores by one workgroup, for calls of a few segments (the centroids of
+// a few dozen heads): such a launch is a matter of instructions per thread - sixteen waves share a CU's four SIMDs, and
+// every line of code is fetched cold - so the program is kept short.  Four keys per thread; one histogram of 2048 bins
+// linear between the smallest and the largest key; the threshold bin from one suffix scan; the entries of that bin and
+// above (k and a handful) ranked by counting, which is also their output position.  When that bin is crowded (ties)
+// the whole segment goes through the sorting network instead.
+// Dynamic LDS: 2 x 4096 composites (the sort and its exchange buffer; the candidates and the selected otherwise).
+__global__ __launch_bounds__(kSelThreads) void select_small_kernel(SelectParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint64_t* sh_all = (uint64_t*)smem;
+  uint64_t* sh_cand = sh_all;
+  uint64_t* sh_sort = sh_all + kSmallMaxCand;
+  __shared__ uint32_t sh_hist[kHistBins];
+  __shared__ uint32_t sh_wtot[kSelWaves];
+  __shared__ uint32_t sh_res[4];
+  __shared__ uint32_t sh_n[3];   // smallest key, largest key, candidates collected
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int seg = blockIdx.x;
+  const uint32_t k = (uint32_t)p.k;
+  const int64_t n = p.seg_len;
+  const float* sc = p.scores + (int64_t)seg * p.seg_stride;
+  uint32_t keys[4], vm;
+  load_keys<4>(sc, (int64_t)tid * 4, n, (((uintptr_t)sc) & 15u) == 0, keys, &vm);
+  sh_hist[2 * tid] = 0;
+  sh_hist[2 * tid + 1] = 0;
+  if (tid == 0) { sh_n[0] = ~0u; sh_n[1] = 0u; sh_n[2] = 0u; sh_res[0] = 0u; sh_res[1] = 0u; sh_res[2] = 0u; }
+  uint32_t kmin = ~0u, kmax = 0u;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (vm >> e & 1u) {
+      kmin = min(kmin, keys[e]);
+      kmax = max(kmax, keys[e]);
+    }
+  }
+  kmin = min(kmin, lane_xor<1>(kmin));   kmax = max(kmax, lane_xor<1>(kmax));
+  kmin = min(kmin, lane_xor<2>(kmin));   kmax = max(kmax, lane_xor<2>(kmax));
+  kmin = min(kmin, lane_xor<4>(kmin));   kmax = max(kmax, lane_xor<4>(kmax));
+  kmin = min(kmin, lane_xor<8>(kmin));   kmax = max(kmax, lane_xor<8>(kmax));
+  kmin = min(kmin, lane_xor<16>(kmin));  kmax = max(kmax, lane_xor<16>(kmax));
+  kmin = min(kmin, lane_xor<32>(kmin));  kmax = max(kmax, lane_xor<32>(kmax));
+  __syncthreads();
+  if (lane == 0) {
+    atomicMin(&sh_n[0], kmin);
+    atomicMax(&sh_n[1], kmax);
+  }
+  __syncthreads();
+  kmin = sh_n[0];
+  kmax = sh_n[1];
+  // bins: the 11 leading bits of key - smallest key, counted from the leading bit of the range
+  const int fixed = kmax == kmin ? 31 : __builtin_clz(kmax - kmin);
+  const int shift = 32 - fixed > kHistBits ? 32 - fixed - kHistBits : 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if (vm >> e & 1u) atomicAdd(&sh_hist[(keys[e] - kmin) >> shift], 1u);
+  __syncthreads();
+  find_threshold_bin_1024(sh_hist, k, sh_wtot, sh_res);
+  const uint32_t d = sh_res[0], n_cand = sh_res[1] + sh_res[2];   // the threshold bin; entries in it and above
+  if (n_cand > (uint32_t)kSmallMaxCand) {
+    // a crowded threshold bin (ties): sort the whole segment
+    uint32_t npad = 64;
+    while (npad < (uint32_t)n) npad <<= 1;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t i = (uint32_t)tid * 4 + e;
+      if (i < npad) sh_all[i] = (vm >> e & 1u) ? composite(keys[e], i) : 0ull;   // pad: below every real composite
+    }
+    __syncthreads();
+    sort_lds_desc(sh_all, sh_all + npad, (int)npad);
+    write_rank_outputs(sh_all, p, seg);
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if ((vm >> e & 1u) && ((keys[e] - kmin) >> shift) >= d) sh_cand[atomicAdd(&sh_n[2], 1u)] = composite(keys[e], (uint32_t)tid * 4 + e);
+  __syncthreads();
+  // rank = number of larger candidates: eight threads per candidate, each with an eighth of the list, add up in LDS
+  // (the histogram is spent)
+  uint32_t* sh_rank = sh_hist;
+  for (uint32_t i = tid; i < n_cand; i += kSelThreads) sh_rank[i] = 0;
+  __syncthreads();
+  {
+    const uint32_t part = (uint32_t)tid >> 7, per = (n_cand + 7u) / 8u;
+    const uint32_t j0 = part * per, j1 = min(j0 + per, n_cand);
+    for (uint32_t i = (uint32_t)tid & 127u; i < n_cand; i += 128u) {
+      const uint64_t x = sh_cand[i];
+      uint32_t larger = 0;
+      for (uint32_t j = j0; j < j1; ++j) larger += sh_cand[j] > x ? 1u : 0u;
+      atomicAdd(&sh_rank[i], larger);
+    }
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < n_cand; i += kSelThreads) {
+    const uint32_t r = sh_rank[i];
+    if (r < k) sh_sort[r] = sh_cand[i];
+  }
+  __syncthreads();
+  write_rank_outputs(sh_sort, p, seg);
+}
+
 // Ascending duplicate-free union of the selected ids with [0,sink) and [n-local,n).
 // One workgroup per segment; the middle part is sorted ascending with the same bitonic network
 // (ids complemented so that "descending" composites are ascending ids).
@@ -1409,6 +1517,18 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
     if (wide) select_rank_kernel<TKA_BF16, 8><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
     else select_rank_kernel<TKA_BF16, 4><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
   }
+  return hip_status(hipGetLastError());
+}
+
+int select_small_max_len() { return kSmallMaxLen; }
+int select_small_max_k() { return kSmallMaxK; }
+
+int launch_select_small(const SelectParams& p, hipStream_t stream) {
+  if (p.seg_len > kSmallMaxLen || p.k > kSmallMaxK || p.k > p.seg_len || !p.out_idx || p.union_idx) return TKA_EINVAL;
+  const int lds = 2 * kSmallMaxLen * (int)sizeof(uint64_t);
+  if (allow_dynamic_lds((const void*)select_small_kernel, lds) != TKA_OK) return TKA_EHIP;
+  LaunchTimer timer("select_small", stream);
+  select_small_kernel<<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 
