@@ -821,18 +821,15 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   }
   __syncthreads();
 
-  // this thread's share for the radix passes: entries tid, tid + 1024, ...
-  uint64_t mine[kCandPerThread];
+  // The passes over the entries (tid, tid + 1024, ...) are rolled loops over the LDS copy: the kernel runs a few workgroups,
+  // every line of its code is fetched cold, and an unrolled pass for the 16 entries per thread that the capacity allows
+  // costs that fetch whether or not the list reaches them.
   uint32_t kmin = ~0u, kmax = 0u;   // smallest and largest key among the entries
-#pragma unroll
-  for (int i = 0; i < kCandPerThread; ++i) {
-    const uint32_t v = (uint32_t)i * kSelThreads + tid;
-    const bool ok = v < n_entries;
-    mine[i] = ok ? sh_ent[v] : 0ull;
-    if (ok) {
-      kmin = min(kmin, (uint32_t)(mine[i] >> 32));
-      kmax = max(kmax, (uint32_t)(mine[i] >> 32));
-    }
+#pragma unroll 1
+  for (uint32_t v = tid; v < n_entries; v += kSelThreads) {
+    const uint32_t key = (uint32_t)(sh_ent[v] >> 32);
+    kmin = min(kmin, key);
+    kmax = max(kmax, key);
   }
 
   uint64_t threshold = 0;   // selected: composite >= threshold
@@ -855,9 +852,6 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     // width of the key range, and the 11 bits below spread the candidates evenly (shared bits of the float
     // keys themselves say little once the scores straddle a power of two).
     const uint64_t base = (uint64_t)kmin << 32;
-#pragma unroll
-    for (int i = 0; i < kCandPerThread; ++i)
-      if ((uint32_t)i * kSelThreads + tid < n_entries) mine[i] -= base;
     int fixed = kmin == kmax ? 32 : __builtin_clz(kmax - kmin);
     uint64_t prefix = 0ull;
     uint32_t need = k;
@@ -869,11 +863,10 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
       sh_hist[2 * tid] = 0;
       sh_hist[2 * tid + 1] = 0;
       __syncthreads();
-#pragma unroll
-      for (int i = 0; i < kCandPerThread; ++i) {
-        const uint64_t c = mine[i];
-        if ((uint32_t)i * kSelThreads + tid < n_entries && (fixed == 0 || (c >> (64 - fixed)) == prefix))
-          atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
+#pragma unroll 1
+      for (uint32_t v = tid; v < n_entries; v += kSelThreads) {
+        const uint64_t c = sh_ent[v] - base;
+        if (fixed == 0 || (c >> (64 - fixed)) == prefix) atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
       }
       __syncthreads();
       find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
@@ -886,10 +879,10 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
         done = true;
       } else if (cnt <= (uint32_t)kSmallBucket) {
         // few entries left in the threshold bucket: every wave ranks them and picks the need-th largest
-#pragma unroll
-        for (int i = 0; i < kCandPerThread; ++i) {
-          const uint64_t c = mine[i];
-          if ((uint32_t)i * kSelThreads + tid < n_entries && (c >> (64 - fixed)) == prefix) sh_small[atomicAdd(&sh_small_cnt, 1u)] = c;
+#pragma unroll 1
+        for (uint32_t v = tid; v < n_entries; v += kSelThreads) {
+          const uint64_t c = sh_ent[v] - base;
+          if ((c >> (64 - fixed)) == prefix) sh_small[atomicAdd(&sh_small_cnt, 1u)] = c;
         }
         __syncthreads();
         const uint64_t e = (uint32_t)lane < cnt ? sh_small[lane] : 0ull;
@@ -909,18 +902,18 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   const int64_t n = p.seg_len;
   const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
   const uint32_t hi = (uint32_t)(n - p.local > lo ? n - p.local : lo);
-  const uint32_t per = (n_entries + kSelThreads - 1) / kSelThreads;
-  uint64_t run[kCandPerThread];
+  const uint32_t per = (n_entries + kSelThreads - 1) / kSelThreads;   // at most kCandPerThread
   uint32_t sel_mask = 0, mid_mask = 0;
-#pragma unroll
-  for (int i = 0; i < kCandPerThread; ++i) {
+#pragma unroll 1
+  for (uint32_t i = 0; i < per; ++i) {
     const uint32_t v = (uint32_t)tid * per + i;
-    const bool ok = (uint32_t)i < per && v < n_entries;
-    run[i] = ok ? sh_ent[v] : 0ull;
-    const bool sel = ok && run[i] >= threshold;
-    const uint32_t idx = ~(uint32_t)run[i];
-    sel_mask |= (sel ? 1u : 0u) << i;
-    mid_mask |= (sel && idx >= lo && idx < hi ? 1u : 0u) << i;
+    if (v < n_entries) {
+      const uint64_t c = sh_ent[v];
+      const bool sel = c >= threshold;
+      const uint32_t idx = ~(uint32_t)c;
+      sel_mask |= (sel ? 1u : 0u) << i;
+      mid_mask |= (sel && idx >= lo && idx < hi ? 1u : 0u) << i;
+    }
   }
   // one scan for both counts (each total is at most 16384)
   uint32_t totals;
@@ -928,15 +921,18 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   if (want_union) {
     int32_t* uo = p.union_idx + (int64_t)seg * (p.k + p.sink + p.local);
     uint32_t pos = lo + (ex & 0xffffu);
-#pragma unroll
-    for (int i = 0; i < kCandPerThread; ++i)
-      if (mid_mask >> i & 1u) uo[pos++] = (int32_t)~(uint32_t)run[i];
+#pragma unroll 1
+    for (uint32_t i = 0; i < per; ++i)
+      if (mid_mask >> i & 1u) uo[pos++] = (int32_t)~(uint32_t)sh_ent[(uint32_t)tid * per + i];
     write_union_edges(uo, p, seg, lo, hi, totals & 0xffffu);
   }
   if (!want_rank) return;
   uint64_t* sh_sort = sh_ent;
   uint64_t* sh_xchg = sh_ent + kpad;
-  __syncthreads();   // every thread holds its run in registers: the entries may be overwritten
+  uint64_t run[kCandPerThread];   // the selected of this thread's run, in registers: the buffer is about to be overwritten
+#pragma unroll
+  for (int i = 0; i < kCandPerThread; ++i) run[i] = (sel_mask >> i & 1u) ? sh_ent[(uint32_t)tid * per + i] : 0ull;
+  __syncthreads();
   {
     uint32_t pos = ex >> 16;
 #pragma unroll
