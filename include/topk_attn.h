@@ -128,8 +128,8 @@ int tka_gemv_topk_gave_up_slices(const tka_gemv_topk_args* args, int32_t* count)
  * change how the candidate route of stage 1 gets to its result, never the result.  NULL restores the defaults
  * (all zero).  Every kernel still runs to its end under any setting: the waits involved are bounded. */
 typedef struct tka_test_hooks {
-  int32_t force_segment_redo;  /* 1: the selection accepts no candidate count, every long segment is redone
-                                  from the keys                                                         */
+  int32_t force_segment_redo;  /* 1: the selection accepts no candidate count, every segment of the routes that
+                                  store candidates above a sampled threshold is redone from the keys    */
   int32_t tau_spin_limit;      /* > 0: polls of a streaming workgroup for its segment's threshold before
                                   it gives up (default 65536)                                           */
   int32_t tau_withhold_mod;    /* > 0: the threshold of segments s with s % mod == rem is withheld ...   */

@@ -343,13 +343,14 @@ def test_long_segment_ragged_length():
     _check_long(K, randn_bits(rng, (1, 4, 128), oracle.BF16), oracle.BF16, 2, 1500)
 
 
-def test_two_level_long_clusters():
-    """Two-level selection whose clusters are long enough for the sampled-threshold path (cluster ids pick the
-    segments)."""
+@pytest.mark.parametrize("CSZ,CLEN", [(4, 65536), (3, 131072)])
+def test_two_level_long_clusters(CSZ, CLEN):
+    """Two-level selection whose clusters are long (cluster ids pick the segments): four segments of 65536 tokens take
+    the common-cut route, four of 131072 the sampled-threshold path of the long segments."""
     from topk_attn_amd import ops
-    announce("cluster_gemv_topk CSZ=4 CLEN=65536 TOPC=2 k=300")
+    announce("cluster_gemv_topk CSZ=%d CLEN=%d TOPC=2 k=300" % (CSZ, CLEN))
     rng = np.random.default_rng(37)
-    H, CSZ, CLEN, TOPC, K = 2, 4, 65536, 2, 300
+    H, TOPC, K = 2, 2, 300
     cen = rng.uniform(-0.5, 0.5, (H, CSZ, 128))
     keys = np.empty((CSZ * CLEN, H, 128), dtype=np.float32)
     for c in range(CSZ):
