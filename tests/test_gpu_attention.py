@@ -378,6 +378,27 @@ def test_sparse_decode_step_union_only(dtype, B, H, G, N, k, sink, local, kind, 
             assert (np.abs(out[b, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_short_token_list_bf16_weights(seed):
+    """A step that attends to 17 tokens only (top 1 + a window of 16), bf16 inputs, grouped queries on the matrix cores,
+    fp16 output: with so few terms nothing averages out, so the softmax weights must reach the P.V product with more than
+    the 8 bits of a bf16 operand (they go in as a high and a low part).  Half the 2e-3 tolerance."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step bf16 G=8, 17 tokens, seed %d" % seed)
+    rng = np.random.default_rng(900 + seed)
+    dtype, B, H, G, N, k, sink, local = oracle.BF16, 2, 2, 8, 6000, 1, 0, 16
+    q, K, V = randn_bits(rng, (B, H * G, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype)
+    out, tidx, tval, uidx, ucnt = ops.sparse_decode_step(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), k, sink,
+                                                         local, SCALE, G, out_dtype=torch.float16, want_topk=False)
+    torch.cuda.synchronize()
+    out = f32_of(out)
+    for b in range(B):
+        for h in range(H):
+            ro, ri, rv, ru = oracle.sparse_decode_step(q[b, h * G:(h + 1) * G], K[b, :, h], V[b, :, h], dtype, G, k, sink,
+                                                       local, SCALE)
+            assert np.abs(out[b, h * G:(h + 1) * G] - ro).max() < 1e-3
+
+
 @pytest.fixture
 def hooks():
     """Testing hooks of the candidate route, restored to their defaults afterwards."""

@@ -170,6 +170,16 @@ __global__ __launch_bounds__(kThreads) void attn_mfma_kernel(AttnParams p) {
     u32x4 pfrag;
 #pragma unroll
     for (int w = 0; w < 4; ++w) pfrag[w] = Mfma<DT>::pack(ps[2 * w], ps[2 * w + 1]);
+    // bf16 keeps 8 bits of a weight: the rest goes through the matrix cores as a second operand (the products are
+    // exact, the sum is fp32), so that a short list of tokens is weighted as precisely as the fp32 sum l above
+    u32x4 pfrag_lo;
+    if constexpr (DT == TKA_BF16) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float r0 = ps[2 * w] - Elem<DT>::widen((uint16_t)pfrag[w]), r1 = ps[2 * w + 1] - Elem<DT>::widen((uint16_t)(pfrag[w] >> 16));
+        pfrag_lo[w] = Mfma<DT>::pack(r0, r1);
+      }
+    }
 
     // ---- rescale the accumulators: element i belongs to head 4j+i, whose alpha sits in lane 4j+i
     float ah[4];
@@ -195,6 +205,7 @@ __global__ __launch_bounds__(kThreads) void attn_mfma_kernel(AttnParams p) {
 #pragma unroll
       for (int w = 0; w < 4; ++w) vt[w] = __builtin_amdgcn_perm(vr[2 * w + 1][c >> 1], vr[2 * w][c >> 1], sel);
       acc[c] = Mfma<DT>::run(pfrag, vt, acc[c]);
+      if constexpr (DT == TKA_BF16) acc[c] = Mfma<DT>::run(pfrag_lo, vt, acc[c]);
     }
     (void)okk;
   }
