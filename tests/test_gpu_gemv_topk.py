@@ -426,9 +426,11 @@ def test_long_segment_threshold_never_published(hooks, withheld):
 
 @pytest.mark.parametrize("dtype,B,H,G,N,k", [(oracle.F16, 1, 1, 1, 32768, 2048), (oracle.BF16, 1, 2, 4, 20011, 1000),
                                              (oracle.F16, 2, 2, 1, 65536, 2048), (oracle.F16, 1, 1, 8, 40000, 1),
-                                             (oracle.BF16, 1, 3, 2, 16385, 2048)])
+                                             (oracle.BF16, 1, 3, 2, 16385, 2048), (oracle.F16, 1, 2, 1, 12000, 400),
+                                             (oracle.BF16, 2, 2, 4, 8193, 300)])
 def test_common_cut_route(dtype, B, H, G, N, k):
-    """Calls of up to 262144 rows with segments of 16385 .. 65536 tokens and no score output: every GEMV workgroup
+    """Calls of up to 262144 rows with segments of 16385 .. 65536 tokens (from 8193 tokens on calls of up to 65536 rows) and
+    no score output: every GEMV workgroup
     derives the same cut from 256 sample rows, eight ranking workgroups per segment rank the candidates.  Ordinary
     data with heavy hitters; no segment is redone from the keys."""
     announce("gemv_topk common-cut route dtype=%d B=%d H=%d G=%d N=%d k=%d" % (dtype, B, H, G, N, k))

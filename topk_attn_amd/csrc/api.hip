@@ -200,7 +200,7 @@ void candidate_plan(const tka_gemv_topk_args* a, int* num_samples, int* sample_r
 int64_t cut_route_min_len() {
   static const int64_t v = [] {
     const char* e = getenv("TKA_CUT_MIN_LEN");
-    return e && *e ? (int64_t)atoll(e) : (int64_t)select_cand_capacity() + 1;
+    return e && *e ? (int64_t)atoll(e) : (int64_t)select_cand_capacity() / 2 + 1;
   }();
   return v;
 }
@@ -214,7 +214,11 @@ void cut_plan(const tka_gemv_topk_args* a, bool want_union, int* num_samples, in
   // Every workgroup of this route scores the sample rows again, which is free while the launch does not fill the GPU.
   // Measured (us per call, k = 2048, this route against the others): 1 x 32768 rows 13.6 / 25.1, 1 x 65536 15.8 / 31.6,
   // 4 x 49152 29.0 / 35.0, 8 x 32768 32.9 / 35.9, 16 x 32768 56.4 / 47.3, 8 x 65536 60.0 / 45.8.
-  if ((int64_t)a->batch * a->num_kv_heads * a->seq_len > kCutMaxRows) return;
+  const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
+  if (rows > kCutMaxRows) return;
+  // Segments that would also fit the registers of one workgroup (8193 .. 16384 rows): up to 65536 rows per call
+  // (1 x 16384 rows, k = 1024: 12.9 / 18.4 us, 4 x 16384: 13.2 / 17.8, 8 x 16384, k = 512: 19.1 / 17.3; at 8192 rows the two are equal).
+  if (chunk_len <= select_cand_capacity() && rows > kCutMaxRows / 4) return;
   *num_samples = s;
   *sample_rank = r;
 }
