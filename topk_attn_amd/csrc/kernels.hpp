@@ -119,6 +119,7 @@ int select_wave_max_k(int64_t seg_len);
 // One workgroup per segment of up to select_small_max_len() scores, k up to select_small_max_k(), rank order: a short
 // program for calls of a few segments.
 int launch_select_small(const SelectParams& p, hipStream_t stream);
+int launch_gemv_select_small(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);   // scores its segments itself
 int select_small_max_len();
 int select_small_max_k();
 

@@ -26,6 +26,7 @@
 // slices), and select_finalize_cand_kernel does step 3 on them from LDS, or, when the slices cannot be
 // used, redoes the segment from the keys (fallback_segment).
 #include <stdlib.h>
+#include <string.h>
 
 #include <mutex>
 #include <utility>
@@ -1175,7 +1176,10 @@ constexpr int kSmallMaxCand = 1024;   // entries of the threshold bucket and abo
 // above (k and a handful) ranked by counting, which is also their output position.  When that bin is crowded (ties)
 // the whole segment goes through the sorting network instead.
 // Dynamic LDS: 2 x 4096 composites (the sort and its exchange buffer; the candidates and the selected otherwise).
-__global__ __launch_bounds__(kSelThreads) void select_small_kernel(SelectParams p) {
+// FROM_KEYS: no GEMV launch before this one; the workgroup scores its segment itself (64 row groups of 16 lanes, 16 rows
+// in flight each, canonical order), the keys go through LDS to the threads that own them.
+template <int DT, bool FROM_KEYS>
+__global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g, SelectParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint64_t* sh_all = (uint64_t*)smem;
   uint64_t* sh_cand = sh_all;
@@ -1190,9 +1194,49 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(SelectParams 
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
   const int64_t n = p.seg_len;
-  const float* sc = p.scores + (int64_t)seg * p.seg_stride;
   uint32_t keys[4], vm;
-  load_keys<4>(sc, (int64_t)tid * 4, n, (((uintptr_t)sc) & 15u) == 0, keys, &vm);
+  if constexpr (FROM_KEYS) {
+    uint32_t* sh_key = (uint32_t*)(sh_all + kSmallMaxLen);   // (the exchange half of the buffer: free until a sort)
+    const int j = tid & 15, rg = tid >> 4;
+    const int chunk = seg % g.num_chunks, bh = seg / g.num_chunks;
+    const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
+    const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
+    const uint16_t* kbase = (const uint16_t*)g.keys + (int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h +
+                            chunk_base * g.key_stride_n + 8 * j;
+    constexpr int kRows = 16;   // rows in flight per lane
+    const int nn = (int)n;
+    float qf[8];
+    for (int base = 0; base < nn; base += (kSelThreads / 16) * kRows) {
+      u32x4 kv[kRows];
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        const int t = base + rg * kRows + u;
+        kv[u] = *(const u32x4*)(kbase + (int64_t)(t < nn ? t : nn - 1) * g.key_stride_n);
+      }
+      __builtin_amdgcn_sched_barrier(0);   // the rows are asked for before the query (whose conversion waits for it)
+      if (base == 0) load_group_query<DT>(g.q, g.q_stride_b, b, h, g.group, j, qf);
+      float mine = 0.0f;
+#pragma unroll
+      for (int u = 0; u < kRows; ++u) {
+        const float s = row_score<DT>(qf, kv[u], g.scale);
+        if (j == u) mine = s;
+      }
+      const int t = base + rg * kRows + j;
+      if (t < nn) sh_key[t] = score_key(mine);
+    }
+    __syncthreads();
+    vm = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int t = 4 * tid + e;
+      const bool ok = t < nn;
+      keys[e] = ok ? sh_key[t] : 0u;
+      vm |= (ok ? 1u : 0u) << e;
+    }
+  } else {
+    const float* sc = p.scores + (int64_t)seg * p.seg_stride;
+    load_keys<4>(sc, (int64_t)tid * 4, n, (((uintptr_t)sc) & 15u) == 0, keys, &vm);
+  }
   sh_hist[2 * tid] = 0;
   sh_hist[2 * tid + 1] = 0;
   if (tid == 0) { sh_n[0] = ~0u; sh_n[1] = 0u; sh_n[2] = 0u; sh_res[0] = 0u; sh_res[1] = 0u; sh_res[2] = 0u; }
@@ -1522,9 +1566,26 @@ int select_small_max_k() { return kSmallMaxK; }
 int launch_select_small(const SelectParams& p, hipStream_t stream) {
   if (p.seg_len > kSmallMaxLen || p.k > kSmallMaxK || p.k > p.seg_len || !p.out_idx || p.union_idx) return TKA_EINVAL;
   const int lds = 2 * kSmallMaxLen * (int)sizeof(uint64_t);
-  if (allow_dynamic_lds((const void*)select_small_kernel, lds) != TKA_OK) return TKA_EHIP;
+  if (allow_dynamic_lds((const void*)select_small_kernel<TKA_F16, false>, lds) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("select_small", stream);
-  select_small_kernel<<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(p);
+  GemvParams none;
+  memset(&none, 0, sizeof none);
+  select_small_kernel<TKA_F16, false><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(none, p);
+  return hip_status(hipGetLastError());
+}
+
+// The same in one launch: every workgroup scores its own segment first (segments of up to select_small_max_len() rows).
+int launch_gemv_select_small(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
+  if (p.seg_len > kSmallMaxLen || p.k > kSmallMaxK || p.k > p.seg_len || !p.out_idx || p.union_idx) return TKA_EINVAL;
+  const int lds = 2 * kSmallMaxLen * (int)sizeof(uint64_t);
+  if (allow_dynamic_lds((const void*)select_small_kernel<TKA_F16, true>, lds) != TKA_OK ||
+      allow_dynamic_lds((const void*)select_small_kernel<TKA_BF16, true>, lds) != TKA_OK)
+    return TKA_EHIP;
+  LaunchTimer timer("gemv_select_small", stream);
+  if (dtype == TKA_F16)
+    select_small_kernel<TKA_F16, true><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p);
+  else
+    select_small_kernel<TKA_BF16, true><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p);
   return hip_status(hipGetLastError());
 }
 
