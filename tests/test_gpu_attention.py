@@ -399,6 +399,34 @@ def test_short_token_list_bf16_weights(seed):
             assert np.abs(out[b, h * G:(h + 1) * G] - ro).max() < 1e-3
 
 
+@pytest.mark.parametrize("layout", ["padded_heads", "head_major"])
+@pytest.mark.parametrize("N,k", [(9000, 1024), (70000, 2048)])
+def test_sparse_decode_step_cache_layouts(layout, N, k):
+    """K and V caches that are views (unused heads on either side of the ones in use; head-major storage): the step
+    must give what it gives on contiguous copies — selection bit for bit, attention within tolerance."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step cache layout %s N=%d k=%d" % (layout, N, k))
+    rng = np.random.default_rng(N + k + 7)
+    dtype, B, H, G, sink, local = oracle.F16, 1, 2, 4, 16, 128
+    q, K, V = randn_bits(rng, (B, H * G, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype)
+
+    def view(x):
+        if layout == "padded_heads":
+            full = randn_bits(rng, (B, N, H + 2, 128), dtype)
+            full[:, :, 1:1 + H] = x
+            return to_dev(full, dtype)[:, :, 1:1 + H]
+        return to_dev(np.ascontiguousarray(x.transpose(0, 2, 1, 3)), dtype).permute(0, 2, 1, 3)
+
+    out, tidx, tval, uidx, ucnt = ops.sparse_decode_step(to_dev(q, dtype), view(K), view(V), k, sink, local, SCALE, G,
+                                                         out_dtype=torch.float16, want_topk=False)
+    torch.cuda.synchronize()
+    out, uidx, ucnt = f32_of(out), uidx.cpu().numpy(), ucnt.cpu().numpy()
+    for h in range(H):
+        ro, ri, rv, ru = oracle.sparse_decode_step(q[0, h * G:(h + 1) * G], K[0, :, h], V[0, :, h], dtype, G, k, sink, local, SCALE)
+        assert ucnt[0, h] == len(ru) and np.array_equal(uidx[0, h, :len(ru)], ru), "union differs (h=%d)" % h
+        assert (np.abs(out[0, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
+
+
 @pytest.fixture
 def hooks():
     """Testing hooks of the candidate route, restored to their defaults afterwards."""

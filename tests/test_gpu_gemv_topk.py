@@ -515,3 +515,36 @@ def test_common_cut_route_chunked():
             ei, ev = oracle.topk_stable(ref[c * 32768:(c + 1) * 32768], k)
             assert np.array_equal(idx[0, h, c * k:(c + 1) * k], ei + c * 32768)
             assert np.array_equal(val[0, h, c * k:(c + 1) * k].view(np.uint32), ev.view(np.uint32))
+
+
+# ---- key caches that are views: padded head dimension, head-major storage ----
+
+@pytest.mark.parametrize("layout", ["padded_heads", "head_major"])
+@pytest.mark.parametrize("N,k", [(1500, 100), (6000, 300), (20000, 700), (40000, 8000), (70000, 1000)])
+def test_key_cache_layouts(layout, N, k):
+    """The key strides are arguments: a cache with unused heads on either side of the ones in use (token stride larger
+    than the heads in use, base pointer inside a row) and a cache stored head-major (token stride 128, head stride
+    N * 128) must give what the contiguous copy gives, on every route (one launch, registers of a workgroup, common
+    cut, dense path, candidate slices)."""
+    from topk_attn_amd import ops
+    announce("gemv_topk key layout %s N=%d k=%d" % (layout, N, k))
+    rng = np.random.default_rng(N + k)
+    dtype, B, H, G = oracle.F16, 2, 2, 2
+    q = randn_bits(rng, (B, H * G, 128), dtype)
+    K = randn_bits(rng, (B, N, H, 128), dtype)
+    if layout == "padded_heads":
+        full = randn_bits(rng, (B, N, H + 3, 128), dtype)
+        full[:, :, 1:1 + H] = K
+        Kd = to_dev(full, dtype)[:, :, 1:1 + H]
+    else:
+        Kd = to_dev(np.ascontiguousarray(K.transpose(0, 2, 1, 3)), dtype).permute(0, 2, 1, 3)
+    assert not Kd.is_contiguous()
+    plan = ops.GemvTopkPlan(to_dev(q, dtype), Kd, k, group=G, scale=SCALE).run()
+    torch.cuda.synchronize()
+    idx, val = plan.idx.cpu().numpy(), plan.val.cpu().numpy()
+    for b in range(B):
+        for h in range(H):
+            ref = oracle.scores_canonical(K[b, :, h, :], dtype, oracle.group_query(q[b, h * G:(h + 1) * G], dtype, G), SCALE)
+            ei, ev = oracle.topk_stable(ref, k)
+            assert np.array_equal(idx[b, h], ei), "indices differ (b=%d h=%d)" % (b, h)
+            assert np.array_equal(val[b, h].view(np.uint32), ev.view(np.uint32))
