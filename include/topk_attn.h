@@ -125,8 +125,9 @@ int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* args, int32_t* count
 int tka_gemv_topk_gave_up_slices(const tka_gemv_topk_args* args, int32_t* count);
 
 /* Testing hooks (no counterpart in the reference).  Process-wide; read once at the start of every call; they
- * change how the candidate route of stage 1 gets to its result, never the result.  NULL restores the defaults
- * (all zero).  Every kernel still runs to its end under any setting: the waits involved are bounded. */
+ * change how the candidate route of stage 1 gets to its result, never the result (union_handoff_order shows a
+ * list in the order in which it is otherwise only handed on).  NULL restores the defaults (all zero).  Every
+ * kernel still runs to its end under any setting: the waits involved are bounded. */
 typedef struct tka_test_hooks {
   int32_t force_segment_redo;  /* 1: the selection accepts no candidate count, every segment of the routes that
                                   store candidates above a sampled threshold is redone from the keys    */
@@ -136,7 +137,9 @@ typedef struct tka_test_hooks {
   int32_t tau_withhold_rem;
   int32_t tau_withhold_mode;   /* ... 0: for good (every slice of the segment gives up); 1: until the
                                   first slice of the segment has given up (the later ones see it)       */
-  int32_t reserved0;
+  int32_t union_handoff_order; /* 1: tka_sparse_decode_step writes out_union_idx the way it hands the list to
+                                  its attention when the caller does not ask for it: the selected tokens
+                                  between the sink range and the local window in the order of the route */
 } tka_test_hooks;
 int tka_set_test_hooks(const tka_test_hooks* hooks);
 
@@ -365,7 +368,8 @@ typedef struct tka_sparse_decode_args {
   int32_t reserved0;
   int32_t* out_topk_idx;  /* device [batch][num_kv_heads][k] rank order; may be NULL (saves a sort) */
   float* out_topk_val;    /* device, same shape; may be NULL; needs out_topk_idx              */
-  int32_t* out_union_idx; /* device [batch][num_kv_heads][k+sink+local]; may be NULL          */
+  int32_t* out_union_idx; /* device [batch][num_kv_heads][k+sink+local], ascending, -1 behind the count; may be NULL
+                             (the step then hands the tokens to the attention in whatever order its route selects them) */
   int32_t* out_union_count;/* device [batch][num_kv_heads]; may be NULL                       */
   void* workspace;
   size_t workspace_bytes;

@@ -435,6 +435,83 @@ def hooks():
     ops.set_test_hooks()
 
 
+@pytest.mark.parametrize("dtype,B,H,G,N,k,sink,local,kind,want_topk,cut", [
+    (oracle.F16, 1, 1, 8, 32768, 2048, 64, 512, "heavy", False, True),
+    (oracle.F16, 1, 1, 8, 32768, 2048, 64, 512, "heavy", True, True),
+    (oracle.BF16, 1, 2, 4, 30000, 1000, 16, 128, "levels", True, True),       # large tie buckets: slices beyond their head entries
+    (oracle.F16, 1, 1, 2, 17000, 1024, 8, 8, "equal", False, True),            # every token ties
+    (oracle.F16, 2, 2, 4, 20000, 1200, 64, 512, "heavy", False, True),
+    (oracle.F16, 1, 1, 1, 65536, 2048, 0, 0, "heavy", False, True),            # no sink range, no window
+    (oracle.F16, 1, 1, 4, 24000, 1400, 6000, 22000, "heavy", True, True),      # range and window overlap: nothing in between
+    (oracle.BF16, 3, 1, 4, 20000, 1200, 1, 19990, "levels", False, True),      # the window covers nearly everything
+    (oracle.F16, 1, 2, 4, 24577, 3000, 300, 300, "heavy", False, False),       # k too large for that route: another one, same list
+    (oracle.F16, 2, 2, 4, 16384, 1024, 64, 512, "heavy", False, False)])       # short enough for the registers of a workgroup
+def test_sparse_decode_step_handoff_order(hooks, dtype, B, H, G, N, k, sink, local, kind, want_topk, cut):
+    """A step that is not asked for its union list hands the tokens to the attention in the order of its route: for a few
+    segments of 8193 .. 65536 tokens the ranking workgroups of the common-cut route write the middle part themselves, part
+    after part.  The union_handoff_order hook makes that list visible: as a set it must be the oracle's, sink range
+    first, local window last, -1 behind the count; rank-ordered top-k (when asked for) bit for bit; attention within tolerance."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step hand-off order dtype=%d B=%d H=%d G=%d N=%d k=%d sink=%d local=%d %s" % (dtype, B, H, G, N, k, sink, local, kind))
+    hooks(union_handoff_order=1)
+    rng = np.random.default_rng(N + 3 * k + sink)
+    if kind == "levels":
+        Kf = np.linspace(-2, 2, 16)[rng.integers(0, 16, (B, N, H, 128))]
+    elif kind == "equal":
+        Kf = np.broadcast_to(rng.standard_normal((1, 1, 1, 128)), (B, N, H, 128)).copy()
+    else:
+        Kf = rng.standard_normal((B, N, H, 128))
+        Kf[:, rng.permutation(N)[:max(1, N // 100)]] *= 4.0
+    q, K, V = randn_bits(rng, (B, H * G, 128), dtype), oracle.to_bits(Kf, dtype), randn_bits(rng, (B, N, H, 128), dtype)
+    plan = ops.SparseDecodePlan(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), k, sink, local, SCALE, G,
+                                out_dtype=torch.float16, want_topk=want_topk)
+    ops.profile_reset()
+    ops.profile_enable(True)
+    plan.step()
+    torch.cuda.synchronize()
+    kernels = ops.profile_read()
+    ops.profile_enable(False)
+    if cut:
+        assert "gemv_cut" in kernels and "select_rank" in kernels, "not the common-cut route: %s" % sorted(kernels)
+        assert plan.redone_segments() == 0
+    out, uidx, ucnt = f32_of(plan.out), plan.union_idx.cpu().numpy(), plan.union_count.cpu().numpy()
+    lo = min(sink, N)
+    hi = max(N - local, lo)
+    for b in range(B):
+        for h in range(H):
+            ro, ri, rv, ru = oracle.sparse_decode_step(q[b, h * G:(h + 1) * G], K[b, :, h], V[b, :, h], dtype, G, k, sink,
+                                                       local, SCALE)
+            got = uidx[b, h]
+            assert ucnt[b, h] == len(ru), "union count differs (b=%d h=%d)" % (b, h)
+            assert np.array_equal(np.sort(got[:len(ru)]), ru), "union differs as a set (b=%d h=%d)" % (b, h)
+            assert np.array_equal(got[:lo], np.arange(lo)) and np.array_equal(got[len(ru) - (N - hi):len(ru)], np.arange(hi, N))
+            assert (got[len(ru):] == -1).all()
+            if want_topk:
+                assert np.array_equal(plan.topk_idx[b, h].cpu().numpy(), ri), "top-k indices differ"
+                assert np.array_equal(plan.topk_val[b, h].cpu().numpy().view(np.uint32), rv.view(np.uint32))
+            assert (np.abs(out[b, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
+
+
+def test_sparse_decode_step_handoff_order_forced_redo(hooks):
+    """The same hand-off when the ranking kernel redoes its segments from the keys (then the list comes ascending)."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step hand-off order, segments redone from the keys (N=20000 k=1200 G=4)")
+    hooks(union_handoff_order=1, force_segment_redo=1)
+    rng = np.random.default_rng(61)
+    dtype, B, H, G, N, k, sink, local = oracle.F16, 1, 2, 4, 20000, 1200, 32, 100
+    q, K, V = randn_bits(rng, (B, H * G, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype)
+    plan = ops.SparseDecodePlan(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), k, sink, local, SCALE, G,
+                                out_dtype=torch.float16, want_topk=False)
+    plan.step()
+    torch.cuda.synchronize()
+    assert plan.redone_segments() == 2
+    out, uidx, ucnt = f32_of(plan.out), plan.union_idx.cpu().numpy(), plan.union_count.cpu().numpy()
+    for h in range(H):
+        ro, ri, rv, ru = oracle.sparse_decode_step(q[0, h * G:(h + 1) * G], K[0, :, h], V[0, :, h], dtype, G, k, sink, local, SCALE)
+        assert ucnt[0, h] == len(ru) and np.array_equal(uidx[0, h, :len(ru)], ru), "union differs (h=%d)" % h
+        assert (np.abs(out[0, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
+
+
 def test_sparse_decode_step_forced_redo(hooks):
     """Union mode of the path that redoes a segment from the keys (force_segment_redo hook), 16-level keys."""
     hooks(force_segment_redo=1)

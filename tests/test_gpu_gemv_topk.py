@@ -490,6 +490,24 @@ def test_common_cut_route_adversarial_sample_falls_back():
     _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k, redone=1)
 
 
+def test_common_cut_route_sample_sits_low():
+    """The sampled rows score lower than the rest (their keys shrunk by a fifth): the cut lands low and more tokens pass
+    than one ranking workgroup may hold (8192).  No part of the order is that large, so the segment keeps the route."""
+    announce("gemv_topk common-cut route, sample below the rest: more than 8192 candidates, none redone")
+    rng = np.random.default_rng(56)
+    N, k, dtype = 65536, 2048, oracle.F16
+    Kf = rng.standard_normal((1, N, 1, 128))
+    pos = _cut_sample_positions(0, N)
+    Kf[0, pos, 0, :] *= 0.8
+    K, q = oracle.to_bits(Kf, dtype), randn_bits(rng, (1, 1, 128), dtype)
+    ref = oracle.scores_canonical(K[0, :, 0, :], dtype, oracle.group_query(q[0, 0:1], dtype, 1), SCALE)
+    m = 256.0 * k / N
+    rank = int(np.ceil(m + 5.5 * np.sqrt(m) + 2.0))
+    cut = np.sort(ref[pos])[::-1][rank - 1]
+    assert 8192 < int((ref >= cut).sum()) < 16384, "the premise of this test: candidates at or above the rank-%d sample" % rank
+    _check_long(K, q, dtype, 1, k, redone=0)
+
+
 def test_common_cut_route_forced_redo(hooks):
     announce("gemv_topk common-cut route, every segment redone from the keys")
     hooks(force_segment_redo=1)

@@ -194,8 +194,15 @@ void candidate_plan(const tka_gemv_topk_args* a, int* num_samples, int* sample_r
     gemv_candidate_plan(chunk_len, (int64_t)a->batch * a->num_kv_heads * a->seq_len, a->k, select_cand_capacity(), num_samples, sample_rank);
 }
 
+struct UnionOut {
+  int32_t* idx;
+  int32_t* count;
+  int sink, local;
+  bool any_order;   // the selected tokens between the sink range and the local window may come in any order
+};
+
 // Samples per segment and rank of the cut when the call takes the common-cut route (a few segments of middling
-// length, rank-ordered output), else 0.  Shorter segments are selected from the registers of one workgroup, longer
+// length; rank-ordered output, and the union list for a caller that takes its middle part in any order), else 0.  Shorter segments are selected from the registers of one workgroup, longer
 // ones (or many of them) by the sampling workgroups of the candidate route.
 int64_t cut_route_min_len() {
   static const int64_t v = [] {
@@ -204,10 +211,10 @@ int64_t cut_route_min_len() {
   }();
   return v;
 }
-void cut_plan(const tka_gemv_topk_args* a, bool want_union, int* num_samples, int* sample_rank) {
+void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, int* sample_rank) {
   *num_samples = *sample_rank = 0;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
-  if (!a->out_idx || want_union || a->out_scores || chunk_len < cut_route_min_len()) return;
+  if ((!a->out_idx && !u) || (u && !u->any_order) || a->out_scores || chunk_len < cut_route_min_len()) return;
   int s = 0, r = 0;
   gemv_cut_plan(chunk_len, a->k, &s, &r);
   if (s == 0) return;
@@ -219,15 +226,13 @@ void cut_plan(const tka_gemv_topk_args* a, bool want_union, int* num_samples, in
   // Segments that would also fit the registers of one workgroup (8193 .. 16384 rows): up to 65536 rows per call
   // (1 x 16384 rows, k = 1024: 12.9 / 18.4 us, 4 x 16384: 13.2 / 17.8, 8 x 16384, k = 512: 19.1 / 17.3; at 8192 rows the two are equal).
   if (chunk_len <= select_cand_capacity() && rows > kCutMaxRows / 4) return;
+  // With the union list for the attention of a decode step (us per step, this route against the others): 1 x 32768 rows
+  // 25.6 / 32.2, 4 x 32768 34.7 / 37.5, 8 x 32768 46.5 / 43.7, 1 x 65536 28.9 / 34.5, 2 x 65536 42.1 / 36.0,
+  // 2 x 49152 (k = 1024) 32.5 / 32.7, 1 x 16384 (k = 1024) 23.7 / 22.5.
+  if (u && (chunk_len <= select_cand_capacity() || rows > (chunk_len <= 32768 ? kCutMaxRows / 2 : kCutMaxRows / 4))) return;
   *num_samples = s;
   *sample_rank = r;
 }
-
-struct UnionOut {
-  int32_t* idx;
-  int32_t* count;
-  int sink, local;
-};
 
 // Runs clear + GEMV (+histogram) + select.  `ws` holds [scores][select workspace].
 // a->out_idx == nullptr skips the rank-order sort (then `u` must ask for the union list).
@@ -295,7 +300,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // A few segments of middling length: every GEMV workgroup derives the segment's cut from common sample rows and
   // stores its candidates, one workgroup per segment ranks them.
   int cut_samples = 0, cut_rank = 0;
-  cut_plan(a, u != nullptr, &cut_samples, &cut_rank);
+  cut_plan(a, u, &cut_samples, &cut_rank);
   if (cut_samples != 0 && !ic) {
     GemvParams cp = gp;
     cp.hist = nullptr;
@@ -314,7 +319,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     sc.hist = nullptr;
     sc.parts = cp.wgs_per_chunk;
     sc.part_len = kCutTokensPerWg;
-    sc.max_entries = current_hooks().force_segment_redo ? 0 : kCutMaxCandidates;
+    sc.max_entries = current_hooks().force_segment_redo ? 0 : kCutMaxSlices * kCutTokensPerWg;   // (no limit of its own)
     sc.scores = scores;
     sc.cut_splits = cp.cut_splits;
     return launch_select_rank(gp, sc, a->dtype, stream);
@@ -563,14 +568,15 @@ int tka_gemv_topk(const tka_gemv_topk_args* a) {
 
 // Per-segment flag words of the last candidate-route call with these arguments (bit 0: redone from the keys,
 // bits 8..: slices whose workgroup gave up waiting for the threshold); empty for calls that take another route.
-static int read_segment_flags(const tka_gemv_topk_args* a, std::vector<uint32_t>* flags) {
+// `u`: the union list that the call asked for (nullptr: none), which decides the route with the other arguments.
+static int read_segment_flags(const tka_gemv_topk_args* a, const UnionOut* u, std::vector<uint32_t>* flags) {
   flags->clear();
   int rc = check_gemv(a, true);
   if (rc != TKA_OK) return rc;
   if (!a->workspace || a->workspace_bytes < tka_gemv_topk_workspace_bytes(a)) return TKA_EWORKSPACE;
   int num_samples = 0, sample_rank = 0;
-  candidate_plan(a, &num_samples, &sample_rank);
-  if (num_samples == 0) cut_plan(a, false, &num_samples, &sample_rank);
+  cut_plan(a, u, &num_samples, &sample_rank);   // (no route between the two writes the flags: those segments are too short for the second)
+  if (num_samples == 0) candidate_plan(a, &num_samples, &sample_rank);
   if (num_samples == 0) return TKA_OK;
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
   SelectParams sp;
@@ -582,20 +588,22 @@ static int read_segment_flags(const tka_gemv_topk_args* a, std::vector<uint32_t>
   return TKA_OK;
 }
 
-int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* a, int32_t* count) {
+static int redone_segments(const tka_gemv_topk_args* a, const UnionOut* u, int32_t* count) {
   if (!count) return TKA_EINVAL;
   *count = 0;
   std::vector<uint32_t> flags;
-  const int rc = read_segment_flags(a, &flags);
+  const int rc = read_segment_flags(a, u, &flags);
   for (uint32_t f : flags) *count += (int32_t)(f & 1u);
   return rc;
 }
+
+int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* a, int32_t* count) { return redone_segments(a, nullptr, count); }
 
 int tka_gemv_topk_gave_up_slices(const tka_gemv_topk_args* a, int32_t* count) {
   if (!count) return TKA_EINVAL;
   *count = 0;
   std::vector<uint32_t> flags;
-  const int rc = read_segment_flags(a, &flags);
+  const int rc = read_segment_flags(a, nullptr, &flags);
   for (uint32_t f : flags) *count += (int32_t)(f >> 8);
   return rc;
 }
@@ -1039,6 +1047,9 @@ static int sd_parts(const tka_sparse_decode_args* a, tka_gemv_topk_args* g, tka_
   return TKA_OK;
 }
 
+// The attention takes the selected tokens in any order; a caller that asks for the list gets it ascending.
+static bool sd_union_any_order(const tka_sparse_decode_args* a) { return !a->out_union_idx || current_hooks().union_handoff_order != 0; }
+
 static int sd_check(const tka_sparse_decode_args* a, tka_gemv_topk_args* g, tka_flash_decode_args* f) {
   int rc = sd_parts(a, g, f);
   if (rc != TKA_OK) return rc;
@@ -1078,7 +1089,8 @@ int tka_sparse_decode_redone_segments(const tka_sparse_decode_args* a, int32_t* 
   if (!a->workspace || a->workspace_bytes < tka_sparse_decode_workspace_bytes(a)) return TKA_EWORKSPACE;
   g.workspace = (unsigned char*)a->workspace + sd_gemv_ws_offset(a, f);
   g.workspace_bytes = tka_gemv_topk_workspace_bytes(&g);
-  return tka_gemv_topk_redone_segments(&g, count);
+  const UnionOut uo = {nullptr, nullptr, a->sink, a->local, sd_union_any_order(a)};
+  return redone_segments(&g, &uo, count);
 }
 
 int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
@@ -1109,7 +1121,7 @@ int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
   g.out_val = a->out_topk_idx ? tval : nullptr;
   g.workspace = ws;
   g.workspace_bytes = gemv_ws;
-  UnionOut uo = {uidx, ucnt, a->sink, a->local};
+  UnionOut uo = {uidx, ucnt, a->sink, a->local, sd_union_any_order(a)};
   rc = run_gemv_topk(&g, nullptr, 0, nullptr, &uo);
   if (rc != TKA_OK) return rc;
   f.kv_idx = uidx;

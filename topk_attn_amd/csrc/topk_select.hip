@@ -971,8 +971,13 @@ __device__ __forceinline__ void write_ranked(const SelectParams& p, int seg, uin
 // part's lower end, cut to its 11 leading bits, gives 2048 buckets in rank order; a histogram and one suffix scan
 // give every bucket its first rank, the composites are scattered to their bucket, and each one counts the larger
 // members of its own bucket.  rank < k: selected, and the rank is the output position.  Heavy ties that fill a bucket
-// send the part to the bitonic network; a segment with fewer than k candidates (the sample misjudged it) or more than
-// fit is redone from the keys by its first workgroup (fallback_segment).
+// send the part to the bitonic network; a segment with fewer than k candidates (the sample misjudged it), with a part
+// of more than kCutMaxCandidates or with more than kCutMaxExtras entries beyond the heads is redone from the keys by
+// its first workgroup (fallback_segment).
+// A caller that takes the selected tokens in any order (the attention of the decode step) gets the union list from the
+// same workgroups: sink range, then the selected tokens between the ranges - part after part, inside a part in the order
+// of its threads; a workgroup's first position is the number of candidates above its part less those of them inside
+// the ranges - then the local window, the count and the padding, written by the workgroup that holds rank k - 1.
 // Dynamic LDS: kCutMaxCandidates composites (the part, as found), then as many again (the part in bucket order;
 // before that, entries from beyond the heads); the tie path and the fallback reuse both.
 // PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256).
@@ -989,7 +994,8 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   __shared__ uint64_t sh_split[kCutParts + 1];
   __shared__ uint32_t sh_ovf[kCutMaxSlices];
   __shared__ uint32_t sh_n[8];   // [0] slices with more than kCutHead entries, [1] entries beyond the heads, [2] candidates,
-                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key
+                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key,
+                                 // [7] candidates above the part inside the sink range or the local window (union list only)
 
   typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
   constexpr int kPairs = PAIRS;
@@ -1002,6 +1008,10 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   const uint32_t k = (uint32_t)p.k;
   const u64x2* heads = (const u64x2*)(p.cand_head + (int64_t)seg * p.parts * kCutHead);
   const int n_pairs = p.parts * (kCutHead / 2);
+  // union list: tokens below `lo` (sink range) and from `hi` on (local window) are listed whether selected or not
+  const bool want_union = p.union_idx != nullptr;
+  const uint32_t lo = (uint32_t)(p.sink < p.seg_len ? p.sink : p.seg_len);
+  const uint32_t hi = (uint32_t)(p.seg_len - p.local > (int64_t)lo ? p.seg_len - p.local : (int64_t)lo);
 
   u64x2 w[kPairs];
 #pragma unroll
@@ -1062,24 +1072,35 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   // all candidates, those above this part, those of the part (collected in LDS), the part's largest key
   const uint64_t t_hi = sh_split[part], t_lo = sh_split[part + 1];
   {
-    uint32_t n_all = 0, n_above = 0, kmax = 0;
-    auto take = [&](uint64_t x) {
+    uint32_t n_all = 0, n_above = 0, kmax = 0, n_edge = 0;
+    // (only the slices that reach into the sink range or the local window can hold tokens of them)
+    const int lo_slices = (int)((lo + (uint32_t)kCutTokensPerWg - 1u) / (uint32_t)kCutTokensPerWg), hi_slice = (int)(hi / (uint32_t)kCutTokensPerWg);
+    auto take = [&](uint64_t x, bool edge_slice) {
       const bool nz = x != 0ull;
       const bool above = part != 0 && x >= t_hi;
       const bool own = nz && !above && x >= t_lo;
       n_all += nz ? 1u : 0u;
       n_above += above ? 1u : 0u;
       if (own) {
-        sh_own[atomicAdd(&sh_n[5], 1u)] = x;
+        const uint32_t at = atomicAdd(&sh_n[5], 1u);
+        if (at < (uint32_t)kCutMaxCandidates) sh_own[at] = x;   // (a part beyond that: the segment is redone, see below)
         kmax = max(kmax, (uint32_t)(x >> 32));
+      }
+      if (edge_slice && above) {
+        const uint32_t t = ~(uint32_t)x;
+        n_edge += t < lo || t >= hi ? 1u : 0u;
       }
     };
 #pragma unroll
-    for (int i = 0; i < kHeadMine; ++i) take(c[i]);
+    for (int i = 0; i < kHeadMine; ++i) {
+      const int slice = ((i / 2) * kSelThreads + tid) / (kCutHead / 2);
+      take(c[i], want_union && (slice < lo_slices || slice >= hi_slice));
+    }
     if (n_ovf) {
 #pragma unroll
-      for (int i = kHeadMine; i < kMine; ++i) take(c[i]);
+      for (int i = kHeadMine; i < kMine; ++i) take(c[i], want_union);
     }
+    if (n_edge) atomicAdd(&sh_n[7], n_edge);
     const uint32_t inc = wave_inclusive_scan((n_all << 16) | n_above);   // (at most 18 x 64 per wave each)
     kmax = max(kmax, lane_xor<1>(kmax));
     kmax = max(kmax, lane_xor<2>(kmax));
@@ -1095,8 +1116,43 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   }
   __syncthreads();
   const uint32_t n_cand = sh_n[2], n_above = sh_n[4], n_own = sh_n[5];
-  const uint32_t cap = (uint32_t)(p.max_entries < kCutMaxCandidates ? p.max_entries : kCutMaxCandidates);
-  const bool redo = n_cand < k || n_cand > cap || n_extra > (uint32_t)kCutMaxExtras;
+  // More candidates than one part may hold (the sample sat low: at 65536 tokens and k = 2048 one call in ten): fine as
+  // long as every part fits, which all workgroups of the segment have to see alike - each counts the sizes of all parts.
+  uint32_t max_part = n_own;
+  if (n_cand > (uint32_t)kCutMaxCandidates) {
+    uint64_t sizes = 0;   // eight counts of 8 bits (a thread holds 24 entries at most)
+    auto count = [&](uint64_t x) {
+      uint32_t below = 0;
+#pragma unroll
+      for (int i = 1; i < kCutParts; ++i) below += x < sh_split[i] ? 1u : 0u;
+      sizes += x != 0ull ? 1ull << (8 * below) : 0ull;
+    };
+#pragma unroll
+    for (int i = 0; i < kHeadMine; ++i) count(c[i]);
+    if (n_ovf) {
+#pragma unroll
+      for (int i = kHeadMine; i < kMine; ++i) count(c[i]);
+    }
+    if (tid < kCutParts) sh_hist[tid] = 0;   // (the histogram's first words: cleared again below)
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kCutParts / 2; ++i) {   // two parts per word, 16 bits each (at most 24 x 64 per wave)
+      const uint32_t two = (uint32_t)(sizes >> (16 * i)) & 0xffu, other = (uint32_t)(sizes >> (16 * i + 8)) & 0xffu;
+      const uint32_t inc = wave_inclusive_scan(two | (other << 16));
+      if (lane == 63) {
+        atomicAdd(&sh_hist[2 * i], inc & 0xffffu);
+        atomicAdd(&sh_hist[2 * i + 1], inc >> 16);
+      }
+    }
+    __syncthreads();
+    max_part = 0;
+#pragma unroll
+    for (int i = 0; i < kCutParts; ++i) max_part = max(max_part, sh_hist[i]);
+    __syncthreads();
+    if (tid < kCutParts) sh_hist[tid] = 0;
+    __syncthreads();
+  }
+  const bool redo = n_cand < k || n_cand > (uint32_t)p.max_entries || n_extra > (uint32_t)kCutMaxExtras || max_part > (uint32_t)kCutMaxCandidates;
   if (tid == 0 && part == 0) p.seg_flags[seg] = redo ? 1u : 0u;
   if (redo) {   // every workgroup of the segment sees the same counts: the first one redoes it, the others leave
     if (part != 0) return;
@@ -1132,6 +1188,22 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   }
   __syncthreads();
   const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len) : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
+  // what a ranked candidate leaves behind (every thread calls it once per round of the loops below: it scans over the
+  // workgroup when the union list is wanted)
+  int32_t* uo = want_union ? p.union_idx + (int64_t)seg * (p.k + p.sink + p.local) : nullptr;
+  uint32_t mid_at = lo + n_above - sh_n[7];   // next place of the middle part: every candidate above the part is selected
+  auto emit = [&](bool valid, uint32_t rank, uint64_t x) {
+    const bool sel = valid && rank < k;
+    if (sel && p.out_idx) write_ranked(p, seg, idx_base, rank, x);
+    if (want_union) {
+      const uint32_t t = ~(uint32_t)x;
+      const bool mid = sel && t >= lo && t < hi;
+      uint32_t total;
+      const uint32_t pos = block_exclusive_scan(mid ? 1u : 0u, sh_wtot, &total);
+      if (mid) uo[mid_at + pos] = (int32_t)t;
+      mid_at += total;
+    }
+  };
   if (sh_n[3] != 0u) {
     // heavy ties: sort the part and take it in order
     uint32_t npad = 64;
@@ -1139,28 +1211,40 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     for (uint32_t i = n_own + tid; i < npad; i += kSelThreads) sh_own[i] = 0;   // pad: below every real composite
     __syncthreads();
     sort_lds_desc(sh_own, sh_x, (int)npad);
-    for (uint32_t i = tid; i < n_own; i += kSelThreads)
-      if (n_above + i < k) write_ranked(p, seg, idx_base, n_above + i, sh_own[i]);
-    return;
-  }
+    __syncthreads();
 #pragma unroll 1
-  for (uint32_t i = tid; i < n_own; i += kSelThreads) {
-    const uint64_t x = sh_own[i];
-    sh_x[atomicAdd(&sh_cur[(uint32_t)((x - base) >> shift)], 1u)] = x;
-  }
-  __syncthreads();
-  // every candidate of the part: its rank is the candidates above the part, plus the first rank of its bucket, plus the
-  // larger members of the bucket
+    for (uint32_t first = 0; first < n_own; first += kSelThreads) {
+      const uint32_t i = first + tid;
+      emit(i < n_own, n_above + i, i < n_own ? sh_own[i] : 0ull);
+    }
+  } else {
 #pragma unroll 1
-  for (uint32_t i = tid; i < n_own; i += kSelThreads) {
-    const uint64_t x = sh_x[i];
-    const uint32_t bin = (uint32_t)((x - base) >> shift);
-    const uint32_t start = sh_off[bin], cnt = sh_hist[bin];
-    uint32_t larger = 0;
-    for (uint32_t j = 0; j < cnt; ++j) larger += sh_x[start + j] > x ? 1u : 0u;
-    const uint32_t rank = n_above + start + larger;
-    if (rank < k) write_ranked(p, seg, idx_base, rank, x);
+    for (uint32_t i = tid; i < n_own; i += kSelThreads) {
+      const uint64_t x = sh_own[i];
+      sh_x[atomicAdd(&sh_cur[(uint32_t)((x - base) >> shift)], 1u)] = x;
+    }
+    __syncthreads();
+    // every candidate of the part: its rank is the candidates above the part, plus the first rank of its bucket, plus the
+    // larger members of the bucket
+#pragma unroll 1
+    for (uint32_t first = 0; first < n_own; first += kSelThreads) {
+      const uint32_t i = first + tid;
+      const bool valid = i < n_own;
+      uint64_t x = 0ull;
+      uint32_t rank = 0;
+      if (valid) {
+        x = sh_x[i];
+        const uint32_t bin = (uint32_t)((x - base) >> shift);
+        const uint32_t start = sh_off[bin], cnt = sh_hist[bin];
+        uint32_t larger = 0;
+        for (uint32_t j = 0; j < cnt; ++j) larger += sh_x[start + j] > x ? 1u : 0u;
+        rank = n_above + start + larger;
+      }
+      emit(valid, rank, x);
+    }
   }
+  // the workgroup whose part holds rank k - 1 knows how long the middle part is
+  if (want_union && n_above + n_own >= k) write_union_edges(uo, p, seg, lo, hi, mid_at - lo);
 }
 
 // ---- a small k out of a few thousand scores, few segments -------------------------------------------------
@@ -1538,8 +1622,8 @@ int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int 
 }
 
 int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
-  if (p.parts < 1 || p.parts > kCutMaxSlices || p.part_len != kCutTokensPerWg || p.k > kCutMaxK || !p.out_idx || p.union_idx || !p.cand_head ||
-      !p.list_cnt || !p.cut_splits)
+  if (p.parts < 1 || p.parts > kCutMaxSlices || p.part_len != kCutTokensPerWg || p.k > kCutMaxK || (!p.out_idx && !p.union_idx) || !p.cand_head ||
+      !p.list_cnt || !p.cut_splits || (p.union_idx && !p.union_count))
     return TKA_EINVAL;
   const int lds = 2 * kCutMaxCandidates * (int)sizeof(uint64_t);
   const void* kernels[4] = {(const void*)select_rank_kernel<TKA_F16, 4>, (const void*)select_rank_kernel<TKA_F16, 8>,
