@@ -961,6 +961,52 @@ __device__ __forceinline__ void write_ranked(const SelectParams& p, int seg, uin
   }
 }
 
+// Size of the largest of the kCutParts parts of a segment's candidates: `pairs` pairs of head entries (zeros are no
+// candidates), `n_extra` entries from beyond the heads, sh_split[1 .. kCutParts - 1] the inner ends of the parts in
+// descending order.  sh_words: kCutParts words that are zero on entry and on exit.  Every thread of the workgroup calls it.
+// Kept out of line: it runs when a segment has more candidates than one part may hold, which is rare, and the kernel
+// around it is one whose every instruction counts.
+__device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_pairs, const uint64_t* extra, uint32_t n_extra,
+                                              const uint64_t* sh_split, uint32_t* sh_words) {
+  typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+  const u64x2* heads = (const u64x2*)heads_flat;
+  const int tid = threadIdx.x, lane = tid & 63;
+  uint64_t sizes = 0;   // eight counts of 8 bits (a thread sees 24 entries at most)
+  auto count = [&](uint64_t x) {
+    uint32_t below = 0;
+#pragma unroll
+    for (int i = 1; i < kCutParts; ++i) below += x < sh_split[i] ? 1u : 0u;
+    sizes += x != 0ull ? 1ull << (8 * below) : 0ull;
+  };
+#pragma unroll 1
+  for (int q = tid; q < n_pairs; q += kSelThreads) {
+    const u64x2 two = heads[q];
+    count(two[0]);
+    count(two[1]);
+  }
+  if (extra) {
+#pragma unroll 1
+    for (uint32_t i = tid; i < n_extra; i += kSelThreads) count(extra[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < kCutParts / 2; ++i) {   // two parts per word, 16 bits each (at most 24 x 64 per wave)
+    const uint32_t one = (uint32_t)(sizes >> (16 * i)) & 0xffu, other = (uint32_t)(sizes >> (16 * i + 8)) & 0xffu;
+    const uint32_t inc = wave_inclusive_scan(one | (other << 16));
+    if (lane == 63) {
+      atomicAdd(&sh_words[2 * i], inc & 0xffffu);
+      atomicAdd(&sh_words[2 * i + 1], inc >> 16);
+    }
+  }
+  __syncthreads();
+  uint32_t largest = 0;
+#pragma unroll
+  for (int i = 0; i < kCutParts; ++i) largest = max(largest, sh_words[i]);
+  __syncthreads();
+  if (tid < kCutParts) sh_words[tid] = 0;
+  __syncthreads();
+  return largest;
+}
+
 // Common-cut route: the slices (256 tokens each, written by gemv_cut_kernel) hold every token at or above the
 // segment's cut, as composites, and kCutParts sample composites split the order into parts of about equal size.
 // kCutParts workgroups per segment (one CU executes 64 lane-operations per cycle, and this is a kernel of a few
@@ -980,8 +1026,8 @@ __device__ __forceinline__ void write_ranked(const SelectParams& p, int seg, uin
 // the ranges - then the local window, the count and the padding, written by the workgroup that holds rank k - 1.
 // Dynamic LDS: kCutMaxCandidates composites (the part, as found), then as many again (the part in bucket order;
 // before that, entries from beyond the heads); the tie path and the fallback reuse both.
-// PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256).
-template <int DT, int PAIRS>
+// PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256); UNION: the union list is written.
+template <int DT, int PAIRS, bool UNION>
 __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, SelectParams p, int kpad) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint64_t* sh_own = (uint64_t*)smem;
@@ -1008,10 +1054,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   const uint32_t k = (uint32_t)p.k;
   const u64x2* heads = (const u64x2*)(p.cand_head + (int64_t)seg * p.parts * kCutHead);
   const int n_pairs = p.parts * (kCutHead / 2);
-  // union list: tokens below `lo` (sink range) and from `hi` on (local window) are listed whether selected or not
-  const bool want_union = p.union_idx != nullptr;
-  const uint32_t lo = (uint32_t)(p.sink < p.seg_len ? p.sink : p.seg_len);
-  const uint32_t hi = (uint32_t)(p.seg_len - p.local > (int64_t)lo ? p.seg_len - p.local : (int64_t)lo);
 
   u64x2 w[kPairs];
 #pragma unroll
@@ -1072,35 +1114,26 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   // all candidates, those above this part, those of the part (collected in LDS), the part's largest key
   const uint64_t t_hi = sh_split[part], t_lo = sh_split[part + 1];
   {
-    uint32_t n_all = 0, n_above = 0, kmax = 0, n_edge = 0;
-    // (only the slices that reach into the sink range or the local window can hold tokens of them)
-    const int lo_slices = (int)((lo + (uint32_t)kCutTokensPerWg - 1u) / (uint32_t)kCutTokensPerWg), hi_slice = (int)(hi / (uint32_t)kCutTokensPerWg);
-    auto take = [&](uint64_t x, bool edge_slice) {
+    uint32_t n_all = 0, n_above = 0, kmax = 0;
+    auto take = [&](uint64_t x) {
       const bool nz = x != 0ull;
       const bool above = part != 0 && x >= t_hi;
       const bool own = nz && !above && x >= t_lo;
       n_all += nz ? 1u : 0u;
       n_above += above ? 1u : 0u;
       if (own) {
-        const uint32_t at = atomicAdd(&sh_n[5], 1u);
-        if (at < (uint32_t)kCutMaxCandidates) sh_own[at] = x;   // (a part beyond that: the segment is redone, see below)
+        // (a part of more than kCutMaxCandidates runs on into the second array, whose last place takes the rest: such a
+        // segment is redone, see below)
+        sh_own[min(atomicAdd(&sh_n[5], 1u), 2u * (uint32_t)kCutMaxCandidates - 1u)] = x;
         kmax = max(kmax, (uint32_t)(x >> 32));
-      }
-      if (edge_slice && above) {
-        const uint32_t t = ~(uint32_t)x;
-        n_edge += t < lo || t >= hi ? 1u : 0u;
       }
     };
 #pragma unroll
-    for (int i = 0; i < kHeadMine; ++i) {
-      const int slice = ((i / 2) * kSelThreads + tid) / (kCutHead / 2);
-      take(c[i], want_union && (slice < lo_slices || slice >= hi_slice));
-    }
+    for (int i = 0; i < kHeadMine; ++i) take(c[i]);
     if (n_ovf) {
 #pragma unroll
-      for (int i = kHeadMine; i < kMine; ++i) take(c[i], want_union);
+      for (int i = kHeadMine; i < kMine; ++i) take(c[i]);
     }
-    if (n_edge) atomicAdd(&sh_n[7], n_edge);
     const uint32_t inc = wave_inclusive_scan((n_all << 16) | n_above);   // (at most 18 x 64 per wave each)
     kmax = max(kmax, lane_xor<1>(kmax));
     kmax = max(kmax, lane_xor<2>(kmax));
@@ -1119,39 +1152,8 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   // More candidates than one part may hold (the sample sat low: at 65536 tokens and k = 2048 one call in ten): fine as
   // long as every part fits, which all workgroups of the segment have to see alike - each counts the sizes of all parts.
   uint32_t max_part = n_own;
-  if (n_cand > (uint32_t)kCutMaxCandidates) {
-    uint64_t sizes = 0;   // eight counts of 8 bits (a thread holds 24 entries at most)
-    auto count = [&](uint64_t x) {
-      uint32_t below = 0;
-#pragma unroll
-      for (int i = 1; i < kCutParts; ++i) below += x < sh_split[i] ? 1u : 0u;
-      sizes += x != 0ull ? 1ull << (8 * below) : 0ull;
-    };
-#pragma unroll
-    for (int i = 0; i < kHeadMine; ++i) count(c[i]);
-    if (n_ovf) {
-#pragma unroll
-      for (int i = kHeadMine; i < kMine; ++i) count(c[i]);
-    }
-    if (tid < kCutParts) sh_hist[tid] = 0;   // (the histogram's first words: cleared again below)
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < kCutParts / 2; ++i) {   // two parts per word, 16 bits each (at most 24 x 64 per wave)
-      const uint32_t two = (uint32_t)(sizes >> (16 * i)) & 0xffu, other = (uint32_t)(sizes >> (16 * i + 8)) & 0xffu;
-      const uint32_t inc = wave_inclusive_scan(two | (other << 16));
-      if (lane == 63) {
-        atomicAdd(&sh_hist[2 * i], inc & 0xffffu);
-        atomicAdd(&sh_hist[2 * i + 1], inc >> 16);
-      }
-    }
-    __syncthreads();
-    max_part = 0;
-#pragma unroll
-    for (int i = 0; i < kCutParts; ++i) max_part = max(max_part, sh_hist[i]);
-    __syncthreads();
-    if (tid < kCutParts) sh_hist[tid] = 0;
-    __syncthreads();
-  }
+  if (n_cand > (uint32_t)kCutMaxCandidates)
+    max_part = max(max_part, largest_part((const uint64_t*)heads, n_pairs, n_ovf ? sh_extra : nullptr, min(n_extra, (uint32_t)kCutMaxExtras), sh_split, sh_hist));
   const bool redo = n_cand < k || n_cand > (uint32_t)p.max_entries || n_extra > (uint32_t)kCutMaxExtras || max_part > (uint32_t)kCutMaxCandidates;
   if (tid == 0 && part == 0) p.seg_flags[seg] = redo ? 1u : 0u;
   if (redo) {   // every workgroup of the segment sees the same counts: the first one redoes it, the others leave
@@ -1161,6 +1163,31 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     return;
   }
   if (n_above >= k || n_own == 0u) return;   // nothing of this part is selected
+
+  // union list: tokens below `lo` (sink range) and from `hi` on (local window) are listed whether selected or not, so the
+  // selected ones among them do not count for the place of this part in the list
+  constexpr bool want_union = UNION;
+  const uint32_t lo = (uint32_t)(p.sink < p.seg_len ? p.sink : p.seg_len);
+  const uint32_t hi = (uint32_t)(p.seg_len - p.local > (int64_t)lo ? p.seg_len - p.local : (int64_t)lo);
+  if (want_union && part != 0) {
+    // (only the slices that reach into the range or the window can hold tokens of them)
+    const int lo_slices = (int)((lo + (uint32_t)kCutTokensPerWg - 1u) / (uint32_t)kCutTokensPerWg), hi_slice = (int)(hi / (uint32_t)kCutTokensPerWg);
+    uint32_t n_edge = 0;
+    auto edge = [&](uint64_t x) {
+      const uint32_t t = ~(uint32_t)x;
+      n_edge += x >= t_hi && (t < lo || t >= hi) ? 1u : 0u;
+    };
+#pragma unroll
+    for (int i = 0; i < kHeadMine; ++i) {
+      const int slice = ((i / 2) * kSelThreads + tid) / (kCutHead / 2);
+      if (slice < lo_slices || slice >= hi_slice) edge(c[i]);
+    }
+    if (n_ovf) {
+#pragma unroll
+      for (int i = kHeadMine; i < kMine; ++i) edge(c[i]);
+    }
+    if (n_edge) atomicAdd(&sh_n[7], n_edge);   // (read behind the barriers of the bucket scan)
+  }
 
   // buckets: linear in the composite between the ends of the part (the first part ends at its largest key)
   const uint64_t base = t_lo;
@@ -1226,21 +1253,28 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     __syncthreads();
     // every candidate of the part: its rank is the candidates above the part, plus the first rank of its bucket, plus the
     // larger members of the bucket
+    auto rank_of = [&](uint64_t x) {
+      const uint32_t bin = (uint32_t)((x - base) >> shift);
+      const uint32_t start = sh_off[bin], cnt = sh_hist[bin];
+      uint32_t larger = 0;
+      for (uint32_t j = 0; j < cnt; ++j) larger += sh_x[start + j] > x ? 1u : 0u;
+      return n_above + start + larger;
+    };
+    if constexpr (want_union) {
 #pragma unroll 1
-    for (uint32_t first = 0; first < n_own; first += kSelThreads) {
-      const uint32_t i = first + tid;
-      const bool valid = i < n_own;
-      uint64_t x = 0ull;
-      uint32_t rank = 0;
-      if (valid) {
-        x = sh_x[i];
-        const uint32_t bin = (uint32_t)((x - base) >> shift);
-        const uint32_t start = sh_off[bin], cnt = sh_hist[bin];
-        uint32_t larger = 0;
-        for (uint32_t j = 0; j < cnt; ++j) larger += sh_x[start + j] > x ? 1u : 0u;
-        rank = n_above + start + larger;
+      for (uint32_t first = 0; first < n_own; first += kSelThreads) {   // (every thread takes every round: emit scans)
+        const uint32_t i = first + tid;
+        const bool valid = i < n_own;
+        const uint64_t x = valid ? sh_x[i] : 0ull;
+        emit(valid, valid ? rank_of(x) : 0u, x);
       }
-      emit(valid, rank, x);
+    } else {
+#pragma unroll 1
+      for (uint32_t i = tid; i < n_own; i += kSelThreads) {
+        const uint64_t x = sh_x[i];
+        const uint32_t rank = rank_of(x);
+        if (rank < k) write_ranked(p, seg, idx_base, rank, x);
+      }
     }
   }
   // the workgroup whose part holds rank k - 1 knows how long the middle part is
@@ -1626,21 +1660,18 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
       !p.list_cnt || !p.cut_splits || (p.union_idx && !p.union_count))
     return TKA_EINVAL;
   const int lds = 2 * kCutMaxCandidates * (int)sizeof(uint64_t);
-  const void* kernels[4] = {(const void*)select_rank_kernel<TKA_F16, 4>, (const void*)select_rank_kernel<TKA_F16, 8>,
-                            (const void*)select_rank_kernel<TKA_BF16, 4>, (const void*)select_rank_kernel<TKA_BF16, 8>};
-  for (const void* kn : kernels)
-    if (allow_dynamic_lds(kn, lds) != TKA_OK) return TKA_EHIP;
+  typedef void (*RankKernel)(GemvParams, SelectParams, int);
+  static const RankKernel kernels[2][2][2] = {   // [dtype][more than 8 head entries per thread][union list]
+      {{select_rank_kernel<TKA_F16, 4, false>, select_rank_kernel<TKA_F16, 4, true>},
+       {select_rank_kernel<TKA_F16, 8, false>, select_rank_kernel<TKA_F16, 8, true>}},
+      {{select_rank_kernel<TKA_BF16, 4, false>, select_rank_kernel<TKA_BF16, 4, true>},
+       {select_rank_kernel<TKA_BF16, 8, false>, select_rank_kernel<TKA_BF16, 8, true>}}};
+  const bool wide = p.parts * kCutHead > 8 * kSelThreads;
+  const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0][p.union_idx ? 1 : 0];
+  if (allow_dynamic_lds((const void*)kernel, lds) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("select_rank", stream);
   const unsigned wgs = (unsigned)p.num_segments * kCutParts;
-  const int kpad = kpad_for(p.k);
-  const bool wide = p.parts * kCutHead > 8 * kSelThreads;   // more head entries than 8 per thread
-  if (dtype == TKA_F16) {
-    if (wide) select_rank_kernel<TKA_F16, 8><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
-    else select_rank_kernel<TKA_F16, 4><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
-  } else {
-    if (wide) select_rank_kernel<TKA_BF16, 8><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
-    else select_rank_kernel<TKA_BF16, 4><<<wgs, kSelThreads, lds, stream>>>(g, p, kpad);
-  }
+  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(kSelThreads), lds, stream, g, p, kpad_for(p.k));
   return hip_status(hipGetLastError());
 }
 
