@@ -74,7 +74,8 @@ class SparseDecode:
     """c4 (and a small variant): the end-to-end step."""
 
     def __init__(self, torch, ops, dev, batch=8, hkv=8, group=4, seq_len=131072, k=2048, sink=64, local=512,
-                 dtype="float16", out_dtype="bfloat16", heavy=0.01, seed=4, name="c4", num_splits=0, levels=False):
+                 dtype="float16", out_dtype="bfloat16", heavy=0.01, seed=4, name="c4", num_splits=0, levels=False,
+                 want_union=True):
         self.torch, self.name = torch, name
         g = torch.Generator(device=dev)
         g.manual_seed(seed)
@@ -96,6 +97,14 @@ class SparseDecode:
         # output (a sort per KV head) is not requested
         self.plan = ops.SparseDecodePlan(self.q, self.K, self.V, k, sink, local, SCALE, G,
                                          out_dtype=getattr(torch, out_dtype), num_splits=num_splits, want_topk=False)
+        self.selected = None
+        if not want_union:
+            # the caller that only wants the attention output: the step hands its token list on in the order of its route;
+            # the size of the list (for the byte count) comes from one step of the plan above
+            self.plan.step()
+            self.selected = int(self.plan.union_count.sum().item())
+            self.plan = ops.SparseDecodePlan(self.q, self.K, self.V, k, sink, local, SCALE, G, out_dtype=getattr(torch, out_dtype),
+                                             num_splits=num_splits, want_topk=False, want_union=False)
         self.desc = "%s: B=%d Hq=%d Hkv=%d D=128 N=%d %s k=%d sink=%d local=%d out=%s" % (
             name, B, H * G, H, N, dtype, k, sink, local, out_dtype)
         self.dominant = "gemv_scores"
@@ -107,7 +116,7 @@ class SparseDecode:
         return self.plan.redone_segments()
 
     def bytes(self):
-        sel = int(self.plan.union_count.sum().item())
+        sel = self.selected if self.selected is not None else int(self.plan.union_count.sum().item())
         gemv = self.B * self.N * self.H * 128 * 2
         sparse = sel * 128 * 2 * 2 + sel * 4 * 2          # gathered K and V rows, index lists written + read
         qo = self.B * self.H * self.G * 128 * 4           # q read, out written (2 bytes each)
@@ -130,16 +139,16 @@ class SparseDecode:
         # sanity (not the parity oracle): same selected sets, outputs close
         N, H = self.N, self.H
         lo, hi = min(self.sink, N), max(N - self.local, min(self.sink, N))
-        same_sets = True
-        for h in range(H):
+        same_sets = None   # (a plan that is not asked for the list has none to compare)
+        for h in range(H if self.plan.union_idx is not None else 0):
             want = set(range(lo)) | set(range(hi, N)) | set(ref_top[h].tolist())
             got = self.plan.union_idx[0, h, :int(self.plan.union_count[0, h])].tolist()
-            same_sets = same_sets and got == sorted(want)
+            same_sets = same_sets is not False and got == sorted(want)
         max_err = (self.plan.out[0].float().cpu() - ref_out).abs().max().item()
         return cpu_s, {"cores": torch.get_num_threads(), "host_cpus": os.cpu_count(), "cpu_model": cpu_model(), "kind": "port",
                        "sample": "batch entry 0 of %d (all %d KV heads, full N=%d), median of %d runs, scaled x%d" % (
                            self.B, H, N, runs, self.B),
-                       "union_sets_equal_gpu": bool(same_sets), "out_max_abs_diff_vs_gpu": round(max_err, 5)}
+                       "union_sets_equal_gpu": same_sets, "out_max_abs_diff_vs_gpu": round(max_err, 5)}
 
 
 class GemvTopk:
@@ -285,6 +294,8 @@ def build_workload(name, torch, ops, dev, args):
         return SparseDecode(torch, ops, dev, num_splits=args.splits)
     if name == "c4-small":
         return SparseDecode(torch, ops, dev, batch=2, seq_len=16384, name="c4-small")
+    if name == "c4-share32k":   # one GPU's share of an 8-way head-sharded model, one sequence of 32768 tokens, output only
+        return SparseDecode(torch, ops, dev, batch=1, hkv=1, group=8, seq_len=32768, name="c4-share32k", want_union=False)
     if name == "c1":
         return GemvTopk(torch, ops, dev, 1, 1, 1, 32768, 2048, "float16", 1, "c1", rotate=args.rotate)
     if name == "c2":
@@ -338,7 +349,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c5", "c5-topk", "ra", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c4-share32k", "c5", "c5-topk", "ra", "copy"])
     ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--score-mode", type=int, default=0, choices=[0, 1],
