@@ -138,8 +138,8 @@ typedef struct tka_test_hooks {
   int32_t tau_withhold_mode;   /* ... 0: for good (every slice of the segment gives up); 1: until the
                                   first slice of the segment has given up (the later ones see it)       */
   int32_t union_handoff_order; /* 1: tka_sparse_decode_step writes out_union_idx the way it hands the list to
-                                  its attention when the caller does not ask for it: the selected tokens
-                                  between the sink range and the local window in the order of the route */
+                                  its attention when the caller does not ask for it: in the order of the
+                                  route, which may list -1 (an id the attention skips) inside the count  */
 } tka_test_hooks;
 int tka_set_test_hooks(const tka_test_hooks* hooks);
 
@@ -369,7 +369,7 @@ typedef struct tka_sparse_decode_args {
   int32_t* out_topk_idx;  /* device [batch][num_kv_heads][k] rank order; may be NULL (saves a sort) */
   float* out_topk_val;    /* device, same shape; may be NULL; needs out_topk_idx              */
   int32_t* out_union_idx; /* device [batch][num_kv_heads][k+sink+local], ascending, -1 behind the count; may be NULL
-                             (the step then hands the tokens to the attention in whatever order its route selects them) */
+                             (the step then hands the tokens to the attention in whatever form its route selects them) */
   int32_t* out_union_count;/* device [batch][num_kv_heads]; may be NULL                       */
   void* workspace;
   size_t workspace_bytes;

@@ -449,8 +449,10 @@ def hooks():
 def test_sparse_decode_step_handoff_order(hooks, dtype, B, H, G, N, k, sink, local, kind, want_topk, cut):
     """A step that is not asked for its union list hands the tokens to the attention in the order of its route: for a few
     segments of 8193 .. 65536 tokens the ranking workgroups of the common-cut route write the middle part themselves, part
-    after part.  The union_handoff_order hook makes that list visible: as a set it must be the oracle's, sink range
-    first, local window last, -1 behind the count; rank-ordered top-k (when asked for) bit for bit; attention within tolerance."""
+    in rank order behind the sink range and the local window, with -1 in the place of a selected token that lies inside the
+    ranges (the attention skips such ids).  The union_handoff_order hook makes that list visible: without the -1 it must be
+    the oracle's as a set, and the oracle's top-k in rank order behind the ranges; -1 behind the count; rank-ordered top-k
+    output (when asked for) bit for bit; attention within tolerance."""
     from topk_attn_amd import ops
     announce("sparse_decode_step hand-off order dtype=%d B=%d H=%d G=%d N=%d k=%d sink=%d local=%d %s" % (dtype, B, H, G, N, k, sink, local, kind))
     hooks(union_handoff_order=1)
@@ -481,11 +483,17 @@ def test_sparse_decode_step_handoff_order(hooks, dtype, B, H, G, N, k, sink, loc
         for h in range(H):
             ro, ri, rv, ru = oracle.sparse_decode_step(q[b, h * G:(h + 1) * G], K[b, :, h], V[b, :, h], dtype, G, k, sink,
                                                        local, SCALE)
-            got = uidx[b, h]
-            assert ucnt[b, h] == len(ru), "union count differs (b=%d h=%d)" % (b, h)
-            assert np.array_equal(np.sort(got[:len(ru)]), ru), "union differs as a set (b=%d h=%d)" % (b, h)
-            assert np.array_equal(got[:lo], np.arange(lo)) and np.array_equal(got[len(ru) - (N - hi):len(ru)], np.arange(hi, N))
-            assert (got[len(ru):] == -1).all()
+            got, cnt = uidx[b, h], int(ucnt[b, h])
+            listed = got[:cnt]
+            assert np.array_equal(np.sort(listed[listed >= 0]), ru), "union differs as a set (b=%d h=%d)" % (b, h)
+            assert (got[cnt:] == -1).all()
+            if cut:   # this route: the two ranges, then a place per rank (-1 where the token lies inside the ranges)
+                assert cnt == lo + (N - hi) + k
+                assert np.array_equal(got[:lo], np.arange(lo)) and np.array_equal(got[lo:lo + N - hi], np.arange(hi, N))
+                mid = ri[(ri >= lo) & (ri < hi)]
+                assert np.array_equal(listed[lo + N - hi:][listed[lo + N - hi:] >= 0], mid), "rank order of the listed tokens"
+            else:
+                assert cnt == len(ru)
             if want_topk:
                 assert np.array_equal(plan.topk_idx[b, h].cpu().numpy(), ri), "top-k indices differ"
                 assert np.array_equal(plan.topk_val[b, h].cpu().numpy().view(np.uint32), rv.view(np.uint32))

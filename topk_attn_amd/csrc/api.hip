@@ -227,8 +227,8 @@ void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, 
   // (1 x 16384 rows, k = 1024: 12.9 / 18.4 us, 4 x 16384: 13.2 / 17.8, 8 x 16384, k = 512: 19.1 / 17.3; at 8192 rows the two are equal).
   if (chunk_len <= select_cand_capacity() && rows > kCutMaxRows / 4) return;
   // With the union list for the attention of a decode step (us per step, this route against the others): 1 x 32768 rows
-  // 25.6 / 32.2, 4 x 32768 34.7 / 37.5, 8 x 32768 46.5 / 43.7, 1 x 65536 28.9 / 34.5, 2 x 65536 42.1 / 36.0,
-  // 2 x 49152 (k = 1024) 32.5 / 32.7, 1 x 16384 (k = 1024) 23.7 / 22.5.
+  // 23.6 / 32.2, 4 x 32768 32.9 / 37.5, 1 x 65536 26.7 / 34.5; and where it is not taken 8 x 32768 about 45 / 43.7,
+  // 2 x 65536 about 40 / 36.0, 2 x 49152 (k = 1024) about 31 / 32.6, 1 x 16384 (k = 1024) about 22.3 / 22.5.
   if (u && (chunk_len <= select_cand_capacity() || rows > (chunk_len <= 32768 ? kCutMaxRows / 2 : kCutMaxRows / 4))) return;
   *num_samples = s;
   *sample_rank = r;

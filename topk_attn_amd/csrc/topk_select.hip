@@ -1020,14 +1020,13 @@ __device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_
 // send the part to the bitonic network; a segment with fewer than k candidates (the sample misjudged it), with a part
 // of more than kCutMaxCandidates or with more than kCutMaxExtras entries beyond the heads is redone from the keys by
 // its first workgroup (fallback_segment).
-// A caller that takes the selected tokens in any order (the attention of the decode step) gets the union list from the
-// same workgroups: sink range, then the selected tokens between the ranges - part after part, inside a part in the order
-// of its threads; a workgroup's first position is the number of candidates above its part less those of them inside
-// the ranges - then the local window, the count and the padding, written by the workgroup that holds rank k - 1.
+// A caller that takes the selected tokens in any order and skips ids outside the cache (the attention of the decode
+// step) gets the union list from the same workgroups: sink range and local window first, then one place per rank,
+// which holds the token, or -1 when the token lies inside the ranges (it is listed there).
 // Dynamic LDS: kCutMaxCandidates composites (the part, as found), then as many again (the part in bucket order;
 // before that, entries from beyond the heads); the tie path and the fallback reuse both.
-// PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256); UNION: the union list is written.
-template <int DT, int PAIRS, bool UNION>
+// PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256).
+template <int DT, int PAIRS>
 __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, SelectParams p, int kpad) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint64_t* sh_own = (uint64_t*)smem;
@@ -1040,8 +1039,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   __shared__ uint64_t sh_split[kCutParts + 1];
   __shared__ uint32_t sh_ovf[kCutMaxSlices];
   __shared__ uint32_t sh_n[8];   // [0] slices with more than kCutHead entries, [1] entries beyond the heads, [2] candidates,
-                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key,
-                                 // [7] candidates above the part inside the sink range or the local window (union list only)
+                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key
 
   typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
   constexpr int kPairs = PAIRS;
@@ -1164,31 +1162,6 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   }
   if (n_above >= k || n_own == 0u) return;   // nothing of this part is selected
 
-  // union list: tokens below `lo` (sink range) and from `hi` on (local window) are listed whether selected or not, so the
-  // selected ones among them do not count for the place of this part in the list
-  constexpr bool want_union = UNION;
-  const uint32_t lo = (uint32_t)(p.sink < p.seg_len ? p.sink : p.seg_len);
-  const uint32_t hi = (uint32_t)(p.seg_len - p.local > (int64_t)lo ? p.seg_len - p.local : (int64_t)lo);
-  if (want_union && part != 0) {
-    // (only the slices that reach into the range or the window can hold tokens of them)
-    const int lo_slices = (int)((lo + (uint32_t)kCutTokensPerWg - 1u) / (uint32_t)kCutTokensPerWg), hi_slice = (int)(hi / (uint32_t)kCutTokensPerWg);
-    uint32_t n_edge = 0;
-    auto edge = [&](uint64_t x) {
-      const uint32_t t = ~(uint32_t)x;
-      n_edge += x >= t_hi && (t < lo || t >= hi) ? 1u : 0u;
-    };
-#pragma unroll
-    for (int i = 0; i < kHeadMine; ++i) {
-      const int slice = ((i / 2) * kSelThreads + tid) / (kCutHead / 2);
-      if (slice < lo_slices || slice >= hi_slice) edge(c[i]);
-    }
-    if (n_ovf) {
-#pragma unroll
-      for (int i = kHeadMine; i < kMine; ++i) edge(c[i]);
-    }
-    if (n_edge) atomicAdd(&sh_n[7], n_edge);   // (read behind the barriers of the bucket scan)
-  }
-
   // buckets: linear in the composite between the ends of the part (the first part ends at its largest key)
   const uint64_t base = t_lo;
   const uint64_t span = (part == 0 ? (((uint64_t)sh_n[6] << 32) | 0xffffffffull) : t_hi) - base;
@@ -1215,20 +1188,28 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   }
   __syncthreads();
   const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len) : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
-  // what a ranked candidate leaves behind (every thread calls it once per round of the loops below: it scans over the
-  // workgroup when the union list is wanted)
+  // What a ranked candidate leaves behind.  The union list of this route: sink range [0, lo) and local window [hi, n)
+  // first, then one place per rank; a selected token that lies inside the ranges is listed there already, and its place
+  // holds -1, which the attention kernels skip like any id outside the cache.  So the place is the rank: nobody needs to
+  // know how many of the tokens above fall into the ranges.
+  const bool want_union = p.union_idx != nullptr;
+  const uint32_t lo = (uint32_t)(p.sink < p.seg_len ? p.sink : p.seg_len);
+  const uint32_t hi = (uint32_t)(p.seg_len - p.local > (int64_t)lo ? p.seg_len - p.local : (int64_t)lo);
+  const uint32_t edges = lo + ((uint32_t)p.seg_len - hi);
   int32_t* uo = want_union ? p.union_idx + (int64_t)seg * (p.k + p.sink + p.local) : nullptr;
-  uint32_t mid_at = lo + n_above - sh_n[7];   // next place of the middle part: every candidate above the part is selected
-  auto emit = [&](bool valid, uint32_t rank, uint64_t x) {
-    const bool sel = valid && rank < k;
-    if (sel && p.out_idx) write_ranked(p, seg, idx_base, rank, x);
+  if (want_union && part == 0) {
+    // the ranges, the count and the padding come from the first workgroup, which always gets this far (its part holds
+    // the first splitter)
+    for (uint32_t i = (uint32_t)tid; i < edges; i += kSelThreads) uo[i] = (int32_t)(i < lo ? i : hi + (i - lo));
+    for (uint32_t i = edges + k + (uint32_t)tid; i < (uint32_t)(p.k + p.sink + p.local); i += kSelThreads) uo[i] = -1;
+    if (tid == 0) p.union_count[seg] = (int32_t)(edges + k);
+  }
+  auto emit = [&](uint32_t rank, uint64_t x) {
+    if (rank >= k) return;
+    if (p.out_idx) write_ranked(p, seg, idx_base, rank, x);
     if (want_union) {
       const uint32_t t = ~(uint32_t)x;
-      const bool mid = sel && t >= lo && t < hi;
-      uint32_t total;
-      const uint32_t pos = block_exclusive_scan(mid ? 1u : 0u, sh_wtot, &total);
-      if (mid) uo[mid_at + pos] = (int32_t)t;
-      mid_at += total;
+      uo[edges + rank] = t >= lo && t < hi ? (int32_t)t : -1;
     }
   };
   if (sh_n[3] != 0u) {
@@ -1238,47 +1219,26 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     for (uint32_t i = n_own + tid; i < npad; i += kSelThreads) sh_own[i] = 0;   // pad: below every real composite
     __syncthreads();
     sort_lds_desc(sh_own, sh_x, (int)npad);
-    __syncthreads();
-#pragma unroll 1
-    for (uint32_t first = 0; first < n_own; first += kSelThreads) {
-      const uint32_t i = first + tid;
-      emit(i < n_own, n_above + i, i < n_own ? sh_own[i] : 0ull);
-    }
-  } else {
-#pragma unroll 1
-    for (uint32_t i = tid; i < n_own; i += kSelThreads) {
-      const uint64_t x = sh_own[i];
-      sh_x[atomicAdd(&sh_cur[(uint32_t)((x - base) >> shift)], 1u)] = x;
-    }
-    __syncthreads();
-    // every candidate of the part: its rank is the candidates above the part, plus the first rank of its bucket, plus the
-    // larger members of the bucket
-    auto rank_of = [&](uint64_t x) {
-      const uint32_t bin = (uint32_t)((x - base) >> shift);
-      const uint32_t start = sh_off[bin], cnt = sh_hist[bin];
-      uint32_t larger = 0;
-      for (uint32_t j = 0; j < cnt; ++j) larger += sh_x[start + j] > x ? 1u : 0u;
-      return n_above + start + larger;
-    };
-    if constexpr (want_union) {
-#pragma unroll 1
-      for (uint32_t first = 0; first < n_own; first += kSelThreads) {   // (every thread takes every round: emit scans)
-        const uint32_t i = first + tid;
-        const bool valid = i < n_own;
-        const uint64_t x = valid ? sh_x[i] : 0ull;
-        emit(valid, valid ? rank_of(x) : 0u, x);
-      }
-    } else {
-#pragma unroll 1
-      for (uint32_t i = tid; i < n_own; i += kSelThreads) {
-        const uint64_t x = sh_x[i];
-        const uint32_t rank = rank_of(x);
-        if (rank < k) write_ranked(p, seg, idx_base, rank, x);
-      }
-    }
+    for (uint32_t i = tid; i < n_own; i += kSelThreads) emit(n_above + i, sh_own[i]);
+    return;
   }
-  // the workgroup whose part holds rank k - 1 knows how long the middle part is
-  if (want_union && n_above + n_own >= k) write_union_edges(uo, p, seg, lo, hi, mid_at - lo);
+#pragma unroll 1
+  for (uint32_t i = tid; i < n_own; i += kSelThreads) {
+    const uint64_t x = sh_own[i];
+    sh_x[atomicAdd(&sh_cur[(uint32_t)((x - base) >> shift)], 1u)] = x;
+  }
+  __syncthreads();
+  // every candidate of the part: its rank is the candidates above the part, plus the first rank of its bucket, plus the
+  // larger members of the bucket
+#pragma unroll 1
+  for (uint32_t i = tid; i < n_own; i += kSelThreads) {
+    const uint64_t x = sh_x[i];
+    const uint32_t bin = (uint32_t)((x - base) >> shift);
+    const uint32_t start = sh_off[bin], cnt = sh_hist[bin];
+    uint32_t larger = 0;
+    for (uint32_t j = 0; j < cnt; ++j) larger += sh_x[start + j] > x ? 1u : 0u;
+    emit(n_above + start + larger, x);
+  }
 }
 
 // ---- a small k out of a few thousand scores, few segments -------------------------------------------------
@@ -1661,13 +1621,10 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
     return TKA_EINVAL;
   const int lds = 2 * kCutMaxCandidates * (int)sizeof(uint64_t);
   typedef void (*RankKernel)(GemvParams, SelectParams, int);
-  static const RankKernel kernels[2][2][2] = {   // [dtype][more than 8 head entries per thread][union list]
-      {{select_rank_kernel<TKA_F16, 4, false>, select_rank_kernel<TKA_F16, 4, true>},
-       {select_rank_kernel<TKA_F16, 8, false>, select_rank_kernel<TKA_F16, 8, true>}},
-      {{select_rank_kernel<TKA_BF16, 4, false>, select_rank_kernel<TKA_BF16, 4, true>},
-       {select_rank_kernel<TKA_BF16, 8, false>, select_rank_kernel<TKA_BF16, 8, true>}}};
+  static const RankKernel kernels[2][2] = {   // [dtype][more than 8 head entries per thread]
+      {select_rank_kernel<TKA_F16, 4>, select_rank_kernel<TKA_F16, 8>}, {select_rank_kernel<TKA_BF16, 4>, select_rank_kernel<TKA_BF16, 8>}};
   const bool wide = p.parts * kCutHead > 8 * kSelThreads;
-  const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0][p.union_idx ? 1 : 0];
+  const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0];
   if (allow_dynamic_lds((const void*)kernel, lds) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("select_rank", stream);
   const unsigned wgs = (unsigned)p.num_segments * kCutParts;
