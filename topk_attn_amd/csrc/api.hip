@@ -198,7 +198,8 @@ struct UnionOut {
   int32_t* idx;
   int32_t* count;
   int sink, local;
-  bool any_order;   // the selected tokens between the sink range and the local window may come in any order
+  bool handoff;     // the list only goes to the attention kernels: the selected tokens may come in any order, and -1 (an
+                    // id those kernels skip) may stand inside the count
 };
 
 // Samples per segment and rank of the cut when the call takes the common-cut route (a few segments of middling
@@ -214,7 +215,7 @@ int64_t cut_route_min_len() {
 void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, int* sample_rank) {
   *num_samples = *sample_rank = 0;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
-  if ((!a->out_idx && !u) || (u && !u->any_order) || a->out_scores || chunk_len < cut_route_min_len()) return;
+  if ((!a->out_idx && !u) || (u && !u->handoff) || a->out_scores || chunk_len < cut_route_min_len()) return;
   int s = 0, r = 0;
   gemv_cut_plan(chunk_len, a->k, &s, &r);
   if (s == 0) return;
@@ -1047,8 +1048,8 @@ static int sd_parts(const tka_sparse_decode_args* a, tka_gemv_topk_args* g, tka_
   return TKA_OK;
 }
 
-// The attention takes the selected tokens in any order; a caller that asks for the list gets it ascending.
-static bool sd_union_any_order(const tka_sparse_decode_args* a) { return !a->out_union_idx || current_hooks().union_handoff_order != 0; }
+// The attention takes the selected tokens in any order and skips -1; a caller that asks for the list gets it ascending and dense.
+static bool sd_union_handoff(const tka_sparse_decode_args* a) { return !a->out_union_idx || current_hooks().union_handoff_order != 0; }
 
 static int sd_check(const tka_sparse_decode_args* a, tka_gemv_topk_args* g, tka_flash_decode_args* f) {
   int rc = sd_parts(a, g, f);
@@ -1089,7 +1090,7 @@ int tka_sparse_decode_redone_segments(const tka_sparse_decode_args* a, int32_t* 
   if (!a->workspace || a->workspace_bytes < tka_sparse_decode_workspace_bytes(a)) return TKA_EWORKSPACE;
   g.workspace = (unsigned char*)a->workspace + sd_gemv_ws_offset(a, f);
   g.workspace_bytes = tka_gemv_topk_workspace_bytes(&g);
-  const UnionOut uo = {nullptr, nullptr, a->sink, a->local, sd_union_any_order(a)};
+  const UnionOut uo = {nullptr, nullptr, a->sink, a->local, sd_union_handoff(a)};
   return redone_segments(&g, &uo, count);
 }
 
@@ -1121,7 +1122,7 @@ int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
   g.out_val = a->out_topk_idx ? tval : nullptr;
   g.workspace = ws;
   g.workspace_bytes = gemv_ws;
-  UnionOut uo = {uidx, ucnt, a->sink, a->local, sd_union_any_order(a)};
+  UnionOut uo = {uidx, ucnt, a->sink, a->local, sd_union_handoff(a)};
   rc = run_gemv_topk(&g, nullptr, 0, nullptr, &uo);
   if (rc != TKA_OK) return rc;
   f.kv_idx = uidx;
