@@ -444,8 +444,10 @@ def hooks():
     (oracle.F16, 1, 1, 1, 65536, 2048, 0, 0, "heavy", False, True),            # no sink range, no window
     (oracle.F16, 1, 1, 4, 24000, 1400, 6000, 22000, "heavy", True, True),      # range and window overlap: nothing in between
     (oracle.BF16, 3, 1, 4, 20000, 1200, 1, 19990, "levels", False, True),      # the window covers nearly everything
-    (oracle.F16, 1, 2, 4, 24577, 3000, 300, 300, "heavy", False, False),       # k too large for that route: another one, same list
-    (oracle.F16, 2, 2, 4, 16384, 1024, 64, 512, "heavy", False, False)])       # short enough for the registers of a workgroup
+    (oracle.F16, 1, 2, 4, 24577, 3000, 300, 300, "heavy", False, False),       # k too large for that route: the dense path, ascending list
+    (oracle.F16, 2, 2, 4, 16384, 1024, 64, 512, "heavy", False, False),        # short enough for the registers of a workgroup
+    (oracle.BF16, 1, 3, 2, 5000, 700, 3000, 3000, "levels", True, False),      # the same with range and window overlapping, ties
+    (oracle.F16, 1, 2, 8, 3000, 100, 5, 9, "equal", False, False)])
 def test_sparse_decode_step_handoff_order(hooks, dtype, B, H, G, N, k, sink, local, kind, want_topk, cut):
     """A step that is not asked for its union list hands the tokens to the attention in the order of its route: for a few
     segments of 8193 .. 65536 tokens the ranking workgroups of the common-cut route write the middle part themselves, part
@@ -487,11 +489,13 @@ def test_sparse_decode_step_handoff_order(hooks, dtype, B, H, G, N, k, sink, loc
             listed = got[:cnt]
             assert np.array_equal(np.sort(listed[listed >= 0]), ru), "union differs as a set (b=%d h=%d)" % (b, h)
             assert (got[cnt:] == -1).all()
-            if cut:   # this route: the two ranges, then a place per rank (-1 where the token lies inside the ranges)
+            if cut or "select_wave" in kernels:
+                # these routes: the two ranges, then a place per selected token (-1 where it lies inside the ranges)
                 assert cnt == lo + (N - hi) + k
                 assert np.array_equal(got[:lo], np.arange(lo)) and np.array_equal(got[lo:lo + N - hi], np.arange(hi, N))
-                mid = ri[(ri >= lo) & (ri < hi)]
-                assert np.array_equal(listed[lo + N - hi:][listed[lo + N - hi:] >= 0], mid), "rank order of the listed tokens"
+                if cut:   # here the places are the ranks
+                    mid = ri[(ri >= lo) & (ri < hi)]
+                    assert np.array_equal(listed[lo + N - hi:][listed[lo + N - hi:] >= 0], mid), "rank order of the listed tokens"
             else:
                 assert cnt == len(ru)
             if want_topk:

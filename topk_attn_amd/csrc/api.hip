@@ -289,6 +289,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     sp.union_count = u->count;
     sp.sink = u->sink;
     sp.local = u->local;
+    sp.union_handoff = u->handoff ? 1 : 0;
   }
 
   GemvParams gp;

@@ -91,6 +91,8 @@ struct SelectParams {
   int segs_per_row;       // chunks per (batch, head): index base = (s % segs_per_row) * seg_len
   int expand;             // cluster_len of the expansion, 0 = none
   int sink, local;        // union mode
+  int union_handoff;      // the union list only goes to the attention kernels: any order, and -1 (an id they skip) may stand
+                          // inside the count (select_wave_kernel, select_rank_kernel)
   int unordered;          // select_wave kernel: out_idx / out_val need not be in rank order
 };
 size_t select_workspace_bytes(int num_segments, int64_t seg_len);

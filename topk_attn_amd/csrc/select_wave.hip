@@ -407,7 +407,30 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
     }
   }
 
-  if (p.union_idx) {
+  if (p.union_idx && p.union_handoff) {
+    // The list only goes to the attention kernels, which take any order and skip -1: sink range [0, lo) and local
+    // window [hi, n) first, then a place for each of the k selected tokens in the order of the threads (one scan instead
+    // of one per group of four registers), holding -1 when the token lies inside the ranges, where it is listed already.
+    const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
+    const uint32_t hi = (uint32_t)(n - p.local > (int)lo ? n - p.local : (int)lo);
+    const uint32_t edges = lo + ((uint32_t)n - hi);
+    const int cap = p.k + p.sink + p.local;
+    int32_t* uo = p.union_idx + (int64_t)seg * cap;
+    const uint32_t mine = ws_count<W, EPT>(rel, tid, selected);
+    uint32_t pos = edges + ws_exclusive<W>(mine, tid, sh);
+    const uint32_t not_t0 = ~(uint32_t)(4 * tid);
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const uint32_t not_t = not_t0 - ws_token_base(e, W);
+      if (selected(rel[e], not_t)) {
+        const uint32_t t = ~not_t;
+        uo[pos++] = t >= lo && t < hi ? (int32_t)t : -1;
+      }
+    }
+    for (uint32_t i = tid; i < edges; i += T) uo[i] = (int32_t)(i < lo ? i : hi + (i - lo));
+    for (uint32_t i = edges + k + tid; i < (uint32_t)cap; i += T) uo[i] = -1;
+    if (tid == 0) p.union_count[seg] = (int32_t)(edges + k);
+  } else if (p.union_idx) {
     // ascending union with the sink range [0, lo) and the local window [hi, n): the selected tokens between them,
     // in token order (register group, thread, register), then the two ranges, -1 padding and the count
     const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
