@@ -1025,8 +1025,9 @@ __device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_
 // which holds the token, or -1 when the token lies inside the ranges (it is listed there).
 // Dynamic LDS: kCutMaxCandidates composites (the part, as found), then as many again (the part in bucket order;
 // before that, entries from beyond the heads); the tie path and the fallback reuse both.
-// PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256).
-template <int DT, int PAIRS>
+// PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256); UNION: the union list is written (the
+// rank-ordered outputs then only if asked for).
+template <int DT, int PAIRS, bool UNION>
 __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, SelectParams p, int kpad) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint64_t* sh_own = (uint64_t*)smem;
@@ -1192,7 +1193,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   // first, then one place per rank; a selected token that lies inside the ranges is listed there already, and its place
   // holds -1, which the attention kernels skip like any id outside the cache.  So the place is the rank: nobody needs to
   // know how many of the tokens above fall into the ranges.
-  const bool want_union = p.union_idx != nullptr;
+  constexpr bool want_union = UNION;
   const uint32_t lo = (uint32_t)(p.sink < p.seg_len ? p.sink : p.seg_len);
   const uint32_t hi = (uint32_t)(p.seg_len - p.local > (int64_t)lo ? p.seg_len - p.local : (int64_t)lo);
   const uint32_t edges = lo + ((uint32_t)p.seg_len - hi);
@@ -1206,7 +1207,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   }
   auto emit = [&](uint32_t rank, uint64_t x) {
     if (rank >= k) return;
-    if (p.out_idx) write_ranked(p, seg, idx_base, rank, x);
+    if (!want_union || p.out_idx) write_ranked(p, seg, idx_base, rank, x);
     if (want_union) {
       const uint32_t t = ~(uint32_t)x;
       uo[edges + rank] = t >= lo && t < hi ? (int32_t)t : -1;
@@ -1621,10 +1622,13 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
     return TKA_EINVAL;
   const int lds = 2 * kCutMaxCandidates * (int)sizeof(uint64_t);
   typedef void (*RankKernel)(GemvParams, SelectParams, int);
-  static const RankKernel kernels[2][2] = {   // [dtype][more than 8 head entries per thread]
-      {select_rank_kernel<TKA_F16, 4>, select_rank_kernel<TKA_F16, 8>}, {select_rank_kernel<TKA_BF16, 4>, select_rank_kernel<TKA_BF16, 8>}};
+  static const RankKernel kernels[2][2][2] = {   // [dtype][more than 8 head entries per thread][union list]
+      {{select_rank_kernel<TKA_F16, 4, false>, select_rank_kernel<TKA_F16, 4, true>},
+       {select_rank_kernel<TKA_F16, 8, false>, select_rank_kernel<TKA_F16, 8, true>}},
+      {{select_rank_kernel<TKA_BF16, 4, false>, select_rank_kernel<TKA_BF16, 4, true>},
+       {select_rank_kernel<TKA_BF16, 8, false>, select_rank_kernel<TKA_BF16, 8, true>}}};
   const bool wide = p.parts * kCutHead > 8 * kSelThreads;
-  const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0];
+  const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0][p.union_idx ? 1 : 0];
   if (allow_dynamic_lds((const void*)kernel, lds) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("select_rank", stream);
   const unsigned wgs = (unsigned)p.num_segments * kCutParts;
