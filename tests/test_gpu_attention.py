@@ -444,6 +444,8 @@ def hooks():
     (oracle.F16, 1, 1, 1, 65536, 2048, 0, 0, "heavy", False, True),            # no sink range, no window
     (oracle.F16, 1, 1, 4, 24000, 1400, 6000, 22000, "heavy", True, True),      # range and window overlap: nothing in between
     (oracle.BF16, 3, 1, 4, 20000, 1200, 1, 19990, "levels", False, True),      # the window covers nearly everything
+    (oracle.F16, 1, 8, 4, 32768, 2048, 64, 512, "heavy", False, True),         # more than 65536 rows: the route in three launches
+    (oracle.BF16, 2, 4, 2, 20001, 1000, 100, 300, "levels", True, True),
     (oracle.F16, 1, 2, 4, 24577, 3000, 300, 300, "heavy", False, False),       # k too large for that route: the dense path, ascending list
     (oracle.F16, 2, 2, 4, 16384, 1024, 64, 512, "heavy", False, False),        # short enough for the registers of a workgroup
     (oracle.BF16, 1, 3, 2, 5000, 700, 3000, 3000, "levels", True, False),      # the same with range and window overlapping, ties
@@ -476,7 +478,7 @@ def test_sparse_decode_step_handoff_order(hooks, dtype, B, H, G, N, k, sink, loc
     kernels = ops.profile_read()
     ops.profile_enable(False)
     if cut:
-        assert "gemv_cut" in kernels and "select_rank" in kernels, "not the common-cut route: %s" % sorted(kernels)
+        assert ("gemv_cut" in kernels or "gemv_cut_slices" in kernels) and "select_rank" in kernels, "not the common-cut route: %s" % sorted(kernels)
         assert plan.redone_segments() == 0
     out, uidx, ucnt = f32_of(plan.out), plan.union_idx.cpu().numpy(), plan.union_count.cpu().numpy()
     lo = min(sink, N)

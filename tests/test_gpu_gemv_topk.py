@@ -427,12 +427,16 @@ def test_long_segment_threshold_never_published(hooks, withheld):
 @pytest.mark.parametrize("dtype,B,H,G,N,k", [(oracle.F16, 1, 1, 1, 32768, 2048), (oracle.BF16, 1, 2, 4, 20011, 1000),
                                              (oracle.F16, 2, 2, 1, 65536, 2048), (oracle.F16, 1, 1, 8, 40000, 1),
                                              (oracle.BF16, 1, 3, 2, 16385, 2048), (oracle.F16, 1, 2, 1, 12000, 400),
-                                             (oracle.BF16, 2, 2, 4, 8193, 300)])
+                                             (oracle.BF16, 2, 2, 4, 8193, 300),
+                                             # more than 65536 rows: the cut from a launch of its own, 512 tokens per GEMV workgroup
+                                             (oracle.F16, 1, 4, 1, 32768, 2048), (oracle.BF16, 2, 3, 2, 20001, 1000),
+                                             (oracle.F16, 1, 8, 4, 49152, 1500), (oracle.F16, 3, 1, 1, 30000, 7)])
 def test_common_cut_route(dtype, B, H, G, N, k):
-    """Calls of up to 262144 rows with segments of 16385 .. 65536 tokens (from 8193 tokens on calls of up to 65536 rows) and
-    no score output: every GEMV workgroup
-    derives the same cut from 256 sample rows, eight ranking workgroups per segment rank the candidates.  Ordinary
-    data with heavy hitters; no segment is redone from the keys."""
+    """Calls of up to 524288 rows with segments of 16385 .. 65536 tokens (from 8193 tokens on calls of up to 65536 rows) and
+    no score output: the cut of a segment comes from 256 sample rows - every GEMV workgroup derives the same one, or, on
+    calls of more than 65536 rows, one workgroup per segment does in a launch before the GEMV - and eight ranking
+    workgroups per segment rank the candidates.  Ordinary data with heavy hitters; ragged lengths (an odd number of
+    slices of 256 tokens); no segment is redone from the keys."""
     announce("gemv_topk common-cut route dtype=%d B=%d H=%d G=%d N=%d k=%d" % (dtype, B, H, G, N, k))
     rng = np.random.default_rng(51)
     K = randn_bits(rng, (B, N, H, 128), dtype)
@@ -440,12 +444,14 @@ def test_common_cut_route(dtype, B, H, G, N, k):
     _check_long(K, randn_bits(rng, (B, H * G, 128), dtype), dtype, G, k, redone=0)
 
 
+@pytest.mark.parametrize("heads", [1, 3])
 @pytest.mark.parametrize("kind", ["levels", "all_equal", "two_buckets", "ramp", "tail_block"])
-def test_common_cut_route_ties_and_clusters(kind):
+def test_common_cut_route_ties_and_clusters(kind, heads):
     """Ties (16-level keys, constant keys, three-valued scores with the k-th inside a bucket of thousands of equal
     scores) and top scores that sit in one place (a ramp over the tokens; all of the top k in the last tokens, so
-    that their slices hold more candidates than the ranking kernel reads in its first round trip)."""
-    announce("gemv_topk common-cut route, %s" % kind)
+    that their slices hold more candidates than the ranking kernel reads in its first round trip).  With three heads
+    (the same keys in each) the call has more than 65536 rows and finds its cuts in a launch of their own."""
+    announce("gemv_topk common-cut route, %s, %d head(s)" % (kind, heads))
     rng = np.random.default_rng(52)
     dtype, N, k = oracle.F16, 32768, 2048
     q = randn_bits(rng, (1, 1, 128), dtype)
@@ -468,6 +474,8 @@ def test_common_cut_route_ties_and_clusters(kind):
         qf = np.zeros((1, 1, 128))
         qf[0, 0, 5] = 1.0            # unit query: the score is one key column
         K, q = oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype)
+    if heads > 1:
+        K, q = np.ascontiguousarray(np.repeat(K, heads, axis=2)), np.ascontiguousarray(np.repeat(q, heads, axis=1))
     _check_long(K, q, dtype, 1, k, scale=1.0, redone=0)
 
 
@@ -487,6 +495,18 @@ def test_common_cut_route_adversarial_sample_falls_back():
     qf = rng.standard_normal((1, 2, 128))
     pos = _cut_sample_positions(0, N)
     Kf[0, pos, 0, :] = qf[0, 0] * rng.uniform(0.5, 1.5, (len(pos), 1))
+    _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k, redone=1)
+
+
+def test_common_cut_route_adversarial_sample_falls_back_in_three_launches():
+    """The same on a call of more than 65536 rows (four heads): the cut of head 2 comes out among the heavy tokens."""
+    announce("gemv_topk common-cut route in three launches, adversarial sample (fallback)")
+    rng = np.random.default_rng(57)
+    N, k, dtype = 32768, 2048, oracle.F16
+    Kf = rng.standard_normal((1, N, 4, 128)) * 0.05
+    qf = rng.standard_normal((1, 4, 128))
+    pos = _cut_sample_positions(2, N)
+    Kf[0, pos, 2, :] = qf[0, 2] * rng.uniform(0.5, 1.5, (len(pos), 1))
     _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k, redone=1)
 
 

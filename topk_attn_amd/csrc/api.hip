@@ -202,13 +202,25 @@ struct UnionOut {
                     // id those kernels skip) may stand inside the count
 };
 
-// Samples per segment and rank of the cut when the call takes the common-cut route (a few segments of middling
-// length; rank-ordered output, and the union list for a caller that takes its middle part in any order), else 0.  Shorter segments are selected from the registers of one workgroup, longer
-// ones (or many of them) by the sampling workgroups of the candidate route.
+// Samples per segment and rank of the cut when the call takes the common-cut route (segments of middling length on
+// calls of up to half a million rows; rank-ordered output, and the union list for a caller that only hands it to the
+// attention), else 0.  Shorter segments are selected from the registers of one workgroup, longer ones (or many of
+// them) by the sampling workgroups of the candidate route.
 int64_t cut_route_min_len() {
   static const int64_t v = [] {
     const char* e = getenv("TKA_CUT_MIN_LEN");
     return e && *e ? (int64_t)atoll(e) : (int64_t)select_cand_capacity() / 2 + 1;
+  }();
+  return v;
+}
+// Rows of a call beyond which the cut is found in a launch of its own (one workgroup per segment) instead of in every
+// GEMV workgroup: scoring the 256 sample rows beside every 256 tokens is free only while the launch does not fill the
+// GPU.  Decode steps, k = 2048, us per step in two / three launches: 1 x 32768 tokens 23.5 / 26.5, 2 x 32768 28.1 / 30.0,
+// 1 x 65536 26.3 / 29.5, 3 x 32768 29.3 / 26.8, 4 x 32768 31.3 / 27.7, 8 x 32768 43.0 / 36.2.
+int64_t cut_split_min_rows() {
+  static const int64_t v = [] {
+    const char* e = getenv("TKA_CUT_SPLIT_ROWS");
+    return e && *e ? (int64_t)atoll(e) : (int64_t)65536;
   }();
   return v;
 }
@@ -219,18 +231,22 @@ void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, 
   int s = 0, r = 0;
   gemv_cut_plan(chunk_len, a->k, &s, &r);
   if (s == 0) return;
-  // Every workgroup of this route scores the sample rows again, which is free while the launch does not fill the GPU.
-  // Measured (us per call, k = 2048, this route against the others): 1 x 32768 rows 13.6 / 25.1, 1 x 65536 15.8 / 31.6,
-  // 4 x 49152 29.0 / 35.0, 8 x 32768 32.9 / 35.9, 16 x 32768 56.4 / 47.3, 8 x 65536 60.0 / 45.8.
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
+  // Measured, decode steps with k = 2048 unless said (us per step, this route against the others): 1 x 32768 tokens
+  // 23.6 / 32.2, 4 x 32768 27.7 / 37.5, 8 x 32768 36.2 / 43.4, 16 x 32768 54.9 / 56.9, 24 x 32768 68.1 / 68.3,
+  // 4 x 49152 33.8 / 42.1, 8 x 49152 45.2 / 51.8, 16 x 20000 (k = 1000) 41.9 / 46.7, 32 x 20000 56.9 / 58.4.
   if (rows > kCutMaxRows) return;
-  // Segments that would also fit the registers of one workgroup (8193 .. 16384 rows): up to 65536 rows per call
-  // (1 x 16384 rows, k = 1024: 12.9 / 18.4 us, 4 x 16384: 13.2 / 17.8, 8 x 16384, k = 512: 19.1 / 17.3; at 8192 rows the two are equal).
-  if (chunk_len <= select_cand_capacity() && rows > kCutMaxRows / 4) return;
-  // With the union list for the attention of a decode step (us per step, this route against the others): 1 x 32768 rows
-  // 23.6 / 32.2, 4 x 32768 32.9 / 37.5, 1 x 65536 26.7 / 34.5; and where it is not taken 8 x 32768 about 45 / 43.7,
-  // 2 x 65536 about 40 / 36.0, 2 x 49152 (k = 1024) about 31 / 32.6, 1 x 16384 (k = 1024) about 22.3 / 22.5.
-  if (u && (chunk_len <= select_cand_capacity() || rows > (chunk_len <= 32768 ? kCutMaxRows / 2 : kCutMaxRows / 4))) return;
+  // Segments that would also fit the registers of one workgroup (8193 .. 16384 rows): rank-ordered output only, up to
+  // 65536 rows per call (1 x 16384 rows, k = 1024: 12.9 / 18.4 us per call, 4 x 16384: 13.2 / 17.8, 8 x 16384, k = 512:
+  // 19.1 / 17.3; at 8192 rows the two are equal; a decode step over 1 x 16384, k = 1024: about 22.3 / 22.5).
+  if (chunk_len <= select_cand_capacity() && (u || rows > 65536)) return;
+  // Segments that the candidate route takes as well (65536 tokens): that route from two segments on
+  // (decode steps: 1 x 65536 26.3 / 34.5, 2 x 65536 35.6 / 35.8, 8 x 65536 55.1 / 49.3).
+  if (rows > 65536) {
+    int cs = 0, cr = 0;
+    candidate_plan(a, &cs, &cr);
+    if (cs != 0) return;
+  }
   *num_samples = s;
   *sample_rank = r;
 }
@@ -315,7 +331,15 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     cp.cand_head = const_cast<uint64_t*>(sp.cand_head);
     cp.cand_count = sp.list_cnt;
     cp.cut_splits = (uint64_t*)sp.hist;   // (the histograms of the dense path: 8 KB per segment, free on this route)
-    int rc = launch_gemv_cut(cp, a->dtype, stream);
+    // a call that fills the GPU finds the cut in a launch of its own instead of in every GEMV workgroup
+    const int64_t rows = (int64_t)segs * chunk_len;
+    int rc;
+    if (rows > cut_split_min_rows()) {
+      rc = launch_cut_samples(cp, a->dtype, stream);
+      if (rc == TKA_OK) rc = launch_gemv_cut_slices(cp, a->dtype, stream);
+    } else {
+      rc = launch_gemv_cut(cp, a->dtype, stream);
+    }
     if (rc != TKA_OK) return rc;
     SelectParams sc = sp;
     sc.hist = nullptr;

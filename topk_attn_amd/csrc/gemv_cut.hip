@@ -23,6 +23,46 @@ namespace {
 constexpr int kCutThreads = 1024;
 constexpr int kCutUnroll = 8;                                        // rows per lane
 
+// Ranks of the S samples of a segment by counting, on 4 S threads (all threads of the workgroup call; sh_rank must be
+// zero and the keys in place behind a barrier): thread (s, q) counts the samples of block q (a quarter of them,
+// broadcast reads) that come before sample s, four threads per sample add up in LDS.  The order is that of the ranking
+// keys (the key with its last 8 bits replaced by S - 1 - sample number): all different, so one compare decides, exactly
+// one sample holds rank R - 1, and samples that share a key (heavy ties) come in token order, as in the full order (key
+// descending, token ascending).  Keys that differ in their last 8 bits only may change places; any sample will do as
+// the cut, it is its rank among the samples that makes the number of candidates what was planned.
+// The sample of rank R is the cut (sh_cut: its key and token); the samples of ranks R g / 8 split the candidates into
+// eight parts of about equal size for the ranking kernel's eight workgroups per segment, and go to `splits` as
+// composites when that is not null (the last one is the cut).  No barrier behind the last write.
+template <int S>
+__device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint32_t* sh_rkey, uint32_t* sh_rank, uint32_t* sh_cut, int seg,
+                                             int64_t stride, uint32_t rank, uint64_t* splits) {
+  const int tid = threadIdx.x;
+  if (tid < 4 * S) {
+    const int s = tid & (S - 1), q = tid / S;   // q is the same for a whole wave
+    const uint32_t ks = sh_rkey[s];
+    const u32x4* blk = (const u32x4*)(sh_rkey + q * (S / 4));
+    uint32_t ahead = 0;
+#pragma unroll
+    for (int i = 0; i < S / 16; ++i) {
+      const u32x4 kj = blk[i];
+      ahead += (kj[0] > ks ? 1u : 0u) + (kj[1] > ks ? 1u : 0u) + (kj[2] > ks ? 1u : 0u) + (kj[3] > ks ? 1u : 0u);
+    }
+    atomicAdd(&sh_rank[s], ahead);
+  }
+  __syncthreads();
+  if (tid < S) {
+    const uint32_t r = sh_rank[tid] + 1u;   // 1-based
+    uint32_t part = 0;   // 1 .. 8 when this sample ends part `part` of the candidates (8: the cut itself)
+#pragma unroll
+    for (uint32_t gq = 1; gq <= (uint32_t)kCutParts; ++gq) part = r == rank * gq / (uint32_t)kCutParts ? gq : part;
+    if (part != 0) {   // (R >= 8: every part has a sample of its own)
+      const uint32_t token = (uint32_t)sample_token(seg, tid, stride);
+      if (part == (uint32_t)kCutParts) { sh_cut[0] = sh_skey[tid]; sh_cut[1] = token; }
+      if (splits) splits[(int64_t)seg * kCutParts + (part - 1)] = composite(sh_skey[tid], token);
+    }
+  }
+}
+
 // Row groups 0 .. 31 score the 256 tokens of the slice, the row groups behind them the S sample tokens (S = 256:
 // sixteen waves), one round of eight loads per lane.
 // Many waves and a short program: few workgroups run at a time on these problems, so a wave pays the first fetch
@@ -83,38 +123,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   if (tid < kCutSamples) sh_rank[tid] = 0;
   __syncthreads();
 
-  // Rank of every sample by counting: thread (s, q) counts the samples of block q (a quarter of them, broadcast reads) that
-  // come before sample s, four threads per sample add up in LDS.  The order is that of the ranking keys (the key with
-  // its last 8 bits replaced by S - 1 - sample number): all different, so one compare decides, exactly one sample holds
-  // rank R - 1, and samples that share a key (heavy ties) come in token order, as in the full order (key descending,
-  // token ascending).  Keys that differ in their last 8 bits only may change places; any sample will do as the cut, it
-  // is its rank among the samples that makes the number of candidates what was planned.
-  // The samples of ranks R g / 8 - 1 split the candidates into eight parts of about equal size for the ranking
-  // kernel's eight workgroups per segment.
-  if (tid < 4 * kCutSamples) {
-    const int s = tid & (kCutSamples - 1), q = tid / kCutSamples;   // q is the same for a whole wave
-    const uint32_t ks = sh_rkey[s];
-    const u32x4* blk = (const u32x4*)(sh_rkey + q * (kCutSamples / 4));
-    uint32_t ahead = 0;
-#pragma unroll
-    for (int i = 0; i < kCutSamples / 16; ++i) {
-      const u32x4 kj = blk[i];
-      ahead += (kj[0] > ks ? 1u : 0u) + (kj[1] > ks ? 1u : 0u) + (kj[2] > ks ? 1u : 0u) + (kj[3] > ks ? 1u : 0u);
-    }
-    atomicAdd(&sh_rank[s], ahead);
-  }
-  __syncthreads();
-  if (tid < kCutSamples) {
-    const uint32_t r = sh_rank[tid] + 1u, rank = (uint32_t)p.sample_rank;   // 1-based
-    uint32_t part = 0;   // 1 .. 8 when this sample ends part `part` of the candidates (8: the cut itself)
-#pragma unroll
-    for (uint32_t gq = 1; gq <= (uint32_t)kCutParts; ++gq) part = r == rank * gq / (uint32_t)kCutParts ? gq : part;
-    if (part != 0) {   // (R >= 8: every part has a sample of its own)
-      const uint32_t token = (uint32_t)sample_token(seg, tid, stride);
-      if (part == (uint32_t)kCutParts) { sh_cut[0] = sh_key[kCutTokensPerWg + tid]; sh_cut[1] = token; }
-      if (slice == 0) p.cut_splits[(int64_t)seg * kCutParts + (part - 1)] = composite(sh_key[kCutTokensPerWg + tid], token);
-    }
-  }
+  rank_samples<S>(sh_key + kCutTokensPerWg, sh_rkey, sh_rank, sh_cut, seg, stride, (uint32_t)p.sample_rank, slice == 0 ? p.cut_splits : nullptr);
   __syncthreads();
   if (tid >= kCutTokensPerWg) return;
 
@@ -147,6 +156,125 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   if (tid == 0) p.cand_count[slice_id] = total;
 }
 
+
+// ---- the same route in three launches, for calls that fill the GPU ---------------------------------------------
+// When a call has more rows than a few CUs' worth, scoring the sample again in every workgroup doubles the work of the
+// launch.  Then one workgroup per segment finds the cut and the part ends first (cut_sample_kernel), and the GEMV
+// workgroups read them (gemv_cut_slices_kernel: 512 tokens, two slices, per workgroup, nothing scored twice).
+
+// One workgroup per segment: the 256 sample rows (64 row groups, four rows per lane), their ranks, cut and part ends.
+template <int DT>
+__global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
+  constexpr int S = 256, kRows = S / (kCutThreads / 16);   // four rows per lane
+  __shared__ uint32_t sh_skey[S];
+  __shared__ __attribute__((aligned(16))) uint32_t sh_rkey[S];
+  __shared__ uint32_t sh_rank[S];
+  __shared__ uint32_t sh_cut[2];
+  const int tid = threadIdx.x;
+  const int j = tid & 15, rg = tid >> 4;
+  const int seg = (int)blockIdx.x;
+  const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
+  const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
+  const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
+  const int64_t stride = p.chunk_len / S;
+  const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
+                          chunk_base * p.key_stride_n + 8 * j;
+  u32x4 kv[kRows];
+#pragma unroll
+  for (int u = 0; u < kRows; ++u) kv[u] = *(const u32x4*)(kbase + sample_token(seg, rg * kRows + u, stride) * p.key_stride_n);
+  __builtin_amdgcn_sched_barrier(0);
+  float qf[8];
+  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  __builtin_amdgcn_sched_barrier(0);
+  float mine = 0.0f;
+#pragma unroll
+  for (int u = 0; u < kRows; ++u) {
+    const float sc = row_score<DT>(qf, kv[u], p.scale);
+    if (j == u) mine = sc;
+  }
+  if (j < kRows) {
+    const int i = rg * kRows + j;
+    const uint32_t key = score_key(mine);
+    sh_skey[i] = key;
+    sh_rkey[i] = (key & ~0xffu) | (uint32_t)(S - 1 - i);
+  }
+  if (tid < S) sh_rank[tid] = 0;
+  __syncthreads();
+  rank_samples<S>(sh_skey, sh_rkey, sh_rank, sh_cut, seg, stride, (uint32_t)p.sample_rank, p.cut_splits);
+}
+
+// One workgroup per 512 tokens (two slices of the ranking kernel's layout): scores, and the tokens at or above the cut
+// that cut_sample_kernel left in p.cut_splits, stored as in gemv_cut_kernel.
+template <int DT>
+__global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams p) {
+  constexpr int kTokens = 2 * kCutTokensPerWg;
+  __shared__ uint32_t sh_key[kTokens];
+  __shared__ uint32_t sh_wcnt[kTokens / kWave];
+  const int tid = threadIdx.x;
+  const int j = tid & 15, rg = tid >> 4;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wgs_per_seg = (p.wgs_per_chunk + 1) / 2;   // p.wgs_per_chunk counts slices
+  const int pair = (int)(blockIdx.x % (uint32_t)wgs_per_seg);
+  const int seg = (int)(blockIdx.x / (uint32_t)wgs_per_seg);
+  const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
+  const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
+  const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
+  const int n = (int)p.chunk_len;
+  const int t_begin = pair * kTokens;
+  const int n_local = n - t_begin < kTokens ? n - t_begin : kTokens;
+
+  const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
+                          chunk_base * p.key_stride_n + 8 * j;
+  u32x4 kv[kCutUnroll];
+#pragma unroll
+  for (int u = 0; u < kCutUnroll; ++u) {
+    const int row = rg * kCutUnroll + u;
+    kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + (int64_t)(t_begin + (row < n_local ? row : n_local - 1)) * p.key_stride_n));
+  }
+  const uint64_t cut = p.cut_splits[(int64_t)seg * kCutParts + (kCutParts - 1)];   // (the same for all: a scalar load beside the rows)
+  __builtin_amdgcn_sched_barrier(0);
+  float qf[8];
+  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  __builtin_amdgcn_sched_barrier(0);
+  float mine = 0.0f;
+#pragma unroll
+  for (int u = 0; u < kCutUnroll; ++u) {
+    const float sc = row_score<DT>(qf, kv[u], p.scale);
+    if (j == u) mine = sc;
+  }
+  if (j < kCutUnroll) sh_key[rg * kCutUnroll + j] = score_key(mine);
+  __syncthreads();
+  if (tid >= kTokens) return;
+
+  // thread t owns token t_begin + t; waves 0 .. 3 make the first slice, waves 4 .. 7 the second
+  const int half = tid / kCutTokensPerWg, t_in = tid % kCutTokensPerWg;
+  const uint32_t token = (uint32_t)(t_begin + tid);
+  const uint64_t mine_c = composite(sh_key[tid], token);
+  const bool pass = tid < n_local && mine_c >= cut;
+  const unsigned long long mask = __ballot(pass);
+  if (lane == 0) sh_wcnt[wave] = (uint32_t)__popcll(mask);
+  __syncthreads();   // (the waves that have ended no longer count)
+  uint32_t ahead = 0, total = 0;
+#pragma unroll
+  for (int v = 0; v < kCutTokensPerWg / kWave; ++v) {
+    const int w = half * (kCutTokensPerWg / kWave) + v;
+    const uint32_t c = sh_wcnt[w];
+    ahead += w < wave ? c : 0u;
+    total += c;
+  }
+  const int slice = 2 * pair + half;
+  if (slice >= p.wgs_per_chunk) return;   // a segment with an odd number of slices: the last workgroup has one
+  const int64_t slice_id = (int64_t)seg * p.wgs_per_chunk + slice;
+  uint64_t* head = p.cand_head + slice_id * kCutHead;
+  uint64_t* wide = p.cand + (int64_t)seg * p.cand_seg_stride + (int64_t)slice * kCutTokensPerWg;
+  if (pass) {
+    const uint32_t pos = ahead + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+    (pos < (uint32_t)kCutHead ? head : wide)[pos] = mine_c;
+  }
+  if ((uint32_t)t_in >= total && t_in < kCutHead) head[t_in] = 0ull;
+  if (t_in == 0) p.cand_count[slice_id] = total;
+}
+
 }  // namespace
 
 int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
@@ -162,6 +290,33 @@ int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
     gemv_cut_kernel<TKA_F16, 256><<<wgs, threads, 0, stream>>>(p);
   else
     gemv_cut_kernel<TKA_BF16, 256><<<wgs, threads, 0, stream>>>(p);
+  return hip_status(hipGetLastError());
+}
+
+// The route in three launches (this one and the next, then launch_select_rank): same arguments and the same outputs
+// as launch_gemv_cut.
+int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream) {
+  const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
+  if (p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples || !p.cut_splits ||
+      segs > 0x7fffffffLL)
+    return TKA_EINVAL;
+  LaunchTimer timer("cut_sample", stream);
+  if (dtype == TKA_F16)
+    cut_sample_kernel<TKA_F16><<<(unsigned)segs, kCutThreads, 0, stream>>>(p);
+  else
+    cut_sample_kernel<TKA_BF16><<<(unsigned)segs, kCutThreads, 0, stream>>>(p);
+  return hip_status(hipGetLastError());
+}
+
+int launch_gemv_cut_slices(const GemvParams& p, int dtype, hipStream_t stream) {
+  const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
+  const int64_t wgs = segs * ((p.wgs_per_chunk + 1) / 2);
+  if (p.tokens_per_wg != kCutTokensPerWg || !p.cand || !p.cand_head || !p.cand_count || !p.cut_splits || wgs > 0x7fffffffLL) return TKA_EINVAL;
+  LaunchTimer timer("gemv_cut_slices", stream);
+  if (dtype == TKA_F16)
+    gemv_cut_slices_kernel<TKA_F16><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
+  else
+    gemv_cut_slices_kernel<TKA_BF16><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 
