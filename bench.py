@@ -294,6 +294,8 @@ def build_workload(name, torch, ops, dev, args):
         return SparseDecode(torch, ops, dev, num_splits=args.splits)
     if name == "c4-small":
         return SparseDecode(torch, ops, dev, batch=2, seq_len=16384, name="c4-small")
+    if name == "c4-b1-32k":     # one sequence of 32768 tokens on one GPU (all 8 KV heads), output only
+        return SparseDecode(torch, ops, dev, batch=1, seq_len=32768, name="c4-b1-32k", want_union=False)
     if name == "c4-share32k":   # one GPU's share of an 8-way head-sharded model, one sequence of 32768 tokens, output only
         return SparseDecode(torch, ops, dev, batch=1, hkv=1, group=8, seq_len=32768, name="c4-share32k", want_union=False)
     if name == "c1":
@@ -349,7 +351,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c4-share32k", "c5", "c5-topk", "ra", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c4-b1-32k", "c4-share32k", "c5", "c5-topk", "ra", "copy"])
     ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--score-mode", type=int, default=0, choices=[0, 1],
@@ -419,6 +421,8 @@ def main():
         dominant = "gemv_candidates"                    # long segments run the candidate-mode GEMV
     if dominant == "gemv_scores" and "gemv_cut" in kern:
         dominant = "gemv_cut"                           # a few segments of middling length: the common-cut GEMV
+    if dominant == "gemv_scores" and "gemv_cut_slices" in kern:
+        dominant = "gemv_cut_slices"                    # the same route on calls that fill the GPU
     dom_us = kern.get(dominant, ms_per_step * 1e3)     # a workload with one foreign kernel: the step itself
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     traffic, traffic_source = recorded_traffic(args.workload, dominant) if not args.splits else (None, None)
