@@ -224,6 +224,20 @@ int64_t cut_split_min_rows() {
   }();
   return v;
 }
+// Whether those cuts come from the first workgroups of the GEMV launch (the default) or from a launch before it.
+bool cut_front_sampling() {
+  static const bool v = [] {
+    const char* e = getenv("TKA_CUT_FRONT_SAMPLING");
+    return !(e && *e) || atoi(e) != 0;
+  }();
+  return v;
+}
+// Tells this call's words in a workspace from older contents: never 0, the cleared state; bit 30 stays free for the
+// "has a cut" mark of the candidate route's threshold words.
+uint32_t next_epoch() {
+  static std::atomic<uint32_t> call_counter{0};
+  return (call_counter.fetch_add(1, std::memory_order_relaxed) & ~kTauHasCut) | 0x80000000u;
+}
 void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, int* sample_rank) {
   *num_samples = *sample_rank = 0;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
@@ -335,14 +349,25 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     const int64_t rows = (int64_t)segs * chunk_len;
     int rc;
     if (rows > cut_split_min_rows()) {
-      rc = launch_cut_samples(cp, a->dtype, stream);
-      if (rc == TKA_OK) rc = launch_gemv_cut_slices(cp, a->dtype, stream);
+      if (cut_front_sampling()) {
+        const tka_test_hooks hooks = current_hooks();
+        cp.tau_words = sp.tau_words;
+        cp.epoch = next_epoch();
+        if (hooks.tau_spin_limit > 0) cp.tau_spin_limit = hooks.tau_spin_limit;
+        cp.withhold_mod = hooks.tau_withhold_mod > 0 ? hooks.tau_withhold_mod : 0;
+        cp.withhold_rem = hooks.tau_withhold_rem;
+        rc = launch_gemv_cut_slices(cp, a->dtype, true, stream);
+      } else {
+        rc = launch_cut_samples(cp, a->dtype, stream);
+        if (rc == TKA_OK) rc = launch_gemv_cut_slices(cp, a->dtype, false, stream);
+      }
     } else {
       rc = launch_gemv_cut(cp, a->dtype, stream);
     }
     if (rc != TKA_OK) return rc;
     SelectParams sc = sp;
     sc.hist = nullptr;
+    sc.tau_words = cp.tau_words;   // (set when the GEMV launch announced the cuts itself)
     sc.parts = cp.wgs_per_chunk;
     sc.part_len = kCutTokensPerWg;
     sc.max_entries = current_hooks().force_segment_redo ? 0 : kCutMaxSlices * kCutTokensPerWg;   // (no limit of its own)
@@ -405,7 +430,6 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // Long segments: sampled threshold, GEMV that stores candidates only, selection straight from the
   // candidate slices.  A segment whose candidates turn out too few (or too many) is redone from the keys by
   // its selection workgroup.
-  static std::atomic<uint32_t> call_counter{0};
   GemvParams cp = gp;
   cp.hist = nullptr;
   cp.tokens_per_wg = kGemvCandTokensPerWg;
@@ -413,8 +437,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   cp.tau_words = sp.tau_words;
   cp.sample_flags = sp.sample_flags;
   cp.sample_pool = sp.sample_pool;
-  // never 0, the cleared state; bit 30 stays free for the "has a cut" mark of the threshold words
-  cp.epoch = (call_counter.fetch_add(1, std::memory_order_relaxed) & ~kTauHasCut) | 0x80000000u;
+  cp.epoch = next_epoch();
   const tka_test_hooks hooks = current_hooks();
   cp.seg_flags = sp.seg_flags;
   if (hooks.tau_spin_limit > 0) cp.tau_spin_limit = hooks.tau_spin_limit;

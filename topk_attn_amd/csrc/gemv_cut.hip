@@ -33,7 +33,9 @@ constexpr int kCutUnroll = 8;                                        // rows per
 // The sample of rank R is the cut (sh_cut: its key and token); the samples of ranks R g / 8 split the candidates into
 // eight parts of about equal size for the ranking kernel's eight workgroups per segment, and go to `splits` as
 // composites when that is not null (the last one is the cut).  No barrier behind the last write.
-template <int S>
+// ANNOUNCED: other workgroups of the same launch are going to read `splits` (see gemv_cut_slices_kernel): the stores go
+// to where every CU sees them and have got there when this function returns.
+template <int S, bool ANNOUNCED = false>
 __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint32_t* sh_rkey, uint32_t* sh_rank, uint32_t* sh_cut, int seg,
                                              int64_t stride, uint32_t rank, uint64_t* splits) {
   const int tid = threadIdx.x;
@@ -58,7 +60,12 @@ __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint
     if (part != 0) {   // (R >= 8: every part has a sample of its own)
       const uint32_t token = (uint32_t)sample_token(seg, tid, stride);
       if (part == (uint32_t)kCutParts) { sh_cut[0] = sh_skey[tid]; sh_cut[1] = token; }
-      if (splits) splits[(int64_t)seg * kCutParts + (part - 1)] = composite(sh_skey[tid], token);
+      if (ANNOUNCED) {
+        __hip_atomic_store(splits + (int64_t)seg * kCutParts + (part - 1), composite(sh_skey[tid], token), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      } else if (splits) {
+        splits[(int64_t)seg * kCutParts + (part - 1)] = composite(sh_skey[tid], token);
+      }
     }
   }
 }
@@ -162,9 +169,10 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
 // launch.  Then one workgroup per segment finds the cut and the part ends first (cut_sample_kernel), and the GEMV
 // workgroups read them (gemv_cut_slices_kernel: 512 tokens, two slices, per workgroup, nothing scored twice).
 
-// One workgroup per segment: the 256 sample rows (64 row groups, four rows per lane), their ranks, cut and part ends.
-template <int DT>
-__global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
+// The work of one workgroup for one segment's cut: the 256 sample rows (64 row groups, four rows per lane), their
+// ranks, cut and part ends (to p.cut_splits).  Every thread of the 1024 calls it.
+template <int DT, bool ANNOUNCED>
+__device__ __forceinline__ void sample_segment(const GemvParams& p, int seg) {
   constexpr int S = 256, kRows = S / (kCutThreads / 16);   // four rows per lane
   __shared__ uint32_t sh_skey[S];
   __shared__ __attribute__((aligned(16))) uint32_t sh_rkey[S];
@@ -172,7 +180,6 @@ __global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
   __shared__ uint32_t sh_cut[2];
   const int tid = threadIdx.x;
   const int j = tid & 15, rg = tid >> 4;
-  const int seg = (int)blockIdx.x;
   const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
   const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
@@ -200,22 +207,49 @@ __global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
   }
   if (tid < S) sh_rank[tid] = 0;
   __syncthreads();
-  rank_samples<S>(sh_skey, sh_rkey, sh_rank, sh_cut, seg, stride, (uint32_t)p.sample_rank, p.cut_splits);
+  rank_samples<S, ANNOUNCED>(sh_skey, sh_rkey, sh_rank, sh_cut, seg, stride, (uint32_t)p.sample_rank, p.cut_splits);
 }
 
-// One workgroup per 512 tokens (two slices of the ranking kernel's layout): scores, and the tokens at or above the cut
-// that cut_sample_kernel left in p.cut_splits, stored as in gemv_cut_kernel.
+// One workgroup per segment, in a launch of its own.
 template <int DT>
+__global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
+  sample_segment<DT, false>(p, (int)blockIdx.x);
+}
+
+// One workgroup per 512 tokens (two slices of the ranking kernel's layout): scores, and the tokens at or above the
+// segment's cut in p.cut_splits, stored as in gemv_cut_kernel.
+// FRONT = false: the cuts are there (cut_sample_kernel ran before).  FRONT = true: the first workgroups of this launch, one
+// per segment, find them (sample_segment) while the others score their tokens; each publishes its cut and part ends and
+// then the call's epoch in the segment's word of p.tau_words, for which the first thread of a scoring workgroup waits
+// before the compare - a bounded wait: a workgroup that never sees the word marks its slices (kCutGaveUp in the count),
+// and the ranking kernel redoes such a segment from the keys.  The sampling workgroups come first in the grid, so they
+// run before any workgroup that waits for them; nothing depends on that but the speed.
+template <int DT, bool FRONT>
 __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams p) {
   constexpr int kTokens = 2 * kCutTokensPerWg;
   __shared__ uint32_t sh_key[kTokens];
   __shared__ uint32_t sh_wcnt[kTokens / kWave];
+  __shared__ uint64_t sh_cutc[2];   // the cut composite, whether it has arrived
   const int tid = threadIdx.x;
+  const int segs = p.batch * p.num_kv_heads * p.num_chunks;
+  if (FRONT && (int)blockIdx.x < segs) {
+    const int seg = (int)blockIdx.x;
+    __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
+    sample_segment<DT, true>(p, seg);
+    // the part ends have completed (rank_samples) before the word that announces them leaves; relaxed device-scope
+    // accesses on both sides, as for the thresholds of the candidate route: a fence would write back and invalidate
+    // whole caches in the middle of the stream
+    __syncthreads();
+    if (tid == 0 && !(p.withhold_mod > 0 && seg % p.withhold_mod == p.withhold_rem))   // (testing: this segment's word is withheld)
+      __hip_atomic_store(p.tau_words + 2 * seg, (uint64_t)p.epoch << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (the epoch where the candidate route keeps its own)
+    return;
+  }
+  const uint32_t wg = blockIdx.x - (FRONT ? (uint32_t)segs : 0u);
   const int j = tid & 15, rg = tid >> 4;
   const int lane = tid & 63, wave = tid >> 6;
   const int wgs_per_seg = (p.wgs_per_chunk + 1) / 2;   // p.wgs_per_chunk counts slices
-  const int pair = (int)(blockIdx.x % (uint32_t)wgs_per_seg);
-  const int seg = (int)(blockIdx.x / (uint32_t)wgs_per_seg);
+  const int pair = (int)(wg % (uint32_t)wgs_per_seg);
+  const int seg = (int)(wg / (uint32_t)wgs_per_seg);
   const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
   const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
@@ -231,7 +265,8 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
     const int row = rg * kCutUnroll + u;
     kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + (int64_t)(t_begin + (row < n_local ? row : n_local - 1)) * p.key_stride_n));
   }
-  const uint64_t cut = p.cut_splits[(int64_t)seg * kCutParts + (kCutParts - 1)];   // (the same for all: a scalar load beside the rows)
+  uint64_t cut = 0;
+  if (!FRONT) cut = p.cut_splits[(int64_t)seg * kCutParts + (kCutParts - 1)];   // (the same for all: a scalar load beside the rows)
   __builtin_amdgcn_sched_barrier(0);
   float qf[8];
   load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
@@ -243,14 +278,32 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
     if (j == u) mine = sc;
   }
   if (j < kCutUnroll) sh_key[rg * kCutUnroll + j] = score_key(mine);
+  bool have_cut = true;
+  if (FRONT) {
+    if (tid == 0) {
+      const uint64_t* word = p.tau_words + 2 * seg;
+      uint64_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int spin = 0; (uint32_t)(v >> 32) != p.epoch && spin < p.tau_spin_limit; ++spin) {
+        __builtin_amdgcn_s_sleep(16);
+        v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      const bool ok = (uint32_t)(v >> 32) == p.epoch;
+      sh_cutc[1] = ok ? 1ull : 0ull;
+      sh_cutc[0] = ok ? __hip_atomic_load(p.cut_splits + (int64_t)seg * kCutParts + (kCutParts - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : ~0ull;
+    }
+  }
   __syncthreads();
   if (tid >= kTokens) return;
+  if (FRONT) {
+    cut = sh_cutc[0];
+    have_cut = sh_cutc[1] != 0ull;
+  }
 
   // thread t owns token t_begin + t; waves 0 .. 3 make the first slice, waves 4 .. 7 the second
   const int half = tid / kCutTokensPerWg, t_in = tid % kCutTokensPerWg;
   const uint32_t token = (uint32_t)(t_begin + tid);
   const uint64_t mine_c = composite(sh_key[tid], token);
-  const bool pass = tid < n_local && mine_c >= cut;
+  const bool pass = have_cut && tid < n_local && mine_c >= cut;
   const unsigned long long mask = __ballot(pass);
   if (lane == 0) sh_wcnt[wave] = (uint32_t)__popcll(mask);
   __syncthreads();   // (the waves that have ended no longer count)
@@ -272,7 +325,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
     (pos < (uint32_t)kCutHead ? head : wide)[pos] = mine_c;
   }
   if ((uint32_t)t_in >= total && t_in < kCutHead) head[t_in] = 0ull;
-  if (t_in == 0) p.cand_count[slice_id] = total;
+  if (t_in == 0) p.cand_count[slice_id] = have_cut ? total : kCutGaveUp;
 }
 
 }  // namespace
@@ -308,15 +361,23 @@ int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream) {
   return hip_status(hipGetLastError());
 }
 
-int launch_gemv_cut_slices(const GemvParams& p, int dtype, hipStream_t stream) {
+// front_sampling: the cuts come from the first workgroups of this launch (p.tau_words, p.epoch, p.tau_spin_limit and the
+// sampling arguments of launch_cut_samples are then needed) instead of from a launch before it.
+int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  const int64_t wgs = segs * ((p.wgs_per_chunk + 1) / 2);
+  const int64_t wgs = segs * ((p.wgs_per_chunk + 1) / 2) + (front_sampling ? segs : 0);
   if (p.tokens_per_wg != kCutTokensPerWg || !p.cand || !p.cand_head || !p.cand_count || !p.cut_splits || wgs > 0x7fffffffLL) return TKA_EINVAL;
+  if (front_sampling && (p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
+                         !p.tau_words || p.epoch == 0 || p.tau_spin_limit < 1))
+    return TKA_EINVAL;
   LaunchTimer timer("gemv_cut_slices", stream);
-  if (dtype == TKA_F16)
-    gemv_cut_slices_kernel<TKA_F16><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
-  else
-    gemv_cut_slices_kernel<TKA_BF16><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
+  if (dtype == TKA_F16) {
+    if (front_sampling) gemv_cut_slices_kernel<TKA_F16, true><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
+    else gemv_cut_slices_kernel<TKA_F16, false><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
+  } else {
+    if (front_sampling) gemv_cut_slices_kernel<TKA_BF16, true><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
+    else gemv_cut_slices_kernel<TKA_BF16, false><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
+  }
   return hip_status(hipGetLastError());
 }
 

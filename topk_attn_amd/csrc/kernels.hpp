@@ -59,7 +59,7 @@ int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream);
 // The same in two launches for calls that fill the GPU: one workgroup per segment finds the cut and the part ends, then the
 // GEMV workgroups (512 tokens each) score nothing twice.
 int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream);
-int launch_gemv_cut_slices(const GemvParams& p, int dtype, hipStream_t stream);
+int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream);
 void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank);
 
 // ---- stage 1: selection -----------------------------------------------------------------------

@@ -1040,7 +1040,8 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   __shared__ uint64_t sh_split[kCutParts + 1];
   __shared__ uint32_t sh_ovf[kCutMaxSlices];
   __shared__ uint32_t sh_n[8];   // [0] slices with more than kCutHead entries, [1] entries beyond the heads, [2] candidates,
-                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key
+                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key,
+                                 // [7] a slice whose workgroup gave up waiting for the cut
 
   typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
   constexpr int kPairs = PAIRS;
@@ -1080,7 +1081,9 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   sh_hist[2 * tid + 1] = 0;
   if (tid < 8) sh_n[tid] = 0;
   __syncthreads();
-  if (slice_cnt > (uint32_t)kCutHead) sh_ovf[atomicAdd(&sh_n[0], 1u)] = (uint32_t)tid | (slice_cnt << 16);
+  // (p.tau_words: the cuts were announced inside the GEMV launch; the slice of a workgroup that never saw its segment's holds no candidates)
+  if (p.tau_words && slice_cnt == kCutGaveUp) sh_n[7] = 1u;
+  else if (slice_cnt > (uint32_t)kCutHead) sh_ovf[atomicAdd(&sh_n[0], 1u)] = (uint32_t)tid | (slice_cnt << 16);
   __syncthreads();
   const uint32_t n_ovf = sh_n[0];
   if (n_ovf) {   // rare: slices whose candidates go beyond the head entries (scores that cluster in one place)
@@ -1153,8 +1156,12 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   uint32_t max_part = n_own;
   if (n_cand > (uint32_t)kCutMaxCandidates)
     max_part = max(max_part, largest_part((const uint64_t*)heads, n_pairs, n_ovf ? sh_extra : nullptr, min(n_extra, (uint32_t)kCutMaxExtras), sh_split, sh_hist));
-  const bool redo = n_cand < k || n_cand > (uint32_t)p.max_entries || n_extra > (uint32_t)kCutMaxExtras || max_part > (uint32_t)kCutMaxCandidates;
-  if (tid == 0 && part == 0) p.seg_flags[seg] = redo ? 1u : 0u;
+  const bool redo = n_cand < k || n_cand > (uint32_t)p.max_entries || n_extra > (uint32_t)kCutMaxExtras || max_part > (uint32_t)kCutMaxCandidates ||
+                    sh_n[7] != 0u;
+  if (tid == 0 && part == 0) {
+    p.seg_flags[seg] = redo ? 1u : 0u;
+    if (p.tau_words) p.tau_words[2 * seg] = 0ull;   // the word that announced the segment's cut: spent (a replayed graph brings the same epoch)
+  }
   if (redo) {   // every workgroup of the segment sees the same counts: the first one redoes it, the others leave
     if (part != 0) return;
     __syncthreads();
@@ -1618,7 +1625,7 @@ int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int 
 
 int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
   if (p.parts < 1 || p.parts > kCutMaxSlices || p.part_len != kCutTokensPerWg || p.k > kCutMaxK || (!p.out_idx && !p.union_idx) || !p.cand_head ||
-      !p.list_cnt || !p.cut_splits || (p.union_idx && !p.union_count))
+      !p.list_cnt || !p.cut_splits || !p.seg_flags || (p.union_idx && !p.union_count))
     return TKA_EINVAL;
   const int lds = 2 * kCutMaxCandidates * (int)sizeof(uint64_t);
   typedef void (*RankKernel)(GemvParams, SelectParams, int);
