@@ -594,6 +594,53 @@ def test_sparse_decode_step_graph_replay():
         assert torch.equal(plan.out, want_out), "replay %d: outputs differ" % it
 
 
+def test_sparse_decode_step_graph_replay_cuts_announced_in_the_launch(hooks):
+    """The same for a step whose GEMV launch finds the cuts of its segments in its first workgroups and announces them
+    to the others (4 x 32768 tokens, output only): a replay brings the same epoch, so the word of one replay must be
+    spent before the next.  Top-k and hand-off list (made visible by the hook) bit for bit, output bit for bit, and no
+    segment redone."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step captured in a graph, 3 replays, cuts announced inside the GEMV launch (4 x 32768, k=2048)")
+    hooks(union_handoff_order=1)
+    rng = np.random.default_rng(79)
+    dtype, B, H, G, N, k, sink, local = oracle.F16, 1, 4, 4, 32768, 2048, 64, 512
+    q = to_dev(randn_bits(rng, (B, H * G, 128), dtype), dtype)
+    K, V = to_dev(randn_bits(rng, (B, N, H, 128), dtype), dtype), to_dev(randn_bits(rng, (B, N, H, 128), dtype), dtype)
+    plan = ops.SparseDecodePlan(q, K, V, k, sink, local, SCALE, G, out_dtype=torch.float16, want_topk=True)
+    ops.profile_reset()
+    ops.profile_enable(True)
+    plan.step()                      # warm-up outside the capture
+    torch.cuda.synchronize()
+    kernels = ops.profile_read()
+    ops.profile_enable(False)
+    assert "gemv_cut_slices" in kernels and "cut_sample" not in kernels, sorted(kernels)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        plan.step()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            plan.step()
+    torch.cuda.synchronize()
+    for it in range(3):
+        q.copy_(to_dev(oracle.to_bits(rng.standard_normal((B, H * G, 128)) * (1.0 + 0.5 * it), dtype), dtype))
+        plan.step()                  # eager, default stream
+        torch.cuda.synchronize()
+        assert plan.redone_segments() == 0
+        want = [t.clone() for t in (plan.out, plan.union_idx, plan.union_count, plan.topk_idx, plan.topk_val)]
+        plan.out.zero_()
+        plan.union_idx.fill_(-7)
+        plan.union_count.zero_()
+        plan.topk_idx.fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert plan.redone_segments() == 0, "replay %d: a segment was redone from the keys" % it
+        for got, ref, what in zip((plan.out, plan.union_idx, plan.union_count, plan.topk_idx, plan.topk_val), want,
+                                  ("outputs", "hand-off lists", "list counts", "top-k indices", "top-k values")):
+            assert torch.equal(got, ref), "replay %d: %s differ" % (it, what)
+
+
 def test_retrieval_attention_graph_replay():
     """The operator captured in a HIP graph (the batch path: shared-key scoring, small-workgroup selection,
     attention that writes the result itself) and replayed with new queries; every replay is compared with the
