@@ -10,6 +10,10 @@
 // k; the ranking kernel (select_rank_kernel) checks that and otherwise redoes the segment from the keys.  About
 // n R / 256 candidates per segment, see gemv_cut_plan.
 //
+// On calls that do fill the GPU (more than 65536 rows) the sample is scored once per segment instead: by the first
+// workgroups of the GEMV launch, whose cut the others wait for (gemv_cut_slices_kernel), or by a launch before it
+// (cut_sample_kernel).  Same cut, same slices, same ranking kernel.
+//
 // The scores are the canonical ones (gemv_topk.cu:303-332 of the reference: fma chain over the lane's 8 dims,
 // xor butterfly over 16 lanes, one multiply).
 #include <math.h>
@@ -164,10 +168,10 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
 }
 
 
-// ---- the same route in three launches, for calls that fill the GPU ---------------------------------------------
+// ---- the same route for calls that fill the GPU -----------------------------------------------------------------
 // When a call has more rows than a few CUs' worth, scoring the sample again in every workgroup doubles the work of the
-// launch.  Then one workgroup per segment finds the cut and the part ends first (cut_sample_kernel), and the GEMV
-// workgroups read them (gemv_cut_slices_kernel: 512 tokens, two slices, per workgroup, nothing scored twice).
+// launch.  Then one workgroup per segment finds the cut and the part ends (sample_segment), and the GEMV workgroups
+// read them (gemv_cut_slices_kernel: 512 tokens, two slices, per workgroup, nothing scored twice).
 
 // The work of one workgroup for one segment's cut: the 256 sample rows (64 row groups, four rows per lane), their
 // ranks, cut and part ends (to p.cut_splits).  Every thread of the 1024 calls it.
