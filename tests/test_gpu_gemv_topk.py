@@ -432,7 +432,7 @@ def test_long_segment_threshold_never_published(hooks, withheld):
                                              (oracle.F16, 1, 4, 1, 32768, 2048), (oracle.BF16, 2, 3, 2, 20001, 1000),
                                              (oracle.F16, 1, 8, 4, 49152, 1500), (oracle.F16, 3, 1, 1, 30000, 7)])
 def test_common_cut_route(dtype, B, H, G, N, k):
-    """Calls of up to 524288 rows with segments of 16385 .. 65536 tokens (from 8193 tokens on calls of up to 65536 rows) and
+    """Calls of up to 655360 rows with segments of 16385 .. 65536 tokens (from 8193 tokens on calls of up to 65536 rows) and
     no score output: the cut of a segment comes from 256 sample rows - every GEMV workgroup derives the same one, or, on
     calls of more than 65536 rows, one workgroup per segment does in a launch before the GEMV - and eight ranking
     workgroups per segment rank the candidates.  Ordinary data with heavy hitters; ragged lengths (an odd number of

@@ -203,7 +203,7 @@ struct UnionOut {
 };
 
 // Samples per segment and rank of the cut when the call takes the common-cut route (segments of middling length on
-// calls of up to half a million rows; rank-ordered output, and the union list for a caller that only hands it to the
+// calls of up to 655360 rows; rank-ordered output, and the union list for a caller that only hands it to the
 // attention), else 0.  Shorter segments are selected from the registers of one workgroup, longer ones (or many of
 // them) by the sampling workgroups of the candidate route.
 int64_t cut_route_min_len() {
@@ -247,8 +247,9 @@ void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, 
   if (s == 0) return;
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   // Measured, decode steps with k = 2048 unless said (us per step, this route against the others): 1 x 32768 tokens
-  // 23.6 / 32.2, 4 x 32768 27.7 / 37.5, 8 x 32768 36.2 / 43.4, 16 x 32768 54.9 / 56.9, 24 x 32768 68.1 / 68.3,
-  // 4 x 49152 33.8 / 42.1, 8 x 49152 45.2 / 51.8, 16 x 20000 (k = 1000) 41.9 / 46.7, 32 x 20000 56.9 / 58.4.
+  // 23.6 / 32.2, 4 x 32768 26.7 / 37.5, 8 x 32768 33.7 / 43.4, 16 x 32768 50.4 / 56.9, 24 x 32768 63.8 / 68.3,
+  // 8 x 49152 42.9 / 51.8, 16 x 20000 (k = 1000) 37.0 / 46.7, 32 x 20000 54.4 / 58.4, 32 x 24576 (k = 1536) 66.5 / 67.7,
+  // 40 x 20000 67.1 / 65.5, 48 x 20000 74.5 / 73.7.
   if (rows > kCutMaxRows) return;
   // Segments that would also fit the registers of one workgroup (8193 .. 16384 rows): rank-ordered output only, up to
   // 65536 rows per call (1 x 16384 rows, k = 1024: 12.9 / 18.4 us per call, 4 x 16384: 13.2 / 17.8, 8 x 16384, k = 512:
