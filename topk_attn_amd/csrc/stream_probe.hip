@@ -52,6 +52,30 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(8, 8)))
   if (acc == 0x12345678u) out[0] = acc;   // (keeps the loads alive; the buffer holds other values)
 }
 
+// The candidate GEMV's shape (512 threads, two rounds of eight loads per lane: a slice of 512 rows) with the last
+// `tail_slices` slices of the grid handled by two workgroups of one round each: does the end of a launch, where
+// workgroups that are out of step finish one by one, cost what shorter workgroups there would save?
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(8, 8))) void read_registers_split_tail(const unsigned char* p, int slices_per_head,
+                                                                                                              int full_slices, unsigned* out) {
+  constexpr int kRowsPerRound = 512 / 16 * 8;
+  const bool half = (int)blockIdx.x >= full_slices;
+  const int slice = half ? full_slices + ((int)blockIdx.x - full_slices) / 2 : (int)blockIdx.x;
+  const int first_round = half ? ((int)blockIdx.x - full_slices) % 2 : 0, rounds = half ? 1 : 2;
+  const int h = slice / slices_per_head, sl = slice % slices_per_head;
+  const int j = threadIdx.x & 15, rg = threadIdx.x >> 4;
+  const size_t stride = (size_t)kHeads * kRowBytes;
+  const unsigned char* base = p + (size_t)h * kRowBytes + (size_t)sl * (2 * kRowsPerRound) * stride + 16 * j;
+  unsigned acc = 0;
+  for (int it = first_round; it < first_round + rounds; ++it) {
+    u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load((const u32x4*)(base + (size_t)(it * kRowsPerRound + rg * 8 + u) * stride));
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  if (acc == 0x12345678u) out[0] = acc;
+}
+
 // Direct-to-LDS loads (global_load_lds_dwordx4): 256 threads, ROWS rows per workgroup (ROWS * 256 B of LDS), all loads
 // of a lane in flight at once, then one pass over the LDS copy.
 template <int ROWS>
@@ -114,6 +138,14 @@ void run_registers(const char* what) {
   std::printf("%-78s %8.1f us  %6.0f GB/s\n", what, us, g_bytes / us / 1e3);
 }
 
+void run_split_tail(int tail_slices, const char* what) {
+  const int sph = (int)(g_rows_per_head / 512), slices = kHeads * sph;
+  if (g_rows_per_head % 512 || tail_slices > slices) return;
+  const int full = slices - tail_slices;
+  const float us = time_us([&] { read_registers_split_tail<<<full + 2 * tail_slices, 512>>>(g_buf, sph, full, g_out); });
+  std::printf("%-78s %8.1f us  %6.0f GB/s\n", what, us, g_bytes / us / 1e3);
+}
+
 template <int ROWS>
 void run_lds(const char* what) {
   if (g_rows_per_head % ROWS) return;
@@ -154,6 +186,9 @@ int main(int argc, char** argv) {
   run_lds<128>("direct to LDS, 256 threads, 128 rows (32 KB)");
   run_lds<256>("direct to LDS, 256 threads, 256 rows (64 KB)");
   run_registers<512, 2, false, true>("512 threads, 2 rounds again");
+  run_split_tail(0, "512 threads, 2 rounds, the rounds as a loop that is not unrolled");
+  run_split_tail(1024, "  the same, the last 1024 slices (one resident set) as two workgroups of one round each");
+  run_split_tail(4096, "  the same, the last 4096 slices so");
   CK(hipFree(g_buf));
   CK(hipFree(g_out));
   return 0;
