@@ -121,7 +121,8 @@ int tka_gemv_scores(const tka_gemv_topk_args* args);
  * redone - exact, but about a millisecond per 131072 tokens.  0 for calls that do not take that path.
  * Waits for the stream. */
 int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* args, int32_t* count);
-/* Same protocol: *count = candidate slices (512 tokens each) of that call whose workgroup gave up waiting. */
+/* Same protocol: *count = candidate slices of that call (512 tokens each; 256 on calls that announce the cut of a
+ * segment of up to 65536 tokens inside the GEMV launch) whose workgroup gave up waiting. */
 int tka_gemv_topk_gave_up_slices(const tka_gemv_topk_args* args, int32_t* count);
 
 /* Testing hooks (no counterpart in the reference).  Process-wide; read once at the start of every call; they

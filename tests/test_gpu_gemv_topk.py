@@ -520,7 +520,7 @@ def test_common_cut_route_cut_never_announced(hooks, mod, rem, affected):
     hooks(tau_spin_limit=64, tau_withhold_mod=mod, tau_withhold_rem=rem, tau_withhold_mode=0)
     rng = np.random.default_rng(58)
     K = randn_bits(rng, (1, 32768, 4, 128), oracle.F16)
-    _check_long(K, randn_bits(rng, (1, 4, 128), oracle.F16), oracle.F16, 1, 2048, redone=affected)
+    _check_long(K, randn_bits(rng, (1, 4, 128), oracle.F16), oracle.F16, 1, 2048, redone=affected, gave_up=affected * 128)
 
 
 def test_common_cut_route_sample_sits_low():

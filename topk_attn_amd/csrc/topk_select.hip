@@ -1041,7 +1041,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   __shared__ uint32_t sh_ovf[kCutMaxSlices];
   __shared__ uint32_t sh_n[8];   // [0] slices with more than kCutHead entries, [1] entries beyond the heads, [2] candidates,
                                  // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key,
-                                 // [7] a slice whose workgroup gave up waiting for the cut
+                                 // [7] slices whose workgroup gave up waiting for the cut
 
   typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
   constexpr int kPairs = PAIRS;
@@ -1082,7 +1082,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   if (tid < 8) sh_n[tid] = 0;
   __syncthreads();
   // (p.tau_words: the cuts were announced inside the GEMV launch; the slice of a workgroup that never saw its segment's holds no candidates)
-  if (p.tau_words && slice_cnt == kCutGaveUp) sh_n[7] = 1u;
+  if (p.tau_words && slice_cnt == kCutGaveUp) atomicAdd(&sh_n[7], 1u);
   else if (slice_cnt > (uint32_t)kCutHead) sh_ovf[atomicAdd(&sh_n[0], 1u)] = (uint32_t)tid | (slice_cnt << 16);
   __syncthreads();
   const uint32_t n_ovf = sh_n[0];
@@ -1159,7 +1159,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   const bool redo = n_cand < k || n_cand > (uint32_t)p.max_entries || n_extra > (uint32_t)kCutMaxExtras || max_part > (uint32_t)kCutMaxCandidates ||
                     sh_n[7] != 0u;
   if (tid == 0 && part == 0) {
-    p.seg_flags[seg] = redo ? 1u : 0u;
+    p.seg_flags[seg] = (redo ? 1u : 0u) | (sh_n[7] << 8);   // (as on the candidate route: bit 0 redone, bits 8.. slices that gave up)
     if (p.tau_words) p.tau_words[2 * seg] = 0ull;   // the word that announced the segment's cut: spent (a replayed graph brings the same epoch)
   }
   if (redo) {   // every workgroup of the segment sees the same counts: the first one redoes it, the others leave
