@@ -430,7 +430,10 @@ def test_long_segment_threshold_never_published(hooks, withheld):
                                              (oracle.BF16, 2, 2, 4, 8193, 300),
                                              # more than 65536 rows: the cut from a launch of its own, 512 tokens per GEMV workgroup
                                              (oracle.F16, 1, 4, 1, 32768, 2048), (oracle.BF16, 2, 3, 2, 20001, 1000),
-                                             (oracle.F16, 1, 8, 4, 49152, 1500), (oracle.F16, 3, 1, 1, 30000, 7)])
+                                             (oracle.F16, 1, 8, 4, 49152, 1500), (oracle.F16, 3, 1, 1, 30000, 7),
+                                             # k above n / 14.5 (up to n / 8): slices of 128 tokens
+                                             (oracle.F16, 1, 1, 1, 20000, 2048), (oracle.BF16, 2, 1, 2, 16384, 2048),
+                                             (oracle.F16, 1, 8, 4, 24577, 2048), (oracle.BF16, 1, 3, 1, 32768, 2048 + 1000)])
 def test_common_cut_route(dtype, B, H, G, N, k):
     """Calls of up to 655360 rows with segments of 16385 .. 65536 tokens (from 8193 tokens on calls of up to 65536 rows) and
     no score output: the cut of a segment comes from 256 sample rows - every GEMV workgroup derives the same one, or, on

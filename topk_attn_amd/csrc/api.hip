@@ -238,13 +238,14 @@ uint32_t next_epoch() {
   static std::atomic<uint32_t> call_counter{0};
   return (call_counter.fetch_add(1, std::memory_order_relaxed) & ~kTauHasCut) | 0x80000000u;
 }
-void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, int* sample_rank) {
+void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, int* sample_rank, int* slice_len = nullptr) {
   *num_samples = *sample_rank = 0;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
   if ((!a->out_idx && !u) || (u && !u->handoff) || a->out_scores || chunk_len < cut_route_min_len()) return;
-  int s = 0, r = 0;
-  gemv_cut_plan(chunk_len, a->k, &s, &r);
+  int s = 0, r = 0, len = 0;
+  gemv_cut_plan(chunk_len, a->k, &s, &r, &len);
   if (s == 0) return;
+  if (slice_len) *slice_len = len;
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   // Measured, decode steps with k = 2048 unless said (us per step, this route against the others): 1 x 32768 tokens
   // 23.6 / 32.2, 4 x 32768 26.7 / 37.5, 8 x 32768 33.7 / 43.4, 16 x 32768 50.4 / 56.9, 24 x 32768 63.8 / 68.3,
@@ -332,13 +333,13 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
 
   // A few segments of middling length: every GEMV workgroup derives the segment's cut from common sample rows and
   // stores its candidates, one workgroup per segment ranks them.
-  int cut_samples = 0, cut_rank = 0;
-  cut_plan(a, u, &cut_samples, &cut_rank);
+  int cut_samples = 0, cut_rank = 0, cut_slice_len = 0;
+  cut_plan(a, u, &cut_samples, &cut_rank, &cut_slice_len);
   if (cut_samples != 0 && !ic) {
     GemvParams cp = gp;
     cp.hist = nullptr;
-    cp.tokens_per_wg = kCutTokensPerWg;
-    cp.wgs_per_chunk = (int)((chunk_len + kCutTokensPerWg - 1) / kCutTokensPerWg);
+    cp.tokens_per_wg = cut_slice_len;
+    cp.wgs_per_chunk = (int)((chunk_len + cut_slice_len - 1) / cut_slice_len);
     cp.num_samples = cut_samples;
     cp.sample_rank = cut_rank;
     cp.cand = sp.list;
@@ -370,7 +371,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     sc.hist = nullptr;
     sc.tau_words = cp.tau_words;   // (set when the GEMV launch announced the cuts itself)
     sc.parts = cp.wgs_per_chunk;
-    sc.part_len = kCutTokensPerWg;
+    sc.part_len = cut_slice_len;
     sc.max_entries = current_hooks().force_segment_redo ? 0 : kCutMaxSlices * kCutTokensPerWg;   // (no limit of its own)
     sc.scores = scores;
     sc.cut_splits = cp.cut_splits;

@@ -74,11 +74,50 @@ __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint
   }
 }
 
+// The candidates of a workgroup's TOKENS tokens (keys in sh_key, thread t owns token t_begin + t; the threads beyond
+// TOKENS have left) to the slices of L tokens that they belong to: tokens at or above `cut` in the order, as composites
+// (key << 32 | ~token, token counted inside the segment) ascending in token; the first kCutHead of a slice go to its
+// place in the dense head array, which is always written whole (zeros behind the last candidate: no composite is
+// zero), the rest to the slice's place in the wide array; the slice's count goes to its own word (kCutGaveUp without a
+// cut).  L: 256, or 128 where k is a larger share of the segment and a slice of 256 would overflow its head entries.
+template <int TOKENS, int L>
+__device__ __forceinline__ void store_slices(const GemvParams& p, int seg, int t_begin, int n_local, const uint32_t* sh_key, uint32_t* sh_wcnt,
+                                             uint64_t cut, bool have_cut) {
+  static_assert(L % kWave == 0 && L >= kCutHead && TOKENS % L == 0, "whole waves per slice, a thread per head entry");
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int sub = tid / L, t_in = tid % L;
+  const uint32_t token = (uint32_t)(t_begin + tid);
+  const uint64_t mine = composite(sh_key[tid], token);
+  const bool pass = have_cut && tid < n_local && mine >= cut;
+  const unsigned long long mask = __ballot(pass);
+  if (lane == 0) sh_wcnt[wave] = (uint32_t)__popcll(mask);
+  __syncthreads();   // (the waves that have ended no longer count)
+  uint32_t ahead = 0, total = 0;
+#pragma unroll
+  for (int v = 0; v < L / kWave; ++v) {
+    const int w = sub * (L / kWave) + v;
+    const uint32_t c = sh_wcnt[w];
+    ahead += w < wave ? c : 0u;
+    total += c;
+  }
+  const int slice = t_begin / L + sub;
+  if (slice >= p.wgs_per_chunk) return;   // (p.wgs_per_chunk counts the slices of a segment: its last workgroup may have fewer)
+  const int64_t slice_id = (int64_t)seg * p.wgs_per_chunk + slice;
+  uint64_t* head = p.cand_head + slice_id * kCutHead;
+  uint64_t* wide = p.cand + (int64_t)seg * p.cand_seg_stride + (int64_t)slice * L;
+  if (pass) {
+    const uint32_t pos = ahead + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+    (pos < (uint32_t)kCutHead ? head : wide)[pos] = mine;
+  }
+  if ((uint32_t)t_in >= total && t_in < kCutHead) head[t_in] = 0ull;
+  if (t_in == 0) p.cand_count[slice_id] = have_cut ? total : kCutGaveUp;
+}
+
 // Row groups 0 .. 31 score the 256 tokens of the slice, the row groups behind them the S sample tokens (S = 256:
 // sixteen waves), one round of eight loads per lane.
 // Many waves and a short program: few workgroups run at a time on these problems, so a wave pays the first fetch
 // of every line of code itself (the same rows on four waves with four rounds each: 9.6 instead of 8.1 us).
-template <int DT, int S>
+template <int DT, int S, int L>
 __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   constexpr int kCutSamples = S;
   constexpr int kCutRows = kCutTokensPerWg + S;
@@ -92,8 +131,9 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   const int tid = threadIdx.x;
   const int j = tid & 15, rg = tid >> 4;
   const int lane = tid & 63, wave = tid >> 6;
-  const int slice = (int)(blockIdx.x % (uint32_t)p.wgs_per_chunk);
-  const int seg = (int)(blockIdx.x / (uint32_t)p.wgs_per_chunk);
+  const uint32_t wgs_per_seg = (uint32_t)((p.chunk_len + kCutTokensPerWg - 1) / kCutTokensPerWg);
+  const int slice = (int)(blockIdx.x % wgs_per_seg);   // this workgroup's 256 tokens inside the segment
+  const int seg = (int)(blockIdx.x / wgs_per_seg);
   const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
   const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
@@ -138,33 +178,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   __syncthreads();
   if (tid >= kCutTokensPerWg) return;
 
-  // thread t owns token t_begin + t.  Entries are composites (key << 32 | ~token, token counted inside the segment),
-  // ascending in token; the first kCutHead of a slice go to its place in the dense head array, which is always
-  // written whole (zeros behind the last candidate: no composite is zero), the rest to the slice's place in the wide
-  // array; the slice's count goes to its own word.
-  const uint32_t tau = sh_cut[0], cut = sh_cut[1];
-  const uint32_t key = sh_key[tid];
-  const uint32_t token = (uint32_t)(t_begin + tid);
-  const bool pass = tid < n_local && (key > tau || (key == tau && token <= cut));
-  const unsigned long long mask = __ballot(pass);
-  if (lane == 0) sh_wcnt[wave] = (uint32_t)__popcll(mask);
-  __syncthreads();   // (the waves that have ended no longer count)
-  uint32_t ahead = 0, total = 0;
-#pragma unroll
-  for (int v = 0; v < kCutTokensPerWg / kWave; ++v) {
-    const uint32_t c = sh_wcnt[v];
-    ahead += v < wave ? c : 0u;
-    total += c;
-  }
-  const int64_t slice_id = (int64_t)seg * p.wgs_per_chunk + slice;
-  uint64_t* head = p.cand_head + slice_id * kCutHead;
-  uint64_t* wide = p.cand + (int64_t)seg * p.cand_seg_stride + (int64_t)slice * kCutTokensPerWg;
-  if (pass) {
-    const uint32_t pos = ahead + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-    (pos < (uint32_t)kCutHead ? head : wide)[pos] = composite(key, token);
-  }
-  if ((uint32_t)tid >= total && tid < kCutHead) head[tid] = 0ull;
-  if (tid == 0) p.cand_count[slice_id] = total;
+  store_slices<kCutTokensPerWg, L>(p, seg, t_begin, n_local, sh_key, sh_wcnt, composite(sh_cut[0], sh_cut[1]), true);
 }
 
 
@@ -228,7 +242,7 @@ __global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
 // before the compare - a bounded wait: a workgroup that never sees the word marks its slices (kCutGaveUp in the count),
 // and the ranking kernel redoes such a segment from the keys.  The sampling workgroups come first in the grid, so they
 // run before any workgroup that waits for them; nothing depends on that but the speed.
-template <int DT, bool FRONT>
+template <int DT, bool FRONT, int L>
 __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams p) {
   constexpr int kTokens = 2 * kCutTokensPerWg;
   __shared__ uint32_t sh_key[kTokens];
@@ -251,7 +265,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
   const uint32_t wg = blockIdx.x - (FRONT ? (uint32_t)segs : 0u);
   const int j = tid & 15, rg = tid >> 4;
   const int lane = tid & 63, wave = tid >> 6;
-  const int wgs_per_seg = (p.wgs_per_chunk + 1) / 2;   // p.wgs_per_chunk counts slices
+  const int wgs_per_seg = (int)((p.chunk_len + kTokens - 1) / kTokens);
   const int pair = (int)(wg % (uint32_t)wgs_per_seg);
   const int seg = (int)(wg / (uint32_t)wgs_per_seg);
   const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
@@ -303,50 +317,34 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
     have_cut = sh_cutc[1] != 0ull;
   }
 
-  // thread t owns token t_begin + t; waves 0 .. 3 make the first slice, waves 4 .. 7 the second
-  const int half = tid / kCutTokensPerWg, t_in = tid % kCutTokensPerWg;
-  const uint32_t token = (uint32_t)(t_begin + tid);
-  const uint64_t mine_c = composite(sh_key[tid], token);
-  const bool pass = have_cut && tid < n_local && mine_c >= cut;
-  const unsigned long long mask = __ballot(pass);
-  if (lane == 0) sh_wcnt[wave] = (uint32_t)__popcll(mask);
-  __syncthreads();   // (the waves that have ended no longer count)
-  uint32_t ahead = 0, total = 0;
-#pragma unroll
-  for (int v = 0; v < kCutTokensPerWg / kWave; ++v) {
-    const int w = half * (kCutTokensPerWg / kWave) + v;
-    const uint32_t c = sh_wcnt[w];
-    ahead += w < wave ? c : 0u;
-    total += c;
-  }
-  const int slice = 2 * pair + half;
-  if (slice >= p.wgs_per_chunk) return;   // a segment with an odd number of slices: the last workgroup has one
-  const int64_t slice_id = (int64_t)seg * p.wgs_per_chunk + slice;
-  uint64_t* head = p.cand_head + slice_id * kCutHead;
-  uint64_t* wide = p.cand + (int64_t)seg * p.cand_seg_stride + (int64_t)slice * kCutTokensPerWg;
-  if (pass) {
-    const uint32_t pos = ahead + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-    (pos < (uint32_t)kCutHead ? head : wide)[pos] = mine_c;
-  }
-  if ((uint32_t)t_in >= total && t_in < kCutHead) head[t_in] = 0ull;
-  if (t_in == 0) p.cand_count[slice_id] = have_cut ? total : kCutGaveUp;
+  store_slices<kTokens, L>(p, seg, t_begin, n_local, sh_key, sh_wcnt, cut, have_cut);
 }
 
 }  // namespace
 
+// p.tokens_per_wg: the slice length (256 or 128), p.wgs_per_chunk: the slices of a segment.
+static bool slices_ok(const GemvParams& p) {
+  return (p.tokens_per_wg == kCutTokensPerWg || p.tokens_per_wg == kCutTokensPerWg / 2) &&
+         p.wgs_per_chunk == (int)((p.chunk_len + p.tokens_per_wg - 1) / p.tokens_per_wg) && p.wgs_per_chunk <= kCutMaxSlices && p.cand &&
+         p.cand_head && p.cand_count && p.cut_splits;
+}
+
 int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  if (p.tokens_per_wg != kCutTokensPerWg || p.num_samples != 256 || p.chunk_len < p.num_samples ||
-      p.sample_rank < kCutParts || p.sample_rank > p.num_samples || !p.cand || !p.cand_head || !p.cand_count || !p.cut_splits ||
-      segs * p.wgs_per_chunk > 0x7fffffffLL)
+  const int64_t wgs = segs * ((p.chunk_len + kCutTokensPerWg - 1) / kCutTokensPerWg);
+  if (!slices_ok(p) || p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
+      wgs > 0x7fffffffLL)
     return TKA_EINVAL;
-  const unsigned wgs = (unsigned)(segs * p.wgs_per_chunk);
   const unsigned threads = (unsigned)(kCutTokensPerWg + p.num_samples) / kCutUnroll * 16;   // 16 lanes per row, 8 rows each
+  const bool short_slices = p.tokens_per_wg != kCutTokensPerWg;
   LaunchTimer timer("gemv_cut", stream);
-  if (dtype == TKA_F16)
-    gemv_cut_kernel<TKA_F16, 256><<<wgs, threads, 0, stream>>>(p);
-  else
-    gemv_cut_kernel<TKA_BF16, 256><<<wgs, threads, 0, stream>>>(p);
+  if (dtype == TKA_F16) {
+    if (short_slices) gemv_cut_kernel<TKA_F16, 256, kCutTokensPerWg / 2><<<(unsigned)wgs, threads, 0, stream>>>(p);
+    else gemv_cut_kernel<TKA_F16, 256, kCutTokensPerWg><<<(unsigned)wgs, threads, 0, stream>>>(p);
+  } else {
+    if (short_slices) gemv_cut_kernel<TKA_BF16, 256, kCutTokensPerWg / 2><<<(unsigned)wgs, threads, 0, stream>>>(p);
+    else gemv_cut_kernel<TKA_BF16, 256, kCutTokensPerWg><<<(unsigned)wgs, threads, 0, stream>>>(p);
+  }
   return hip_status(hipGetLastError());
 }
 
@@ -369,19 +367,21 @@ int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream) {
 // sampling arguments of launch_cut_samples are then needed) instead of from a launch before it.
 int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  const int64_t wgs = segs * ((p.wgs_per_chunk + 1) / 2) + (front_sampling ? segs : 0);
-  if (p.tokens_per_wg != kCutTokensPerWg || !p.cand || !p.cand_head || !p.cand_count || !p.cut_splits || wgs > 0x7fffffffLL) return TKA_EINVAL;
+  const int64_t wgs = segs * ((p.chunk_len + 2 * kCutTokensPerWg - 1) / (2 * kCutTokensPerWg)) + (front_sampling ? segs : 0);
+  if (!slices_ok(p) || wgs > 0x7fffffffLL) return TKA_EINVAL;
   if (front_sampling && (p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
                          !p.tau_words || p.epoch == 0 || p.tau_spin_limit < 1))
     return TKA_EINVAL;
   LaunchTimer timer("gemv_cut_slices", stream);
-  if (dtype == TKA_F16) {
-    if (front_sampling) gemv_cut_slices_kernel<TKA_F16, true><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
-    else gemv_cut_slices_kernel<TKA_F16, false><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
-  } else {
-    if (front_sampling) gemv_cut_slices_kernel<TKA_BF16, true><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
-    else gemv_cut_slices_kernel<TKA_BF16, false><<<(unsigned)wgs, kCutThreads, 0, stream>>>(p);
-  }
+  typedef void (*Kernel)(GemvParams);
+  constexpr int kLong = kCutTokensPerWg, kShort = kCutTokensPerWg / 2;
+  static const Kernel kernels[2][2][2] = {   // [dtype][cuts from the first workgroups][slices of 128 tokens]
+      {{gemv_cut_slices_kernel<TKA_F16, false, kLong>, gemv_cut_slices_kernel<TKA_F16, false, kShort>},
+       {gemv_cut_slices_kernel<TKA_F16, true, kLong>, gemv_cut_slices_kernel<TKA_F16, true, kShort>}},
+      {{gemv_cut_slices_kernel<TKA_BF16, false, kLong>, gemv_cut_slices_kernel<TKA_BF16, false, kShort>},
+       {gemv_cut_slices_kernel<TKA_BF16, true, kLong>, gemv_cut_slices_kernel<TKA_BF16, true, kShort>}}};
+  hipLaunchKernelGGL(kernels[dtype == TKA_F16 ? 0 : 1][front_sampling ? 1 : 0][p.tokens_per_wg == kShort ? 1 : 0], dim3((unsigned)wgs),
+                     dim3(kCutThreads), 0, stream, p);
   return hip_status(hipGetLastError());
 }
 
@@ -389,22 +389,26 @@ int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, 
 // does not serve the shape.  With S = 256 samples spread evenly and m = k S / n of them expected inside the top k,
 // the rank is R = m + 5.5 sqrt(m) + 2 (at least 8: every part of the candidates ends with a sample of its own):
 // "fewer than k tokens pass" (the segment is then redone from the keys, still exact) needs R of the samples inside
-// the top k, more than five deviations out; about n R / S candidates are stored.  Limits: a slice of 256 tokens
-// should stay within the kCutHead entries that the ranking kernel reads in its first round trip (40 expected at
-// most), and a segment within what it ranks in one go.
+// the top k, more than five deviations out; about n R / S candidates are stored.  Limits: a slice should stay within
+// the kCutHead entries that the ranking kernel reads in its first round trip (40 expected at most: k up to about
+// n / 14.5 with slices of 256 tokens; a larger k, up to n / 8, takes slices of 128 tokens where the segment then
+// still has no more than kCutMaxSlices of them), and a segment within what it ranks in one go.
 // (With 64 samples - enough for a small k on segments of a few thousand rows - the route was measured too: 32 x 4096
 // rows, k = 64: 19.5 us against 13.3 on the route that selects in the registers of one workgroup per segment.)
-void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank) {
-  *num_samples = *sample_rank = 0;
+void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank, int* slice_len) {
+  *num_samples = *sample_rank = *slice_len = 0;
   if (chunk_len < 2048 || chunk_len > (int64_t)kCutMaxSlices * kCutTokensPerWg || k > kCutMaxK || (int64_t)k * 8 > chunk_len) return;
   const int s = 256;
   const double m = (double)k * s / (double)chunk_len;
   int r = (int)ceil(m + 5.5 * sqrt(m) + 2.0);
   if (r < kCutParts) r = kCutParts;
-  const double per_slice = (double)kCutTokensPerWg * r / s, per_segment = (double)chunk_len * r / s;
-  if (r * 2 > s || per_slice > 40.0 || per_segment * 1.2 > (double)kCutMaxCandidates) return;
+  int len = kCutTokensPerWg;
+  if ((double)len * r / s > 40.0) len /= 2;
+  const double per_slice = (double)len * r / s, per_segment = (double)chunk_len * r / s;
+  if (r * 2 > s || per_slice > 40.0 || (chunk_len + len - 1) / len > kCutMaxSlices || per_segment * 1.2 > (double)kCutMaxCandidates) return;
   *num_samples = s;
   *sample_rank = r;
+  *slice_len = len;
 }
 
 }  // namespace tka

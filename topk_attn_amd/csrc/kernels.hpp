@@ -54,13 +54,13 @@ void gemv_candidate_plan(int64_t chunk_len, int64_t total_rows, int k, int max_c
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);
 // Common-cut route: every workgroup derives the segment's cut from the same sample rows and stores its slice's candidates
 // (p.cand_head: the first kCutHead of a slice as composites, zeros behind; p.cand: the rest; p.cand_count; p.num_samples /
-// p.sample_rank from gemv_cut_plan).
+// p.sample_rank and the slice length p.tokens_per_wg from gemv_cut_plan; p.wgs_per_chunk: the slices of a segment).
 int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream);
 // The same in two launches for calls that fill the GPU: one workgroup per segment finds the cut and the part ends, then the
 // GEMV workgroups (512 tokens each) score nothing twice.
 int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream);
 int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream);
-void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank);
+void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank, int* slice_len);
 
 // ---- stage 1: selection -----------------------------------------------------------------------
 struct SelectParams {

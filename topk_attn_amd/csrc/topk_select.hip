@@ -1026,8 +1026,10 @@ __device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_
 // Dynamic LDS: kCutMaxCandidates composites (the part, as found), then as many again (the part in bucket order;
 // before that, entries from beyond the heads); the tie path and the fallback reuse both.
 // PAIRS: pairs of head entries per thread, 4 (up to 128 slices) or 8 (up to 256); UNION: the union list is written (the
-// rank-ordered outputs then only if asked for).
-template <int DT, int PAIRS, bool UNION>
+// rank-ordered outputs then only if asked for); ANNOUNCED: the GEMV launch announced the cuts to its own workgroups
+// (p.tau_words), some of which may have given up waiting.  (Template arguments, not flags: a dozen instructions of
+// bookkeeping on this kernel's straight path cost 0.4 of its 6.5 us.)
+template <int DT, int PAIRS, bool UNION, bool ANNOUNCED>
 __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, SelectParams p, int kpad) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint64_t* sh_own = (uint64_t*)smem;
@@ -1062,6 +1064,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     w[e] = q < n_pairs ? heads[q] : (u64x2){0ull, 0ull};
   }
   const uint32_t slice_cnt = tid < p.parts ? p.list_cnt[(int64_t)seg * p.parts + tid] : 0u;
+
   // ends of the parts, in descending order: [part] above this workgroup's part, [part + 1] its lower end
   // (as a running minimum: the samples were ranked by keys whose last bits were replaced, so two of them may come
   // in the other order here)
@@ -1081,8 +1084,8 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   sh_hist[2 * tid + 1] = 0;
   if (tid < 8) sh_n[tid] = 0;
   __syncthreads();
-  // (p.tau_words: the cuts were announced inside the GEMV launch; the slice of a workgroup that never saw its segment's holds no candidates)
-  if (p.tau_words && slice_cnt == kCutGaveUp) atomicAdd(&sh_n[7], 1u);
+  // (the slice of a workgroup that never saw its segment's cut holds no candidates)
+  if (ANNOUNCED && slice_cnt == kCutGaveUp) atomicAdd(&sh_n[7], 1u);
   else if (slice_cnt > (uint32_t)kCutHead) sh_ovf[atomicAdd(&sh_n[0], 1u)] = (uint32_t)tid | (slice_cnt << 16);
   __syncthreads();
   const uint32_t n_ovf = sh_n[0];
@@ -1092,7 +1095,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
       const uint32_t sl = sh_ovf[i] & 0xffffu, cnt = sh_ovf[i] >> 16;
       const uint32_t j = (uint32_t)kCutHead + (uint32_t)tid;
       if (j < cnt) {
-        const uint64_t x = wide[(int64_t)sl * kCutTokensPerWg + j];
+        const uint64_t x = wide[(int64_t)sl * p.part_len + j];
         const uint32_t pos = atomicAdd(&sh_n[1], 1u);
         if (pos < (uint32_t)kCutMaxExtras) sh_extra[pos] = x;
       }
@@ -1156,11 +1159,12 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   uint32_t max_part = n_own;
   if (n_cand > (uint32_t)kCutMaxCandidates)
     max_part = max(max_part, largest_part((const uint64_t*)heads, n_pairs, n_ovf ? sh_extra : nullptr, min(n_extra, (uint32_t)kCutMaxExtras), sh_split, sh_hist));
+  const uint32_t n_gave_up = ANNOUNCED ? sh_n[7] : 0u;
   const bool redo = n_cand < k || n_cand > (uint32_t)p.max_entries || n_extra > (uint32_t)kCutMaxExtras || max_part > (uint32_t)kCutMaxCandidates ||
-                    sh_n[7] != 0u;
+                    n_gave_up != 0u;
   if (tid == 0 && part == 0) {
-    p.seg_flags[seg] = (redo ? 1u : 0u) | (sh_n[7] << 8);   // (as on the candidate route: bit 0 redone, bits 8.. slices that gave up)
-    if (p.tau_words) p.tau_words[2 * seg] = 0ull;   // the word that announced the segment's cut: spent (a replayed graph brings the same epoch)
+    p.seg_flags[seg] = (redo ? 1u : 0u) | (n_gave_up << 8);   // (as on the candidate route: bit 0 redone, bits 8.. slices that gave up)
+    if (ANNOUNCED) p.tau_words[2 * seg] = 0ull;   // the word that announced the segment's cut: spent (a replayed graph brings the same epoch)
   }
   if (redo) {   // every workgroup of the segment sees the same counts: the first one redoes it, the others leave
     if (part != 0) return;
@@ -1496,7 +1500,9 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   // head entries of the slices: the candidate route (32 per slice of 512 tokens) or the common-cut route (64 per slice of 256)
   const size_t cut_segs = seg_len <= (int64_t)kCutMaxSlices * kCutTokensPerWg ? (size_t)num_segments : 0;
   const size_t head_cand = cand_segs * (size_t)(seg_len / kGemvCandTokensPerWg + 1) * kCandHead * sizeof(uint64_t);
-  const size_t head_cut = cut_segs * (size_t)(seg_len / kCutTokensPerWg + 1) * kCutHead * sizeof(uint64_t);
+  // (slices of 128 tokens where a segment has no more than kCutMaxSlices of them, see gemv_cut_plan)
+  const int64_t cut_slices = seg_len <= (int64_t)kCutMaxSlices * (kCutTokensPerWg / 2) ? seg_len / (kCutTokensPerWg / 2) + 1 : seg_len / kCutTokensPerWg + 1;
+  const size_t head_cut = cut_segs * (size_t)cut_slices * kCutHead * sizeof(uint64_t);
   l.head = take(head_cand > head_cut ? head_cand : head_cut);
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
@@ -1624,18 +1630,19 @@ int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int 
 }
 
 int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
-  if (p.parts < 1 || p.parts > kCutMaxSlices || p.part_len != kCutTokensPerWg || p.k > kCutMaxK || (!p.out_idx && !p.union_idx) || !p.cand_head ||
+  if (p.parts < 1 || p.parts > kCutMaxSlices || (p.part_len != kCutTokensPerWg && p.part_len != kCutTokensPerWg / 2) || p.k > kCutMaxK || (!p.out_idx && !p.union_idx) || !p.cand_head ||
       !p.list_cnt || !p.cut_splits || !p.seg_flags || (p.union_idx && !p.union_count))
     return TKA_EINVAL;
   const int lds = 2 * kCutMaxCandidates * (int)sizeof(uint64_t);
   typedef void (*RankKernel)(GemvParams, SelectParams, int);
-  static const RankKernel kernels[2][2][2] = {   // [dtype][more than 8 head entries per thread][union list]
-      {{select_rank_kernel<TKA_F16, 4, false>, select_rank_kernel<TKA_F16, 4, true>},
-       {select_rank_kernel<TKA_F16, 8, false>, select_rank_kernel<TKA_F16, 8, true>}},
-      {{select_rank_kernel<TKA_BF16, 4, false>, select_rank_kernel<TKA_BF16, 4, true>},
-       {select_rank_kernel<TKA_BF16, 8, false>, select_rank_kernel<TKA_BF16, 8, true>}}};
+#define TKA_RANK_KERNELS(DT, PAIRS) \
+  {{select_rank_kernel<DT, PAIRS, false, false>, select_rank_kernel<DT, PAIRS, false, true>}, \
+   {select_rank_kernel<DT, PAIRS, true, false>, select_rank_kernel<DT, PAIRS, true, true>}}
+  static const RankKernel kernels[2][2][2][2] = {   // [dtype][more than 8 head entries per thread][union list][cuts announced in the GEMV launch]
+      {TKA_RANK_KERNELS(TKA_F16, 4), TKA_RANK_KERNELS(TKA_F16, 8)}, {TKA_RANK_KERNELS(TKA_BF16, 4), TKA_RANK_KERNELS(TKA_BF16, 8)}};
+#undef TKA_RANK_KERNELS
   const bool wide = p.parts * kCutHead > 8 * kSelThreads;
-  const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0][p.union_idx ? 1 : 0];
+  const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0][p.union_idx ? 1 : 0][p.tau_words ? 1 : 0];
   if (allow_dynamic_lds((const void*)kernel, lds) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("select_rank", stream);
   const unsigned wgs = (unsigned)p.num_segments * kCutParts;
