@@ -131,11 +131,17 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   const int tid = threadIdx.x;
   const int j = tid & 15, rg = tid >> 4;
   const int lane = tid & 63, wave = tid >> 6;
-  const uint32_t wgs_per_seg = (uint32_t)((p.chunk_len + kCutTokensPerWg - 1) / kCutTokensPerWg);
-  const int slice = (int)(blockIdx.x % wgs_per_seg);   // this workgroup's 256 tokens inside the segment
-  const int seg = (int)(blockIdx.x / wgs_per_seg);
-  const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
-  const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
+  // Grid: x = this workgroup's 256 tokens inside the segment, y = KV head and chunk, z = batch entry: no division on the
+  // way to the first load (the hardware has none: each costs some twenty-five instructions, and the five of a flat grid
+  // stood in front of every load of this short kernel).
+  const int slice = (int)blockIdx.x;
+  const int b = (int)blockIdx.z;
+  int h = (int)blockIdx.y, chunk = 0;
+  if (p.num_chunks != 1) {
+    h = (int)(blockIdx.y / (uint32_t)p.num_chunks);
+    chunk = (int)blockIdx.y - h * p.num_chunks;
+  }
+  const int seg = b * (int)gridDim.y + (int)blockIdx.y;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
   const int n = (int)p.chunk_len;
   const int t_begin = slice * kCutTokensPerWg;
@@ -146,14 +152,18 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   // otherwise stand in front of the row loads (one more round trip to memory in a kernel made of a few)
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
                           chunk_base * p.key_stride_n + 8 * j;
-  const bool sampler = rg >= kCutTokensPerWg / kCutUnroll;
+  const bool sampler = rg >= kCutTokensPerWg / kCutUnroll;   // (whole waves: each runs one side of the branch only)
   u32x4 kv[kCutUnroll];
+  if (sampler) {
 #pragma unroll
-  for (int u = 0; u < kCutUnroll; ++u) {
-    const int row = rg * kCutUnroll + u;   // 0 .. 255 the slice, from 256 on the sample
-    const int64_t ts = sample_token(seg, row & (kCutSamples - 1), stride);
-    const int64_t to = (int64_t)(t_begin + (row < n_local ? row : n_local - 1));
-    kv[u] = *(const u32x4*)(kbase + (sampler ? ts : to) * p.key_stride_n);
+    for (int u = 0; u < kCutUnroll; ++u)
+      kv[u] = *(const u32x4*)(kbase + sample_token(seg, (rg * kCutUnroll + u) & (kCutSamples - 1), stride) * p.key_stride_n);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kCutUnroll; ++u) {
+      const int row = rg * kCutUnroll + u;
+      kv[u] = *(const u32x4*)(kbase + (int64_t)(t_begin + (row < n_local ? row : n_local - 1)) * p.key_stride_n);
+    }
   }
   __builtin_amdgcn_sched_barrier(0);
   float qf[8];
@@ -331,19 +341,20 @@ static bool slices_ok(const GemvParams& p) {
 
 int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  const int64_t wgs = segs * ((p.chunk_len + kCutTokensPerWg - 1) / kCutTokensPerWg);
+  const int64_t wgs_per_seg = (p.chunk_len + kCutTokensPerWg - 1) / kCutTokensPerWg;
   if (!slices_ok(p) || p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
-      wgs > 0x7fffffffLL)
+      segs * wgs_per_seg > 0x7fffffffLL || (int64_t)p.num_kv_heads * p.num_chunks > 65535 || p.batch > 65535)
     return TKA_EINVAL;
+  const dim3 wgs((unsigned)wgs_per_seg, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
   const unsigned threads = (unsigned)(kCutTokensPerWg + p.num_samples) / kCutUnroll * 16;   // 16 lanes per row, 8 rows each
   const bool short_slices = p.tokens_per_wg != kCutTokensPerWg;
   LaunchTimer timer("gemv_cut", stream);
   if (dtype == TKA_F16) {
-    if (short_slices) gemv_cut_kernel<TKA_F16, 256, kCutTokensPerWg / 2><<<(unsigned)wgs, threads, 0, stream>>>(p);
-    else gemv_cut_kernel<TKA_F16, 256, kCutTokensPerWg><<<(unsigned)wgs, threads, 0, stream>>>(p);
+    if (short_slices) gemv_cut_kernel<TKA_F16, 256, kCutTokensPerWg / 2><<<wgs, threads, 0, stream>>>(p);
+    else gemv_cut_kernel<TKA_F16, 256, kCutTokensPerWg><<<wgs, threads, 0, stream>>>(p);
   } else {
-    if (short_slices) gemv_cut_kernel<TKA_BF16, 256, kCutTokensPerWg / 2><<<(unsigned)wgs, threads, 0, stream>>>(p);
-    else gemv_cut_kernel<TKA_BF16, 256, kCutTokensPerWg><<<(unsigned)wgs, threads, 0, stream>>>(p);
+    if (short_slices) gemv_cut_kernel<TKA_BF16, 256, kCutTokensPerWg / 2><<<wgs, threads, 0, stream>>>(p);
+    else gemv_cut_kernel<TKA_BF16, 256, kCutTokensPerWg><<<wgs, threads, 0, stream>>>(p);
   }
   return hip_status(hipGetLastError());
 }

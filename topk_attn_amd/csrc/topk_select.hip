@@ -1052,7 +1052,9 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int seg = blockIdx.x / kCutParts, part = blockIdx.x % kCutParts;
+  // (grid: x = chunk and part, y = batch entry and KV head: no division by a run-time value anywhere on the straight path)
+  const int chunk = (int)(blockIdx.x / (uint32_t)kCutParts), part = (int)(blockIdx.x % (uint32_t)kCutParts);
+  const int seg = (int)blockIdx.y * p.segs_per_row + chunk;
   const uint32_t k = (uint32_t)p.k;
   const u64x2* heads = (const u64x2*)(p.cand_head + (int64_t)seg * p.parts * kCutHead);
   const int n_pairs = p.parts * (kCutHead / 2);
@@ -1199,7 +1201,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     sh_off[2 * tid] = sh_cur[2 * tid] = above + ge - h0;             // buckets > 2t
   }
   __syncthreads();
-  const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len) : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
+  const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len) : (uint32_t)(chunk * p.seg_len);
   // What a ranked candidate leaves behind.  The union list of this route: sink range [0, lo) and local window [hi, n)
   // first, then one place per rank; a selected token that lies inside the ranges is listed there already, and its place
   // holds -1, which the attention kernels skip like any id outside the cache.  So the place is the rank: nobody needs to
@@ -1645,8 +1647,9 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
   const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0][p.union_idx ? 1 : 0][p.tau_words ? 1 : 0];
   if (allow_dynamic_lds((const void*)kernel, lds) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("select_rank", stream);
-  const unsigned wgs = (unsigned)p.num_segments * kCutParts;
-  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(kSelThreads), lds, stream, g, p, kpad_for(p.k));
+  if (p.segs_per_row < 1 || p.num_segments % p.segs_per_row || p.num_segments / p.segs_per_row > 65535) return TKA_EINVAL;
+  const dim3 wgs((unsigned)(p.segs_per_row * kCutParts), (unsigned)(p.num_segments / p.segs_per_row));
+  hipLaunchKernelGGL(kernel, wgs, dim3(kSelThreads), lds, stream, g, p, kpad_for(p.k));
   return hip_status(hipGetLastError());
 }
 
