@@ -74,6 +74,45 @@ __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint
   }
 }
 
+// Where a workgroup of these kernels works.  Their grids have y = KV head and chunk and z = batch entry (x: the place
+// inside the segment), so that no division by a run-time value stands in front of the first load - the hardware has
+// none: each costs some twenty-five instructions, and the five of a flat grid were 0.8 us of c1's 13.5.
+struct SegPos {
+  int b, h, chunk, seg;
+};
+__device__ __forceinline__ SegPos seg_position(const GemvParams& p) {
+  SegPos s;
+  s.b = (int)blockIdx.z;
+  s.h = (int)blockIdx.y;
+  s.chunk = 0;
+  if (p.num_chunks != 1) {
+    s.h = (int)(blockIdx.y / (uint32_t)p.num_chunks);
+    s.chunk = (int)blockIdx.y - s.h * p.num_chunks;
+  }
+  s.seg = s.b * (int)gridDim.y + (int)blockIdx.y;
+  return s;
+}
+// The same from a segment number (a flat grid): divisions only where a call has several chunks per head, or several
+// batch entries.
+__device__ __forceinline__ SegPos seg_position_flat(const GemvParams& p, int seg) {
+  SegPos s;
+  s.seg = seg;
+  int bh = seg;
+  s.chunk = 0;
+  if (p.num_chunks != 1) {
+    bh = (int)((uint32_t)seg / (uint32_t)p.num_chunks);
+    s.chunk = seg - bh * p.num_chunks;
+  }
+  s.b = 0;
+  s.h = bh;
+  if (p.batch != 1) {
+    s.b = (int)((uint32_t)bh / (uint32_t)p.num_kv_heads);
+    s.h = bh - s.b * p.num_kv_heads;
+  }
+  return s;
+}
+static bool grid_ok(const GemvParams& p) { return (int64_t)p.num_kv_heads * p.num_chunks <= 65535 && p.batch <= 65535; }
+
 // The candidates of a workgroup's TOKENS tokens (keys in sh_key, thread t owns token t_begin + t; the threads beyond
 // TOKENS have left) to the slices of L tokens that they belong to: tokens at or above `cut` in the order, as composites
 // (key << 32 | ~token, token counted inside the segment) ascending in token; the first kCutHead of a slice go to its
@@ -130,18 +169,9 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
 
   const int tid = threadIdx.x;
   const int j = tid & 15, rg = tid >> 4;
-  const int lane = tid & 63, wave = tid >> 6;
-  // Grid: x = this workgroup's 256 tokens inside the segment, y = KV head and chunk, z = batch entry: no division on the
-  // way to the first load (the hardware has none: each costs some twenty-five instructions, and the five of a flat grid
-  // stood in front of every load of this short kernel).
-  const int slice = (int)blockIdx.x;
-  const int b = (int)blockIdx.z;
-  int h = (int)blockIdx.y, chunk = 0;
-  if (p.num_chunks != 1) {
-    h = (int)(blockIdx.y / (uint32_t)p.num_chunks);
-    chunk = (int)blockIdx.y - h * p.num_chunks;
-  }
-  const int seg = b * (int)gridDim.y + (int)blockIdx.y;
+  const int slice = (int)blockIdx.x;   // this workgroup's 256 tokens inside the segment
+  const SegPos at = seg_position(p);
+  const int b = at.b, h = at.h, chunk = at.chunk, seg = at.seg;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
   const int n = (int)p.chunk_len;
   const int t_begin = slice * kCutTokensPerWg;
@@ -200,7 +230,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
 // The work of one workgroup for one segment's cut: the 256 sample rows (64 row groups, four rows per lane), their
 // ranks, cut and part ends (to p.cut_splits).  Every thread of the 1024 calls it.
 template <int DT, bool ANNOUNCED>
-__device__ __forceinline__ void sample_segment(const GemvParams& p, int seg) {
+__device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos& at) {
   constexpr int S = 256, kRows = S / (kCutThreads / 16);   // four rows per lane
   __shared__ uint32_t sh_skey[S];
   __shared__ __attribute__((aligned(16))) uint32_t sh_rkey[S];
@@ -208,8 +238,7 @@ __device__ __forceinline__ void sample_segment(const GemvParams& p, int seg) {
   __shared__ uint32_t sh_cut[2];
   const int tid = threadIdx.x;
   const int j = tid & 15, rg = tid >> 4;
-  const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
-  const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
+  const int b = at.b, h = at.h, chunk = at.chunk, seg = at.seg;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
   const int64_t stride = p.chunk_len / S;
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
@@ -241,7 +270,7 @@ __device__ __forceinline__ void sample_segment(const GemvParams& p, int seg) {
 // One workgroup per segment, in a launch of its own.
 template <int DT>
 __global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
-  sample_segment<DT, false>(p, (int)blockIdx.x);
+  sample_segment<DT, false>(p, seg_position(p));
 }
 
 // One workgroup per 512 tokens (two slices of the ranking kernel's layout): scores, and the tokens at or above the
@@ -259,11 +288,30 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
   __shared__ uint32_t sh_wcnt[kTokens / kWave];
   __shared__ uint64_t sh_cutc[2];   // the cut composite, whether it has arrived
   const int tid = threadIdx.x;
-  const int segs = p.batch * p.num_kv_heads * p.num_chunks;
-  if (FRONT && (int)blockIdx.x < segs) {
-    const int seg = (int)blockIdx.x;
+  // FRONT: a flat grid, the sampling workgroups of all segments first (in a grid with the segments in y and z every
+  // segment's own would come right before its scoring workgroups - too late on calls of several generations of
+  // workgroups: 16 x 32768 tokens 56 instead of 50 us per decode step), then the scoring workgroups segment by segment
+  int pair;
+  SegPos at;
+  if (FRONT) {
+    const int segs = p.batch * p.num_kv_heads * p.num_chunks;
+    if ((int)blockIdx.x < segs) {
+      at = seg_position_flat(p, (int)blockIdx.x);
+      pair = -1;
+    } else {
+      const uint32_t wg = blockIdx.x - (uint32_t)segs, per_seg = (uint32_t)((p.chunk_len + kTokens - 1) / kTokens);
+      const uint32_t seg = (per_seg & (per_seg - 1u)) == 0u ? wg >> (31 - __builtin_clz(per_seg)) : wg / per_seg;   // (mostly a power of two)
+      at = seg_position_flat(p, (int)seg);
+      pair = (int)(wg - seg * per_seg);
+    }
+  } else {
+    at = seg_position(p);
+    pair = (int)blockIdx.x;   // this workgroup's 512 tokens inside the segment
+  }
+  const int b = at.b, h = at.h, chunk = at.chunk, seg = at.seg;
+  if (FRONT && pair < 0) {
     __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
-    sample_segment<DT, true>(p, seg);
+    sample_segment<DT, true>(p, at);
     // the part ends have completed (rank_samples) before the word that announces them leaves; relaxed device-scope
     // accesses on both sides, as for the thresholds of the candidate route: a fence would write back and invalidate
     // whole caches in the middle of the stream
@@ -272,14 +320,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
       __hip_atomic_store(p.tau_words + 2 * seg, (uint64_t)p.epoch << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (the epoch where the candidate route keeps its own)
     return;
   }
-  const uint32_t wg = blockIdx.x - (FRONT ? (uint32_t)segs : 0u);
   const int j = tid & 15, rg = tid >> 4;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int wgs_per_seg = (int)((p.chunk_len + kTokens - 1) / kTokens);
-  const int pair = (int)(wg % (uint32_t)wgs_per_seg);
-  const int seg = (int)(wg / (uint32_t)wgs_per_seg);
-  const int chunk = seg % p.num_chunks, bh = seg / p.num_chunks;
-  const int h = bh % p.num_kv_heads, b = bh / p.num_kv_heads;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
   const int n = (int)p.chunk_len;
   const int t_begin = pair * kTokens;
@@ -343,7 +384,7 @@ int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
   const int64_t wgs_per_seg = (p.chunk_len + kCutTokensPerWg - 1) / kCutTokensPerWg;
   if (!slices_ok(p) || p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
-      segs * wgs_per_seg > 0x7fffffffLL || (int64_t)p.num_kv_heads * p.num_chunks > 65535 || p.batch > 65535)
+      segs * wgs_per_seg > 0x7fffffffLL || !grid_ok(p))
     return TKA_EINVAL;
   const dim3 wgs((unsigned)wgs_per_seg, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
   const unsigned threads = (unsigned)(kCutTokensPerWg + p.num_samples) / kCutUnroll * 16;   // 16 lanes per row, 8 rows each
@@ -364,13 +405,14 @@ int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
 int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
   if (p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples || !p.cut_splits ||
-      segs > 0x7fffffffLL)
+      segs > 0x7fffffffLL || !grid_ok(p))
     return TKA_EINVAL;
+  const dim3 wgs(1u, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
   LaunchTimer timer("cut_sample", stream);
   if (dtype == TKA_F16)
-    cut_sample_kernel<TKA_F16><<<(unsigned)segs, kCutThreads, 0, stream>>>(p);
+    cut_sample_kernel<TKA_F16><<<wgs, kCutThreads, 0, stream>>>(p);
   else
-    cut_sample_kernel<TKA_BF16><<<(unsigned)segs, kCutThreads, 0, stream>>>(p);
+    cut_sample_kernel<TKA_BF16><<<wgs, kCutThreads, 0, stream>>>(p);
   return hip_status(hipGetLastError());
 }
 
@@ -378,8 +420,10 @@ int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream) {
 // sampling arguments of launch_cut_samples are then needed) instead of from a launch before it.
 int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  const int64_t wgs = segs * ((p.chunk_len + 2 * kCutTokensPerWg - 1) / (2 * kCutTokensPerWg)) + (front_sampling ? segs : 0);
-  if (!slices_ok(p) || wgs > 0x7fffffffLL) return TKA_EINVAL;
+  const int64_t wgs_per_seg = (p.chunk_len + 2 * kCutTokensPerWg - 1) / (2 * kCutTokensPerWg);
+  if (!slices_ok(p) || segs * (wgs_per_seg + 1) > 0x7fffffffLL || !grid_ok(p)) return TKA_EINVAL;
+  const dim3 wgs = front_sampling ? dim3((unsigned)(segs * (wgs_per_seg + 1)))
+                                  : dim3((unsigned)wgs_per_seg, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
   if (front_sampling && (p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
                          !p.tau_words || p.epoch == 0 || p.tau_spin_limit < 1))
     return TKA_EINVAL;
@@ -391,8 +435,8 @@ int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, 
        {gemv_cut_slices_kernel<TKA_F16, true, kLong>, gemv_cut_slices_kernel<TKA_F16, true, kShort>}},
       {{gemv_cut_slices_kernel<TKA_BF16, false, kLong>, gemv_cut_slices_kernel<TKA_BF16, false, kShort>},
        {gemv_cut_slices_kernel<TKA_BF16, true, kLong>, gemv_cut_slices_kernel<TKA_BF16, true, kShort>}}};
-  hipLaunchKernelGGL(kernels[dtype == TKA_F16 ? 0 : 1][front_sampling ? 1 : 0][p.tokens_per_wg == kShort ? 1 : 0], dim3((unsigned)wgs),
-                     dim3(kCutThreads), 0, stream, p);
+  hipLaunchKernelGGL(kernels[dtype == TKA_F16 ? 0 : 1][front_sampling ? 1 : 0][p.tokens_per_wg == kShort ? 1 : 0], wgs, dim3(kCutThreads), 0,
+                     stream, p);
   return hip_status(hipGetLastError());
 }
 
