@@ -171,11 +171,12 @@ __device__ __forceinline__ void write_union_edges(int32_t* uo, const SelectParam
 }
 
 // Rank-ordered outputs of one segment from the sorted composites in sh_sort[0 .. k).
-__device__ __forceinline__ void write_rank_outputs(const uint64_t* sh_sort, const SelectParams& p, int seg) {
+// (`chunk`: the segment's number inside its row, for a caller that has it without a division; -1: seg % p.segs_per_row)
+__device__ __forceinline__ void write_rank_outputs(const uint64_t* sh_sort, const SelectParams& p, int seg, int chunk = -1) {
   const int tid = threadIdx.x;
   const uint32_t k = (uint32_t)p.k;
   const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
-                                           : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
+                                           : (uint32_t)((chunk >= 0 ? chunk : seg % p.segs_per_row) * p.seg_len);
   int32_t* oi = p.out_idx + (int64_t)seg * p.out_stride;
   float* ov = p.out_val ? p.out_val + (int64_t)seg * p.out_stride : nullptr;
   for (uint32_t r = tid; r < k; r += kSelThreads) {
@@ -1283,15 +1284,21 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int seg = blockIdx.x;
+  // (grid: x = the segment inside its row, y = batch entry and KV head: a division by a run-time value is some
+  // twenty-five instructions, and this kernel's every instruction counts)
+  const int chunk = (int)blockIdx.x;
+  const int seg = (int)blockIdx.y * (int)gridDim.x + chunk;
   const uint32_t k = (uint32_t)p.k;
   const int64_t n = p.seg_len;
   uint32_t keys[4], vm;
   if constexpr (FROM_KEYS) {
     uint32_t* sh_key = (uint32_t*)(sh_all + kSmallMaxLen);   // (the exchange half of the buffer: free until a sort)
     const int j = tid & 15, rg = tid >> 4;
-    const int chunk = seg % g.num_chunks, bh = seg / g.num_chunks;
-    const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
+    int b = 0, h = (int)blockIdx.y;
+    if (g.batch != 1) {
+      b = (int)(blockIdx.y / (uint32_t)g.num_kv_heads);
+      h = (int)blockIdx.y - b * g.num_kv_heads;
+    }
     const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
     const uint16_t* kbase = (const uint16_t*)g.keys + (int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h +
                             chunk_base * g.key_stride_n + 8 * j;
@@ -1374,7 +1381,7 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
     }
     __syncthreads();
     sort_lds_desc(sh_all, sh_all + npad, (int)npad);
-    write_rank_outputs(sh_all, p, seg);
+    write_rank_outputs(sh_all, p, seg, chunk);
     return;
   }
 #pragma unroll
@@ -1402,7 +1409,7 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
     if (r < k) sh_sort[r] = sh_cand[i];
   }
   __syncthreads();
-  write_rank_outputs(sh_sort, p, seg);
+  write_rank_outputs(sh_sort, p, seg, chunk);
 }
 
 // Ascending duplicate-free union of the selected ids with [0,sink) and [n-local,n).
@@ -1660,10 +1667,12 @@ int launch_select_small(const SelectParams& p, hipStream_t stream) {
   if (p.seg_len > kSmallMaxLen || p.k > kSmallMaxK || p.k > p.seg_len || !p.out_idx || p.union_idx) return TKA_EINVAL;
   const int lds = 2 * kSmallMaxLen * (int)sizeof(uint64_t);
   if (allow_dynamic_lds((const void*)select_small_kernel<TKA_F16, false>, lds) != TKA_OK) return TKA_EHIP;
+  if (p.segs_per_row < 1 || p.num_segments % p.segs_per_row || p.num_segments / p.segs_per_row > 65535) return TKA_EINVAL;
+  const dim3 small_grid((unsigned)p.segs_per_row, (unsigned)(p.num_segments / p.segs_per_row));
   LaunchTimer timer("select_small", stream);
   GemvParams none;
   memset(&none, 0, sizeof none);
-  select_small_kernel<TKA_F16, false><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(none, p);
+  select_small_kernel<TKA_F16, false><<<small_grid, kSelThreads, lds, stream>>>(none, p);
   return hip_status(hipGetLastError());
 }
 
@@ -1674,11 +1683,14 @@ int launch_gemv_select_small(const GemvParams& g, const SelectParams& p, int dty
   if (allow_dynamic_lds((const void*)select_small_kernel<TKA_F16, true>, lds) != TKA_OK ||
       allow_dynamic_lds((const void*)select_small_kernel<TKA_BF16, true>, lds) != TKA_OK)
     return TKA_EHIP;
+  if (p.segs_per_row != g.num_chunks || p.num_segments != g.batch * g.num_kv_heads * g.num_chunks || p.num_segments / p.segs_per_row > 65535)
+    return TKA_EINVAL;
+  const dim3 small_grid((unsigned)p.segs_per_row, (unsigned)(p.num_segments / p.segs_per_row));
   LaunchTimer timer("gemv_select_small", stream);
   if (dtype == TKA_F16)
-    select_small_kernel<TKA_F16, true><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p);
+    select_small_kernel<TKA_F16, true><<<small_grid, kSelThreads, lds, stream>>>(g, p);
   else
-    select_small_kernel<TKA_BF16, true><<<(unsigned)p.num_segments, kSelThreads, lds, stream>>>(g, p);
+    select_small_kernel<TKA_BF16, true><<<small_grid, kSelThreads, lds, stream>>>(g, p);
   return hip_status(hipGetLastError());
 }
 
