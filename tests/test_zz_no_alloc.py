@@ -87,6 +87,47 @@ def test_noalloc_step_matches_the_workspace_form_on_calls_in_a_row():
         _one_case(rng, dtype, B, H, G, N, k, sink, local, kind)
 
 
+@pytest.mark.gpu
+def test_noalloc_step_without_list_outputs():
+    """The production form (attention output only, no token list asked for) on the routes it opens: a few segments of
+    middling length where the ranking workgroups hand the list to the attention themselves - one segment, then four
+    (whose GEMV launch announces the cuts to its own workgroups through words of the scratch buffer), then a smaller
+    input.  Output and rank-ordered top-k of the two entry points bit for bit, the top-k as the oracle's."""
+    lib = L.lib()
+    rng = np.random.default_rng(2025)
+    for dtype, B, H, G, N, k, sink, local in [(oracle.F16, 1, 1, 8, 32768, 2048, 64, 512), (oracle.BF16, 1, 4, 4, 32768, 2048, 64, 512),
+                                              (oracle.F16, 2, 1, 2, 20000, 1200, 0, 100)]:
+        announce("sparse_decode_step_noalloc vs sparse_decode_step, no list outputs: dtype=%d B=%d H=%d G=%d N=%d k=%d" % (dtype, B, H, G, N, k))
+        qb, Kb, Vb = randn_bits(rng, (B, H * G, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype), randn_bits(rng, (B, N, H, 128), dtype)
+        q, K, V = to_dev(qb, dtype), to_dev(Kb, dtype), to_dev(Vb, dtype)
+        outs = []
+        for noalloc in (False, True):
+            out = torch.full((B, H * G, 128), 7.0, dtype=torch.float16, device="cuda")
+            tidx = torch.full((B, H, k), -7, dtype=torch.int32, device="cuda")
+            tval = torch.full((B, H, k), -7.0, dtype=torch.float32, device="cuda")
+            a = _args(q, K, V, out, k, sink, local, G, tidx, tval, tidx, tidx)
+            a.out_union_idx, a.out_union_count = None, None
+            if noalloc:
+                a.workspace, a.workspace_bytes = None, 0
+                L.check(lib.tka_sparse_decode_step_noalloc(C.byref(a)), "tka_sparse_decode_step_noalloc")
+            else:
+                need = lib.tka_sparse_decode_workspace_bytes(C.byref(a))
+                assert 0 < need <= L.TKA_NOALLOC_SCRATCH_BYTES
+                ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+                a.workspace, a.workspace_bytes = ws.data_ptr(), need
+                L.check(lib.tka_sparse_decode_step(C.byref(a)), "tka_sparse_decode_step")
+            torch.cuda.synchronize()
+            outs.append((out, tidx, tval))
+        for name, r, g in zip(("out", "topk_idx", "topk_val"), outs[0], outs[1]):
+            assert torch.equal(r.contiguous().view(torch.uint8), g.contiguous().view(torch.uint8)), "%s differs between the two entry points" % name
+        tidx, outf = outs[1][1].cpu().numpy(), outs[1][0].float().cpu().numpy()
+        for b in range(B):
+            for h in range(H):
+                ro, ri, rv, ru = oracle.sparse_decode_step(qb[b, h * G:(h + 1) * G], Kb[b, :, h], Vb[b, :, h], dtype, G, k, sink, local, SCALE)
+                assert np.array_equal(tidx[b, h], ri)
+                assert (np.abs(outf[b, h * G:(h + 1) * G] - ro) < 2e-3).all()
+
+
 def test_noalloc_step_rejects_what_does_not_fit():
     """Batch 16 of the 128k configuration needs 203 MiB of scratch: refused with TKA_ESCRATCH before any HIP call
     (so this runs without a GPU)."""
