@@ -137,7 +137,9 @@ typedef struct tka_test_hooks {
   int32_t tau_withhold_mod;    /* > 0: the threshold of segments s with s % mod == rem is withheld ...   */
   int32_t tau_withhold_rem;
   int32_t tau_withhold_mode;   /* ... 0: for good (every slice of the segment gives up); 1: until the
-                                  first slice of the segment has given up (the later ones see it)       */
+                                  first slice of the segment has given up (the later ones see it).  On
+                                  calls that announce the CUT of a segment of up to 65536 tokens inside
+                                  the GEMV launch the same hooks withhold that word, always for good     */
   int32_t union_handoff_order; /* 1: tka_sparse_decode_step writes out_union_idx the way it hands the list to
                                   its attention when the caller does not ask for it: in the order of the
                                   route, which may list -1 (an id the attention skips) inside the count  */
