@@ -485,7 +485,7 @@ def test_common_cut_route_ties_and_clusters(kind, heads):
 def _cut_sample_positions(seg, n):
     """Token positions of the 256 sample rows of a segment on the common-cut route."""
     stride = n // 256
-    return [i * stride + ((_mix32((seg * 0x9e3779b9 + i) & 0xFFFFFFFF) * stride) >> 32) for i in range(256)]
+    return [i * stride + (((((i + seg * 0x85ebca6b) & 0xFFFFFFFF) * 0x9e3779b9) & 0xFFFFFFFF) * stride >> 32) for i in range(256)]
 
 
 def test_common_cut_route_adversarial_sample_falls_back():

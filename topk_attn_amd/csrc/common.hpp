@@ -211,6 +211,13 @@ __device__ __forceinline__ int64_t sample_token(int seg, int i, int64_t stride) 
   return (int64_t)i * stride + (int64_t)__umulhi(mix32((uint32_t)seg * 0x9e3779b9u + (uint32_t)i), (uint32_t)stride);
 }
 
+// The same for the common-cut route, whose kernels are a few microseconds long and pay for every instruction: the
+// offset inside the stride is the fractional part of a multiple of the golden ratio (a sequence that fills the stride
+// evenly), shifted per segment - three instructions instead of the hash's ten.
+__device__ __forceinline__ int64_t cut_sample_token(int seg, int i, int64_t stride) {
+  return (int64_t)i * stride + (int64_t)__umulhi(((uint32_t)i + (uint32_t)seg * 0x85ebca6bu) * 0x9e3779b9u, (uint32_t)stride);
+}
+
 // ---- block-wide threshold search (1024 threads, 2048 bins) --------------------------------------
 
 // Finds the bin d with  count(bins > d) < need <= count(bins >= d)  in sh_hist[2048]; every one of the 1024

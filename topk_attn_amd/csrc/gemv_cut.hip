@@ -62,7 +62,7 @@ __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint
 #pragma unroll
     for (uint32_t gq = 1; gq <= (uint32_t)kCutParts; ++gq) part = r == rank * gq / (uint32_t)kCutParts ? gq : part;
     if (part != 0) {   // (R >= 8: every part has a sample of its own)
-      const uint32_t token = (uint32_t)sample_token(seg, tid, stride);
+      const uint32_t token = (uint32_t)cut_sample_token(seg, tid, stride);
       if (part == (uint32_t)kCutParts) { sh_cut[0] = sh_skey[tid]; sh_cut[1] = token; }
       if (ANNOUNCED) {
         __hip_atomic_store(splits + (int64_t)seg * kCutParts + (part - 1), composite(sh_skey[tid], token), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -187,7 +187,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   if (sampler) {
 #pragma unroll
     for (int u = 0; u < kCutUnroll; ++u)
-      kv[u] = *(const u32x4*)(kbase + sample_token(seg, (rg * kCutUnroll + u) & (kCutSamples - 1), stride) * p.key_stride_n);
+      kv[u] = *(const u32x4*)(kbase + cut_sample_token(seg, (rg * kCutUnroll + u) & (kCutSamples - 1), stride) * p.key_stride_n);
   } else {
 #pragma unroll
     for (int u = 0; u < kCutUnroll; ++u) {
@@ -245,7 +245,7 @@ __device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos
                           chunk_base * p.key_stride_n + 8 * j;
   u32x4 kv[kRows];
 #pragma unroll
-  for (int u = 0; u < kRows; ++u) kv[u] = *(const u32x4*)(kbase + sample_token(seg, rg * kRows + u, stride) * p.key_stride_n);
+  for (int u = 0; u < kRows; ++u) kv[u] = *(const u32x4*)(kbase + cut_sample_token(seg, rg * kRows + u, stride) * p.key_stride_n);
   __builtin_amdgcn_sched_barrier(0);
   float qf[8];
   load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
