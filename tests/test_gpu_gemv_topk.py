@@ -482,10 +482,10 @@ def test_common_cut_route_ties_and_clusters(kind, heads):
     _check_long(K, q, dtype, 1, k, scale=1.0, redone=0)
 
 
-def _cut_sample_positions(seg, n):
-    """Token positions of the 256 sample rows of a segment on the common-cut route."""
-    stride = n // 256
-    return [i * stride + (((((i + seg * 0x85ebca6b) & 0xFFFFFFFF) * 0x9e3779b9) & 0xFFFFFFFF) * stride >> 32) for i in range(256)]
+def _cut_sample_positions(seg, n, samples=256):
+    """Token positions of the sample rows of a segment on the common-cut route."""
+    stride = n // samples
+    return [i * stride + (((((i + seg * 0x85ebca6b) & 0xFFFFFFFF) * 0x9e3779b9) & 0xFFFFFFFF) * stride >> 32) for i in range(samples)]
 
 
 def test_common_cut_route_adversarial_sample_falls_back():

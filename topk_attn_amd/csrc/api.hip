@@ -242,11 +242,11 @@ void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, 
   *num_samples = *sample_rank = 0;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
   if ((!a->out_idx && !u) || (u && !u->handoff) || a->out_scores || chunk_len < cut_route_min_len()) return;
+  const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   int s = 0, r = 0, len = 0;
-  gemv_cut_plan(chunk_len, a->k, &s, &r, &len);
+  gemv_cut_plan(chunk_len, a->k, rows > cut_split_min_rows(), &s, &r, &len);
   if (s == 0) return;
   if (slice_len) *slice_len = len;
-  const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   // Measured, decode steps with k = 2048 unless said (us per step, this route against the others): 1 x 32768 tokens
   // 23.6 / 32.2, 4 x 32768 26.7 / 37.5, 8 x 32768 33.7 / 43.4, 16 x 32768 50.4 / 56.9, 24 x 32768 63.8 / 68.3,
   // 8 x 49152 42.9 / 51.8, 16 x 20000 (k = 1000) 37.0 / 46.7, 32 x 20000 54.4 / 58.4, 32 x 24576 (k = 1536) 66.5 / 67.7,

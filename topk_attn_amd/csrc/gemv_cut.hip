@@ -27,10 +27,10 @@ namespace {
 constexpr int kCutThreads = 1024;
 constexpr int kCutUnroll = 8;                                        // rows per lane
 
-// Ranks of the S samples of a segment by counting, on 4 S threads (all threads of the workgroup call; sh_rank must be
-// zero and the keys in place behind a barrier): thread (s, q) counts the samples of block q (a quarter of them,
-// broadcast reads) that come before sample s, four threads per sample add up in LDS.  The order is that of the ranking
-// keys (the key with its last 8 bits replaced by S - 1 - sample number): all different, so one compare decides, exactly
+// Ranks of the S samples of a segment by counting, on the workgroup's 1024 threads (sh_rank must be zero and the keys in
+// place behind a barrier): thread (s, q) counts the samples of block q (a quarter or a half of them, broadcast reads)
+// that come before sample s, the threads of a sample add up in LDS.  The order is that of the ranking keys (the key
+// with its last bits replaced by S - 1 - sample number, see ranking_key): all different, so one compare decides, exactly
 // one sample holds rank R - 1, and samples that share a key (heavy ties) come in token order, as in the full order (key
 // descending, token ascending).  Keys that differ in their last 8 bits only may change places; any sample will do as
 // the cut, it is its rank among the samples that makes the number of candidates what was planned.
@@ -39,17 +39,24 @@ constexpr int kCutUnroll = 8;                                        // rows per
 // composites when that is not null (the last one is the cut).  No barrier behind the last write.
 // ANNOUNCED: other workgroups of the same launch are going to read `splits` (see gemv_cut_slices_kernel): the stores go
 // to where every CU sees them and have got there when this function returns.
+template <int S>
+__device__ __forceinline__ uint32_t ranking_key(uint32_t key, int i) {
+  return (key & ~(uint32_t)(S - 1)) | (uint32_t)(S - 1 - i);
+}
+
 template <int S, bool ANNOUNCED = false>
 __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint32_t* sh_rkey, uint32_t* sh_rank, uint32_t* sh_cut, int seg,
                                              int64_t stride, uint32_t rank, uint64_t* splits) {
   const int tid = threadIdx.x;
-  if (tid < 4 * S) {
+  constexpr int kShare = kCutThreads / S;   // threads per sample: 4 (S = 256) or 2 (S = 512), each with 1 / kShare of the samples
+  static_assert(kShare * S == kCutThreads && (S / kShare) % 4 == 0, "all threads count");
+  {
     const int s = tid & (S - 1), q = tid / S;   // q is the same for a whole wave
     const uint32_t ks = sh_rkey[s];
-    const u32x4* blk = (const u32x4*)(sh_rkey + q * (S / 4));
+    const u32x4* blk = (const u32x4*)(sh_rkey + q * (S / kShare));
     uint32_t ahead = 0;
-#pragma unroll
-    for (int i = 0; i < S / 16; ++i) {
+#pragma unroll 16
+    for (int i = 0; i < S / kShare / 4; ++i) {
       const u32x4 kj = blk[i];
       ahead += (kj[0] > ks ? 1u : 0u) + (kj[1] > ks ? 1u : 0u) + (kj[2] > ks ? 1u : 0u) + (kj[3] > ks ? 1u : 0u);
     }
@@ -209,7 +216,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
     const int row = rg * kCutUnroll + j;
     const uint32_t key = score_key(mine);
     sh_key[row] = key;
-    if (sampler) sh_rkey[row - kCutTokensPerWg] = (key & ~0xffu) | (uint32_t)(kCutSamples - 1 - (row - kCutTokensPerWg));
+    if (sampler) sh_rkey[row - kCutTokensPerWg] = ranking_key<S>(key, row - kCutTokensPerWg);
   }
   if (tid < kCutSamples) sh_rank[tid] = 0;
   __syncthreads();
@@ -227,11 +234,14 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
 // launch.  Then one workgroup per segment finds the cut and the part ends (sample_segment), and the GEMV workgroups
 // read them (gemv_cut_slices_kernel: 512 tokens, two slices, per workgroup, nothing scored twice).
 
-// The work of one workgroup for one segment's cut: the 256 sample rows (64 row groups, four rows per lane), their
-// ranks, cut and part ends (to p.cut_splits).  Every thread of the 1024 calls it.
+// The work of one workgroup for one segment's cut: the kCutSamplesOnce sample rows (64 row groups, four rows per lane),
+// their ranks, cut and part ends (to p.cut_splits).  Every thread of the 1024 calls it.  (With 512 samples the cut sits
+// tighter - a fifth fewer candidates - and the part ends are steadier, eight samples per part instead of five; but the
+// scoring workgroups wait for this one, and its longer counting cost them more than the ranking kernel gained: 8 x 32768
+// tokens 37.8 instead of 33.9 us per decode step.)
 template <int DT, bool ANNOUNCED>
 __device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos& at) {
-  constexpr int S = 256, kRows = S / (kCutThreads / 16);   // four rows per lane
+  constexpr int S = kCutSamplesOnce, kRows = S / (kCutThreads / 16);
   __shared__ uint32_t sh_skey[S];
   __shared__ __attribute__((aligned(16))) uint32_t sh_rkey[S];
   __shared__ uint32_t sh_rank[S];
@@ -260,7 +270,7 @@ __device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos
     const int i = rg * kRows + j;
     const uint32_t key = score_key(mine);
     sh_skey[i] = key;
-    sh_rkey[i] = (key & ~0xffu) | (uint32_t)(S - 1 - i);
+    sh_rkey[i] = ranking_key<S>(key, i);
   }
   if (tid < S) sh_rank[tid] = 0;
   __syncthreads();
@@ -404,8 +414,8 @@ int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
 // as launch_gemv_cut.
 int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  if (p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples || !p.cut_splits ||
-      segs > 0x7fffffffLL || !grid_ok(p))
+  if (p.num_samples != kCutSamplesOnce || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
+      !p.cut_splits || segs > 0x7fffffffLL || !grid_ok(p))
     return TKA_EINVAL;
   const dim3 wgs(1u, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
   LaunchTimer timer("cut_sample", stream);
@@ -424,7 +434,7 @@ int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, 
   if (!slices_ok(p) || segs * (wgs_per_seg + 1) > 0x7fffffffLL || !grid_ok(p)) return TKA_EINVAL;
   const dim3 wgs = front_sampling ? dim3((unsigned)(segs * (wgs_per_seg + 1)))
                                   : dim3((unsigned)wgs_per_seg, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
-  if (front_sampling && (p.num_samples != 256 || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
+  if (front_sampling && (p.num_samples != kCutSamplesOnce || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
                          !p.tau_words || p.epoch == 0 || p.tau_spin_limit < 1))
     return TKA_EINVAL;
   LaunchTimer timer("gemv_cut_slices", stream);
@@ -450,10 +460,10 @@ int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, 
 // still has no more than kCutMaxSlices of them), and a segment within what it ranks in one go.
 // (With 64 samples - enough for a small k on segments of a few thousand rows - the route was measured too: 32 x 4096
 // rows, k = 64: 19.5 us against 13.3 on the route that selects in the registers of one workgroup per segment.)
-void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank, int* slice_len) {
+void gemv_cut_plan(int64_t chunk_len, int k, bool sampled_once, int* num_samples, int* sample_rank, int* slice_len) {
   *num_samples = *sample_rank = *slice_len = 0;
   if (chunk_len < 2048 || chunk_len > (int64_t)kCutMaxSlices * kCutTokensPerWg || k > kCutMaxK || (int64_t)k * 8 > chunk_len) return;
-  const int s = 256;
+  const int s = sampled_once ? kCutSamplesOnce : 256;   // (one workgroup per segment scores the sample, or every workgroup does)
   const double m = (double)k * s / (double)chunk_len;
   int r = (int)ceil(m + 5.5 * sqrt(m) + 2.0);
   if (r < kCutParts) r = kCutParts;

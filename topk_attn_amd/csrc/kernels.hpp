@@ -60,7 +60,8 @@ int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream);
 // GEMV workgroups (512 tokens each) score nothing twice.
 int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream);
 int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream);
-void gemv_cut_plan(int64_t chunk_len, int k, int* num_samples, int* sample_rank, int* slice_len);
+// sampled_once: the plan for launch_cut_samples / launch_gemv_cut_slices (kCutSamplesOnce samples) instead of launch_gemv_cut (256).
+void gemv_cut_plan(int64_t chunk_len, int k, bool sampled_once, int* num_samples, int* sample_rank, int* slice_len);
 
 // ---- stage 1: selection -----------------------------------------------------------------------
 struct SelectParams {
