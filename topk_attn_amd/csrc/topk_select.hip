@@ -972,12 +972,14 @@ __device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_
   typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
   const u64x2* heads = (const u64x2*)heads_flat;
   const int tid = threadIdx.x, lane = tid & 63;
-  uint64_t sizes = 0;   // eight counts of 8 bits (a thread sees 24 entries at most)
+  static_assert(kCutParts % 8 == 0, "eight counts per word");
+  uint64_t sizes[kCutParts / 8] = {};   // counts of 8 bits (a thread sees 24 entries at most)
   auto count = [&](uint64_t x) {
     uint32_t below = 0;
 #pragma unroll
     for (int i = 1; i < kCutParts; ++i) below += x < sh_split[i] ? 1u : 0u;
-    sizes += x != 0ull ? 1ull << (8 * below) : 0ull;
+#pragma unroll
+    for (int w = 0; w < kCutParts / 8; ++w) sizes[w] += x != 0ull && (int)(below >> 3) == w ? 1ull << (8 * (below & 7u)) : 0ull;
   };
 #pragma unroll 1
   for (int q = tid; q < n_pairs; q += kSelThreads) {
@@ -991,7 +993,8 @@ __device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_
   }
 #pragma unroll
   for (int i = 0; i < kCutParts / 2; ++i) {   // two parts per word, 16 bits each (at most 24 x 64 per wave)
-    const uint32_t one = (uint32_t)(sizes >> (16 * i)) & 0xffu, other = (uint32_t)(sizes >> (16 * i + 8)) & 0xffu;
+    const uint64_t word = sizes[i / 4];
+    const uint32_t one = (uint32_t)(word >> (16 * (i % 4))) & 0xffu, other = (uint32_t)(word >> (16 * (i % 4) + 8)) & 0xffu;
     const uint32_t inc = wave_inclusive_scan(one | (other << 16));
     if (lane == 63) {
       atomicAdd(&sh_words[2 * i], inc & 0xffffu);
