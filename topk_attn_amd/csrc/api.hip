@@ -151,6 +151,7 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->tau_spin_limit = kTauSpinLimit;
   g->withhold_mod = g->withhold_rem = g->withhold_mode = 0;
   g->num_samples = g->sample_rank = g->sample_wgs = g->early_wgs = 0;
+  g->split_ranks = 0;
   g->cand = nullptr;
   g->cand_seg_stride = 0;
   g->cand_head = nullptr;
@@ -342,6 +343,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     cp.wgs_per_chunk = (int)((chunk_len + cut_slice_len - 1) / cut_slice_len);
     cp.num_samples = cut_samples;
     cp.sample_rank = cut_rank;
+    cp.split_ranks = gemv_cut_split_ranks(chunk_len, a->k, cut_samples, cut_rank);
     cp.cand = sp.list;
     cp.cand_seg_stride = sp.list_stride;
     cp.cand_head = const_cast<uint64_t*>(sp.cand_head);

@@ -34,9 +34,10 @@ constexpr int kCutUnroll = 8;                                        // rows per
 // one sample holds rank R - 1, and samples that share a key (heavy ties) come in token order, as in the full order (key
 // descending, token ascending).  Keys that differ in their last 8 bits only may change places; any sample will do as
 // the cut, it is its rank among the samples that makes the number of candidates what was planned.
-// The sample of rank R is the cut (sh_cut: its key and token); the samples of ranks R g / 8 split the candidates into
-// eight parts of about equal size for the ranking kernel's eight workgroups per segment, and go to `splits` as
-// composites when that is not null (the last one is the cut).  No barrier behind the last write.
+// The sample of rank R is the cut (sh_cut: its key and token); the samples whose ranks the bytes of `ranks` name (the last
+// one is R, see gemv_cut_split_ranks) split the candidates into eight parts for the ranking kernel's eight workgroups
+// per segment, and go to `splits` as composites when that is not null (the last one is the cut).  No barrier behind
+// the last write.
 // ANNOUNCED: other workgroups of the same launch are going to read `splits` (see gemv_cut_slices_kernel): the stores go
 // to where every CU sees them and have got there when this function returns.
 template <int S>
@@ -46,7 +47,7 @@ __device__ __forceinline__ uint32_t ranking_key(uint32_t key, int i) {
 
 template <int S, bool ANNOUNCED = false>
 __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint32_t* sh_rkey, uint32_t* sh_rank, uint32_t* sh_cut, int seg,
-                                             int64_t stride, uint32_t rank, uint64_t* splits) {
+                                             int64_t stride, uint64_t ranks, uint64_t* splits) {
   const int tid = threadIdx.x;
   constexpr int kShare = kCutThreads / S;   // threads per sample: 4 (S = 256) or 2 (S = 512), each with 1 / kShare of the samples
   static_assert(kShare * S == kCutThreads && (S / kShare) % 4 == 0, "all threads count");
@@ -67,8 +68,8 @@ __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint
     const uint32_t r = sh_rank[tid] + 1u;   // 1-based
     uint32_t part = 0;   // 1 .. 8 when this sample ends part `part` of the candidates (8: the cut itself)
 #pragma unroll
-    for (uint32_t gq = 1; gq <= (uint32_t)kCutParts; ++gq) part = r == rank * gq / (uint32_t)kCutParts ? gq : part;
-    if (part != 0) {   // (R >= 8: every part has a sample of its own)
+    for (uint32_t gq = 1; gq <= (uint32_t)kCutParts; ++gq) part = r == ((uint32_t)(ranks >> (8 * (gq - 1))) & 0xffu) ? gq : part;
+    if (part != 0) {   // (the ranks are all different: every part has a sample of its own)
       const uint32_t token = (uint32_t)cut_sample_token(seg, tid, stride);
       if (part == (uint32_t)kCutParts) { sh_cut[0] = sh_skey[tid]; sh_cut[1] = token; }
       if (ANNOUNCED) {
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
   if (tid < kCutSamples) sh_rank[tid] = 0;
   __syncthreads();
 
-  rank_samples<S>(sh_key + kCutTokensPerWg, sh_rkey, sh_rank, sh_cut, seg, stride, (uint32_t)p.sample_rank, slice == 0 ? p.cut_splits : nullptr);
+  rank_samples<S>(sh_key + kCutTokensPerWg, sh_rkey, sh_rank, sh_cut, seg, stride, p.split_ranks, slice == 0 ? p.cut_splits : nullptr);
   __syncthreads();
   if (tid >= kCutTokensPerWg) return;
 
@@ -274,7 +275,7 @@ __device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos
   }
   if (tid < S) sh_rank[tid] = 0;
   __syncthreads();
-  rank_samples<S, ANNOUNCED>(sh_skey, sh_rkey, sh_rank, sh_cut, seg, stride, (uint32_t)p.sample_rank, p.cut_splits);
+  rank_samples<S, ANNOUNCED>(sh_skey, sh_rkey, sh_rank, sh_cut, seg, stride, p.split_ranks, p.cut_splits);
 }
 
 // One workgroup per segment, in a launch of its own.
@@ -474,6 +475,31 @@ void gemv_cut_plan(int64_t chunk_len, int k, bool sampled_once, int* num_samples
   *num_samples = s;
   *sample_rank = r;
   *slice_len = len;
+}
+
+// Ranks (1-based, among the samples in descending order) of the samples that end the kCutParts parts of a segment's
+// candidates, one per byte.  Only the parts that reach into the top k are ranked at all, and the top k ends near sample
+// rank m = k S / n, far above the cut at rank R: seven parts share the ranks up to m + 2 sqrt(m) + 1 evenly, and the
+// last part takes the rest down to the cut - it is ranked in one call in fifty (the k-th token two deviations below
+// its expected place among the samples).  Splitting all R ranks evenly left five of the eight ranking workgroups
+// without work and gave the others parts of twice the size.
+uint64_t gemv_cut_split_ranks(int64_t chunk_len, int k, int num_samples, int sample_rank) {
+  static_assert(kCutParts == 8, "one byte per part");
+  const double m = (double)k * num_samples / (double)chunk_len;
+  int upper = (int)ceil(m + 2.0 * sqrt(m) + 1.0);
+  if (upper > sample_rank - 1) upper = sample_rank - 1;
+  if (upper < kCutParts - 1) upper = kCutParts - 1;
+  uint64_t ranks = 0;
+  int last = 0;
+  for (int g = 1; g < kCutParts; ++g) {
+    int r = (upper * g + (kCutParts - 2)) / (kCutParts - 1);   // ceil(upper g / 7)
+    if (r <= last) r = last + 1;
+    last = r;
+    ranks |= (uint64_t)r << (8 * (g - 1));
+  }
+  // (sample_rank >= kCutParts and upper <= sample_rank - 1: the last of the seven lies below sample_rank)
+  ranks |= (uint64_t)sample_rank << (8 * (kCutParts - 1));
+  return ranks;
 }
 
 }  // namespace tka

@@ -27,6 +27,8 @@ struct GemvParams {
   // (mode 0) or published only once a slice of the segment has given up, after a bounded wait (mode 1); 0 = off
   int withhold_mod, withhold_rem, withhold_mode;
   int num_samples, sample_rank;   // per segment
+  uint64_t split_ranks;       // common-cut route: byte g - 1 holds the 1-based rank of the sample that ends part g of the candidates
+                              // (ascending; byte kCutParts - 1 equals sample_rank), see gemv_cut_split_ranks
   int sample_wgs;             // sampling workgroups at the front of the candidate grid (set by the launcher)
   int early_wgs;              // streaming workgroups behind them that take several slices each (set by the launcher)
   uint64_t* cand;             // [segments][wgs_per_chunk][tokens_per_wg] one slice per workgroup, ascending index:
@@ -62,6 +64,7 @@ int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream);
 int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream);
 // sampled_once: the plan for launch_cut_samples / launch_gemv_cut_slices (kCutSamplesOnce samples) instead of launch_gemv_cut (256).
 void gemv_cut_plan(int64_t chunk_len, int k, bool sampled_once, int* num_samples, int* sample_rank, int* slice_len);
+uint64_t gemv_cut_split_ranks(int64_t chunk_len, int k, int num_samples, int sample_rank);
 
 // ---- stage 1: selection -----------------------------------------------------------------------
 struct SelectParams {

@@ -949,6 +949,20 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
 
 // ---- ranking of the common-cut route ---------------------------------------------------------------
 
+// One lane's add to a 64-bit word in LDS, returning the word's old value.  (Written out: around an atomic that one lane of
+// a wave executes the compiler builds its wave-wide aggregation - three loops over the active lanes - and this kernel
+// pays for every instruction sixteen times.)
+__device__ __forceinline__ uint64_t lds_add_rtn_u64(uint64_t* word, uint64_t v) {
+  uint64_t old;
+  const uint32_t offset = (uint32_t)(uintptr_t)word;   // (the low half of a shared-memory address is its place in LDS)
+  asm volatile("ds_add_rtn_u64 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=v"(old) : "v"(offset), "v"(v) : "memory");
+  return old;
+}
+__device__ __forceinline__ void lds_max_u32(uint32_t* word, uint32_t v) {
+  const uint32_t offset = (uint32_t)(uintptr_t)word;
+  asm volatile("ds_max_u32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(offset), "v"(v) : "memory");
+}
+
 constexpr uint32_t kCutBucketMax = 192;   // a bucket with more members than this sends the part to the sorting network
 
 // Rank-ordered outputs of one candidate: index, value and expansion at position `rank` of segment `seg`.
@@ -962,13 +976,14 @@ __device__ __forceinline__ void write_ranked(const SelectParams& p, int seg, uin
   }
 }
 
-// Size of the largest of the kCutParts parts of a segment's candidates: `pairs` pairs of head entries (zeros are no
+// Size of the largest of those of the kCutParts parts of a segment's candidates that reach into the top k (the parts
+// with fewer than k candidates above them; the others are never ranked): `pairs` pairs of head entries (zeros are no
 // candidates), `n_extra` entries from beyond the heads, sh_split[1 .. kCutParts - 1] the inner ends of the parts in
 // descending order.  sh_words: kCutParts words that are zero on entry and on exit.  Every thread of the workgroup calls it.
 // Kept out of line: it runs when a segment has more candidates than one part may hold, which is rare, and the kernel
 // around it is one whose every instruction counts.
 __device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_pairs, const uint64_t* extra, uint32_t n_extra,
-                                              const uint64_t* sh_split, uint32_t* sh_words) {
+                                              const uint64_t* sh_split, uint32_t* sh_words, uint32_t k) {
   typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
   const u64x2* heads = (const u64x2*)heads_flat;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1002,9 +1017,13 @@ __device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_
     }
   }
   __syncthreads();
-  uint32_t largest = 0;
+  uint32_t largest = 0, above = 0;
 #pragma unroll
-  for (int i = 0; i < kCutParts; ++i) largest = max(largest, sh_words[i]);
+  for (int i = 0; i < kCutParts; ++i) {
+    const uint32_t size = sh_words[i];
+    largest = above < k ? max(largest, size) : largest;
+    above += size;
+  }
   __syncthreads();
   if (tid < kCutParts) sh_words[tid] = 0;
   __syncthreads();
@@ -1012,7 +1031,8 @@ __device__ __noinline__ uint32_t largest_part(const uint64_t* heads_flat, int n_
 }
 
 // Common-cut route: the slices (256 tokens each, written by gemv_cut_kernel) hold every token at or above the
-// segment's cut, as composites, and kCutParts sample composites split the order into parts of about equal size.
+// segment's cut, as composites, and kCutParts sample composites split the order into parts: seven of about equal size
+// that cover the top k with some room, and the rest down to the cut (gemv_cut_split_ranks).
 // kCutParts workgroups per segment (one CU executes 64 lane-operations per cycle, and this is a kernel of a few
 // workgroups: what one workgroup would spend on all candidates is the kernel's duration).  Each reads the head
 // entries of ALL slices (a dense array, zeros behind a slice's last candidate) and the slice counts in one round
@@ -1045,9 +1065,9 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   __shared__ uint64_t sh_mm[3];
   __shared__ uint64_t sh_split[kCutParts + 1];
   __shared__ uint32_t sh_ovf[kCutMaxSlices];
-  __shared__ uint32_t sh_n[8];   // [0] slices with more than kCutHead entries, [1] entries beyond the heads, [2] candidates,
-                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part, [6] its largest key,
-                                 // [7] slices whose workgroup gave up waiting for the cut
+  __shared__ __attribute__((aligned(8))) uint32_t sh_n[8];   // [0] slices with more than kCutHead entries, [1] entries beyond the heads, [2] candidates,
+                                 // [3] a bucket too large, [4] candidates above the part, [5] candidates of the part (one 64-bit word
+                                 // with [4]), [6] the largest key, [7] slices whose workgroup gave up waiting for the cut
 
   typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
   constexpr int kPairs = PAIRS;
@@ -1056,9 +1076,15 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  // (grid: x = chunk and part, y = batch entry and KV head: no division by a run-time value anywhere on the straight path)
-  const int chunk = (int)(blockIdx.x / (uint32_t)kCutParts), part = (int)(blockIdx.x % (uint32_t)kCutParts);
-  const int seg = (int)blockIdx.y * p.segs_per_row + chunk;
+  // Grid: workgroups go to the eight XCDs in turn, and every workgroup of a segment reads all of the segment's candidates,
+  // which the GEMV launch left in memory - with workgroup w on XCD w % 8, the eight of a segment are given numbers that
+  // put them on one XCD, whose L2 they share (sixty-four workgroups of eight segments: 1.1 us less than with every XCD
+  // fetching every segment).  The grid is rounded up to whole groups of eight segments; the workgroups of the others leave.
+  static_assert(kCutParts == 8, "a segment's workgroups: one per step of eight in the grid");
+  const int part = (int)(blockIdx.x >> 3) & 7;
+  const int seg = (int)((blockIdx.x >> 6) << 3 | (blockIdx.x & 7u));
+  if (seg >= p.num_segments) return;
+  const int chunk = p.segs_per_row == 1 ? 0 : seg % p.segs_per_row;   // (a division only where a call has chunks)
   const uint32_t k = (uint32_t)p.k;
   const u64x2* heads = (const u64x2*)(p.cand_head + (int64_t)seg * p.parts * kCutHead);
   const int n_pairs = p.parts * (kCutHead / 2);
@@ -1093,6 +1119,10 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   // (the slice of a workgroup that never saw its segment's cut holds no candidates)
   if (ANNOUNCED && slice_cnt == kCutGaveUp) atomicAdd(&sh_n[7], 1u);
   else if (slice_cnt > (uint32_t)kCutHead) sh_ovf[atomicAdd(&sh_n[0], 1u)] = (uint32_t)tid | (slice_cnt << 16);
+  if ((tid & ~63) < p.parts) {   // the segment's candidates: the sum of the slice counts, in the waves that hold them
+    const uint32_t total = wave_inclusive_scan(ANNOUNCED && slice_cnt == kCutGaveUp ? 0u : slice_cnt);
+    if (lane == 63) atomicAdd(&sh_n[2], total);
+  }
   __syncthreads();
   const uint32_t n_ovf = sh_n[0];
   if (n_ovf) {   // rare: slices whose candidates go beyond the head entries (scores that cluster in one place)
@@ -1116,55 +1146,65 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     c[2 * e + 1] = w[e][1];
   }
 #pragma unroll
-  for (int e = 0; e < kCutMaxExtras / kSelThreads; ++e) {
-    const uint32_t i = (uint32_t)e * kSelThreads + tid;
-    c[2 * kPairs + e] = (n_ovf && i < n_extra && i < (uint32_t)kCutMaxExtras) ? sh_extra[i] : 0ull;
+  for (int e = 0; e < kCutMaxExtras / kSelThreads; ++e) c[2 * kPairs + e] = 0ull;
+  if (n_ovf) {
+#pragma unroll
+    for (int e = 0; e < kCutMaxExtras / kSelThreads; ++e) {
+      const uint32_t i = (uint32_t)e * kSelThreads + tid;
+      if (i < n_extra && i < (uint32_t)kCutMaxExtras) c[2 * kPairs + e] = sh_extra[i];
+    }
+    __syncthreads();   // the extras are in registers: their place becomes the bucket-ordered part
   }
-  if (n_ovf) __syncthreads();   // the extras are in registers: their place becomes the bucket-ordered part
 
-  // all candidates, those above this part, those of the part (collected in LDS), the part's largest key
+  // the candidates above this part, those of the part (marked here, collected below once the part is known to be ranked:
+  // one add per wave gives them their places - an add per candidate on one LDS word is a cycle or more per candidate
+  // of the workgroup, 0.3 to 1.5 us of this kernel), the part's largest key
   const uint64_t t_hi = sh_split[part], t_lo = sh_split[part + 1];
+  uint32_t own_mask = 0, own_pos = 0;
   {
-    uint32_t n_all = 0, n_above = 0, kmax = 0;
-    auto take = [&](uint64_t x) {
-      const bool nz = x != 0ull;
+    // (no candidate is zero and no end of a part is: an empty place is below every part)
+    uint32_t n_above = 0;
+    auto take = [&](uint64_t x, int i) {
       const bool above = part != 0 && x >= t_hi;
-      const bool own = nz && !above && x >= t_lo;
-      n_all += nz ? 1u : 0u;
       n_above += above ? 1u : 0u;
-      if (own) {
-        // (a part of more than kCutMaxCandidates runs on into the second array, whose last place takes the rest: such a
-        // segment is redone, see below)
-        sh_own[min(atomicAdd(&sh_n[5], 1u), 2u * (uint32_t)kCutMaxCandidates - 1u)] = x;
-        kmax = max(kmax, (uint32_t)(x >> 32));
-      }
+      own_mask |= (!above && x >= t_lo ? 1u : 0u) << i;
     };
 #pragma unroll
-    for (int i = 0; i < kHeadMine; ++i) take(c[i]);
+    for (int i = 0; i < kHeadMine; ++i) take(c[i], i);
     if (n_ovf) {
 #pragma unroll
-      for (int i = kHeadMine; i < kMine; ++i) take(c[i]);
+      for (int i = kHeadMine; i < kMine; ++i) take(c[i], i);
     }
-    const uint32_t inc = wave_inclusive_scan((n_all << 16) | n_above);   // (at most 18 x 64 per wave each)
-    kmax = max(kmax, lane_xor<1>(kmax));
-    kmax = max(kmax, lane_xor<2>(kmax));
-    kmax = max(kmax, lane_xor<4>(kmax));
-    kmax = max(kmax, lane_xor<8>(kmax));
-    kmax = max(kmax, lane_xor<16>(kmax));
-    kmax = max(kmax, lane_xor<32>(kmax));
-    if (lane == 63) {
-      atomicAdd(&sh_n[2], inc >> 16);
-      atomicAdd(&sh_n[4], inc & 0xffffu);
-      atomicMax(&sh_n[6], kmax);
+    const uint32_t mine = (uint32_t)__builtin_popcount(own_mask);
+    const uint32_t inc = wave_inclusive_scan((mine << 16) | n_above);   // (at most 22 x 64 per wave each)
+    uint64_t before = 0;
+    if (lane == 63) before = lds_add_rtn_u64((uint64_t*)&sh_n[4], ((uint64_t)(inc >> 16) << 32) | (inc & 0xffffu));
+    own_pos = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(before >> 32), 63) + (inc >> 16) - mine;
+    if (part == 0) {   // the first part ends at the segment's largest key
+      uint32_t kmax = 0;
+#pragma unroll
+      for (int i = 0; i < kHeadMine; ++i) kmax = max(kmax, (uint32_t)(c[i] >> 32));
+      if (n_ovf) {
+#pragma unroll
+        for (int i = kHeadMine; i < kMine; ++i) kmax = max(kmax, (uint32_t)(c[i] >> 32));
+      }
+      kmax = max(kmax, lane_xor<1>(kmax));
+      kmax = max(kmax, lane_xor<2>(kmax));
+      kmax = max(kmax, lane_xor<4>(kmax));
+      kmax = max(kmax, lane_xor<8>(kmax));
+      kmax = max(kmax, lane_xor<16>(kmax));
+      kmax = max(kmax, lane_xor<32>(kmax));
+      if (lane == 63) lds_max_u32(&sh_n[6], kmax);
     }
   }
   __syncthreads();
   const uint32_t n_cand = sh_n[2], n_above = sh_n[4], n_own = sh_n[5];
   // More candidates than one part may hold (the sample sat low: at 65536 tokens and k = 2048 one call in ten): fine as
-  // long as every part fits, which all workgroups of the segment have to see alike - each counts the sizes of all parts.
-  uint32_t max_part = n_own;
+  // long as every part that reaches into the top k fits, which all workgroups of the segment have to see alike - each
+  // counts the sizes of all parts.
+  uint32_t max_part = 0;   // (no more candidates than one part may hold: every part fits)
   if (n_cand > (uint32_t)kCutMaxCandidates)
-    max_part = max(max_part, largest_part((const uint64_t*)heads, n_pairs, n_ovf ? sh_extra : nullptr, min(n_extra, (uint32_t)kCutMaxExtras), sh_split, sh_hist));
+    max_part = largest_part((const uint64_t*)heads, n_pairs, n_ovf ? sh_extra : nullptr, min(n_extra, (uint32_t)kCutMaxExtras), sh_split, sh_hist, k);
   const uint32_t n_gave_up = ANNOUNCED ? sh_n[7] : 0u;
   const bool redo = n_cand < k || n_cand > (uint32_t)p.max_entries || n_extra > (uint32_t)kCutMaxExtras || max_part > (uint32_t)kCutMaxCandidates ||
                     n_gave_up != 0u;
@@ -1185,6 +1225,16 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   const uint64_t span = (part == 0 ? (((uint64_t)sh_n[6] << 32) | 0xffffffffull) : t_hi) - base;
   const int fixed = __builtin_clzll(span | 1ull);
   const int shift = 64 - fixed > kHistBits ? 64 - fixed - kHistBits : 0;
+  // (a part that is ranked holds at most kCutMaxCandidates, see the checks above)
+#pragma unroll
+  for (int i = 0; i < kHeadMine; ++i)
+    if (own_mask >> i & 1u) sh_own[own_pos++] = c[i];
+  if (n_ovf) {
+#pragma unroll
+    for (int i = kHeadMine; i < kMine; ++i)
+      if (own_mask >> i & 1u) sh_own[own_pos++] = c[i];
+  }
+  __syncthreads();
 #pragma unroll 1
   for (uint32_t i = tid; i < n_own; i += kSelThreads) atomicAdd(&sh_hist[(uint32_t)((sh_own[i] - base) >> shift)], 1u);
   __syncthreads();
@@ -1657,8 +1707,8 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
   const RankKernel kernel = kernels[dtype == TKA_F16 ? 0 : 1][wide ? 1 : 0][p.union_idx ? 1 : 0][p.tau_words ? 1 : 0];
   if (allow_dynamic_lds((const void*)kernel, lds) != TKA_OK) return TKA_EHIP;
   LaunchTimer timer("select_rank", stream);
-  if (p.segs_per_row < 1 || p.num_segments % p.segs_per_row || p.num_segments / p.segs_per_row > 65535) return TKA_EINVAL;
-  const dim3 wgs((unsigned)(p.segs_per_row * kCutParts), (unsigned)(p.num_segments / p.segs_per_row));
+  if (p.segs_per_row < 1 || p.num_segments % p.segs_per_row || p.num_segments > (1 << 24)) return TKA_EINVAL;
+  const dim3 wgs((unsigned)((p.num_segments + 7) / 8 * 8 * kCutParts));   // (see the kernel)
   hipLaunchKernelGGL(kernel, wgs, dim3(kSelThreads), lds, stream, g, p, kpad_for(p.k));
   return hip_status(hipGetLastError());
 }
