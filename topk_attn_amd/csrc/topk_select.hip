@@ -1162,19 +1162,25 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   const uint64_t t_hi = sh_split[part], t_lo = sh_split[part + 1];
   uint32_t own_mask = 0, own_pos = 0;
   {
-    // (no candidate is zero and no end of a part is: an empty place is below every part)
-    uint32_t n_above = 0;
-    auto take = [&](uint64_t x, int i) {
-      const bool above = part != 0 && x >= t_hi;
-      n_above += above ? 1u : 0u;
-      own_mask |= (!above && x >= t_lo ? 1u : 0u) << i;
-    };
+    // Two compares per entry and nothing else: at or above the part's lower end, and above the part (beyond the largest
+    // composite below its upper end; nothing is above the first part).  No candidate is zero and no end of a part is: an
+    // empty place is below every part.
+    const uint64_t t_top = part == 0 ? ~0ull : t_hi - 1ull;
+    uint32_t in_mask = 0, above_mask = 0;
 #pragma unroll
-    for (int i = 0; i < kHeadMine; ++i) take(c[i], i);
+    for (int i = 0; i < kHeadMine; ++i) {
+      in_mask |= (c[i] >= t_lo ? 1u : 0u) << i;
+      above_mask |= (c[i] > t_top ? 1u : 0u) << i;
+    }
     if (n_ovf) {
 #pragma unroll
-      for (int i = kHeadMine; i < kMine; ++i) take(c[i], i);
+      for (int i = kHeadMine; i < kMine; ++i) {
+        in_mask |= (c[i] >= t_lo ? 1u : 0u) << i;
+        above_mask |= (c[i] > t_top ? 1u : 0u) << i;
+      }
     }
+    own_mask = in_mask & ~above_mask;
+    const uint32_t n_above = (uint32_t)__builtin_popcount(above_mask);
     const uint32_t mine = (uint32_t)__builtin_popcount(own_mask);
     const uint32_t inc = wave_inclusive_scan((mine << 16) | n_above);   // (at most 22 x 64 per wave each)
     uint64_t before = 0;
@@ -1226,13 +1232,16 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   const int fixed = __builtin_clzll(span | 1ull);
   const int shift = 64 - fixed > kHistBits ? 64 - fixed - kHistBits : 0;
   // (a part that is ranked holds at most kCutMaxCandidates, see the checks above)
+  {
+    uint64_t* place = sh_own + own_pos;
 #pragma unroll
-  for (int i = 0; i < kHeadMine; ++i)
-    if (own_mask >> i & 1u) sh_own[own_pos++] = c[i];
-  if (n_ovf) {
+    for (int i = 0; i < kHeadMine; ++i)
+      if (own_mask >> i & 1u) *place++ = c[i];
+    if (n_ovf) {
 #pragma unroll
-    for (int i = kHeadMine; i < kMine; ++i)
-      if (own_mask >> i & 1u) sh_own[own_pos++] = c[i];
+      for (int i = kHeadMine; i < kMine; ++i)
+        if (own_mask >> i & 1u) *place++ = c[i];
+    }
   }
   __syncthreads();
 #pragma unroll 1
@@ -1249,8 +1258,14 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
     if (lane == 0) sh_wtot[wave] = ge;
     if (h0 > kCutBucketMax || h1 > kCutBucketMax) sh_n[3] = 1u;
     __syncthreads();
-    uint32_t above = 0;
-    for (int v = wave + 1; v < kSelWaves; ++v) above += sh_wtot[v];
+    // the composites of the waves above: one read and a sum across the wave instead of a loop of up to fifteen reads
+    static_assert(kSelWaves <= 64, "one lane per wave");
+    uint32_t above = lane > wave && lane < kSelWaves ? sh_wtot[lane] : 0u;
+    above += lane_xor<1>(above);
+    above += lane_xor<2>(above);
+    above += lane_xor<4>(above);
+    above += lane_xor<8>(above);
+    above = (uint32_t)__builtin_amdgcn_readfirstlane((int)above);   // (sixteen waves: the sum stands in each of lanes 0 .. 15)
     sh_off[2 * tid + 1] = sh_cur[2 * tid + 1] = above + ge - mine;   // buckets > 2t+1
     sh_off[2 * tid] = sh_cur[2 * tid] = above + ge - h0;             // buckets > 2t
   }
