@@ -234,8 +234,13 @@ __device__ __forceinline__ void find_threshold_bin_1024(const uint32_t* sh_hist,
   const uint32_t v = wave_total - inc + mine;  // suffix sum over lanes >= lane
   if (lane == 0) sh_wtot[wave] = v;
   __syncthreads();
-  uint32_t above = 0;
-  for (int w = wave + 1; w < 16; ++w) above += sh_wtot[w];
+  // the totals of the waves above: one read and a sum across sixteen lanes instead of a loop of up to fifteen reads
+  uint32_t above = lane > wave && lane < 16 ? sh_wtot[lane] : 0u;
+  above += lane_xor<1>(above);
+  above += lane_xor<2>(above);
+  above += lane_xor<4>(above);
+  above += lane_xor<8>(above);
+  above = (uint32_t)__builtin_amdgcn_readfirstlane((int)above);
   const uint32_t ge0 = above + v;   // count(bins >= 2*tid)
   const uint32_t ge1 = ge0 - h0;    // count(bins >= 2*tid+1)
   const uint32_t gt1 = ge1 - h1;    // count(bins >  2*tid+1)

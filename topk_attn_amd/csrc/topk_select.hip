@@ -1348,7 +1348,8 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
   __shared__ uint32_t sh_hist[kHistBins];
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
-  __shared__ uint32_t sh_n[3];   // smallest key, largest key, candidates collected
+  __shared__ uint32_t sh_n[3];   // (two spare words), candidates collected
+  __shared__ __attribute__((aligned(8))) uint32_t sh_wmm[2 * kSelWaves];   // smallest and largest key of every wave
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1421,14 +1422,18 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
   kmin = min(kmin, lane_xor<8>(kmin));   kmax = max(kmax, lane_xor<8>(kmax));
   kmin = min(kmin, lane_xor<16>(kmin));  kmax = max(kmax, lane_xor<16>(kmax));
   kmin = min(kmin, lane_xor<32>(kmin));  kmax = max(kmax, lane_xor<32>(kmax));
+  // (the waves' extremes through LDS, one lane per wave, and across sixteen lanes: one barrier and no atomics)
+  if (lane == 0) { sh_wmm[2 * (tid >> 6)] = kmin; sh_wmm[2 * (tid >> 6) + 1] = kmax; }
   __syncthreads();
-  if (lane == 0) {
-    atomicMin(&sh_n[0], kmin);
-    atomicMax(&sh_n[1], kmax);
+  {
+    static_assert(kSelWaves == 16, "sixteen lanes hold the waves' extremes");
+    const uint2 mm = *(const uint2*)&sh_wmm[2 * (lane & 15)];
+    kmin = mm.x;  kmax = mm.y;
+    kmin = min(kmin, lane_xor<1>(kmin));   kmax = max(kmax, lane_xor<1>(kmax));
+    kmin = min(kmin, lane_xor<2>(kmin));   kmax = max(kmax, lane_xor<2>(kmax));
+    kmin = min(kmin, lane_xor<4>(kmin));   kmax = max(kmax, lane_xor<4>(kmax));
+    kmin = min(kmin, lane_xor<8>(kmin));   kmax = max(kmax, lane_xor<8>(kmax));
   }
-  __syncthreads();
-  kmin = sh_n[0];
-  kmax = sh_n[1];
   // bins: the 11 leading bits of key - smallest key, counted from the leading bit of the range
   const int fixed = kmax == kmin ? 31 : __builtin_clz(kmax - kmin);
   const int shift = 32 - fixed > kHistBits ? 32 - fixed - kHistBits : 0;
@@ -1456,25 +1461,21 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
   for (int e = 0; e < 4; ++e)
     if ((vm >> e & 1u) && ((keys[e] - kmin) >> shift) >= d) sh_cand[atomicAdd(&sh_n[2], 1u)] = composite(keys[e], (uint32_t)tid * 4 + e);
   __syncthreads();
-  // rank = number of larger candidates: eight threads per candidate, each with an eighth of the list, add up in LDS
-  // (the histogram is spent)
-  uint32_t* sh_rank = sh_hist;
-  for (uint32_t i = tid; i < n_cand; i += kSelThreads) sh_rank[i] = 0;
-  __syncthreads();
+  // rank = number of larger candidates: eight neighbouring lanes per candidate, each with an eighth of the list, add up
+  // across the lanes; the rank is the place
   {
-    const uint32_t part = (uint32_t)tid >> 7, per = (n_cand + 7u) / 8u;
+    const uint32_t part = (uint32_t)tid & 7u, per = (n_cand + 7u) / 8u;
     const uint32_t j0 = part * per, j1 = min(j0 + per, n_cand);
-    for (uint32_t i = (uint32_t)tid & 127u; i < n_cand; i += 128u) {
-      const uint64_t x = sh_cand[i];
+    for (uint32_t first = 0; first < n_cand; first += kSelThreads / 8) {
+      const uint32_t i = first + ((uint32_t)tid >> 3);
+      const uint64_t x = sh_cand[i < n_cand ? i : 0u];
       uint32_t larger = 0;
       for (uint32_t j = j0; j < j1; ++j) larger += sh_cand[j] > x ? 1u : 0u;
-      atomicAdd(&sh_rank[i], larger);
+      larger += lane_xor<1>(larger);
+      larger += lane_xor<2>(larger);
+      larger += lane_xor<4>(larger);
+      if (part == 0u && i < n_cand && larger < k) sh_sort[larger] = x;
     }
-  }
-  __syncthreads();
-  for (uint32_t i = tid; i < n_cand; i += kSelThreads) {
-    const uint32_t r = sh_rank[i];
-    if (r < k) sh_sort[r] = sh_cand[i];
   }
   __syncthreads();
   write_rank_outputs(sh_sort, p, seg, chunk);
