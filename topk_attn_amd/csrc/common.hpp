@@ -111,6 +111,24 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
   return v;
 }
 
+// Largest and smallest value of the wave, valid in lane 63 only: two steps inside the quads, the two mirrors of a DPP
+// row, and the row results carried forward as in the scan - six DPP operands and no trip through the LDS crossbar
+// (lane_xor takes one for distances 4, 16 and 32).  A lane without a source keeps its own value.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_self(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ uint32_t wave_max_in_last_lane(uint32_t v) {
+  v = max(v, dpp_or_self<0xB1, 0xf>(v));    // quad_perm [1,0,3,2]
+  v = max(v, dpp_or_self<0x4E, 0xf>(v));    // quad_perm [2,3,0,1]
+  v = max(v, dpp_or_self<0x141, 0xf>(v));   // row_half_mirror
+  v = max(v, dpp_or_self<0x140, 0xf>(v));   // row_mirror
+  v = max(v, dpp_or_self<0x142, 0xa>(v));   // row_bcast:15 into rows 1 and 3
+  v = max(v, dpp_or_self<0x143, 0xc>(v));   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_min_in_last_lane(uint32_t v) { return ~wave_max_in_last_lane(~v); }
+
 __device__ __forceinline__ int lane_id() {
   return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }

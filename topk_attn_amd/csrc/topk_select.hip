@@ -1194,12 +1194,7 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
 #pragma unroll
         for (int i = kHeadMine; i < kMine; ++i) kmax = max(kmax, (uint32_t)(c[i] >> 32));
       }
-      kmax = max(kmax, lane_xor<1>(kmax));
-      kmax = max(kmax, lane_xor<2>(kmax));
-      kmax = max(kmax, lane_xor<4>(kmax));
-      kmax = max(kmax, lane_xor<8>(kmax));
-      kmax = max(kmax, lane_xor<16>(kmax));
-      kmax = max(kmax, lane_xor<32>(kmax));
+      kmax = wave_max_in_last_lane(kmax);
       if (lane == 63) lds_max_u32(&sh_n[6], kmax);
     }
   }
@@ -1416,14 +1411,10 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
       kmax = max(kmax, keys[e]);
     }
   }
-  kmin = min(kmin, lane_xor<1>(kmin));   kmax = max(kmax, lane_xor<1>(kmax));
-  kmin = min(kmin, lane_xor<2>(kmin));   kmax = max(kmax, lane_xor<2>(kmax));
-  kmin = min(kmin, lane_xor<4>(kmin));   kmax = max(kmax, lane_xor<4>(kmax));
-  kmin = min(kmin, lane_xor<8>(kmin));   kmax = max(kmax, lane_xor<8>(kmax));
-  kmin = min(kmin, lane_xor<16>(kmin));  kmax = max(kmax, lane_xor<16>(kmax));
-  kmin = min(kmin, lane_xor<32>(kmin));  kmax = max(kmax, lane_xor<32>(kmax));
+  kmin = wave_min_in_last_lane(kmin);
+  kmax = wave_max_in_last_lane(kmax);
   // (the waves' extremes through LDS, one lane per wave, and across sixteen lanes: one barrier and no atomics)
-  if (lane == 0) { sh_wmm[2 * (tid >> 6)] = kmin; sh_wmm[2 * (tid >> 6) + 1] = kmax; }
+  if (lane == 63) { sh_wmm[2 * (tid >> 6)] = kmin; sh_wmm[2 * (tid >> 6) + 1] = kmax; }
   __syncthreads();
   {
     static_assert(kSelWaves == 16, "sixteen lanes hold the waves' extremes");
