@@ -58,15 +58,16 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s
   __syncthreads();  // sh_wtot may still be read by the previous call
   if (lane == 63) sh_wtot[wave] = inc;
   __syncthreads();
-  uint32_t before = 0, all = 0;
-#pragma unroll
-  for (int w = 0; w < kSelWaves; ++w) {
-    const uint32_t t = sh_wtot[w];
-    before += w < wave ? t : 0u;
-    all += t;
-  }
-  *total = all;
-  return before + inc - v;
+  // the waves' totals: one read by sixteen lanes and two sums across them instead of sixteen reads per thread
+  static_assert(kSelWaves == 16, "one lane per wave, summed across sixteen lanes");
+  const uint32_t t = lane < kSelWaves ? sh_wtot[lane] : 0u;
+  uint32_t all = t, before = lane < wave ? t : 0u;
+  all += lane_xor<1>(all);   before += lane_xor<1>(before);
+  all += lane_xor<2>(all);   before += lane_xor<2>(before);
+  all += lane_xor<4>(all);   before += lane_xor<4>(before);
+  all += lane_xor<8>(all);   before += lane_xor<8>(before);
+  *total = (uint32_t)__builtin_amdgcn_readfirstlane((int)all);
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)before) + inc - v;
 }
 
 // Loads the `per_thread` (4 or 16) consecutive scores of this thread as keys; positions at or beyond
@@ -637,7 +638,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   __shared__ uint32_t sh_pos[kCandMaxParts + 1];   // start positions of all slices (segments with more than kRound slices)
   __shared__ uint32_t sh_wtot[kSelWaves];
   __shared__ uint32_t sh_res[4];
-  __shared__ uint32_t sh_kminmax[2];
+  __shared__ __attribute__((aligned(8))) uint32_t sh_wmm[2 * kSelWaves];   // smallest and largest key of every wave's entries
   __shared__ uint64_t sh_mm[3];
   __shared__ uint64_t sh_small[kSmallBucket];
   __shared__ uint32_t sh_small_cnt;
@@ -648,6 +649,8 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   const int seg = blockIdx.x;
   const uint32_t k = (uint32_t)p.k;
   if (tid == 0) sh_gave_up = 0u;
+  sh_hist[2 * tid] = 0;       // (for the first radix pass: cleared here, in front of barriers that are needed anyway)
+  sh_hist[2 * tid + 1] = 0;
   __syncthreads();
 
   // Copy the slices into LDS.  Up to kRound slices: 32 lanes per slice load its first 32 entries (entry 0 carries
@@ -659,6 +662,9 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   static_assert(kSliceLanes == kCandHead, "one lane per head entry");
   const int sub = tid & (kSliceLanes - 1), grp = tid / kSliceLanes;
   uint32_t n_entries = 0;
+  // (where the copy below has every entry in a register on its way, the smallest and the largest key are taken there)
+  uint32_t reg_kmin = ~0u, reg_kmax = 0u;
+  bool reg_minmax = false;
   if (p.from_keys) {
     // Short segments: no GEMV launch before this one.  The workgroup scores its segment itself (64 row groups
     // of 16 lanes, 16 rows in flight each, canonical order) and every token becomes an entry.
@@ -732,15 +738,21 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
         const int sl = s0 + u * kGroups + grp;
         const uint32_t start = sh_start[u * kGroups + grp];
         const uint32_t idx0 = (uint32_t)sl * (uint32_t)p.part_len;
-        if ((uint32_t)sub < cnt[u] && start + sub < cap)
+        if ((uint32_t)sub < cnt[u] && start + sub < cap) {
           sh_ent[start + sub] = (first[u] & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)first[u] & 0x1ffu));
+          reg_kmin = min(reg_kmin, (uint32_t)(first[u] >> 32));
+          reg_kmax = max(reg_kmax, (uint32_t)(first[u] >> 32));
+        }
         for (uint32_t j = kSliceLanes + sub; j < cnt[u] && start + j < cap; j += kSliceLanes) {   // rare: a slice with more than 32 candidates
           const uint64_t w = lists[(int64_t)sl * p.part_len + j];
           sh_ent[start + j] = (w & 0xffffffff00000000ull) | (uint32_t)~(idx0 + ((uint32_t)w & 0x1ffu));
+          reg_kmin = min(reg_kmin, (uint32_t)(w >> 32));
+          reg_kmax = max(reg_kmax, (uint32_t)(w >> 32));
         }
       }
       n_entries += total;
     }
+    reg_minmax = true;
   } else {
     // many slices: all counts first (one round trip), one scan, then the entries with no barrier in between
     uint32_t c4[4], sum = 0;
@@ -796,8 +808,6 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   const bool redo = !whole && (n_entries < k || n_entries > cap || n_gave_up != 0u);
   if (tid == 0) {
     sh_small_cnt = 0;
-    sh_kminmax[0] = ~0u;
-    sh_kminmax[1] = 0u;
   }
   if (!whole) {
     if (tid == 0) p.seg_flags[seg] = (redo ? 1u : 0u) | (n_gave_up << 8);
@@ -826,30 +836,33 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   // The passes over the entries (tid, tid + 1024, ...) are rolled loops over the LDS copy: the kernel runs a few workgroups,
   // every line of its code is fetched cold, and an unrolled pass for the 16 entries per thread that the capacity allows
   // costs that fetch whether or not the list reaches them.
-  uint32_t kmin = ~0u, kmax = 0u;   // smallest and largest key among the entries
+  uint32_t kmin = reg_kmin, kmax = reg_kmax;   // smallest and largest key among the entries
+  if (!reg_minmax) {
 #pragma unroll 1
-  for (uint32_t v = tid; v < n_entries; v += kSelThreads) {
-    const uint32_t key = (uint32_t)(sh_ent[v] >> 32);
-    kmin = min(kmin, key);
-    kmax = max(kmax, key);
+    for (uint32_t v = tid; v < n_entries; v += kSelThreads) {
+      const uint32_t key = (uint32_t)(sh_ent[v] >> 32);
+      kmin = min(kmin, key);
+      kmax = max(kmax, key);
+    }
   }
 
   uint64_t threshold = 0;   // selected: composite >= threshold
   if (n_entries > k) {
     // common prefix of all keys: the passes start below it (all keys equal: they start at the index bits)
-    kmin = min(kmin, lane_xor<1>(kmin));   kmax = max(kmax, lane_xor<1>(kmax));
-    kmin = min(kmin, lane_xor<2>(kmin));   kmax = max(kmax, lane_xor<2>(kmax));
-    kmin = min(kmin, lane_xor<4>(kmin));   kmax = max(kmax, lane_xor<4>(kmax));
-    kmin = min(kmin, lane_xor<8>(kmin));   kmax = max(kmax, lane_xor<8>(kmax));
-    kmin = min(kmin, lane_xor<16>(kmin));  kmax = max(kmax, lane_xor<16>(kmax));
-    kmin = min(kmin, lane_xor<32>(kmin));  kmax = max(kmax, lane_xor<32>(kmax));
-    if (lane == 0) {
-      atomicMin(&sh_kminmax[0], kmin);
-      atomicMax(&sh_kminmax[1], kmax);
-    }
+    // (the waves' extremes through LDS, one lane per wave, and across sixteen lanes: no atomics)
+    kmin = wave_min_in_last_lane(kmin);
+    kmax = wave_max_in_last_lane(kmax);
+    if (lane == 63) { sh_wmm[2 * (tid >> 6)] = kmin; sh_wmm[2 * (tid >> 6) + 1] = kmax; }
     __syncthreads();
-    kmin = sh_kminmax[0];
-    kmax = sh_kminmax[1];
+    {
+      static_assert(kSelWaves == 16, "sixteen lanes hold the waves' extremes");
+      const uint2 mm = *(const uint2*)&sh_wmm[2 * (lane & 15)];
+      kmin = mm.x;  kmax = mm.y;
+      kmin = min(kmin, lane_xor<1>(kmin));   kmax = max(kmax, lane_xor<1>(kmax));
+      kmin = min(kmin, lane_xor<2>(kmin));   kmax = max(kmax, lane_xor<2>(kmax));
+      kmin = min(kmin, lane_xor<4>(kmin));   kmax = max(kmax, lane_xor<4>(kmax));
+      kmin = min(kmin, lane_xor<8>(kmin));   kmax = max(kmax, lane_xor<8>(kmax));
+    }
     // Radix passes on the composites relative to the smallest key: their leading bits are zero down to the
     // width of the key range, and the 11 bits below spread the candidates evenly (shared bits of the float
     // keys themselves say little once the scores straddle a power of two).
@@ -857,14 +870,17 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     int fixed = kmin == kmax ? 32 : __builtin_clz(kmax - kmin);
     uint64_t prefix = 0ull;
     uint32_t need = k;
-    bool done = false;
+    bool done = false, first_pass = true;
     while (!done) {
       const int bits = (64 - fixed) >= kHistBits ? kHistBits : (64 - fixed);
       const int shift = 64 - fixed - bits;
-      __syncthreads();
-      sh_hist[2 * tid] = 0;
-      sh_hist[2 * tid + 1] = 0;
-      __syncthreads();
+      if (!first_pass) {
+        __syncthreads();
+        sh_hist[2 * tid] = 0;
+        sh_hist[2 * tid + 1] = 0;
+        __syncthreads();
+      }
+      first_pass = false;
 #pragma unroll 1
       for (uint32_t v = tid; v < n_entries; v += kSelThreads) {
         const uint64_t c = sh_ent[v] - base;
