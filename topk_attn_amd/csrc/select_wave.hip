@@ -34,23 +34,12 @@ constexpr int kWsBins = 2048;
 constexpr int kWsMaxWaves = 16;
 constexpr int kWsMaxLen = kWsMaxWaves * kWave * 16;   // 16384 keys per segment at most
 
+// (the same value in every lane: six DPP steps bring it to the last lane, one read hands it out)
 __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
-  v = min(v, lane_xor<1>(v));
-  v = min(v, lane_xor<2>(v));
-  v = min(v, lane_xor<4>(v));
-  v = min(v, lane_xor<8>(v));
-  v = min(v, lane_xor<16>(v));
-  v = min(v, lane_xor<32>(v));
-  return v;
+  return (uint32_t)__builtin_amdgcn_readlane((int)wave_min_in_last_lane(v), 63);
 }
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-  v = max(v, lane_xor<1>(v));
-  v = max(v, lane_xor<2>(v));
-  v = max(v, lane_xor<4>(v));
-  v = max(v, lane_xor<8>(v));
-  v = max(v, lane_xor<16>(v));
-  v = max(v, lane_xor<32>(v));
-  return v;
+  return (uint32_t)__builtin_amdgcn_readlane((int)wave_max_in_last_lane(v), 63);
 }
 
 // Order-preserving key of a score, as score_key() (NaN lowest, -0 == +0).
@@ -388,8 +377,10 @@ __global__ __launch_bounds__(W * kWave) void select_wave_kernel(SelectParams p, 
       __syncthreads();
     }
     // out; the composites carry relative keys: key = (rel >> lshift) + kmin
-    const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
-                                             : (uint32_t)((seg % p.segs_per_row) * p.seg_len);
+    // (a modulo by a run-time value is some forty instructions on this hardware: none for one or a power of two of chunks)
+    const uint32_t spr = (uint32_t)p.segs_per_row;
+    const uint32_t chunk = spr == 1u ? 0u : (spr & (spr - 1u)) == 0u ? (uint32_t)seg & (spr - 1u) : (uint32_t)seg % spr;
+    const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len) : (uint32_t)(chunk * p.seg_len);
     int32_t* oi = p.out_idx + (int64_t)seg * p.out_stride;
     float* ov = p.out_val ? p.out_val + (int64_t)seg * p.out_stride : nullptr;
     for (uint32_t r = tid; r < k; r += T) {
