@@ -1142,15 +1142,30 @@ __global__ __launch_bounds__(kSelThreads) void select_rank_kernel(GemvParams g, 
   __syncthreads();
   const uint32_t n_ovf = sh_n[0];
   if (n_ovf) {   // rare: slices whose candidates go beyond the head entries (scores that cluster in one place)
+    // One such slice per wave, sixteen at a time, every load asked for before the first one is used: one round trip for
+    // up to sixteen slices (slice after slice, each with its own trip, cost 1.6 us on a step of eight heads whose cuts
+    // sat low).  A slice holds at most kCutTokensPerWg - kCutHead entries beyond its head: three per lane.
     const uint64_t* wide = p.list + (int64_t)seg * p.list_stride;
-    for (uint32_t i = 0; i < n_ovf; ++i) {
-      const uint32_t sl = sh_ovf[i] & 0xffffu, cnt = sh_ovf[i] >> 16;
-      const uint32_t j = (uint32_t)kCutHead + (uint32_t)tid;
-      if (j < cnt) {
-        const uint64_t x = wide[(int64_t)sl * p.part_len + j];
-        const uint32_t pos = atomicAdd(&sh_n[1], 1u);
-        if (pos < (uint32_t)kCutMaxExtras) sh_extra[pos] = x;
+    constexpr int kBeyond = (kCutTokensPerWg - kCutHead + kWave - 1) / kWave;
+    for (uint32_t first = 0; first < n_ovf; first += kSelWaves) {
+      const uint32_t i = first + (uint32_t)(tid >> 6);
+      uint64_t x[kBeyond];
+#pragma unroll
+      for (int u = 0; u < kBeyond; ++u) x[u] = 0ull;   // (no composite is zero)
+      if (i < n_ovf) {
+        const uint32_t sl = sh_ovf[i] & 0xffffu, cnt = sh_ovf[i] >> 16;
+#pragma unroll
+        for (int u = 0; u < kBeyond; ++u) {
+          const uint32_t j = (uint32_t)kCutHead + (uint32_t)lane + (uint32_t)(u * kWave);
+          if (j < cnt) x[u] = wide[(int64_t)sl * p.part_len + j];
+        }
       }
+#pragma unroll
+      for (int u = 0; u < kBeyond; ++u)
+        if (x[u] != 0ull) {
+          const uint32_t pos = atomicAdd(&sh_n[1], 1u);
+          if (pos < (uint32_t)kCutMaxExtras) sh_extra[pos] = x[u];
+        }
     }
     __syncthreads();
   }
