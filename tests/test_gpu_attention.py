@@ -447,7 +447,10 @@ def hooks():
     (oracle.F16, 1, 8, 4, 32768, 2048, 64, 512, "heavy", False, True),         # more than 65536 rows: the route in three launches
     (oracle.BF16, 2, 4, 2, 20001, 1000, 100, 300, "levels", True, True),
     (oracle.F16, 1, 2, 4, 24577, 3000, 300, 300, "heavy", False, False),       # k too large for that route: the dense path, ascending list
-    (oracle.F16, 2, 2, 4, 16384, 1024, 64, 512, "heavy", False, False),        # short enough for the registers of a workgroup
+    (oracle.F16, 2, 2, 4, 16384, 1024, 64, 512, "heavy", False, True),         # would also fit the registers of a workgroup
+    (oracle.F16, 1, 8, 4, 12000, 1024, 64, 512, "heavy", False, True),         # the same on a call of more than 65536 rows
+    (oracle.BF16, 3, 8, 2, 28000, 1500, 64, 512, "heavy", False, True),        # more than 655360 rows
+    (oracle.F16, 2, 2, 4, 8000, 512, 64, 512, "heavy", False, False),          # short enough for the registers of a workgroup
     (oracle.BF16, 1, 3, 2, 5000, 700, 3000, 3000, "levels", True, False),      # the same with range and window overlapping, ties
     (oracle.F16, 1, 2, 8, 3000, 100, 5, 9, "equal", False, False)])
 def test_sparse_decode_step_handoff_order(hooks, dtype, B, H, G, N, k, sink, local, kind, want_topk, cut):

@@ -433,9 +433,14 @@ def test_long_segment_threshold_never_published(hooks, withheld):
                                              (oracle.F16, 1, 8, 4, 49152, 1500), (oracle.F16, 3, 1, 1, 30000, 7),
                                              # k above n / 14.5 (up to n / 8): slices of 128 tokens
                                              (oracle.F16, 1, 1, 1, 20000, 2048), (oracle.BF16, 2, 1, 2, 16384, 2048),
-                                             (oracle.F16, 1, 8, 4, 24577, 2048), (oracle.BF16, 1, 3, 1, 32768, 2048 + 1000)])
+                                             (oracle.F16, 1, 8, 4, 24577, 2048), (oracle.BF16, 1, 3, 1, 32768, 2048 + 1000),
+                                             # segments of 8193 .. 16384 tokens on calls of more than 65536 rows
+                                             (oracle.F16, 1, 8, 1, 16384, 1024), (oracle.BF16, 2, 8, 4, 9001, 512),
+                                             (oracle.F16, 1, 5, 2, 16384, 2048),
+                                             # more than 655360 rows (several generations of GEMV workgroups)
+                                             (oracle.F16, 3, 8, 1, 32768, 2048), (oracle.BF16, 5, 8, 2, 20000, 1000)])
 def test_common_cut_route(dtype, B, H, G, N, k):
-    """Calls of up to 655360 rows with segments of 16385 .. 65536 tokens (from 8193 tokens on calls of up to 65536 rows) and
+    """Calls of up to 1572864 rows with segments of 8193 .. 65536 tokens and
     no score output: the cut of a segment comes from 256 sample rows - every GEMV workgroup derives the same one, or, on
     calls of more than 65536 rows, one workgroup per segment does in a launch before the GEMV - and eight ranking
     workgroups per segment rank the candidates.  Ordinary data with heavy hitters; ragged lengths (an odd number of

@@ -204,7 +204,7 @@ struct UnionOut {
 };
 
 // Samples per segment and rank of the cut when the call takes the common-cut route (segments of middling length on
-// calls of up to 655360 rows; rank-ordered output, and the union list for a caller that only hands it to the
+// calls of up to 1572864 rows; rank-ordered output, and the union list for a caller that only hands it to the
 // attention), else 0.  Shorter segments are selected from the registers of one workgroup, longer ones (or many of
 // them) by the sampling workgroups of the candidate route.
 int64_t cut_route_min_len() {
@@ -249,17 +249,17 @@ void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, 
   if (s == 0) return;
   if (slice_len) *slice_len = len;
   // Measured, decode steps with k = 2048 unless said (us per step, this route against the others): 1 x 32768 tokens
-  // 23.6 / 32.2, 4 x 32768 26.7 / 37.5, 8 x 32768 33.7 / 43.4, 16 x 32768 50.4 / 56.9, 24 x 32768 63.8 / 68.3,
-  // 8 x 49152 42.9 / 51.8, 16 x 20000 (k = 1000) 37.0 / 46.7, 32 x 20000 54.4 / 58.4, 32 x 24576 (k = 1536) 66.5 / 67.7,
-  // 40 x 20000 67.1 / 65.5, 48 x 20000 74.5 / 73.7.
+  // 21.1 / 32.2, 8 x 32768 30.7 / 43.4, 24 x 32768 54.6 / 68.8, 32 x 32768 67.6 / 73.2, 48 x 32768 94.4 / 95.9,
+  // 64 x 32768 118.9 / 118.7, 16 x 49152 55.3 / 70.0, 32 x 49152 89.7 / 92.1, 40 x 20000 (k = 1000) 58.7 / 64.6,
+  // 64 x 20000 81.3 / 88.5; segments that would also fit the registers of one workgroup (8193 .. 16384 tokens):
+  // 1 x 16384 (k = 1024) 20.8 / 22.0, 8 x 16384 23.8 / 25.6, 8 x 12000 22.0 / 25.6, 16 x 16384 32.1 / 35.2, 32 x 16384
+  // 46.1 / 48.3, 48 x 16384 58.8 / 58.9, 96 x 16384 100.4 / 102.2; rank-ordered top-k per call: 8 x 16384 (k = 1024)
+  // 14.2 / 20.2, 16 x 16384 (k = 2048) 17.9 / 29.1, 32 x 16384 32.7 / 42.3, 8 x 9000 (k = 512) 13.7 / 15.9.  Up to 8192
+  // tokens the registers of one workgroup win (8 x 8192, k = 512: 21.1 / 20.1 per step, 8 x 4096: 20.1 / 17.6).
   if (rows > kCutMaxRows) return;
-  // Segments that would also fit the registers of one workgroup (8193 .. 16384 rows): rank-ordered output only, up to
-  // 65536 rows per call (1 x 16384 rows, k = 1024: 12.9 / 18.4 us per call, 4 x 16384: 13.2 / 17.8, 8 x 16384, k = 512:
-  // 19.1 / 17.3; at 8192 rows the two are equal; a decode step over 1 x 16384, k = 1024: about 22.3 / 22.5).
-  if (chunk_len <= select_cand_capacity() && (u || rows > 65536)) return;
   // Segments that the candidate route takes as well (65536 tokens): that route from two segments on
-  // (decode steps: 1 x 65536 26.3 / 34.5, 2 x 65536 35.6 / 35.8, 8 x 65536 55.1 / 49.3).
-  if (rows > 65536) {
+  // (decode steps: 1 x 65536 26.3 / 34.5, 16 x 65536 68.2 / 68.9, 32 x 65536 113.8 / 111.6, 64 x 65536 208.6 / 198.6).
+  if (rows > 65536 && chunk_len >= 65536) {
     int cs = 0, cr = 0;
     candidate_plan(a, &cs, &cr);
     if (cs != 0) return;

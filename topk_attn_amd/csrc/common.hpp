@@ -42,7 +42,7 @@ constexpr int kCutMaxCandidates = 8192;    // candidates of one segment that the
 constexpr int kCutMaxExtras = 6144;        // of them, entries beyond the first kCutHead of their slices
 constexpr int kCutSamplesOnce = 256;        // sample rows of a segment where one workgroup scores them for all (256 or 512)
 constexpr uint32_t kCutGaveUp = 0xffffffffu; // slice count of a workgroup that never saw its segment's cut
-constexpr int64_t kCutMaxRows = 655360;    // rows of a call (all segments) up to which the route is taken
+constexpr int64_t kCutMaxRows = 1572864;   // rows of a call (all segments) up to which the route is taken
 constexpr int kCutParts = 8;                // ranking workgroups per segment, each with its own range of the order
 
 // ---- lane exchanges ---------------------------------------------------------------------------

@@ -82,6 +82,43 @@ __device__ __forceinline__ void rank_samples(const uint32_t* sh_skey, const uint
   }
 }
 
+// The group's query heads summed per dim, for a kernel that is short of registers (eight rows in flight per lane and two
+// workgroups of 1024 threads per CU leave 64; with the heads of a group in registers beside the rows the kernel took
+// 107 and ran one workgroup per CU): the first 16 G threads load one 16-byte piece of one head each, the
+// converted values go through LDS (sh_q: 8 x 128 floats), and behind a barrier of the whole workgroup every thread adds up
+// its 8 dims head after head - the order of load_group_query, so the sums are the same bit for bit.
+// The piece of the query that this thread brings (one of the first 16 G threads: 16 bytes of head tid / 16), asked for
+// here and used in group_query_through_lds.
+__device__ __forceinline__ u32x4 group_query_piece(const GemvParams& p, int b, int h, int j) {
+  const int tid = threadIdx.x;
+  u32x4 w = (u32x4){0u, 0u, 0u, 0u};
+  if (tid < 16 * p.group)
+    w = *(const u32x4*)((const uint16_t*)p.q + (int64_t)b * p.q_stride_b + ((int64_t)h * p.group + (tid >> 4)) * kHeadDim + 8 * j);
+  return w;
+}
+template <int DT>
+__device__ __forceinline__ void group_query_through_lds(const GemvParams& p, const u32x4& w, int j, float* sh_q, float (&qf)[8]) {
+  const int tid = threadIdx.x;
+  if (tid < 16 * p.group) {
+    float* dst = sh_q + (tid >> 4) * kHeadDim + 8 * j;
+    *(f32x4*)dst = (f32x4){Elem<DT>::get(w, 0), Elem<DT>::get(w, 1), Elem<DT>::get(w, 2), Elem<DT>::get(w, 3)};
+    *(f32x4*)(dst + 4) = (f32x4){Elem<DT>::get(w, 4), Elem<DT>::get(w, 5), Elem<DT>::get(w, 6), Elem<DT>::get(w, 7)};
+  }
+  __syncthreads();
+  const float* src = sh_q + 8 * j;
+  f32x4 lo = *(const f32x4*)src, hi = *(const f32x4*)(src + 4);
+#pragma unroll 1
+  for (int g = 1; g < p.group; ++g) {
+    lo += *(const f32x4*)(src + g * kHeadDim);
+    hi += *(const f32x4*)(src + g * kHeadDim + 4);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    qf[i] = lo[i];
+    qf[4 + i] = hi[i];
+  }
+}
+
 // Where a workgroup of these kernels works.  Their grids have y = KV head and chunk and z = batch entry (x: the place
 // inside the segment), so that no division by a run-time value stands in front of the first load - the hardware has
 // none: each costs some twenty-five instructions, and the five of a flat grid were 0.8 us of c1's 13.5.
@@ -240,8 +277,9 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_kernel(GemvParams p) {
 // tighter - a fifth fewer candidates - and the part ends are steadier, eight samples per part instead of five; but the
 // scoring workgroups wait for this one, and its longer counting cost them more than the ranking kernel gained: 8 x 32768
 // tokens 37.8 instead of 33.9 us per decode step.)
-template <int DT, bool ANNOUNCED>
-__device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos& at) {
+// QLDS: the query through LDS (sh_q, see group_query_through_lds) instead of through registers.
+template <int DT, bool ANNOUNCED, bool QLDS = false>
+__device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos& at, float* sh_q = nullptr) {
   constexpr int S = kCutSamplesOnce, kRows = S / (kCutThreads / 16);
   __shared__ uint32_t sh_skey[S];
   __shared__ __attribute__((aligned(16))) uint32_t sh_rkey[S];
@@ -259,7 +297,8 @@ __device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos
   for (int u = 0; u < kRows; ++u) kv[u] = *(const u32x4*)(kbase + cut_sample_token(seg, rg * kRows + u, stride) * p.key_stride_n);
   __builtin_amdgcn_sched_barrier(0);
   float qf[8];
-  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  if (QLDS) group_query_through_lds<DT>(p, group_query_piece(p, b, h, j), j, sh_q, qf);
+  else load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
   __builtin_amdgcn_sched_barrier(0);
   float mine = 0.0f;
 #pragma unroll
@@ -293,11 +332,12 @@ __global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
 // and the ranking kernel redoes such a segment from the keys.  The sampling workgroups come first in the grid, so they
 // run before any workgroup that waits for them; nothing depends on that but the speed.
 template <int DT, bool FRONT, int L>
-__global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams p) {
+__global__ __launch_bounds__(kCutThreads, 8) void gemv_cut_slices_kernel(GemvParams p) {
   constexpr int kTokens = 2 * kCutTokensPerWg;
   __shared__ uint32_t sh_key[kTokens];
   __shared__ uint32_t sh_wcnt[kTokens / kWave];
   __shared__ uint64_t sh_cutc[2];   // the cut composite, whether it has arrived
+  __shared__ __attribute__((aligned(16))) float sh_q[8 * kHeadDim];   // the query heads of the group, converted
   const int tid = threadIdx.x;
   // FRONT: a flat grid, the sampling workgroups of all segments first (in a grid with the segments in y and z every
   // segment's own would come right before its scoring workgroups - too late on calls of several generations of
@@ -322,7 +362,7 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
   const int b = at.b, h = at.h, chunk = at.chunk, seg = at.seg;
   if (FRONT && pair < 0) {
     __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
-    sample_segment<DT, true>(p, at);
+    sample_segment<DT, true, true>(p, at, sh_q);
     // the part ends have completed (rank_samples) before the word that announces them leaves; relaxed device-scope
     // accesses on both sides, as for the thresholds of the candidate route: a fence would write back and invalidate
     // whole caches in the middle of the stream
@@ -339,6 +379,8 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
 
   const uint16_t* kbase = (const uint16_t*)p.keys + (int64_t)b * p.key_stride_b + (int64_t)h * p.key_stride_h +
                           chunk_base * p.key_stride_n + 8 * j;
+  // (the query piece first: it has arrived, and is converted, while the rows are still on their way)
+  const u32x4 qpiece = group_query_piece(p, b, h, j);
   u32x4 kv[kCutUnroll];
 #pragma unroll
   for (int u = 0; u < kCutUnroll; ++u) {
@@ -349,13 +391,14 @@ __global__ __launch_bounds__(kCutThreads) void gemv_cut_slices_kernel(GemvParams
   if (!FRONT) cut = p.cut_splits[(int64_t)seg * kCutParts + (kCutParts - 1)];   // (the same for all: a scalar load beside the rows)
   __builtin_amdgcn_sched_barrier(0);
   float qf[8];
-  load_group_query<DT>(p.q, p.q_stride_b, b, h, p.group, j, qf);
+  group_query_through_lds<DT>(p, qpiece, j, sh_q, qf);
   __builtin_amdgcn_sched_barrier(0);
   float mine = 0.0f;
 #pragma unroll
   for (int u = 0; u < kCutUnroll; ++u) {
     const float sc = row_score<DT>(qf, kv[u], p.scale);
     if (j == u) mine = sc;
+    __builtin_amdgcn_sched_barrier(0);   // row after row: scheduled together, the rows' converted values take 100 registers
   }
   if (j < kCutUnroll) sh_key[rg * kCutUnroll + j] = score_key(mine);
   bool have_cut = true;
