@@ -181,6 +181,7 @@ __device__ __forceinline__ void sum_group_query(const uint16_t* qb, float (&qf)[
     for (int g = 0; g < P; ++g)
 #pragma unroll
       for (int i = 0; i < 8; ++i) qf[i] = (g0 + g == 0) ? Elem<DT>::get(w[g], i) : qf[i] + Elem<DT>::get(w[g], i);
+    if (P < G && PAR >= 2) __builtin_amdgcn_sched_barrier(0);   // (batch after batch: scheduled together they would all be in flight after all)
   }
 }
 template <int DT, int PAR = 8>

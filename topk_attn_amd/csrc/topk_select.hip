@@ -1408,12 +1408,13 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
         kv[u] = *(const u32x4*)(kbase + (int64_t)(t < nn ? t : nn - 1) * g.key_stride_n);
       }
       __builtin_amdgcn_sched_barrier(0);   // the rows are asked for before the query (whose conversion waits for it)
-      if (base == 0) load_group_query<DT>(g.q, g.q_stride_b, b, h, g.group, j, qf);
+      if (base == 0) load_group_query<DT, 1>(g.q, g.q_stride_b, b, h, g.group, j, qf);   // (head after head: sixteen rows per lane are in flight, and two heads beside them spilled registers)
       float mine = 0.0f;
 #pragma unroll
       for (int u = 0; u < kRows; ++u) {
         const float s = row_score<DT>(qf, kv[u], g.scale);
         if (j == u) mine = s;
+        if (u % 4 == 3) __builtin_amdgcn_sched_barrier(0);   // (four rows at a time: all sixteen scheduled together spilled registers)
       }
       const int t = base + rg * kRows + j;
       if (t < nn) sh_key[t] = score_key(mine);
