@@ -42,6 +42,18 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_readlane((int)wave_max_in_last_lane(v), 63);
 }
 
+// The per-wave slots of a workgroup of W waves, combined by the first W lanes of every wave: one LDS read and log2(W)
+// steps across the lanes instead of W reads per thread.  `lane` < `below` picks the slots that count (W: all of them).
+template <int W>
+__device__ __forceinline__ uint32_t ws_slots_sum(const uint32_t* slots, int lane, int from, int below) {
+  uint32_t v = lane >= from && lane < below ? slots[lane < W ? lane : 0] : 0u;
+  if (W > 1) v += lane_xor<1>(v);
+  if (W > 2) v += lane_xor<2>(v);
+  if (W > 4) v += lane_xor<4>(v);
+  if (W > 8) v += lane_xor<8>(v);
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
+}
+
 // Order-preserving key of a score, as score_key() (NaN lowest, -0 == +0).
 __device__ __forceinline__ uint32_t ws_key(float x) {
   const uint32_t u = __builtin_bit_cast(uint32_t, x + 0.0f);
@@ -102,8 +114,7 @@ __device__ __forceinline__ void ws_find_bin(WsShared<W>& sh, uint32_t need, int 
   uint32_t higher = wave_total - inc;            // entries in the bins of higher lanes of this wave
   if (lane == 0) sh.wave_a[wave] = wave_total;
   __syncthreads();
-#pragma unroll
-  for (int w = 1; w < W; ++w) higher += w > wave ? sh.wave_a[w] : 0u;
+  higher += ws_slots_sum<W>(sh.wave_a, lane, wave + 1, W);   // the waves above
   if (higher < need && need <= higher + tot) {   // exactly one thread
     sh.owner[0] = (uint32_t)tid;
     sh.owner[1] = higher;
@@ -159,14 +170,8 @@ __device__ __forceinline__ uint32_t ws_exclusive(uint32_t mine, int tid, WsShare
   __syncthreads();
   if (lane == 63) sh.wave_a[wave] = inc;
   __syncthreads();
-  uint32_t all = 0;
-#pragma unroll
-  for (int w = 0; w < W; ++w) {
-    const uint32_t s = sh.wave_a[w];
-    pos += w < wave ? s : 0u;
-    all += s;
-  }
-  if (total) *total = all;
+  pos += ws_slots_sum<W>(sh.wave_a, lane, 0, wave);   // the waves before
+  if (total) *total = ws_slots_sum<W>(sh.wave_a, lane, 0, W);
   return pos;
 }
 
