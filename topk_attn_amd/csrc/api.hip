@@ -257,9 +257,10 @@ void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, 
   // 14.2 / 20.2, 16 x 16384 (k = 2048) 17.9 / 29.1, 32 x 16384 32.7 / 42.3, 8 x 9000 (k = 512) 13.7 / 15.9.  Up to 8192
   // tokens the registers of one workgroup win (8 x 8192, k = 512: 21.1 / 20.1 per step, 8 x 4096: 20.1 / 17.6).
   if (rows > kCutMaxRows) return;
-  // Segments that the candidate route takes as well (65536 tokens): that route from two segments on
-  // (decode steps: 1 x 65536 26.3 / 34.5, 16 x 65536 68.2 / 68.9, 32 x 65536 113.8 / 111.6, 64 x 65536 208.6 / 198.6).
-  if (rows > 65536 && chunk_len >= 65536) {
+  // Segments that the candidate route takes as well (65536 tokens): that route beyond sixteen segments
+  // (decode steps: 1 x 65536 22.2 / 34.5, 2 x 65536 23.3 / 33.9, 4 x 65536 33.6 / 40.6, 8 x 65536 45.8 / 49.1,
+  // 16 x 65536 68.0 / 68.5, 32 x 65536 113.8 / 111.6, 64 x 65536 208.6 / 198.6).
+  if (rows > (int64_t)1 << 20 && chunk_len >= 65536) {
     int cs = 0, cr = 0;
     candidate_plan(a, &cs, &cr);
     if (cs != 0) return;
