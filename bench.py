@@ -298,8 +298,12 @@ def build_workload(name, torch, ops, dev, args):
         return SparseDecode(torch, ops, dev, batch=1, seq_len=32768, name="c4-b1-32k", want_union=False)
     if name == "c4-share32k":   # one GPU's share of an 8-way head-sharded model, one sequence of 32768 tokens, output only
         return SparseDecode(torch, ops, dev, batch=1, hkv=1, group=8, seq_len=32768, name="c4-share32k", want_union=False)
+    if name == "c4-b1-16k":     # the same at 16384 tokens: segments that would also fit the registers of one workgroup
+        return SparseDecode(torch, ops, dev, batch=1, seq_len=16384, k=1024, name="c4-b1-16k", want_union=False)
     if name == "c1":
         return GemvTopk(torch, ops, dev, 1, 1, 1, 32768, 2048, "float16", 1, "c1", rotate=args.rotate)
+    if name == "c1-8x16k":      # rank-ordered top-k of eight heads of 16384 keys
+        return GemvTopk(torch, ops, dev, 1, 8, 1, 16384, 1024, "float16", 1, "c1-8x16k", rotate=args.rotate)
     if name == "c2":
         return CenterTopk(torch, ops, dev, rotate=args.rotate)
     if name == "c2-ref":   # the problem of the reference's recorded latencies (center_only_topk/gemv_topk.cu:2-7)
@@ -351,7 +355,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c2-ref", "c3", "c4", "c4-small", "c4-b1-32k", "c4-share32k", "c5", "c5-topk", "ra", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c1-8x16k", "c2", "c2-ref", "c3", "c4", "c4-small", "c4-b1-32k", "c4-b1-16k", "c4-share32k", "c5", "c5-topk", "ra", "copy"])
     ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--score-mode", type=int, default=0, choices=[0, 1],
