@@ -160,7 +160,8 @@ def test_lse_combine_matches_unsplit():
         assert abs(lse[r].item() - ref_lse) < 1e-3
 
 
-@pytest.mark.parametrize("k,sink,local,n", [(2048, 64, 512, 131072), (100, 0, 0, 5000), (300, 16, 16, 400), (64, 64, 64, 100)])
+@pytest.mark.parametrize("k,sink,local,n", [(2048, 64, 512, 131072), (100, 0, 0, 5000), (300, 16, 16, 400), (64, 64, 64, 100),
+                                            (2048, 64, 512, 65536), (4096, 0, 1, 65535)])
 def test_index_union(k, sink, local, n):
     from topk_attn_amd import ops
     announce("index_union k=%d sink=%d local=%d n=%d" % (k, sink, local, n))
@@ -349,7 +350,13 @@ def test_sparse_decode_step(dtype, out_dt, B, H, G, N, k, sink, local):
     (oracle.F16, 1, 1, 8, 16384, 4000, 64, 512, "equal"),
     (oracle.F16, 1, 2, 2, 5000, 700, 3000, 3000, "heavy"),        # sink range and local window overlap
     (oracle.BF16, 3, 2, 4, 9000, 2048, 1, 8999, "levels"),        # the window covers nearly everything
-    (oracle.F16, 2, 2, 1, 12289, 2048, 5, 7, "equal")])
+    (oracle.F16, 2, 2, 1, 12289, 2048, 5, 7, "equal"),
+    # 16385 .. 65536 tokens with the list asked for: the common-cut route with a list of its own for the attention, the
+    # caller's ascending list from the rank-ordered ids by one more launch (a bitmap of the sequence)
+    (oracle.F16, 1, 2, 4, 32768, 2048, 64, 512, "heavy"),
+    (oracle.BF16, 2, 3, 2, 20001, 1000, 100, 300, "levels"),
+    (oracle.F16, 1, 8, 4, 24000, 1400, 6000, 22000, "heavy"),     # more than 65536 rows; range and window overlap
+    (oracle.F16, 1, 1, 2, 65536, 2048, 0, 0, "equal")])
 def test_sparse_decode_step_union_only(dtype, B, H, G, N, k, sink, local, kind, out_dt=torch.float16):
     """Production form of the step: no rank-ordered output.  The union list must still equal the oracle's bit for
     bit — with heavy hitters, with 16-level keys (large tie buckets), with all keys equal (every token ties) and

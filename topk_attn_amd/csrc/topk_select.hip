@@ -1504,6 +1504,50 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
   write_rank_outputs(sh_sort, p, seg, chunk);
 }
 
+// The same for sequences of up to 65536 tokens, without a sort: the selected ids between the ranges are marked in a
+// bitmap of the sequence in LDS (8 KB), every thread counts the bits of its 64 tokens, one scan gives it its place, and it
+// writes its tokens in order - ascending because the threads own ascending stretches of the sequence.  Ids outside the
+// sequence are dropped, an id given twice is listed once (as the sorting form does).
+constexpr int kUnionBitmapMaxLen = 65536;
+__global__ __launch_bounds__(kSelThreads) void index_union_bitmap_kernel(UnionParams p) {
+  __shared__ uint32_t sh_bits[kUnionBitmapMaxLen / 32];
+  __shared__ uint32_t sh_wtot[kSelWaves];
+  const int tid = threadIdx.x;
+  const int seg = blockIdx.x;
+  const uint32_t n = (uint32_t)p.seq_len;
+  const uint32_t lo = (uint32_t)(p.sink < p.seq_len ? p.sink : p.seq_len);
+  const uint32_t hi = (uint32_t)(p.seq_len - p.local > (int64_t)lo ? p.seq_len - p.local : (int64_t)lo);
+  const int32_t* in = p.idx + (int64_t)seg * p.k;
+  sh_bits[2 * tid] = 0u;
+  sh_bits[2 * tid + 1] = 0u;
+  __syncthreads();
+  for (int i = tid; i < p.k; i += kSelThreads) {
+    const uint32_t id = (uint32_t)in[i];   // (a negative id is a large one here)
+    if (id >= lo && id < hi) atomicOr(&sh_bits[id >> 5], 1u << (id & 31u));
+  }
+  __syncthreads();
+  uint32_t w0 = sh_bits[2 * tid], w1 = sh_bits[2 * tid + 1];
+  uint32_t total;
+  const uint32_t before = block_exclusive_scan((uint32_t)__builtin_popcount(w0) + (uint32_t)__builtin_popcount(w1), sh_wtot, &total);
+  int32_t* out = p.out_idx + (int64_t)seg * (p.k + p.sink + p.local);
+  const uint32_t cap = (uint32_t)(p.k + p.sink + p.local);
+  uint32_t pos = lo + before;
+  const uint32_t first = 64u * (uint32_t)tid;
+  while (w0) {
+    out[pos++] = (int32_t)(first + (uint32_t)__builtin_ctz(w0));
+    w0 &= w0 - 1u;
+  }
+  while (w1) {
+    out[pos++] = (int32_t)(first + 32u + (uint32_t)__builtin_ctz(w1));
+    w1 &= w1 - 1u;
+  }
+  const uint32_t count = lo + total + (n - hi);
+  for (uint32_t i = (uint32_t)tid; i < lo; i += kSelThreads) out[i] = (int32_t)i;
+  for (uint32_t i = (uint32_t)tid; i < n - hi; i += kSelThreads) out[lo + total + i] = (int32_t)(hi + i);
+  for (uint32_t i = count + (uint32_t)tid; i < cap; i += kSelThreads) out[i] = -1;
+  if (tid == 0) p.out_count[seg] = (int32_t)count;
+}
+
 // Ascending duplicate-free union of the selected ids with [0,sink) and [n-local,n).
 // One workgroup per segment; the middle part is sorted ascending with the same bitonic network
 // (ids complemented so that "descending" composites are ascending ids).
@@ -1793,6 +1837,11 @@ int launch_select(const SelectParams& p, hipStream_t stream) {
 }
 
 int launch_index_union(const UnionParams& p, hipStream_t stream) {
+  if (p.seq_len <= kUnionBitmapMaxLen) {
+    LaunchTimer timer("index_union", stream);
+    index_union_bitmap_kernel<<<(unsigned)p.num_segments, kSelThreads, 0, stream>>>(p);
+    return hip_status(hipGetLastError());
+  }
   const int kpad = kpad_for(p.k);
   const size_t lds = 2 * (size_t)kpad * sizeof(uint64_t);
   if (allow_dynamic_lds((const void*)index_union_kernel, 144 * 1024) != TKA_OK) return TKA_EHIP;
