@@ -161,7 +161,7 @@ def test_lse_combine_matches_unsplit():
 
 
 @pytest.mark.parametrize("k,sink,local,n", [(2048, 64, 512, 131072), (100, 0, 0, 5000), (300, 16, 16, 400), (64, 64, 64, 100),
-                                            (2048, 64, 512, 65536), (4096, 0, 1, 65535)])
+                                            (2048, 64, 512, 65536), (4096, 0, 1, 65535), (2048, 64, 512, 262144), (1024, 8, 8, 300000)])
 def test_index_union(k, sink, local, n):
     from topk_attn_amd import ops
     announce("index_union k=%d sink=%d local=%d n=%d" % (k, sink, local, n))

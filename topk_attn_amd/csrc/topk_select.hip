@@ -1504,13 +1504,15 @@ __global__ __launch_bounds__(kSelThreads) void select_small_kernel(GemvParams g,
   write_rank_outputs(sh_sort, p, seg, chunk);
 }
 
-// The same for sequences of up to 65536 tokens, without a sort: the selected ids between the ranges are marked in a
-// bitmap of the sequence in LDS (8 KB), every thread counts the bits of its 64 tokens, one scan gives it its place, and it
-// writes its tokens in order - ascending because the threads own ascending stretches of the sequence.  Ids outside the
-// sequence are dropped, an id given twice is listed once (as the sorting form does).
-constexpr int kUnionBitmapMaxLen = 65536;
+// The same for sequences of up to 262144 tokens, without a sort: the selected ids between the ranges are marked in a
+// bitmap of the sequence in LDS (WORDS x 4 KB: 8 KB for 65536 tokens), every thread counts the bits of its 32 WORDS
+// tokens, one scan gives it its place, and it writes its tokens in order - ascending because the threads own ascending
+// stretches of the sequence.  Ids outside the sequence are dropped, an id given twice is listed once (as the sorting form
+// does).
+constexpr int kUnionBitmapMaxLen = 262144;
+template <int WORDS>
 __global__ __launch_bounds__(kSelThreads) void index_union_bitmap_kernel(UnionParams p) {
-  __shared__ uint32_t sh_bits[kUnionBitmapMaxLen / 32];
+  __shared__ uint32_t sh_bits[WORDS * kSelThreads];
   __shared__ uint32_t sh_wtot[kSelWaves];
   const int tid = threadIdx.x;
   const int seg = blockIdx.x;
@@ -1518,28 +1520,33 @@ __global__ __launch_bounds__(kSelThreads) void index_union_bitmap_kernel(UnionPa
   const uint32_t lo = (uint32_t)(p.sink < p.seq_len ? p.sink : p.seq_len);
   const uint32_t hi = (uint32_t)(p.seq_len - p.local > (int64_t)lo ? p.seq_len - p.local : (int64_t)lo);
   const int32_t* in = p.idx + (int64_t)seg * p.k;
-  sh_bits[2 * tid] = 0u;
-  sh_bits[2 * tid + 1] = 0u;
+#pragma unroll
+  for (int w = 0; w < WORDS; ++w) sh_bits[WORDS * tid + w] = 0u;
   __syncthreads();
   for (int i = tid; i < p.k; i += kSelThreads) {
     const uint32_t id = (uint32_t)in[i];   // (a negative id is a large one here)
     if (id >= lo && id < hi) atomicOr(&sh_bits[id >> 5], 1u << (id & 31u));
   }
   __syncthreads();
-  uint32_t w0 = sh_bits[2 * tid], w1 = sh_bits[2 * tid + 1];
+  uint32_t bits[WORDS], mine = 0;
+#pragma unroll
+  for (int w = 0; w < WORDS; ++w) {
+    bits[w] = sh_bits[WORDS * tid + w];
+    mine += (uint32_t)__builtin_popcount(bits[w]);
+  }
   uint32_t total;
-  const uint32_t before = block_exclusive_scan((uint32_t)__builtin_popcount(w0) + (uint32_t)__builtin_popcount(w1), sh_wtot, &total);
+  const uint32_t before = block_exclusive_scan(mine, sh_wtot, &total);
   int32_t* out = p.out_idx + (int64_t)seg * (p.k + p.sink + p.local);
   const uint32_t cap = (uint32_t)(p.k + p.sink + p.local);
   uint32_t pos = lo + before;
-  const uint32_t first = 64u * (uint32_t)tid;
-  while (w0) {
-    out[pos++] = (int32_t)(first + (uint32_t)__builtin_ctz(w0));
-    w0 &= w0 - 1u;
-  }
-  while (w1) {
-    out[pos++] = (int32_t)(first + 32u + (uint32_t)__builtin_ctz(w1));
-    w1 &= w1 - 1u;
+#pragma unroll
+  for (int w = 0; w < WORDS; ++w) {
+    const uint32_t first = 32u * (uint32_t)(WORDS * tid + w);
+    uint32_t left = bits[w];
+    while (left) {
+      out[pos++] = (int32_t)(first + (uint32_t)__builtin_ctz(left));
+      left &= left - 1u;
+    }
   }
   const uint32_t count = lo + total + (n - hi);
   for (uint32_t i = (uint32_t)tid; i < lo; i += kSelThreads) out[i] = (int32_t)i;
@@ -1839,7 +1846,8 @@ int launch_select(const SelectParams& p, hipStream_t stream) {
 int launch_index_union(const UnionParams& p, hipStream_t stream) {
   if (p.seq_len <= kUnionBitmapMaxLen) {
     LaunchTimer timer("index_union", stream);
-    index_union_bitmap_kernel<<<(unsigned)p.num_segments, kSelThreads, 0, stream>>>(p);
+    if (p.seq_len <= 65536) index_union_bitmap_kernel<2><<<(unsigned)p.num_segments, kSelThreads, 0, stream>>>(p);
+    else index_union_bitmap_kernel<8><<<(unsigned)p.num_segments, kSelThreads, 0, stream>>>(p);
     return hip_status(hipGetLastError());
   }
   const int kpad = kpad_for(p.k);
