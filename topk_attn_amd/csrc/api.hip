@@ -1109,7 +1109,8 @@ static bool sd_union_handoff(const tka_sparse_decode_args* a) { return !a->out_u
 // hand-off list of its own in the workspace, and the caller's list is made from the rank-ordered ids by one more launch
 // behind the attention (8 x 32768 tokens: 36 instead of 43 us per step).  `g`: the stage-1 arguments of the step.
 static bool sd_list_behind(const tka_sparse_decode_args* a, const tka_gemv_topk_args& g) {
-  if (sd_union_handoff(a) || a->seq_len <= select_cand_capacity()) return false;
+  // (beyond a million rows the routes that make the list themselves are as quick: 48 x 32768 tokens 98.2 / 95.9 us)
+  if (sd_union_handoff(a) || a->seq_len <= select_cand_capacity() || (int64_t)a->batch * a->num_kv_heads * a->seq_len > (int64_t)1 << 20) return false;
   tka_gemv_topk_args probe = g;
   int32_t di;
   probe.out_idx = &di;
