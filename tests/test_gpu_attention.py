@@ -542,6 +542,16 @@ def test_sparse_decode_step_forced_redo(hooks):
     test_sparse_decode_step_union_only(oracle.BF16, 1, 2, 4, 66001, 1500, 32, 100, "levels")
 
 
+def test_sparse_decode_step_list_behind_forced_redo(hooks):
+    """A caller that asks for the ascending list on segments that the common-cut route takes (the list for the attention stays
+    in the workspace, the caller's list is made from the rank-ordered ids by one more launch), with every segment redone from
+    the keys by its first ranking workgroup; and the same with the cuts of every other segment never announced."""
+    hooks(force_segment_redo=1)
+    test_sparse_decode_step_union_only(oracle.F16, 1, 2, 4, 30001, 1500, 32, 100, "levels")
+    hooks(tau_spin_limit=64, tau_withhold_mod=2, tau_withhold_rem=1, tau_withhold_mode=0)
+    test_sparse_decode_step_union_only(oracle.F16, 1, 8, 2, 20000, 1000, 64, 512, "heavy")
+
+
 def test_sparse_decode_step_threshold_never_published(hooks):
     """Union mode when the streaming workgroups of one segment run out of their wait for the threshold: that segment
     is redone from the keys, the other keeps the candidate route, union lists and outputs as the oracle's."""
