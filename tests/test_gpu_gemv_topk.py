@@ -518,17 +518,18 @@ def test_common_cut_route_adversarial_sample_falls_back_in_three_launches():
     _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k, redone=1)
 
 
-@pytest.mark.parametrize("mod,rem,affected", [(1, 0, 4), (2, 1, 2)])
-def test_common_cut_route_cut_never_announced(hooks, mod, rem, affected):
+@pytest.mark.parametrize("H,N,k,mod,rem,affected", [(4, 32768, 2048, 1, 0, 4), (4, 32768, 2048, 2, 1, 2), (20, 16384, 1024, 3, 1, 7)])
+def test_common_cut_route_cut_never_announced(hooks, H, N, k, mod, rem, affected):
     """Calls of more than 65536 rows find their cuts in the first workgroups of the GEMV launch, and the scoring
     workgroups wait for their segment's word - a bounded wait.  With the word of chosen segments withheld and the wait
     shortened, every slice of those segments is marked and the ranking kernel redoes them from the keys; the others keep
-    the route.  Every kernel runs to its end."""
-    announce("gemv_topk common-cut route, the cut of segments s %% %d == %d is never announced" % (mod, rem))
+    the route.  Every kernel runs to its end.  The call of twenty heads has more scoring workgroups than run at once:
+    there the sampling workgroups score tokens themselves afterwards, and wait like the others."""
+    announce("gemv_topk common-cut route, %d x %d tokens, the cut of segments s %% %d == %d is never announced" % (H, N, mod, rem))
     hooks(tau_spin_limit=64, tau_withhold_mod=mod, tau_withhold_rem=rem, tau_withhold_mode=0)
     rng = np.random.default_rng(58)
-    K = randn_bits(rng, (1, 32768, 4, 128), oracle.F16)
-    _check_long(K, randn_bits(rng, (1, 4, 128), oracle.F16), oracle.F16, 1, 2048, redone=affected, gave_up=affected * 128)
+    K = randn_bits(rng, (1, N, H, 128), oracle.F16)
+    _check_long(K, randn_bits(rng, (1, H, 128), oracle.F16), oracle.F16, 1, k, redone=affected, gave_up=affected * (N // 256))
 
 
 def test_common_cut_route_sample_sits_low():

@@ -330,7 +330,9 @@ __global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
 // then the call's epoch in the segment's word of p.tau_words, for which the first thread of a scoring workgroup waits
 // before the compare - a bounded wait: a workgroup that never sees the word marks its slices (kCutGaveUp in the count),
 // and the ranking kernel redoes such a segment from the keys.  The sampling workgroups come first in the grid, so they
-// run before any workgroup that waits for them; nothing depends on that but the speed.
+// run before any workgroup that waits for them; nothing depends on that but the speed.  With p.samplers_score they are not
+// extra workgroups: having published their segment's cut they score the tokens that their place in the grid names, like
+// the others (the cut they then wait for is that of a sampling workgroup no later in the grid than themselves).
 template <int DT, bool FRONT, int L>
 __global__ __launch_bounds__(kCutThreads, 8) void gemv_cut_slices_kernel(GemvParams p) {
   constexpr int kTokens = 2 * kCutTokensPerWg;
@@ -346,31 +348,31 @@ __global__ __launch_bounds__(kCutThreads, 8) void gemv_cut_slices_kernel(GemvPar
   SegPos at;
   if (FRONT) {
     const int segs = p.batch * p.num_kv_heads * p.num_chunks;
+    uint32_t wg = blockIdx.x;
     if ((int)blockIdx.x < segs) {
-      at = seg_position_flat(p, (int)blockIdx.x);
-      pair = -1;
-    } else {
-      const uint32_t wg = blockIdx.x - (uint32_t)segs, per_seg = (uint32_t)((p.chunk_len + kTokens - 1) / kTokens);
-      const uint32_t seg = (per_seg & (per_seg - 1u)) == 0u ? wg >> (31 - __builtin_clz(per_seg)) : wg / per_seg;   // (mostly a power of two)
-      at = seg_position_flat(p, (int)seg);
-      pair = (int)(wg - seg * per_seg);
+      __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
+      const SegPos mine = seg_position_flat(p, (int)blockIdx.x);
+      sample_segment<DT, true, true>(p, mine, sh_q);
+      // the part ends have completed (rank_samples) before the word that announces them leaves; relaxed device-scope
+      // accesses on both sides, as for the thresholds of the candidate route: a fence would write back and invalidate
+      // whole caches in the middle of the stream
+      __syncthreads();
+      if (tid == 0 && !(p.withhold_mod > 0 && mine.seg % p.withhold_mod == p.withhold_rem))   // (testing: this segment's word is withheld)
+        __hip_atomic_store(p.tau_words + 2 * mine.seg, (uint64_t)p.epoch << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (the epoch where the candidate route keeps its own)
+      if (!p.samplers_score) return;
+      __builtin_amdgcn_s_setprio(0);
+    } else if (!p.samplers_score) {
+      wg -= (uint32_t)segs;
     }
+    const uint32_t per_seg = (uint32_t)((p.chunk_len + kTokens - 1) / kTokens);
+    const uint32_t seg = (per_seg & (per_seg - 1u)) == 0u ? wg >> (31 - __builtin_clz(per_seg)) : wg / per_seg;   // (mostly a power of two)
+    at = seg_position_flat(p, (int)seg);
+    pair = (int)(wg - seg * per_seg);
   } else {
     at = seg_position(p);
     pair = (int)blockIdx.x;   // this workgroup's 512 tokens inside the segment
   }
   const int b = at.b, h = at.h, chunk = at.chunk, seg = at.seg;
-  if (FRONT && pair < 0) {
-    __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
-    sample_segment<DT, true, true>(p, at, sh_q);
-    // the part ends have completed (rank_samples) before the word that announces them leaves; relaxed device-scope
-    // accesses on both sides, as for the thresholds of the candidate route: a fence would write back and invalidate
-    // whole caches in the middle of the stream
-    __syncthreads();
-    if (tid == 0 && !(p.withhold_mod > 0 && seg % p.withhold_mod == p.withhold_rem))   // (testing: this segment's word is withheld)
-      __hip_atomic_store(p.tau_words + 2 * seg, (uint64_t)p.epoch << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (the epoch where the candidate route keeps its own)
-    return;
-  }
   const int j = tid & 15, rg = tid >> 4;
   const int64_t chunk_base = p.cluster_ids ? (int64_t)p.cluster_ids[seg] * p.chunk_len : (int64_t)chunk * p.chunk_len;
   const int n = (int)p.chunk_len;
@@ -476,7 +478,7 @@ int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, 
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
   const int64_t wgs_per_seg = (p.chunk_len + 2 * kCutTokensPerWg - 1) / (2 * kCutTokensPerWg);
   if (!slices_ok(p) || segs * (wgs_per_seg + 1) > 0x7fffffffLL || !grid_ok(p)) return TKA_EINVAL;
-  const dim3 wgs = front_sampling ? dim3((unsigned)(segs * (wgs_per_seg + 1)))
+  const dim3 wgs = front_sampling ? dim3((unsigned)(segs * (wgs_per_seg + (p.samplers_score ? 0 : 1))))
                                   : dim3((unsigned)wgs_per_seg, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
   if (front_sampling && (p.num_samples != kCutSamplesOnce || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
                          !p.tau_words || p.epoch == 0 || p.tau_spin_limit < 1))
