@@ -152,7 +152,7 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
   g->withhold_mod = g->withhold_rem = g->withhold_mode = 0;
   g->num_samples = g->sample_rank = g->sample_wgs = g->early_wgs = 0;
   g->split_ranks = 0;
-  g->samplers_score = 0;
+  g->samplers_score = g->interleave_segs = 0;
   g->cand = nullptr;
   g->cand_seg_stride = 0;
   g->cand_head = nullptr;
@@ -367,6 +367,12 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
         // tokens 34.05 -> 33.8 us per decode step, 8 x 65536 46.7 -> 46.35).  Where all run at once the samplers would then
         // be the last to finish (2 x 65536: 23.35 -> 25.0).
         cp.samplers_score = (int64_t)segs * ((chunk_len + 2 * kCutTokensPerWg - 1) / (2 * kCutTokensPerWg)) > 512 ? 1 : 0;
+        // Consecutive scoring workgroups take the same tokens of consecutive segments when the number of segments is a power
+        // of two, instead of consecutive tokens of one segment: with sixteen or thirty-two heads a token's rows of one head
+        // lie 4 or 8 KB apart, and the workgroups that run together, all on the same few heads, crowd the same memory
+        // channels (per decode step, 16 x 32768 tokens 49.3 -> 43.8 us, 32 x 32768 78.8 -> 69.8, 2 x 8 x 32768 44.3 -> 43.0,
+        // 16 x 16384 33.9 -> 32.9, 8 x 32768 30.35 -> 30.1; 12 and 24 x 32768 would lose 0.6-0.7 and keep the other order).
+        cp.interleave_segs = (segs & (segs - 1)) == 0 ? 1 : 0;
         rc = launch_gemv_cut_slices(cp, a->dtype, true, stream);
       } else {
         rc = launch_cut_samples(cp, a->dtype, stream);

@@ -343,7 +343,9 @@ __global__ __launch_bounds__(kCutThreads, 8) void gemv_cut_slices_kernel(GemvPar
   const int tid = threadIdx.x;
   // FRONT: a flat grid, the sampling workgroups of all segments first (in a grid with the segments in y and z every
   // segment's own would come right before its scoring workgroups - too late on calls of several generations of
-  // workgroups: 16 x 32768 tokens 56 instead of 50 us per decode step), then the scoring workgroups segment by segment
+  // workgroups: 16 x 32768 tokens 56 instead of 50 us per decode step), then the scoring workgroups segment by segment -
+  // or, with p.interleave_segs, token range by token range: consecutive workgroups then read neighbouring heads' rows of
+  // the same tokens, which lie side by side in a cache of the usual layout
   int pair;
   SegPos at;
   if (FRONT) {
@@ -364,10 +366,18 @@ __global__ __launch_bounds__(kCutThreads, 8) void gemv_cut_slices_kernel(GemvPar
     } else if (!p.samplers_score) {
       wg -= (uint32_t)segs;
     }
-    const uint32_t per_seg = (uint32_t)((p.chunk_len + kTokens - 1) / kTokens);
-    const uint32_t seg = (per_seg & (per_seg - 1u)) == 0u ? wg >> (31 - __builtin_clz(per_seg)) : wg / per_seg;   // (mostly a power of two)
+    uint32_t seg;
+    if (p.interleave_segs) {
+      const uint32_t usegs = (uint32_t)segs;
+      const uint32_t q = (usegs & (usegs - 1u)) == 0u ? wg >> (31 - __builtin_clz(usegs)) : wg / usegs;
+      seg = wg - q * usegs;
+      pair = (int)q;
+    } else {
+      const uint32_t per_seg = (uint32_t)((p.chunk_len + kTokens - 1) / kTokens);
+      seg = (per_seg & (per_seg - 1u)) == 0u ? wg >> (31 - __builtin_clz(per_seg)) : wg / per_seg;   // (mostly a power of two)
+      pair = (int)(wg - seg * per_seg);
+    }
     at = seg_position_flat(p, (int)seg);
-    pair = (int)(wg - seg * per_seg);
   } else {
     at = seg_position(p);
     pair = (int)blockIdx.x;   // this workgroup's 512 tokens inside the segment

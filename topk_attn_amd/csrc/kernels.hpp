@@ -27,6 +27,7 @@ struct GemvParams {
   // (mode 0) or published only once a slice of the segment has given up, after a bounded wait (mode 1); 0 = off
   int withhold_mod, withhold_rem, withhold_mode;
   int num_samples, sample_rank;   // per segment
+  int interleave_segs;        // the same kernel: consecutive scoring workgroups take the same tokens of consecutive segments
   int samplers_score;         // gemv_cut_slices_kernel with front sampling: the sampling workgroups go on to score tokens like the others
   uint64_t split_ranks;       // common-cut route: byte g - 1 holds the 1-based rank of the sample that ends part g of the candidates
                               // (ascending; byte kCutParts - 1 equals sample_rank), see gemv_cut_split_ranks
