@@ -406,6 +406,15 @@ def test_long_segment_forced_redo(hooks):
     _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 3000, redone=2)
 
 
+def test_long_segments_sixteen_heads():
+    """Sixteen KV heads: the rows of one head lie 4 KB apart, and the streaming workgroups take their slices in units
+    that go round the segments instead of segment by segment (137 slices per segment: the last unit of each is short)."""
+    announce("gemv_topk long segments, sixteen heads (N=70001 k=2048): slices taken round the segments")
+    rng = np.random.default_rng(44)
+    K = randn_bits(rng, (1, 70001, 16, 128), oracle.F16)
+    _check_long(K, randn_bits(rng, (1, 16, 128), oracle.F16), oracle.F16, 1, 2048, redone=0)
+
+
 @pytest.mark.parametrize("withheld", [(2, 1), (1, 0)])
 def test_long_segment_threshold_never_published(hooks, withheld):
     """The bounded wait of the streaming workgroups runs out: the threshold of one of the two segments (then of
