@@ -509,11 +509,11 @@ __device__ __forceinline__ void stream_slice(const unsigned char* sbase, uint32_
 
 // Grid: p.sample_wgs sampling workgroups first (so that they are resident before any workgroup that waits for
 // them), then the streaming workgroups.  Slices (512 tokens) are numbered segment-major (or, with
-// p.interleave_segs, in units that go round the segments, see launch_gemv_candidates).  The first
+// ROUND, in units that go round the segments, see launch_gemv_candidates).  The first
 // p.early_wgs streaming workgroups take kEarlySlices consecutive slices each, all later ones a single slice:
 // the workgroups that start together with the sampling would otherwise sit idle on their CU until the
 // thresholds arrive; with more rows to stream they reach that point when the thresholds are there.
-template <int DT>
+template <int DT, bool ROUND>
 __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8, 8))) void gemv_candidates_kernel(GemvParams p) {
   __shared__ uint32_t sh[kHistBins + 16];   // streaming: keys of kEarlySlices * 512 tokens + wave counts; sampling: histogram
   static_assert(kEarlySlices * kCandThreads <= kHistBins, "LDS of the streaming role");
@@ -539,7 +539,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
 
   int64_t first_seg;
   int first_wg;
-  if (p.interleave_segs) {
+  if (ROUND) {
     // slices numbered in units of kEarlySlices consecutive slices of one segment, the units segment after segment and
     // then on through the tokens: unit u = slices kEarlySlices (u / segs) ... of segment u % segs (a segment's last
     // unit may be short: the numbers behind its end name no slice)
@@ -730,10 +730,13 @@ int launch_gemv_candidates(const GemvParams& p0, int dtype, hipStream_t stream) 
   const int64_t wgs = p.sample_wgs + early + (slices - early * kEarlySlices);
   if (wgs > 0x7fffffffLL) return TKA_EUNSUPPORTED;
   LaunchTimer timer("gemv_candidates", stream);
-  if (dtype == TKA_F16)
-    gemv_candidates_kernel<TKA_F16><<<(unsigned)wgs, kCandThreads, 0, stream>>>(p);
-  else
-    gemv_candidates_kernel<TKA_BF16><<<(unsigned)wgs, kCandThreads, 0, stream>>>(p);
+  if (dtype == TKA_F16) {
+    if (p.interleave_segs) gemv_candidates_kernel<TKA_F16, true><<<(unsigned)wgs, kCandThreads, 0, stream>>>(p);
+    else gemv_candidates_kernel<TKA_F16, false><<<(unsigned)wgs, kCandThreads, 0, stream>>>(p);
+  } else {
+    if (p.interleave_segs) gemv_candidates_kernel<TKA_BF16, true><<<(unsigned)wgs, kCandThreads, 0, stream>>>(p);
+    else gemv_candidates_kernel<TKA_BF16, false><<<(unsigned)wgs, kCandThreads, 0, stream>>>(p);
+  }
   return hip_status(hipGetLastError());
 }
 
