@@ -178,3 +178,25 @@ def test_c3_dense_flash_decode_full_size():
         ref = torch.softmax(logits, dim=-1) @ V[0, :, h].float()
         for o in (out, out_1, out_37):
             assert float((o[0, h * G:(h + 1) * G].float() - ref).abs().max()) < 2e-3
+
+
+def test_dense_flash_decode_sixteen_heads_full_size():
+    """Sixteen KV heads over 131072 tokens: a head's rows lie 4 KB apart and the cache of one batch entry is half a
+    gigabyte, so the matrix-core kernel's grid counts the heads in x and the splits in y.  Against torch fp32
+    attention (tolerance 2e-3), and across split counts."""
+    from topk_attn_amd import ops
+    B, H, G, N = 1, 16, 2, 131072
+    announce("full size: Hq=%d Hkv=%d N=%d dense flash-decoding, heads in the grid's x" % (H * G, H, N))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(304)
+    q = torch.randn((B, H * G, 128), generator=gen, device="cuda").to(torch.float16)
+    K = _randn16((B, N, H, 128), torch.float16, gen)
+    V = _randn16((B, N, H, 128), torch.float16, gen)
+    out = ops.flash_decode(q, K, V, SCALE, group=G)
+    out_5 = ops.flash_decode(q, K, V, SCALE, group=G, num_splits=5)
+    torch.cuda.synchronize()
+    for h in range(H):
+        logits = (q[0, h * G:(h + 1) * G].float() @ K[0, :, h].float().T) * SCALE
+        ref = torch.softmax(logits, dim=-1) @ V[0, :, h].float()
+        for o in (out, out_5):
+            assert float((o[0, h * G:(h + 1) * G].float() - ref).abs().max()) < 2e-3

@@ -160,6 +160,7 @@ struct AttnParams {
   int batch, num_kv_heads, group, num_splits;
   int idx_len;
   int tokens_per_split;     // positions per workgroup
+  int head_fastest;         // matrix-core kernel: the grid's x counts the KV heads and its y the splits (set by its launcher)
   float scale_log2e;        // scale * log2(e)
   // One split per row: the VALU kernel normalises and writes the result itself (no combine launch) when out is set.
   void* out;                // [batch][query heads][128] or nullptr
