@@ -34,7 +34,9 @@ def _dense_ref(q, K, V, dtype, G, scale):
 
 @pytest.mark.parametrize("dtype,B,H,G,N,splits", [
     (oracle.F16, 1, 8, 4, 4096, 0), (oracle.F16, 2, 2, 1, 1000, 3), (oracle.BF16, 1, 2, 8, 3333, 7),
-    (oracle.F16, 1, 1, 2, 77, 1), (oracle.BF16, 2, 4, 4, 2048, 64), (oracle.BF16, 3, 2, 1, 700, 1)])
+    (oracle.F16, 1, 1, 2, 77, 1), (oracle.BF16, 2, 4, 4, 2048, 64), (oracle.BF16, 3, 2, 1, 700, 1),
+    # sixteen and thirty-two KV heads with one query head each (rows of a head 4 and 8 KB apart: the heads in the grid's x)
+    (oracle.F16, 2, 16, 1, 1500, 0), (oracle.BF16, 1, 32, 1, 999, 5), (oracle.F16, 1, 16, 1, 300, 1)])
 def test_flash_decode_dense(dtype, B, H, G, N, splits):
     from topk_attn_amd import ops
     announce("flash_decode dense dtype=%d B=%d H=%d G=%d N=%d splits=%d" % (dtype, B, H, G, N, splits))

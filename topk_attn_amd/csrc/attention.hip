@@ -39,8 +39,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
   const int tid = threadIdx.x;
   const int j = tid & 15;
   const int rg = tid >> 4;
-  const int split = blockIdx.x;
-  const int h = blockIdx.y;
+  const int split = MODE == MODE_DENSE && p.head_fastest ? blockIdx.y : blockIdx.x;   // (see launch_attn_partial)
+  const int h = MODE == MODE_DENSE && p.head_fastest ? blockIdx.x : blockIdx.y;
   const int b = blockIdx.z;
   const int64_t seg = (int64_t)b * p.num_kv_heads + h;
 
@@ -333,8 +333,16 @@ int launch_partial_dt(const AttnParams& p, dim3 grid, hipStream_t stream) {
 
 }  // namespace
 
-int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream) {
+int launch_attn_partial(const AttnParams& p0, int dtype, hipStream_t stream) {
+  AttnParams p = p0;
+  // The dense scan where a head's rows lie a multiple of 4 KB apart (16 or 32 KV heads in a cache laid out
+  // [token][head][128]): the heads in the grid's x, so that the workgroups that run together take the same tokens of all heads
+  // instead of long runs of a few heads, which crowd the same memory channels (one query head per KV head: 2 x 16 heads x
+  // 131072 tokens 375 -> 345 us, 32 heads 417 -> 361, 16 x 65536 115 -> 95).  Other strides lose 1-5 % that way and keep
+  // the splits in x (4 x 8 x 131072: 335 against 330).
+  p.head_fastest = !p.kv_idx && !p.kv_logit && p.num_splits <= 65535 && (p.kv_stride_n * 2) % 4096 == 0 ? 1 : 0;
   dim3 grid((unsigned)p.num_splits, (unsigned)p.num_kv_heads, (unsigned)p.batch);
+  if (p.head_fastest) grid = dim3((unsigned)p.num_kv_heads, (unsigned)p.num_splits, (unsigned)p.batch);
   LaunchTimer timer(p.kv_logit ? "attn_partial_logit" : (p.kv_idx ? "attn_partial_indexed" : "attn_partial_dense"), stream);
   return dtype == TKA_F16 ? launch_partial_dt<TKA_F16>(p, grid, stream) : launch_partial_dt<TKA_BF16>(p, grid, stream);
 }
