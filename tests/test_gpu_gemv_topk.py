@@ -446,6 +446,8 @@ def test_long_segment_threshold_never_published(hooks, withheld):
                                              # segments of 8193 .. 16384 tokens on calls of more than 65536 rows
                                              (oracle.F16, 1, 8, 1, 16384, 1024), (oracle.BF16, 2, 8, 4, 9001, 512),
                                              (oracle.F16, 1, 5, 2, 16384, 2048),
+                                             # sixteen heads (rows of a head 4 KB apart) in a number of segments that is no power of two
+                                             (oracle.F16, 3, 16, 1, 9000, 500),
                                              # more than 655360 rows (several generations of GEMV workgroups)
                                              (oracle.F16, 3, 8, 1, 32768, 2048), (oracle.BF16, 5, 8, 2, 20000, 1000)])
 def test_common_cut_route(dtype, B, H, G, N, k):
