@@ -292,6 +292,8 @@ def build_workload(name, torch, ops, dev, args):
         return PlainCopy(torch, dev)
     if name == "c4":
         return SparseDecode(torch, ops, dev, num_splits=args.splits)
+    if name == "c4-out":        # the same step for a caller that wants the output alone
+        return SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-out", want_union=False)
     if name == "c4-small":
         return SparseDecode(torch, ops, dev, batch=2, seq_len=16384, name="c4-small")
     if name == "c4-b1-32k":     # one sequence of 32768 tokens on one GPU (all 8 KV heads), output only
@@ -315,6 +317,9 @@ def build_workload(name, torch, ops, dev, args):
     if name == "c5":       # the tie-stress step: selection under exact ties at 1M tokens, attention over the selected tokens
         return SparseDecode(torch, ops, dev, batch=1, hkv=8, group=8, seq_len=1048576, k=4096, sink=0, local=0,
                             dtype="bfloat16", heavy=0.0, seed=5, name="c5", levels=True)
+    if name == "c5-out":   # the same step for a caller that wants the output alone
+        return SparseDecode(torch, ops, dev, batch=1, hkv=8, group=8, seq_len=1048576, k=4096, sink=0, local=0,
+                            dtype="bfloat16", heavy=0.0, seed=5, name="c5-out", levels=True, want_union=False)
     if name == "c5-topk":  # its selection stage alone, rank-ordered output
         return GemvTopk(torch, ops, dev, 1, 8, 8, 1048576, 4096, "bfloat16", 5, "c5-topk", levels=True)
     raise ValueError(name)
@@ -355,7 +360,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c1-8x16k", "c2", "c2-ref", "c3", "c4", "c4-small", "c4-b1-32k", "c4-b1-16k", "c4-share32k", "c5", "c5-topk", "ra", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c1-8x16k", "c2", "c2-ref", "c3", "c4", "c4-out", "c4-small", "c4-b1-32k", "c4-b1-16k", "c4-share32k", "c5", "c5-out", "c5-topk", "ra", "copy"])
     ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--score-mode", type=int, default=0, choices=[0, 1],

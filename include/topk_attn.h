@@ -143,6 +143,9 @@ typedef struct tka_test_hooks {
   int32_t union_handoff_order; /* 1: tka_sparse_decode_step writes out_union_idx the way it hands the list to
                                   its attention when the caller does not ask for it: in the order of the
                                   route, which may list -1 (an id the attention skips) inside the count  */
+  int32_t fused_tail;          /* the launch that selects and attends in one (tka_sparse_decode_step of a
+                                  caller that asks for the output alone, long segments): 0 = where it is the
+                                  quicker form (calls of 64 segments and more), 1 = wherever it fits, 2 = never */
 } tka_test_hooks;
 int tka_set_test_hooks(const tka_test_hooks* hooks);
 

@@ -245,9 +245,10 @@ def test_sparse_decode_rejects_values_without_indices():
 def test_test_hooks_validation():
     lib = L.lib()
     assert lib.tka_set_test_hooks(None) == L.TKA_OK
-    assert lib.tka_set_test_hooks(C.byref(L.TestHooks(1, 64, 2, 1, 1, 0))) == L.TKA_OK
+    assert lib.tka_set_test_hooks(C.byref(L.TestHooks(1, 64, 2, 1, 1, 0, 1))) == L.TKA_OK
     assert lib.tka_set_test_hooks(C.byref(L.TestHooks(0, -1, 0, 0, 0, 0))) == L.TKA_EINVAL
-    assert lib.tka_set_test_hooks(C.byref(L.TestHooks(0, 0, 0, 0, 2, 0))) == L.TKA_EINVAL
+    assert lib.tka_set_test_hooks(C.byref(L.TestHooks(0, 0, 0, 0, 2, 0, 0))) == L.TKA_EINVAL
+    assert lib.tka_set_test_hooks(C.byref(L.TestHooks(0, 0, 0, 0, 0, 0, 3))) == L.TKA_EINVAL
     assert lib.tka_set_test_hooks(None) == L.TKA_OK
 
 

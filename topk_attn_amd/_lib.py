@@ -81,7 +81,7 @@ class SparseDecodeArgs(C.Structure):
 
 class TestHooks(C.Structure):
     _fields_ = [("force_segment_redo", _i32), ("tau_spin_limit", _i32), ("tau_withhold_mod", _i32),
-                ("tau_withhold_rem", _i32), ("tau_withhold_mode", _i32), ("union_handoff_order", _i32)]
+                ("tau_withhold_rem", _i32), ("tau_withhold_mode", _i32), ("union_handoff_order", _i32), ("fused_tail", _i32)]
 
 
 RA_VARIANTS = ("", "_global", "_pipelined", "_pipelined_global", "_two_kernels", "_gather_baseline")

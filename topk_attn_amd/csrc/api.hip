@@ -87,7 +87,7 @@ namespace {
 
 // Testing hooks (tka_set_test_hooks): process-wide, read once per call.
 std::mutex g_hooks_mutex;
-tka_test_hooks g_hooks = {0, 0, 0, 0, 0, 0};
+tka_test_hooks g_hooks = {0, 0, 0, 0, 0, 0, 0};
 tka_test_hooks current_hooks() {
   std::lock_guard<std::mutex> lock(g_hooks_mutex);
   return g_hooks;
@@ -294,8 +294,13 @@ bool wave_route(const tka_gemv_topk_args* a, bool want_union) {
          (chunk_len > kFusedMaxSegLen || a->out_scores || segs >= wave_select_min_segments());
 }
 
+struct FusedTail;
+bool fused_tail_take(FusedTail* ft, const GemvParams& g, const SelectParams& s);
+
+// `ft`: the caller can run selection and attention of the candidate route in one launch (launch_attn_select_mfma);
+// when the call takes that route and the launch fits, only the GEMV is launched here and *ft is filled.
 int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, const int32_t* cluster_ids = nullptr,
-                  const UnionOut* u = nullptr, bool any_order = false, const InlineCentres* ic = nullptr) {
+                  const UnionOut* u = nullptr, bool any_order = false, const InlineCentres* ic = nullptr, FusedTail* ft = nullptr) {
   hipStream_t stream = (hipStream_t)a->stream;
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
@@ -477,6 +482,9 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   // testing hook: no candidate count is acceptable, every segment is redone from the keys
   sc.max_entries = hooks.force_segment_redo ? 0 : select_cand_capacity();
   sc.scores = scores;
+  if (ft && !sc.out_idx && sc.union_idx && a->num_chunks == 1 && !cluster_ids && attn_select_fits(sc.parts, a->group) &&
+      fused_tail_take(ft, gp, sc))
+    return TKA_OK;
   return launch_select_finalize_cand(gp, sc, a->dtype, stream);
 }
 
@@ -540,10 +548,8 @@ size_t flash_bytes(const tka_flash_decode_args* a) {
   return align_up(rows * splits * sizeof(float), 256) * 2 + align_up(rows * splits * TKA_HEAD_DIM * sizeof(float), 256);
 }
 
-int run_flash(const tka_flash_decode_args* a, void* workspace) {
-  hipStream_t stream = (hipStream_t)a->stream;
-  int splits, tps;
-  flash_plan(a, &splits, &tps);
+// Parameter block of the attention kernels for a call and its plan; the partials lie at the head of `workspace`.
+void fill_attn_params(const tka_flash_decode_args* a, void* workspace, int splits, int tps, AttnParams* out) {
   const size_t rows = (size_t)a->batch * a->num_kv_heads * a->group;
   unsigned char* ws = (unsigned char*)workspace;
   AttnParams ap;
@@ -571,6 +577,31 @@ int run_flash(const tka_flash_decode_args* a, void* workspace) {
   ap.idx_len = a->idx_len;
   ap.tokens_per_split = tps;
   ap.scale_log2e = a->scale * 1.44269504088896340736f;
+  *out = ap;
+}
+
+void fill_combine_params(const tka_flash_decode_args* a, const AttnParams& ap, CombineParams* out) {
+  CombineParams cp;
+  memset(&cp, 0, sizeof cp);
+  cp.part_m = ap.part_m;
+  cp.part_l = ap.part_l;
+  cp.part_acc = ap.part_acc;
+  cp.out = a->out;
+  cp.out_lse = a->out_lse;
+  cp.out_stride_b = a->out_stride_b;
+  cp.rows_per_batch = a->num_kv_heads * a->group;
+  cp.rows = a->batch * a->num_kv_heads * a->group;
+  cp.num_splits = ap.num_splits;
+  cp.out_dtype = a->out_dtype;
+  *out = cp;
+}
+
+int run_flash(const tka_flash_decode_args* a, void* workspace) {
+  hipStream_t stream = (hipStream_t)a->stream;
+  int splits, tps;
+  flash_plan(a, &splits, &tps);
+  AttnParams ap;
+  fill_attn_params(a, workspace, splits, tps, &ap);
   // grouped queries go to the matrix cores; one query head per KV head (and supplied logits) stay on VALU
   const bool mfma = a->group >= 2 && !a->kv_logit;
   if (!mfma && splits == 1) {   // nothing to combine: the kernel writes the result itself
@@ -583,18 +614,64 @@ int run_flash(const tka_flash_decode_args* a, void* workspace) {
   int rc = mfma ? launch_attn_partial_mfma(ap, a->dtype, stream) : launch_attn_partial(ap, a->dtype, stream);
   if (rc != TKA_OK) return rc;
   CombineParams cp;
-  memset(&cp, 0, sizeof cp);
-  cp.part_m = ap.part_m;
-  cp.part_l = ap.part_l;
-  cp.part_acc = ap.part_acc;
-  cp.out = a->out;
-  cp.out_lse = a->out_lse;
-  cp.out_stride_b = a->out_stride_b;
-  cp.rows_per_batch = a->num_kv_heads * a->group;
-  cp.rows = (int)rows;
-  cp.num_splits = splits;
-  cp.out_dtype = a->out_dtype;
+  fill_combine_params(a, ap, &cp);
   return launch_lse_combine(cp, stream);
+}
+
+// Filled by run_gemv_topk when it leaves the selection of the candidate route to the attention launch
+// (launch_attn_select_mfma): the stage-1 parameters that launch and the redo of flagged segments need.
+struct FusedTail {
+  bool taken;
+  GemvParams g;
+  SelectParams s;
+};
+
+bool fused_tail_take(FusedTail* ft, const GemvParams& g, const SelectParams& s) {
+  ft->taken = true;
+  ft->g = g;
+  ft->s = s;
+  return true;
+}
+
+// Selection + attention in one launch, then the combine launch that also redoes flagged segments.  f.kv_idx / f.kv_count:
+// the list and count arrays of the step's workspace (only a redone segment writes and reads them).
+int run_fused_tail(const tka_flash_decode_args* f, const FusedTail& ft, void* workspace) {
+  hipStream_t stream = (hipStream_t)f->stream;
+  // Every split of a segment finds the segment's threshold again, and a workgroup holds the candidates in LDS (two per
+  // CU): about 512 workgroups, not the thousand of the attention that reads its list from memory.  (The workspace is
+  // sized for that plan, which has at least as many splits.)
+  tka_flash_decode_args fa = *f;
+  int splits, tps;
+  flash_plan(&fa, &splits, &tps);
+  if (fa.num_splits <= 0) {
+    int64_t want = 512 / ((int64_t)fa.batch * fa.num_kv_heads);
+    if (want < 1) want = 1;
+    if (want < splits) {
+      fa.num_splits = (int)want;
+      flash_plan(&fa, &splits, &tps);
+    }
+  }
+  AttnParams ap;
+  fill_attn_params(f, workspace, splits, tps, &ap);
+  FusedSelectParams fs;
+  memset(&fs, 0, sizeof fs);
+  fs.cand_head = ft.s.cand_head;
+  fs.cand = ft.s.list;
+  fs.cand_seg_stride = ft.s.list_stride;
+  fs.tau_words = ft.s.tau_words;
+  fs.sample_flags = ft.s.sample_flags;
+  fs.seg_flags = ft.s.seg_flags;
+  fs.parts = ft.s.parts;
+  fs.part_len = ft.s.part_len;
+  fs.k = ft.s.k;
+  fs.sink = ft.s.sink;
+  fs.local = ft.s.local;
+  fs.max_entries = ft.s.max_entries;
+  int rc = launch_attn_select_mfma(ap, fs, f->dtype, stream);
+  if (rc != TKA_OK) return rc;
+  CombineParams cp;
+  fill_combine_params(f, ap, &cp);
+  return launch_lse_combine_redo(cp, ft.g, ft.s, ap, f->dtype, stream);
 }
 
 }  // namespace
@@ -677,11 +754,11 @@ int tka_gemv_topk_gave_up_slices(const tka_gemv_topk_args* a, int32_t* count) {
 
 int tka_set_test_hooks(const tka_test_hooks* hooks) {
   if (hooks && (hooks->tau_spin_limit < 0 || hooks->tau_withhold_mod < 0 || hooks->tau_withhold_rem < 0 ||
-                (hooks->tau_withhold_mode != 0 && hooks->tau_withhold_mode != 1)))
+                (hooks->tau_withhold_mode != 0 && hooks->tau_withhold_mode != 1) || hooks->fused_tail < 0 || hooks->fused_tail > 2))
     return TKA_EINVAL;
   std::lock_guard<std::mutex> lock(g_hooks_mutex);
   if (hooks) g_hooks = *hooks;
-  else g_hooks = tka_test_hooks{0, 0, 0, 0, 0, 0};
+  else g_hooks = tka_test_hooks{0, 0, 0, 0, 0, 0, 0};
   return TKA_OK;
 }
 
@@ -1210,10 +1287,21 @@ int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
   g.workspace = ws;
   g.workspace_bytes = gemv_ws;
   UnionOut uo = {uidx, ucnt, a->sink, a->local, sd_union_handoff(a) || behind};
-  rc = run_gemv_topk(&g, nullptr, 0, nullptr, &uo);
+  // A caller that asks for neither list (the output alone): on long segments the attention launch selects the tokens
+  // itself from the candidates of the GEMV launch, and the ids never leave the chip.  Every split of a segment finds the
+  // segment's threshold again, which costs what the launch saves until the call has many segments (us per step, one
+  // launch / two, 131072 tokens, k = 2048: 8 segments 66.4 / 64.1, 32 segments 188.1 / 186.2, 64 segments 344.2 / 344.7,
+  // 128 segments of 65536 tokens 366.5 / 372.9), so it is taken from 64 segments on.
+  FusedTail ft;
+  ft.taken = false;
+  const tka_test_hooks hooks = current_hooks();
+  const bool output_only = !a->out_topk_idx && !a->out_union_idx && hooks.union_handoff_order == 0 && a->group >= 2 &&
+                           (hooks.fused_tail == 1 || (hooks.fused_tail == 0 && segs >= 64));
+  rc = run_gemv_topk(&g, nullptr, 0, nullptr, &uo, false, nullptr, output_only ? &ft : nullptr);
   if (rc != TKA_OK) return rc;
   f.kv_idx = uidx;
   f.kv_count = ucnt;
+  if (ft.taken) return run_fused_tail(&f, ft, ws + gemv_ws);
   rc = run_flash(&f, ws + gemv_ws);
   if (rc != TKA_OK || !behind) return rc;
   UnionParams up;

@@ -646,8 +646,11 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
     uint64_t* slice = p.cand + seg * p.cand_seg_stride + (int64_t)wg_in_chunk * kCandThreads;
     uint64_t* head = p.cand_head + (seg * p.wgs_per_chunk + wg_in_chunk) * kCandHead;
     if (pass) {
+      // (stored through to memory: a plain store leaves a dirty line in this XCD's L2 to be written back when the kernel
+      // ends, and the launch measured 1.6 us longer with it, 317.3 against 315.7 us for 2 GiB of keys)
       const uint32_t pos = before + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-      (pos < (uint32_t)kCandHead ? head : slice)[pos] = ((uint64_t)key << 32) | (pos == 0 ? total << 9 : 0u) | (uint32_t)tid;
+      __hip_atomic_store((pos < (uint32_t)kCandHead ? head : slice) + pos, ((uint64_t)key << 32) | (pos == 0 ? total << 9 : 0u) | (uint32_t)tid,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (tid == 0 && total == 0) head[0] = tau_ready ? 0ull : (uint64_t)(kSliceGaveUp << 9);
     if (tid == 0 && !tau_ready) __hip_atomic_store(p.seg_flags + seg, p.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

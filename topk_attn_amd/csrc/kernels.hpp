@@ -111,6 +111,8 @@ size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p
 size_t select_epoch_words(void* ws, int num_segments, int64_t seg_len, uint32_t** words);
 void select_plan(int64_t seg_len, int num_segments, SelectParams* p);
 int launch_zero_u32(uint32_t* ptr, size_t count, hipStream_t stream);
+// Raises a kernel's dynamic-LDS limit once per (kernel, device); safe to call from several host threads.
+int allow_dynamic_lds(const void* kernel, int bytes);
 int launch_select_hist(const SelectParams& p, hipStream_t stream);
 int launch_select(const SelectParams& p, hipStream_t stream);   // filter + finalize
 int launch_select_filter(const SelectParams& p, hipStream_t stream);
@@ -171,6 +173,25 @@ struct AttnParams {
 int launch_attn_partial(const AttnParams& p, int dtype, hipStream_t stream);       // VALU path (any group, logits)
 int launch_attn_partial_mfma(const AttnParams& p, int dtype, hipStream_t stream);  // matrix-core path, group >= 2
 
+// Selection and attention of the candidate route in one launch (attention_select.hip): every attention workgroup
+// derives its segment's k-th largest composite from the candidate slices of the GEMV launch and keeps its split's
+// share of the token list in LDS.  A segment whose candidates cannot be used gets empty partials and bit 0 of its
+// seg_flags word; launch_lse_combine_redo then redoes it from the keys.
+struct FusedSelectParams {
+  const uint64_t* cand_head;  // [segments][parts][kCandHead], see GemvParams
+  const uint64_t* cand;       // [segments][cand_seg_stride]
+  int64_t cand_seg_stride;
+  uint64_t* tau_words;        // [segments][2]  cleared by split 0 of every segment, like the selection kernel does
+  uint32_t* sample_flags;     // [segments][64]
+  uint32_t* seg_flags;        // [segments] bit 0: to be redone from the keys; bits 8..: slices that gave up
+  int parts, part_len;        // slices per segment, tokens per slice
+  int k, sink, local;
+  int max_entries;            // a segment with more candidates is redone (0: every segment, the testing hook)
+  int lds_entries;            // candidates of a segment that a workgroup keeps in LDS (set by the launcher)
+};
+bool attn_select_fits(int parts, int group);
+int launch_attn_select_mfma(const AttnParams& p, const FusedSelectParams& f, int dtype, hipStream_t stream);
+
 struct CombineParams {
   const float* part_m;
   const float* part_l;
@@ -182,5 +203,11 @@ struct CombineParams {
   int rows, num_splits, out_dtype;
 };
 int launch_lse_combine(const CombineParams& p, hipStream_t stream);
+// The combine launch behind launch_attn_select_mfma: rows of unflagged segments are combined as usual; behind them in
+// the grid one workgroup per segment looks at the segment's flag and, when it is set, redoes the segment from the keys
+// (selection by fallback_segment into s.union_idx / s.union_count, attention over that list, output written directly).
+// g, s: the stage-1 parameters of the step (s.out_idx must be null: no rank order); a: q, values, strides, scale.
+int launch_lse_combine_redo(const CombineParams& c, const GemvParams& g, const SelectParams& s, const AttnParams& a, int dtype,
+                            hipStream_t stream);
 
 }  // namespace tka

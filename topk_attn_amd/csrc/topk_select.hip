@@ -34,6 +34,7 @@
 
 #include "kernels.hpp"
 #include "bitonic.hpp"
+#include "lse_combine.hpp"
 
 namespace tka {
 
@@ -963,6 +964,111 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   write_rank_outputs(sh_sort, p, seg);
 }
 
+// ---- combine launch of the fused selection + attention, with the redo of flagged segments ----------------
+
+// Attention of one workgroup of 1024 threads over a token list in memory, all G query heads of one KV head, result
+// written directly (the only "split" of its rows).  The slow path of a slow path: one head after the other, a 16-lane
+// row group per token, four rows in flight.  sh_acc: 64 x 128 floats, sh_ml: 128 floats.
+template <int DT>
+__device__ __forceinline__ void redo_attention(const AttnParams& a, const int32_t* list, int count, int b, int h, void* out,
+                                               int64_t out_stride_b, int out_dtype, float* sh_acc, float* sh_ml) {
+  constexpr int kRowGroups = kSelThreads / 16, U = 4;
+  const int tid = threadIdx.x, j = tid & 15, rg = tid >> 4;
+  const int64_t head_off = (int64_t)b * a.kv_stride_b + (int64_t)h * a.kv_stride_h + 8 * j;
+  const uint16_t* kbase = (const uint16_t*)a.keys + head_off;
+  const uint16_t* vbase = (const uint16_t*)a.values + head_off;
+  for (int g = 0; g < a.group; ++g) {
+    float qf[8];
+    {
+      const u32x4 v = *(const u32x4*)((const uint16_t*)a.q + (int64_t)b * a.q_stride_b + ((int64_t)h * a.group + g) * kHeadDim + 8 * j);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[i] = Elem<DT>::get(v, i);
+    }
+    float m = -INFINITY, l = 0.0f, acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int base = 0; base < count; base += kRowGroups * U) {
+      u32x4 kv[U], vv[U];
+      bool ok[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int pos = base + rg * U + u;
+        int64_t t = pos < count ? (int64_t)list[pos] : -1;
+        ok[u] = t >= 0 && t < a.seq_len;
+        if (!ok[u]) t = 0;
+        kv[u] = *(const u32x4*)(kbase + t * a.kv_stride_n);
+        vv[u] = *(const u32x4*)(vbase + t * a.kv_stride_n);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s = __builtin_fmaf(qf[i], Elem<DT>::get(kv[u], i), s);
+        s = row16_sum(s) * a.scale_log2e;
+        if (!ok[u]) continue;   // (uniform over the row group; a skipped row is never multiplied)
+        const float mx = fmaxf(m, s);
+        const float alpha = __builtin_amdgcn_exp2f(m - mx), pu = __builtin_amdgcn_exp2f(s - mx);
+        m = mx;
+        l = l * alpha + pu;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pu, Elem<DT>::get(vv[u], i), acc[i] * alpha);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sh_acc[rg * kHeadDim + 8 * j + i] = acc[i];
+    if (j == 0) { sh_ml[rg] = m; sh_ml[kRowGroups + rg] = l; }
+    __syncthreads();
+    if (tid < kHeadDim) {
+      float M = -INFINITY;
+      for (int r = 0; r < kRowGroups; ++r) M = fmaxf(M, sh_ml[r]);
+      float L = 0.0f, o = 0.0f;
+      if (M != -INFINITY) {
+        for (int r = 0; r < kRowGroups; ++r) {
+          const float w = __builtin_amdgcn_exp2f(sh_ml[r] - M);
+          L += sh_ml[kRowGroups + r] * w;
+          o += sh_acc[r * kHeadDim + tid] * w;
+        }
+      }
+      const float res = L > 0.0f ? o / L : 0.0f;
+      uint16_t* dst = (uint16_t*)out + (int64_t)b * out_stride_b + ((int64_t)h * a.group + g) * kHeadDim;
+      dst[tid] = out_dtype == TKA_F16 ? Elem<TKA_F16>::narrow(res) : Elem<TKA_BF16>::narrow(res);
+    }
+  }
+}
+
+// Grid: c.rows combine workgroups, then one redo workgroup per segment (they come last so that the combine rows are
+// not held up by workgroups that in all likelihood look at one word and leave).
+template <int DT, int ODT>
+__global__ __launch_bounds__(kSelThreads) void lse_combine_redo_kernel(CombineParams c, GemvParams g, SelectParams p, AttnParams a) {
+  static_assert(kCombineThreads == kSelThreads, "one workgroup shape for both roles");
+  struct RedoLds {
+    uint32_t hist[kHistBins], off[kHistBins], wtot[kSelWaves], res[4];
+    uint64_t mm[3];
+    float acc[(kSelThreads / 16) * kHeadDim], ml[2 * (kSelThreads / 16)];
+  };
+  union Lds {
+    CombineLds combine;
+    RedoLds redo;
+  };
+  __shared__ __attribute__((aligned(16))) unsigned char raw[sizeof(Lds)];
+  if ((int)blockIdx.x < c.rows) {
+    const int row = (int)blockIdx.x;
+    if (p.seg_flags[row / a.group] & 1u) return;   // its segment is redone: the redo workgroup writes the row
+    lse_combine_row<ODT>(c, row, *(CombineLds*)raw);
+    return;
+  }
+  const int seg = (int)blockIdx.x - c.rows;
+  if (!(p.seg_flags[seg] & 1u)) return;
+  RedoLds& sh = *(RedoLds*)raw;
+  fallback_segment<DT>(g, p, seg, 0, nullptr, sh.hist, sh.off, sh.wtot, sh.res, sh.mm);
+  __threadfence_block();
+  __syncthreads();   // the list and its count, written by this workgroup, are read by it below
+  const int count = p.union_count[seg];
+  redo_attention<DT>(a, p.union_idx + (int64_t)seg * (p.k + p.sink + p.local), count, seg / g.num_kv_heads, seg % g.num_kv_heads,
+                     c.out, c.out_stride_b, c.out_dtype, sh.acc, sh.ml);
+}
+
 // ---- ranking of the common-cut route ---------------------------------------------------------------
 
 // One lane's add to a 64-bit word in LDS, returning the word's old value.  (Written out: around an atomic that one lane of
@@ -1715,7 +1821,7 @@ int launch_select_hist(const SelectParams& p, hipStream_t stream) {
 }
 
 // Raises a kernel's dynamic-LDS limit once per (kernel, device); safe to call from several host threads.
-static int allow_dynamic_lds(const void* kernel, int bytes) {
+int allow_dynamic_lds(const void* kernel, int bytes) {
   static std::mutex guard;
   static std::vector<std::pair<const void*, int>> done;
   int device = 0;
@@ -1800,6 +1906,24 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
   if (p.segs_per_row < 1 || p.num_segments % p.segs_per_row || p.num_segments > (1 << 24)) return TKA_EINVAL;
   const dim3 wgs((unsigned)((p.num_segments + 7) / 8 * 8 * kCutParts));   // (see the kernel)
   hipLaunchKernelGGL(kernel, wgs, dim3(kSelThreads), lds, stream, g, p, kpad_for(p.k));
+  return hip_status(hipGetLastError());
+}
+
+int launch_lse_combine_redo(const CombineParams& c, const GemvParams& g, const SelectParams& s, const AttnParams& a, int dtype,
+                            hipStream_t stream) {
+  if (s.out_idx || !s.union_idx || !s.union_count || !s.seg_flags || g.num_chunks != 1 || c.rows != s.num_segments * a.group)
+    return TKA_EINVAL;
+  LaunchTimer timer("lse_combine_redo", stream);
+  const unsigned grid = (unsigned)(c.rows + s.num_segments);
+#define TKA_LAUNCH_COMBINE_REDO(DT, ODT) lse_combine_redo_kernel<DT, ODT><<<grid, kSelThreads, 0, stream>>>(c, g, s, a)
+  if (dtype == TKA_F16) {
+    if (c.out_dtype == TKA_F16) TKA_LAUNCH_COMBINE_REDO(TKA_F16, TKA_F16);
+    else TKA_LAUNCH_COMBINE_REDO(TKA_F16, TKA_BF16);
+  } else {
+    if (c.out_dtype == TKA_F16) TKA_LAUNCH_COMBINE_REDO(TKA_BF16, TKA_F16);
+    else TKA_LAUNCH_COMBINE_REDO(TKA_BF16, TKA_BF16);
+  }
+#undef TKA_LAUNCH_COMBINE_REDO
   return hip_status(hipGetLastError());
 }
 

@@ -384,9 +384,10 @@ def sparse_decode_step(q, keys, values, k, sink, local, scale, group, out_dtype=
 
 
 def set_test_hooks(force_segment_redo=0, tau_spin_limit=0, tau_withhold_mod=0, tau_withhold_rem=0, tau_withhold_mode=0,
-                   union_handoff_order=0):
+                   union_handoff_order=0, fused_tail=0):
     """Testing hooks (see tka_test_hooks in include/topk_attn.h); no arguments = defaults."""
-    h = L.TestHooks(force_segment_redo, tau_spin_limit, tau_withhold_mod, tau_withhold_rem, tau_withhold_mode, union_handoff_order)
+    h = L.TestHooks(force_segment_redo, tau_spin_limit, tau_withhold_mod, tau_withhold_rem, tau_withhold_mode, union_handoff_order,
+                    fused_tail)
     L.check(L.lib().tka_set_test_hooks(C.byref(h)), "tka_set_test_hooks")
 
 
