@@ -75,7 +75,7 @@ class SparseDecode:
 
     def __init__(self, torch, ops, dev, batch=8, hkv=8, group=4, seq_len=131072, k=2048, sink=64, local=512,
                  dtype="float16", out_dtype="bfloat16", heavy=0.01, seed=4, name="c4", num_splits=0, levels=False,
-                 want_union=True):
+                 want_union=True, shared=False):
         self.torch, self.name = torch, name
         g = torch.Generator(device=dev)
         g.manual_seed(seed)
@@ -83,16 +83,20 @@ class SparseDecode:
         B, H, G, N = batch, hkv, group, seq_len
         self.B, self.H, self.G, self.N, self.k, self.sink, self.local = B, H, G, N, k, sink, local
         self.q = randn16(torch, (B, H * G, 128), dt, g, dev, chunk_dim0=False)
+        self.shared = shared
+        KB = 1 if shared else B       # shared: one cache [N, H, 128] for all batch entries (kv_stride_b = 0)
         if levels:  # 16 uniform levels in [-2, 2]: many exact score ties
-            self.K = levels16(torch, (B, N, H, 128), dt, g, dev)
+            self.K = levels16(torch, (KB, N, H, 128), dt, g, dev)
         else:
-            self.K = randn16(torch, (B, N, H, 128), dt, g, dev)
-        self.V = randn16(torch, (B, N, H, 128), dt, g, dev)
+            self.K = randn16(torch, (KB, N, H, 128), dt, g, dev)
+        self.V = randn16(torch, (KB, N, H, 128), dt, g, dev)
         n_heavy = int(N * heavy)
-        for b in range(B):
+        for b in range(KB):
             for h in range(H):
                 hh = torch.randperm(N, generator=g, device=dev)[:n_heavy]
                 self.K[b, hh, h] = (self.K[b, hh, h].float() * 4.0).to(dt)
+        if shared:
+            self.K, self.V = self.K[0], self.V[0]
         # production configuration: the attention consumes the union list; the optional rank-ordered top-k
         # output (a sort per KV head) is not requested
         self.plan = ops.SparseDecodePlan(self.q, self.K, self.V, k, sink, local, SCALE, G,
@@ -117,7 +121,7 @@ class SparseDecode:
 
     def bytes(self):
         sel = self.selected if self.selected is not None else int(self.plan.union_count.sum().item())
-        gemv = self.B * self.N * self.H * 128 * 2
+        gemv = (1 if self.shared else self.B) * self.N * self.H * 128 * 2   # a shared cache is streamed once for the batch
         sparse = sel * 128 * 2 * 2 + sel * 4 * 2          # gathered K and V rows, index lists written + read
         qo = self.B * self.H * self.G * 128 * 4           # q read, out written (2 bytes each)
         return gemv + sparse + qo, gemv, {"selected_tokens": sel}
@@ -126,7 +130,7 @@ class SparseDecode:
         torch = self.torch
         from oracle.cpu_baseline import sparse_decode_cpu
         # bounded sample: batch entry 0 (1/B of the step); the step is B independent copies of it
-        qc, Kc, Vc = self.q[0].cpu(), self.K[0].cpu(), self.V[0].cpu()
+        qc, Kc, Vc = self.q[0].cpu(), (self.K if self.shared else self.K[0]).cpu(), (self.V if self.shared else self.V[0]).cpu()
         times = []
         for r in range(runs + 2):   # two warm-ups, then the timed runs
             c0 = time.perf_counter()
@@ -292,6 +296,8 @@ def build_workload(name, torch, ops, dev, args):
         return PlainCopy(torch, dev)
     if name == "c4":
         return SparseDecode(torch, ops, dev, num_splits=args.splits)
+    if name == "c4-shared":     # the same shapes over ONE cache that the batch shares (a common prefix: kv_stride_b = 0)
+        return SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-shared", shared=True)
     if name == "c4-out":        # the same step for a caller that wants the output alone
         return SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-out", want_union=False)
     if name == "c4-small":
@@ -360,7 +366,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c1-8x16k", "c2", "c2-ref", "c3", "c4", "c4-out", "c4-small", "c4-b1-32k", "c4-b1-16k", "c4-share32k", "c5", "c5-out", "c5-topk", "ra", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c1-8x16k", "c2", "c2-ref", "c3", "c4", "c4-out", "c4-shared", "c4-small", "c4-b1-32k", "c4-b1-16k", "c4-share32k", "c5", "c5-out", "c5-topk", "ra", "copy"])
     ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--score-mode", type=int, default=0, choices=[0, 1],
@@ -426,6 +432,8 @@ def main():
     ops.profile_enable(False)
     kern = {name: ms / max(n, 1) * 1e3 for name, (ms, n) in prof.items()}  # us per launch
     dominant = w.dominant
+    if dominant == "gemv_scores" and "gemv_candidates_shared" in kern:
+        dominant = "gemv_candidates_shared"             # ... over keys that the batch shares
     if dominant == "gemv_scores" and "gemv_candidates" in kern:
         dominant = "gemv_candidates"                    # long segments run the candidate-mode GEMV
     if dominant == "gemv_scores" and "gemv_cut" in kern:

@@ -387,6 +387,31 @@ def test_sparse_decode_step_union_only(dtype, B, H, G, N, k, sink, local, kind, 
             assert (np.abs(out[b, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
 
 
+def test_sparse_decode_step_shared_cache_long():
+    """The step over ONE cache that the batch shares (kv_stride_b = 0) at a length of the candidate route: the keys are
+    scored for a tile of batch entries per pass; top-k, union list and output of every (entry, head) against the oracle."""
+    from topk_attn_amd import ops
+    announce("sparse_decode_step, cache shared by a batch of 5, N=70000 k=1024 G=4")
+    rng = np.random.default_rng(4242)
+    dtype, B, H, G, N, k, sink, local = oracle.F16, 5, 2, 4, 70000, 1024, 16, 128
+    q, K, V = randn_bits(rng, (B, H * G, 128), dtype), randn_bits(rng, (N, H, 128), dtype), randn_bits(rng, (N, H, 128), dtype)
+    ops.profile_reset()
+    ops.profile_enable(True)
+    out, tidx, tval, uidx, ucnt = ops.sparse_decode_step(to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype), k, sink, local,
+                                                         SCALE, G, out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    ran = ops.profile_read()
+    ops.profile_enable(False)
+    assert "gemv_candidates_shared" in ran, sorted(ran)
+    out, tidx, tval, uidx, ucnt = f32_of(out), tidx.cpu().numpy(), tval.cpu().numpy(), uidx.cpu().numpy(), ucnt.cpu().numpy()
+    for b in range(B):
+        for h in range(H):
+            ro, ri, rv, ru = oracle.sparse_decode_step(q[b, h * G:(h + 1) * G], K[:, h], V[:, h], dtype, G, k, sink, local, SCALE)
+            assert np.array_equal(tidx[b, h], ri) and np.array_equal(tval[b, h].view(np.uint32), rv.view(np.uint32))
+            assert ucnt[b, h] == len(ru) and np.array_equal(uidx[b, h, :len(ru)], ru), "union differs (b=%d h=%d)" % (b, h)
+            assert (np.abs(out[b, h * G:(h + 1) * G] - ro) < out_tol(ro, False)).all()
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3, 4])
 def test_short_token_list_bf16_weights(seed):
     """A step that attends to 17 tokens only (top 1 + a window of 16), bf16 inputs, grouped queries on the matrix cores,

@@ -335,6 +335,66 @@ def test_long_segment_chunked_shared_kv():
                 assert np.array_equal(val[b, h, c * k:(c + 1) * k].view(np.uint32), ev.view(np.uint32))
 
 
+@pytest.mark.parametrize("dtype,B,H,G,N,k,kind", [
+    (oracle.F16, 8, 2, 1, 131072, 2048, "heavy"),      # one tile of eight entries
+    (oracle.BF16, 3, 2, 4, 70001, 1000, "levels"),     # a tile of four with one entry missing, grouped queries, ties, ragged slice
+    (oracle.F16, 2, 1, 8, 100000, 2048, "normal"),     # a tile of two
+    (oracle.F16, 9, 1, 2, 66000, 1024, "equal"),       # two tiles of eight, the second with one entry; every score of an entry ties
+    (oracle.BF16, 6, 3, 1, 65536, 512, "normal")])     # 18 segments of 65536 tokens: more than a million rows
+def test_long_segment_shared_keys(dtype, B, H, G, N, k, kind):
+    """Long segments over a key cache that the batch shares (key_stride_b = 0): one pass over the keys scores a tile of
+    batch entries, thresholds and candidate slices are per (entry, head).  Indices and values bit for bit, no segment
+    redone, and the kernel that ran."""
+    from topk_attn_amd import ops
+    announce("gemv_topk long segments, keys shared by the batch: dtype=%d B=%d H=%d G=%d N=%d k=%d %s" % (dtype, B, H, G, N, k, kind))
+    rng = np.random.default_rng(B * 1000 + N % 997)
+    if kind == "levels":
+        K = oracle.to_bits(np.linspace(-2, 2, 16)[rng.integers(0, 16, (N, H, 128))], dtype)
+    elif kind == "equal":
+        K = np.broadcast_to(randn_bits(rng, (1, 1, 128), dtype), (N, H, 128)).copy()
+    else:
+        Kf = rng.standard_normal((N, H, 128))
+        if kind == "heavy":
+            Kf[rng.permutation(N)[:N // 100]] *= 4.0
+        K = oracle.to_bits(Kf, dtype)
+    q = randn_bits(rng, (B, H * G, 128), dtype)
+    plan = ops.GemvTopkPlan(to_dev(q, dtype), to_dev(K, dtype), k, group=G, scale=SCALE)
+    ops.profile_reset()
+    ops.profile_enable(True)
+    plan.run()
+    torch.cuda.synchronize()
+    ran = ops.profile_read()
+    ops.profile_enable(False)
+    assert "gemv_candidates_shared" in ran, sorted(ran)
+    assert plan.redone_segments() == 0 and plan.gave_up_slices() == 0
+    idx, val = plan.idx.cpu().numpy(), plan.val.cpu().numpy()
+    for b in range(B):
+        for h in range(H):
+            ref = oracle.scores_canonical(K[:, h, :], dtype, oracle.group_query(q[b, h * G:(h + 1) * G], dtype, G), SCALE)
+            ei, ev = oracle.topk_stable(ref, k)
+            assert np.array_equal(idx[b, h], ei), "indices differ (b=%d h=%d)" % (b, h)
+            assert np.array_equal(val[b, h].view(np.uint32), ev.view(np.uint32))
+
+
+def test_long_segment_shared_keys_threshold_withheld(hooks):
+    """The same with the thresholds of every third segment withheld: their slices are marked as given up by the
+    workgroups that score them for the whole tile, those segments are redone from the keys, the others are not."""
+    from topk_attn_amd import ops
+    announce("gemv_topk long segments, shared keys, thresholds of segments 1, 4, 7 withheld")
+    hooks(tau_spin_limit=64, tau_withhold_mod=3, tau_withhold_rem=1, tau_withhold_mode=0)
+    rng = np.random.default_rng(91)
+    dtype, B, H, N, k = oracle.F16, 4, 2, 70000, 1024
+    K, q = randn_bits(rng, (N, H, 128), dtype), randn_bits(rng, (B, H, 128), dtype)
+    plan = ops.GemvTopkPlan(to_dev(q, dtype), to_dev(K, dtype), k, group=1, scale=SCALE).run()
+    torch.cuda.synchronize()
+    assert plan.redone_segments() == 3
+    idx = plan.idx.cpu().numpy()
+    for b in range(B):
+        for h in range(H):
+            ref = oracle.scores_canonical(K[:, h, :], dtype, oracle.group_query(q[b, h:h + 1], dtype, 1), SCALE)
+            assert np.array_equal(idx[b, h], oracle.topk_stable(ref, k)[0]), "indices differ (b=%d h=%d)" % (b, h)
+
+
 def test_long_segment_ragged_length():
     """Segment length that is no multiple of the 256-token slice (nor of 4): the last slice is partial."""
     announce("gemv_topk long segment N=100003 k=1500 bf16 G=2")

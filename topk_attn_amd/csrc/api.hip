@@ -472,7 +472,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   cp.cand = sp.list;
   cp.cand_seg_stride = sp.list_stride;
   cp.cand_head = const_cast<uint64_t*>(sp.cand_head);
-  int rc = launch_gemv_candidates(cp, a->dtype, stream);
+  // (keys shared by the batch: one pass over them scores a tile of batch entries)
+  int rc = shared_keys && a->num_chunks == 1 ? launch_gemv_candidates_shared(cp, a->dtype, stream) : launch_gemv_candidates(cp, a->dtype, stream);
   if (rc != TKA_OK) return rc;
   SelectParams sc = sp;
   sc.hist = nullptr;

@@ -54,6 +54,8 @@ int launch_gemv_scores_shared(const GemvParams& p, int dtype, hipStream_t stream
 // The same on the matrix cores (one query head per KV head): scores to a few units in the last place of the canonical ones.
 int launch_gemv_scores_mfma(const GemvParams& p, int dtype, hipStream_t stream);
 int launch_gemv_candidates(const GemvParams& p, int dtype, hipStream_t stream);   // thresholds + candidate slices
+// The same over keys shared by the batch (key_stride_b == 0, batch >= 2): one pass over the keys scores a tile of batch entries.
+int launch_gemv_candidates_shared(const GemvParams& p, int dtype, hipStream_t stream);
 void gemv_candidate_plan(int64_t chunk_len, int64_t total_rows, int k, int max_candidates, int* num_samples, int* sample_rank);
 int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);
 // Common-cut route: every workgroup derives the segment's cut from the same sample rows and stores its slice's candidates
