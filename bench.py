@@ -291,7 +291,43 @@ class PlainCopy:
         return 2 * self.nbytes, 2 * self.nbytes, {}
 
 
+class ReadProbes:
+    """probe-stream / probe-gather: kernels that only read, in the access patterns of the two kernels that carry the
+    bytes of the c4 step (the long-segment GEMV: rows of 256 B of one head per workgroup; the gathered attention: the K
+    and V rows of 2624 tokens per (batch entry, KV head) at random places)."""
+
+    def __init__(self, torch, ops, dev, kind, threads, rounds):
+        g = torch.Generator(device=dev)
+        g.manual_seed(8)
+        B, N, H = 8, 131072, 8
+        self.K = torch.ones((B, N, H, 128), dtype=torch.float16, device=dev)
+        if kind == "gather":
+            self.V = torch.ones((B, N, H, 128), dtype=torch.float16, device=dev)
+            L = 2624
+            idx = torch.stack([torch.randperm(N, generator=g, device=dev)[:L] for _ in range(B * H)]).view(B, H, L)
+            idx = idx.sort(dim=-1).values.to(torch.int32).contiguous()       # ascending, like the union list
+            self.probe = ops.ReadProbe(self.K, self.V, idx, tokens_per_wg=256)
+            self.nbytes = B * H * L * 512
+            self.desc = "probe-gather: K and V rows of %d tokens per (batch entry, KV head), B=%d Hkv=%d N=%d" % (L, B, H, N)
+            self.dominant = "probe_gather"
+        else:
+            self.probe = ops.ReadProbe(self.K, threads=threads, rounds=rounds)
+            self.nbytes = B * N * H * 256
+            self.desc = "probe-stream: B=%d N=%d Hkv=%d, %d threads x %d rounds of 8 loads per lane" % (B, N, H, threads, rounds)
+            self.dominant = "probe_stream"
+
+    def step(self):
+        self.probe.run()
+
+    def bytes(self):
+        return self.nbytes, self.nbytes, {}
+
+
 def build_workload(name, torch, ops, dev, args):
+    if name == "probe-stream":
+        return ReadProbes(torch, ops, dev, "stream", args.probe_threads, args.probe_rounds)
+    if name == "probe-gather":
+        return ReadProbes(torch, ops, dev, "gather", 0, 0)
     if name == "copy":
         return PlainCopy(torch, dev)
     if name == "c4":
@@ -300,6 +336,9 @@ def build_workload(name, torch, ops, dev, args):
         return SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-shared", shared=True)
     if name == "c4-out":        # the same step for a caller that wants the output alone
         return SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-out", want_union=False)
+    if name == "c4-one-launch":  # ... with selection and attention in one launch (the library takes that form from 256 segments on)
+        ops.set_test_hooks(fused_tail=1)
+        return SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-one-launch", want_union=False)
     if name == "c4-small":
         return SparseDecode(torch, ops, dev, batch=2, seq_len=16384, name="c4-small")
     if name == "c4-b1-32k":     # one sequence of 32768 tokens on one GPU (all 8 KV heads), output only
@@ -366,7 +405,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c1-8x16k", "c2", "c2-ref", "c3", "c4", "c4-out", "c4-shared", "c4-small", "c4-b1-32k", "c4-b1-16k", "c4-share32k", "c5", "c5-out", "c5-topk", "ra", "copy"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c1-8x16k", "c2", "c2-ref", "c3", "c4", "c4-out", "c4-one-launch", "c4-shared", "c4-small", "c4-b1-32k", "c4-b1-16k", "c4-share32k", "c5", "c5-out", "c5-topk", "ra", "copy",
+                                                       "probe-stream", "probe-gather"])
     ap.add_argument("--batch", type=int, default=4, help="ra: batch entries")
     ap.add_argument("--topk", type=int, default=128, choices=[32, 128, 256, 512, 1024], help="ra: K per chunk")
     ap.add_argument("--score-mode", type=int, default=0, choices=[0, 1],
@@ -374,6 +414,8 @@ def main():
     ap.add_argument("--splits", type=int, default=0, help="c3, c4: split count of the attention (0 = library default)")
     ap.add_argument("--rotate", type=int, default=0,
                     help="c1, c2, c2-ref, ra: number of key sets taken in turn (working set beyond the Infinity Cache)")
+    ap.add_argument("--probe-threads", type=int, default=512, choices=[256, 512], help="probe-stream: threads per workgroup")
+    ap.add_argument("--probe-rounds", type=int, default=2, help="probe-stream: rounds of eight loads per lane (512 x 2 = the GEMV's shape)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-runs", type=int, default=5)
     args = ap.parse_args()

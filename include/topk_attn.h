@@ -13,6 +13,8 @@
  *   - Return value is a tka_status; nothing here prints or exits.  Argument validation happens before
  *     the first HIP call, so a bad call returns TKA_EINVAL / TKA_EUNSUPPORTED on a machine with no GPU.
  *   - Tensor element types are IEEE binary16 (TKA_F16) or bfloat16 (TKA_BF16); head_dim must be 128.
+ *   - Fields named reserved* must be zero (a later version may give them a meaning, as version 2.0.0 did with
+ *     score_mode); zero the argument block before filling it in.
  *   - Strides are in ELEMENTS.  Offsets are 64-bit everywhere (the reference's int32 offsets overflow
  *     beyond 524288 tokens at 32 heads, retrieval_attn/retrieval_attention.cu:323).
  *
@@ -65,7 +67,9 @@ typedef enum tka_softmax_mode {
  *   scores come from the matrix cores (v_mfma_f32_16x16x32, fp32 accumulation in the unit's own order): within a
  *   few units in the last place of the canonical ones (1e-5 of the exact dot product), not bit-identical to them.
  *   The selection is exact on the scores the call computed: out_idx / out_val are the first k of a stable
- *   descending sort of what out_scores would hold.  Calls it does not apply to run as TKA_SCORE_CANONICAL.
+ *   descending sort of what out_scores would hold.  A call it does not apply to (grouped queries, keys not shared, a
+ *   batch of one, a top-k over chunks of more than 16384 keys) returns TKA_EUNSUPPORTED: the scoring order that ran
+ *   is always the one that was asked for.
  *   (The batch pipeline of retrieval_attention.cu:654-896 as a skinny GEMM; about 4x quicker at batch 32.) */
 typedef enum tka_score_mode { TKA_SCORE_CANONICAL = 0, TKA_SCORE_MATRIX = 1 } tka_score_mode;
 
@@ -145,7 +149,7 @@ typedef struct tka_test_hooks {
                                   route, which may list -1 (an id the attention skips) inside the count  */
   int32_t fused_tail;          /* the launch that selects and attends in one (tka_sparse_decode_step of a
                                   caller that asks for the output alone, long segments): 0 = where it is the
-                                  quicker form (calls of 64 segments and more), 1 = wherever it fits, 2 = never */
+                                  form that is as quick (calls of 256 segments and more), 1 = wherever it fits, 2 = never */
 } tka_test_hooks;
 int tka_set_test_hooks(const tka_test_hooks* hooks);
 
@@ -376,7 +380,7 @@ typedef struct tka_sparse_decode_args {
   float* out_topk_val;    /* device, same shape; may be NULL; needs out_topk_idx              */
   int32_t* out_union_idx; /* device [batch][num_kv_heads][k+sink+local], ascending, -1 behind the count; may be NULL
                              (the step then hands the tokens to the attention in whatever form its route selects them) */
-  int32_t* out_union_count;/* device [batch][num_kv_heads]; may be NULL                       */
+  int32_t* out_union_count;/* device [batch][num_kv_heads]; may be NULL; needs out_union_idx (TKA_EINVAL otherwise) */
   void* workspace;
   size_t workspace_bytes;
   void* stream;
@@ -393,12 +397,46 @@ int tka_sparse_decode_step(const tka_sparse_decode_args* args);
  * larger returns TKA_ESCRATCH before anything is launched (batch 8 x 8 KV heads x 131072 tokens, k = 2048 needs
  * 102 MiB; 8 heads x 1048576 tokens, k = 4096 needs 98 MiB).  Outputs are identical to tka_sparse_decode_step's.
  * All calls on one GPU share that one buffer: two calls may only overlap in time if they run on different
- * GPUs; on one GPU they must be ordered (one stream, or events between streams), otherwise they race. */
+ * GPUs; on one GPU they must be ordered (one stream, or events between streams), otherwise they race.
+ * The buffer's address on a GPU is looked up by the first call made with that GPU current (which must also be the
+ * GPU of args->stream): make that first call outside any stream capture; later calls may be captured and replayed. */
 int tka_sparse_decode_step_noalloc(const tka_sparse_decode_args* args);
 
 /* Diagnostic, as tka_gemv_topk_redone_segments: segments of the last step with these arguments (same workspace)
  * that the selection kernel redid from the keys.  Waits for the stream. */
 int tka_sparse_decode_redone_segments(const tka_sparse_decode_args* args, int32_t* count);
+
+/* ------------------------------------------------------------------------------------------------
+ * Read probes (measurement; no counterpart in the reference): launch a kernel that only READS a KV cache in the
+ * access pattern of one of the two kernels that carry the bytes of the decode step, so that their achieved
+ * bandwidth can be set against what the memory system gives to that pattern on the same machine.
+ *   TKA_PROBE_STREAM  every row of every (batch entry, head), one head per workgroup, `threads` (256 or 512) threads,
+ *                     `rounds` rounds of eight 16-byte loads per lane (512 x 2 is the shape of the long-segment GEMV);
+ *   TKA_PROBE_GATHER  the K and V rows of the token lists idx[batch][num_heads][idx_len] (ids outside the cache read
+ *                     row 0), `tokens_per_wg` ids per workgroup: the pattern of the gathered attention.
+ * Nothing is written but, never in practice, the word `sink`.  Asynchronous on `stream`; time it with events.
+ * ---------------------------------------------------------------------------------------------- */
+typedef enum tka_probe_kind { TKA_PROBE_STREAM = 0, TKA_PROBE_GATHER = 1 } tka_probe_kind;
+typedef struct tka_probe_args {
+  const void* keys;       /* device; row (b,t,h) at keys + b*kv_stride_b + t*kv_stride_n + h*kv_stride_h (elements of 2 bytes) */
+  const void* values;     /* device; gather only, same strides                                 */
+  const int32_t* idx;     /* device; gather only                                               */
+  uint32_t* sink;         /* device; one word                                                  */
+  int32_t kind;           /* tka_probe_kind                                                    */
+  int32_t batch;
+  int32_t num_kv_heads;
+  int32_t idx_len;        /* gather: ids per list                                              */
+  int32_t threads;        /* stream: 256 or 512                                                */
+  int32_t rounds;         /* stream: 1 .. 64                                                   */
+  int32_t nontemporal;    /* stream: 1 = loads with the streaming hint (what the GEMV uses)    */
+  int32_t tokens_per_wg;  /* gather: ids per workgroup (a multiple of 128)                     */
+  int64_t seq_len;
+  int64_t kv_stride_b;
+  int64_t kv_stride_n;
+  int64_t kv_stride_h;
+  void* stream;
+} tka_probe_args;
+int tka_probe_read(const tka_probe_args* args);
 
 /* ------------------------------------------------------------------------------------------------
  * Per-kernel timing.  When enabled, every kernel launch made by this library is bracketed by a pair

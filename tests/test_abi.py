@@ -35,7 +35,7 @@ def _declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = L.lib()
     declared = _declared_symbols()
-    assert len(declared) == 27 + 30
+    assert len(declared) == 28 + 30
     for name in sorted(declared):
         assert hasattr(lib, name), "libtka.so does not export %s" % name
     assert declared == set(L.PROTOTYPES), "ctypes prototypes and headers disagree"
@@ -71,7 +71,7 @@ def test_bind_cpp_style_caller_links_unchanged():
 STRUCTS = {"tka_gemv_topk_args": L.GemvTopkArgs, "tka_topk_args": L.TopkArgs, "tka_center_topk_args": L.CenterTopkArgs,
            "tka_cluster_topk_args": L.ClusterTopkArgs, "tka_index_union_args": L.IndexUnionArgs,
            "tka_flash_decode_args": L.FlashDecodeArgs, "tka_lse_combine_args": L.LseCombineArgs, "tka_ra_args": L.RaArgs,
-           "tka_sparse_decode_args": L.SparseDecodeArgs, "tka_test_hooks": L.TestHooks}
+           "tka_sparse_decode_args": L.SparseDecodeArgs, "tka_test_hooks": L.TestHooks, "tka_probe_args": L.ProbeArgs}
 
 
 def test_ctypes_structs_match_the_c_layout():
@@ -98,7 +98,7 @@ def test_ctypes_structs_match_the_c_layout():
 
 def test_status_strings_and_version():
     lib = L.lib()
-    assert lib.tka_version() >= 100
+    assert lib.tka_version() >= 200            # 2.0.0: score_mode took the place of a reserved field
     assert L.status_string(L.TKA_OK) == "ok"
     assert "workspace" in L.status_string(L.TKA_EWORKSPACE)
     assert L.status_string(99) == "unknown status"
@@ -154,6 +154,20 @@ def test_gemv_topk_validation():
     b = _valid_gemv()
     b.out_scores = None
     assert lib.tka_gemv_scores(C.byref(b)) == L.TKA_EINVAL            # the GEMV phase alone needs out_scores
+    b = _valid_gemv()
+    b.reserved1 = 1
+    assert lib.tka_gemv_topk(C.byref(b)) == L.TKA_EINVAL              # reserved fields must be zero
+    # scores on the matrix cores: only where they apply (keys shared by a batch of two or more, one query head per KV
+    # head, chunks of up to 16384 keys); anywhere else the call is refused, never silently scored in the other order
+    b = _valid_gemv()
+    b.score_mode = L.TKA_SCORE_MATRIX
+    assert lib.tka_gemv_topk(C.byref(b)) == L.TKA_EUNSUPPORTED        # grouped queries, keys per batch entry
+    b.group, b.key_stride_b, b.q_stride_b = 1, 0, 8 * 128
+    assert lib.tka_gemv_topk(C.byref(b)) == L.TKA_EWORKSPACE          # applies: valid, no workspace
+    b.batch = 1
+    assert lib.tka_gemv_topk(C.byref(b)) == L.TKA_EUNSUPPORTED        # a batch of one
+    b.batch, b.seq_len = 2, 32768
+    assert lib.tka_gemv_topk(C.byref(b)) == L.TKA_EUNSUPPORTED        # chunks of more than 16384 keys
 
 
 def test_topk_validation():
@@ -236,10 +250,27 @@ def test_sparse_decode_rejects_values_without_indices():
     assert lib.tka_sparse_decode_step(C.byref(a)) == L.TKA_EWORKSPACE     # valid arguments, no workspace
     a.out_topk_val = 0x5000                                              # values without the rank-ordered ids
     assert lib.tka_sparse_decode_step(C.byref(a)) == L.TKA_EINVAL
-    n = C.c_int32(-1)
     a.out_topk_val = None
+    a.out_union_count = 0x6000                                           # the count of a list that is not asked for
+    assert lib.tka_sparse_decode_step(C.byref(a)) == L.TKA_EINVAL
+    a.out_union_count = None
+    n = C.c_int32(-1)
     assert lib.tka_sparse_decode_redone_segments(C.byref(a), C.byref(n)) == L.TKA_EWORKSPACE
     assert lib.tka_sparse_decode_redone_segments(C.byref(a), None) == L.TKA_EINVAL
+
+
+def test_probe_read_validation():
+    lib = L.lib()
+    a = L.ProbeArgs()
+    assert lib.tka_probe_read(None) == L.TKA_EINVAL
+    assert lib.tka_probe_read(C.byref(a)) == L.TKA_EINVAL            # no cache, no sink
+    a.keys, a.sink, a.batch, a.num_kv_heads, a.seq_len = 4096, 8192, 1, 1, 1000
+    a.kv_stride_n, a.kv_stride_h, a.kind, a.threads, a.rounds = 128, 128, L.TKA_PROBE_STREAM, 300, 2
+    assert lib.tka_probe_read(C.byref(a)) == L.TKA_EINVAL            # threads must be 256 or 512
+    a.kind = L.TKA_PROBE_GATHER
+    assert lib.tka_probe_read(C.byref(a)) == L.TKA_EINVAL            # gather without values and ids
+    a.kind = 7
+    assert lib.tka_probe_read(C.byref(a)) == L.TKA_EUNSUPPORTED
 
 
 def test_test_hooks_validation():

@@ -310,6 +310,46 @@ def test_reference_named_launchers():
             assert np.abs(got[b, h] - ref).max() < TOL
 
 
+_LAUNCHER_MATRIX_SCORES = r"""
+import sys
+import numpy as np, torch
+sys.path.insert(0, sys.argv[1])
+import oracle
+from topk_attn_amd import _lib as L, ops
+from tests.util import f32_of, randn_bits, to_dev
+rng = np.random.default_rng(12)
+dtype = oracle.F16
+q, K, V = randn_bits(rng, (4, 32, 128), dtype, 0.1), randn_bits(rng, (8192, 32, 128), dtype, 0.1), randn_bits(rng, (8192, 32, 128), dtype, 0.1)
+qd, Kd, Vd = to_dev(q, dtype), to_dev(K, dtype), to_dev(V, dtype)
+out = torch.zeros((4, 32, 128), dtype=torch.float16, device="cuda")
+torch.cuda.synchronize()
+ops.profile_enable(True)
+L.lib().launch_retrieval_attention_128(qd.data_ptr(), Kd.data_ptr(), Vd.data_ptr(), out.data_ptr(), 4)
+torch.cuda.synchronize()
+ran = ops.profile_read()
+assert "gemv_scores_mfma" in ran, sorted(ran)
+got = f32_of(out)
+for b, h in ((0, 0), (3, 31), (2, 7)):
+    ref, _, _ = oracle.retrieval_attention(q[b, h], K[:, h], V[:, h], dtype, 4, 128, 1.0)
+    assert np.abs(got[b, h] - ref).max() < 2e-3
+print("launcher with matrix-core scores ok")
+"""
+
+
+def test_ra_launchers_matrix_core_scores_by_environment():
+    """TKA_RA_SCORE_MODE=1 makes the thirty fixed-shape launchers (which have no argument for it) score on the matrix
+    cores.  The variable is read once per process, so the case runs in a child process started with it set, before
+    any GPU call: the kernel that ran, and the output against the oracle at 2e-3."""
+    import os
+    import subprocess
+    import sys
+    announce("launch_retrieval_attention_128 in a child process with TKA_RA_SCORE_MODE=1")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, TKA_RA_SCORE_MODE="1")
+    done = subprocess.run([sys.executable, "-c", _LAUNCHER_MATRIX_SCORES, root], env=env, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0 and "ok" in done.stdout, done.stdout[-2000:] + done.stderr[-4000:]
+
+
 @pytest.mark.parametrize("dtype,out_dt,B,H,G,N,k,sink,local", [
     (oracle.F16, torch.bfloat16, 2, 2, 4, 16384, 2048, 64, 512),
     (oracle.BF16, torch.bfloat16, 1, 2, 8, 8192, 512, 16, 128),

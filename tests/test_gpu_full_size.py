@@ -84,16 +84,22 @@ def test_c4_end_to_end_full_size():
             K[b, hh, h] = (K[b, hh, h].float() * 4.0).to(torch.float16)
     out, tidx, tval, uidx, ucnt = ops.sparse_decode_step(q, K, V, k, sink, local, SCALE, G, out_dtype=torch.bfloat16)
     out16, tidx16, tval16, uidx16, ucnt16 = ops.sparse_decode_step(q, K, V, k, sink, local, SCALE, G, out_dtype=torch.float16)
-    # and for a caller that asks for the output alone: 64 segments, so selection and attention run in one launch
+    # and for a caller that asks for the output alone, with selection and attention in one launch (the rule takes that
+    # form from 256 segments on; the hook takes it here)
     plan_out = ops.SparseDecodePlan(q, K, V, k, sink, local, SCALE, G, out_dtype=torch.float16, want_topk=False, want_union=False)
-    ops.profile_reset()
-    ops.profile_enable(True)
-    out_only = plan_out.step()
-    torch.cuda.synchronize()
-    ran = ops.profile_read()
-    ops.profile_enable(False)
+    ops.set_test_hooks(fused_tail=1)
+    try:
+        ops.profile_reset()
+        ops.profile_enable(True)
+        out_only = plan_out.step()
+        torch.cuda.synchronize()
+        ran = ops.profile_read()
+        ops.profile_enable(False)
+        redone_only = plan_out.redone_segments()
+    finally:
+        ops.set_test_hooks()
     assert "attn_select_mfma" in ran and "lse_combine_redo" in ran and "select_finalize_cand" not in ran, sorted(ran)
-    assert plan_out.redone_segments() == 0
+    assert redone_only == 0
     scores = ops.gemv_scores(q, K, group=G, scale=SCALE)
     torch.cuda.synchronize()
     _check_selection(scores, tidx, tval, k)

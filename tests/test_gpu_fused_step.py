@@ -17,9 +17,9 @@ SCALE = float(np.float32(1.0 / np.sqrt(128.0)))
 
 @pytest.fixture
 def hooks():
-    """The one-launch form is taken by default from 64 segments on; the cases here have a few segments (the CPU oracle
-    checks every one of them) and ask for it through the testing hook.  tests/test_gpu_full_size.py runs the
-    default rule on 64 segments."""
+    """The one-launch form is taken by default from 256 segments on; the cases here have a few segments (the CPU oracle
+    checks every one of them) and ask for it through the testing hook, as tests/test_gpu_full_size.py does at 64
+    segments of 131072 tokens."""
     from topk_attn_amd import ops
 
     def set_hooks(**kw):

@@ -577,9 +577,9 @@ def test_common_cut_route_adversarial_sample_falls_back():
     _check_long(oracle.to_bits(Kf, dtype), oracle.to_bits(qf, dtype), dtype, 1, k, redone=1)
 
 
-def test_common_cut_route_adversarial_sample_falls_back_in_three_launches():
+def test_common_cut_route_adversarial_sample_falls_back_on_a_call_that_fills_the_gpu():
     """The same on a call of more than 65536 rows (four heads): the cut of head 2 comes out among the heavy tokens."""
-    announce("gemv_topk common-cut route in three launches, adversarial sample (fallback)")
+    announce("gemv_topk common-cut route, cuts announced inside the GEMV launch, adversarial sample (fallback)")
     rng = np.random.default_rng(57)
     N, k, dtype = 32768, 2048, oracle.F16
     Kf = rng.standard_normal((1, N, 4, 128)) * 0.05

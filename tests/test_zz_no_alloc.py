@@ -128,6 +128,64 @@ def test_noalloc_step_without_list_outputs():
                 assert (np.abs(outf[b, h * G:(h + 1) * G] - ro) < 2e-3).all()
 
 
+@pytest.mark.gpu
+def test_noalloc_step_captured_in_a_graph():
+    """The use the entry point is for: captured into a HIP graph (after one eager call, which looks up the address of the
+    built-in buffer) and replayed - twice, with new queries each time and, between the replays, an eager call of another
+    shape that leaves the buffer in another layout.  Every replay must give what the eager call with the workspace gives."""
+    lib = L.lib()
+    announce("sparse_decode_step_noalloc captured in a graph, two replays with another layout of the scratch in between")
+    rng = np.random.default_rng(2026)
+    dtype, B, H, G, N, k, sink, local = oracle.F16, 1, 2, 4, 70000, 1024, 16, 128
+
+    def tensors(B, H, G, N, k, sink, local):
+        q = to_dev(randn_bits(rng, (B, H * G, 128), dtype), dtype)
+        K, V = to_dev(randn_bits(rng, (B, N, H, 128), dtype), dtype), to_dev(randn_bits(rng, (B, N, H, 128), dtype), dtype)
+        out = torch.zeros((B, H * G, 128), dtype=torch.float16, device="cuda")
+        tidx = torch.zeros((B, H, k), dtype=torch.int32, device="cuda")
+        tval = torch.zeros((B, H, k), dtype=torch.float32, device="cuda")
+        uidx = torch.zeros((B, H, k + sink + local), dtype=torch.int32, device="cuda")
+        ucnt = torch.zeros((B, H), dtype=torch.int32, device="cuda")
+        return q, K, V, out, tidx, tval, uidx, ucnt
+
+    q, K, V, out, tidx, tval, uidx, ucnt = tensors(B, H, G, N, k, sink, local)
+    q2, K2, V2, out2, tidx2, tval2, uidx2, ucnt2 = tensors(2, 2, 2, 5000, 300, 8, 8)       # the other layout
+    a = _args(q, K, V, out, k, sink, local, G, tidx, tval, uidx, ucnt)
+    other = _args(q2, K2, V2, out2, 300, 8, 8, 2, tidx2, tval2, uidx2, ucnt2)
+    L.check(lib.tka_sparse_decode_step_noalloc(C.byref(a)), "first call, eager")
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        a.stream = side.cuda_stream
+        L.check(lib.tka_sparse_decode_step_noalloc(C.byref(a)), "warm-up on the side stream")
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            a.stream = torch.cuda.current_stream().cuda_stream
+            L.check(lib.tka_sparse_decode_step_noalloc(C.byref(a)), "captured call")
+    torch.cuda.synchronize()
+    # the reference for every replay: the workspace form, eager
+    ref_out, ref_tidx, ref_uidx, ref_ucnt = (torch.zeros_like(t) for t in (out, tidx, uidx, ucnt))
+    ref_tval = torch.zeros_like(tval)
+    r = _args(q, K, V, ref_out, k, sink, local, G, ref_tidx, ref_tval, ref_uidx, ref_ucnt)
+    need = lib.tka_sparse_decode_workspace_bytes(C.byref(r))
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    r.workspace, r.workspace_bytes = ws.data_ptr(), need
+    for it in range(2):
+        q.copy_(to_dev(randn_bits(rng, (B, H * G, 128), dtype), dtype))
+        r.stream = other.stream = torch.cuda.current_stream().cuda_stream
+        L.check(lib.tka_sparse_decode_step(C.byref(r)), "reference step")
+        L.check(lib.tka_sparse_decode_step_noalloc(C.byref(other)), "eager call of another shape")   # another layout in the scratch
+        for t in (out, tidx, tval, uidx, ucnt):
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, g_, r_ in (("out", out, ref_out), ("topk_idx", tidx, ref_tidx), ("topk_val", tval, ref_tval), ("union_idx", uidx, ref_uidx),
+                             ("union_count", ucnt, ref_ucnt)):
+            assert torch.equal(g_.view(torch.uint8), r_.view(torch.uint8)), "replay %d: %s differs from the eager step" % (it, name)
+
+
 def test_noalloc_step_rejects_what_does_not_fit():
     """Batch 16 of the 128k configuration needs 203 MiB of scratch: refused with TKA_ESCRATCH before any HIP call
     (so this runs without a GPU)."""

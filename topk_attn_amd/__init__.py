@@ -11,7 +11,7 @@ TORCH_EXT_PATH = os.path.join(_HERE, "lib", "retrieval_attention_cpp.so")
 
 
 STAMP_PATH = os.path.join(_HERE, "lib", "BUILD_STAMP")
-ARTEFACTS = ("libtka.so", "tka_standalone", "tka_bind_link_check", "tka_stream_probe", "retrieval_attention_cpp.so")
+ARTEFACTS = ("libtka.so", "tka_standalone", "tka_bind_link_check", "retrieval_attention_cpp.so")
 
 
 def source_digest():

@@ -88,6 +88,14 @@ RA_VARIANTS = ("", "_global", "_pipelined", "_pipelined_global", "_two_kernels",
 RA_TOPKS = (32, 128, 256, 512, 1024)
 
 # name -> (restype, argtypes); every symbol include/*.h declares
+class ProbeArgs(C.Structure):
+    _fields_ = [("keys", _p), ("values", _p), ("idx", _p), ("sink", _p), ("kind", _i32), ("batch", _i32), ("num_kv_heads", _i32),
+                ("idx_len", _i32), ("threads", _i32), ("rounds", _i32), ("nontemporal", _i32), ("tokens_per_wg", _i32),
+                ("seq_len", _i64), ("kv_stride_b", _i64), ("kv_stride_n", _i64), ("kv_stride_h", _i64), ("stream", _p)]
+
+
+TKA_PROBE_STREAM, TKA_PROBE_GATHER = 0, 1
+
 PROTOTYPES = {
     "tka_status_string": (C.c_char_p, [C.c_int]),
     "tka_version": (C.c_int, []),
@@ -97,6 +105,7 @@ PROTOTYPES = {
     "tka_gemv_topk_redone_segments": (C.c_int, [C.POINTER(GemvTopkArgs), C.POINTER(C.c_int32)]),
     "tka_gemv_topk_gave_up_slices": (C.c_int, [C.POINTER(GemvTopkArgs), C.POINTER(C.c_int32)]),
     "tka_set_test_hooks": (C.c_int, [C.POINTER(TestHooks)]),
+    "tka_probe_read": (C.c_int, [C.POINTER(ProbeArgs)]),
     "tka_topk_workspace_bytes": (_sz, [C.POINTER(TopkArgs)]),
     "tka_topk_f32": (C.c_int, [C.POINTER(TopkArgs)]),
     "tka_center_topk_expand_workspace_bytes": (_sz, [C.POINTER(CenterTopkArgs)]),

@@ -103,6 +103,7 @@ int check_gemv(const tka_gemv_topk_args* a, bool need_topk) {
   if (a->head_dim != TKA_HEAD_DIM || !dtype_ok(a->dtype) || !group_ok(a->group)) return TKA_EUNSUPPORTED;
   if (a->batch < 1 || a->num_kv_heads < 1 || a->seq_len < 1 || a->num_chunks < 1) return TKA_EINVAL;
   if (a->score_mode != TKA_SCORE_CANONICAL && a->score_mode != TKA_SCORE_MATRIX) return TKA_EUNSUPPORTED;
+  if (a->reserved1 != 0) return TKA_EINVAL;   // reserved fields must be zero
   if (a->batch > 65535 || a->num_kv_heads > 65535) return TKA_EUNSUPPORTED;
   if (a->seq_len > 0x7fffffffLL) return TKA_EUNSUPPORTED;  // token ids are int32
   if (a->seq_len % a->num_chunks != 0) return TKA_EINVAL;
@@ -117,7 +118,17 @@ int check_gemv(const tka_gemv_topk_args* a, bool need_topk) {
   } else if (!a->out_scores) {
     return TKA_EINVAL;
   }
+  if (a->score_mode == TKA_SCORE_MATRIX && (a->batch >= 1 && a->num_kv_heads >= 1) &&
+      !(a->group == 1 && a->key_stride_b == 0 && a->batch >= 2 && (!need_topk || a->seq_len / a->num_chunks <= 16384)))
+    return TKA_EUNSUPPORTED;
   return TKA_OK;
+}
+
+// TKA_SCORE_MATRIX is served where keys are shared by a batch of at least two entries, one query head per KV head, and the
+// scores are written out whole (the GEMV alone, or chunks of up to 16384 keys); a call that asks for it elsewhere is refused
+// rather than silently scored in the canonical order.
+bool matrix_scores_apply(const tka_gemv_topk_args* a) {
+  return a->group == 1 && a->key_stride_b == 0 && a->batch >= 2;
 }
 
 size_t gemv_scores_bytes(const tka_gemv_topk_args* a) {
@@ -166,22 +177,11 @@ void fill_gemv_params(const tka_gemv_topk_args* a, float* scores, uint32_t* hist
 // Segments of up to 16384 scores (k up to 1024, 2048 beyond 4096 scores): one workgroup per segment selects from
 // plain scores with the keys in its registers.  Segments of up to 2048 rows that still have to be scored take this
 // route only in numbers: a few are quicker scored and selected by one workgroup each in one launch.
-int wave_select_min_segments() {
-  static const int v = [] {
-    const char* e = getenv("TKA_WAVE_MIN_SEGS");
-    return e && *e ? atoi(e) : 128;
-  }();
-  return v;
-}
-int small_select_max_segments() {
-  static const int v = [] {
-    const char* e = getenv("TKA_SMALL_MAX_SEGS");
-    return e && *e ? atoi(e) : 64;
-  }();
-  return v;
-}
+constexpr int kWaveSelectMinSegments = 128;
+// A small k out of a few thousand scores: one big workgroup per segment with a short program, up to this many segments.
+constexpr int kSmallSelectMaxSegments = 64;
 bool small_select_fits(int64_t seg_len, int k, int segs) {
-  return seg_len > kFusedMaxSegLen && seg_len <= select_small_max_len() && k <= select_small_max_k() && segs <= small_select_max_segments();
+  return seg_len > kFusedMaxSegLen && seg_len <= select_small_max_len() && k <= select_small_max_k() && segs <= kSmallSelectMaxSegments;
 }
 bool wave_select_fits(int64_t seg_len, int k) { return seg_len <= select_wave_max_len() && k <= select_wave_max_k(seg_len); }
 
@@ -208,32 +208,12 @@ struct UnionOut {
 // calls of up to 1572864 rows; rank-ordered output, and the union list for a caller that only hands it to the
 // attention), else 0.  Shorter segments are selected from the registers of one workgroup, longer ones (or many of
 // them) by the sampling workgroups of the candidate route.
-int64_t cut_route_min_len() {
-  static const int64_t v = [] {
-    const char* e = getenv("TKA_CUT_MIN_LEN");
-    return e && *e ? (int64_t)atoll(e) : (int64_t)select_cand_capacity() / 2 + 1;
-  }();
-  return v;
-}
-// Rows of a call beyond which the cut is found in a launch of its own (one workgroup per segment) instead of in every
+int64_t cut_route_min_len() { return (int64_t)select_cand_capacity() / 2 + 1; }
+// Rows of a call beyond which the cut is found once per segment (by the first workgroups of the GEMV launch) instead of in every
 // GEMV workgroup: scoring the 256 sample rows beside every 256 tokens is free only while the launch does not fill the
 // GPU.  Decode steps, k = 2048, us per step in two / three launches: 1 x 32768 tokens 23.5 / 26.5, 2 x 32768 28.1 / 30.0,
 // 1 x 65536 26.3 / 29.5, 3 x 32768 29.3 / 26.8, 4 x 32768 31.3 / 27.7, 8 x 32768 43.0 / 36.2.
-int64_t cut_split_min_rows() {
-  static const int64_t v = [] {
-    const char* e = getenv("TKA_CUT_SPLIT_ROWS");
-    return e && *e ? (int64_t)atoll(e) : (int64_t)65536;
-  }();
-  return v;
-}
-// Whether those cuts come from the first workgroups of the GEMV launch (the default) or from a launch before it.
-bool cut_front_sampling() {
-  static const bool v = [] {
-    const char* e = getenv("TKA_CUT_FRONT_SAMPLING");
-    return !(e && *e) || atoi(e) != 0;
-  }();
-  return v;
-}
+constexpr int64_t kCutSplitMinRows = 65536;
 // Tells this call's words in a workspace from older contents: never 0, the cleared state; bit 30 stays free for the
 // "has a cut" mark of the candidate route's threshold words.
 uint32_t next_epoch() {
@@ -244,9 +224,10 @@ void cut_plan(const tka_gemv_topk_args* a, const UnionOut* u, int* num_samples, 
   *num_samples = *sample_rank = 0;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
   if ((!a->out_idx && !u) || (u && !u->handoff) || a->out_scores || chunk_len < cut_route_min_len()) return;
+  if (a->score_mode == TKA_SCORE_MATRIX) return;   // (the matrix cores score into a plain score array: the routes that select from one)
   const int64_t rows = (int64_t)a->batch * a->num_kv_heads * a->seq_len;
   int s = 0, r = 0, len = 0;
-  gemv_cut_plan(chunk_len, a->k, rows > cut_split_min_rows(), &s, &r, &len);
+  gemv_cut_plan(chunk_len, a->k, rows > kCutSplitMinRows, &s, &r, &len);
   if (s == 0) return;
   if (slice_len) *slice_len = len;
   // Measured, decode steps with k = 2048 unless said (us per step, this route against the others): 1 x 32768 tokens
@@ -291,7 +272,7 @@ bool wave_route(const tka_gemv_topk_args* a, bool want_union) {
   const int segs = a->batch * a->num_kv_heads * a->num_chunks;
   const int64_t chunk_len = a->seq_len / a->num_chunks;
   return (a->out_idx || want_union) && wave_select_fits(chunk_len, a->k) &&
-         (chunk_len > kFusedMaxSegLen || a->out_scores || segs >= wave_select_min_segments());
+         (chunk_len > kFusedMaxSegLen || a->out_scores || segs >= kWaveSelectMinSegments);
 }
 
 struct FusedTail;
@@ -359,8 +340,8 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
     // a call that fills the GPU finds the cut in a launch of its own instead of in every GEMV workgroup
     const int64_t rows = (int64_t)segs * chunk_len;
     int rc;
-    if (rows > cut_split_min_rows()) {
-      if (cut_front_sampling()) {
+    if (rows > kCutSplitMinRows) {
+      {
         const tka_test_hooks hooks = current_hooks();
         cp.tau_words = sp.tau_words;
         cp.epoch = next_epoch();
@@ -379,10 +360,7 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
         // 16 x 16384 33.9 -> 32.9, 8 x 32768 30.35 -> 30.1; 12 and 24 x 32768 would lose 0.6-0.7 and keep the other order).
         // Also for any number of segments where a head's rows lie a multiple of 4 KB apart (3 x 16 x 32768 tokens 106 -> 95.5).
         cp.interleave_segs = (segs & (segs - 1)) == 0 || (a->key_stride_n * 2) % 4096 == 0 ? 1 : 0;
-        rc = launch_gemv_cut_slices(cp, a->dtype, true, stream);
-      } else {
-        rc = launch_cut_samples(cp, a->dtype, stream);
-        if (rc == TKA_OK) rc = launch_gemv_cut_slices(cp, a->dtype, false, stream);
+        rc = launch_gemv_cut_slices(cp, a->dtype, stream);
       }
     } else {
       rc = launch_gemv_cut(cp, a->dtype, stream);
@@ -694,7 +672,7 @@ const char* tka_status_string(int status) {
   }
 }
 
-int tka_version(void) { return 100; }
+int tka_version(void) { return 200; }
 
 // ---- stage 1 ----------------------------------------------------------------------------------
 
@@ -1263,6 +1241,8 @@ int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
   int rc = sd_check(a, &g, &f);
   if (rc != TKA_OK) return rc;
   if (a->out_topk_val && !a->out_topk_idx) return TKA_EINVAL;   // values come with the rank-ordered ids only
+  if (a->out_union_count && !a->out_union_idx) return TKA_EINVAL;   // the count belongs to the list (without the list the step
+                                                                     // hands its tokens on in a form whose count is not the union's)
   const size_t need = tka_sparse_decode_workspace_bytes(a);
   if (!a->workspace || a->workspace_bytes < need) return TKA_EWORKSPACE;
   const size_t segs = (size_t)a->batch * a->num_kv_heads;
@@ -1288,16 +1268,19 @@ int tka_sparse_decode_step(const tka_sparse_decode_args* a) {
   g.workspace = ws;
   g.workspace_bytes = gemv_ws;
   UnionOut uo = {uidx, ucnt, a->sink, a->local, sd_union_handoff(a) || behind};
-  // A caller that asks for neither list (the output alone): on long segments the attention launch selects the tokens
-  // itself from the candidates of the GEMV launch, and the ids never leave the chip.  Every split of a segment finds the
-  // segment's threshold again, which costs what the launch saves until the call has many segments (us per step, one
-  // launch / two, 131072 tokens, k = 2048: 8 segments 66.4 / 64.1, 32 segments 188.1 / 186.2, 64 segments 344.2 / 344.7,
-  // 128 segments of 65536 tokens 366.5 / 372.9), so it is taken from 64 segments on.
+  // A caller that asks for neither list (the output alone): on long segments the attention launch can select the tokens
+  // itself from the candidates of the GEMV launch, and the ids never leave the chip.  Every split of a segment then finds
+  // the segment's threshold again, and that costs what the saved launch gives: us per step, one launch / two, k = 2048:
+  // 64 segments of 131072 tokens 344.5 / 342.8, 96 segments 507.0 / 503.2, 128 segments 667.1 / 665.5, 128 segments of 65536
+  // tokens 366.5 / 366.4, 192 segments 524.4 / 519.8, 256 segments 724.1 / 725.2.  (A form in which one split per segment
+  // selects and the others wait for its list - a bounded wait - was 2 us slower still: the selection is a chain of
+  // dependent steps that takes its 8-10 us whether or not the other splits keep out of its way.)  So the two launches
+  // stay the rule and the one launch is taken from 256 segments on.
   FusedTail ft;
   ft.taken = false;
   const tka_test_hooks hooks = current_hooks();
   const bool output_only = !a->out_topk_idx && !a->out_union_idx && hooks.union_handoff_order == 0 && a->group >= 2 &&
-                           (hooks.fused_tail == 1 || (hooks.fused_tail == 0 && segs >= 64));
+                           (hooks.fused_tail == 1 || (hooks.fused_tail == 0 && segs >= 256));
   rc = run_gemv_topk(&g, nullptr, 0, nullptr, &uo, false, nullptr, output_only ? &ft : nullptr);
   if (rc != TKA_OK) return rc;
   f.kv_idx = uidx;
@@ -1361,6 +1344,34 @@ int tka_sparse_decode_step_noalloc(const tka_sparse_decode_args* a) {
   b.workspace = ptr;
   b.workspace_bytes = (size_t)TKA_NOALLOC_SCRATCH_BYTES;
   return tka_sparse_decode_step(&b);
+}
+
+// ---- read probes --------------------------------------------------------------------------------
+
+int tka_probe_read(const tka_probe_args* a) {
+  if (!a || !a->keys || !a->sink) return TKA_EINVAL;
+  if (a->batch < 1 || a->num_kv_heads < 1 || a->seq_len < 1 || a->seq_len > 0x7fffffffLL) return TKA_EINVAL;
+  if (a->kv_stride_n < TKA_HEAD_DIM || a->kv_stride_h < 0 || a->kv_stride_b < 0 || ((a->kv_stride_n | a->kv_stride_h | a->kv_stride_b) & 7)) return TKA_EINVAL;
+  if (!aligned16(a->keys)) return TKA_EINVAL;
+  ProbeParams p;
+  memset(&p, 0, sizeof p);
+  p.base = a->keys;
+  p.base2 = a->values;
+  p.idx = a->idx;
+  p.sink = a->sink;
+  p.seq_len = a->seq_len;
+  p.stride_b = a->kv_stride_b;
+  p.stride_n = a->kv_stride_n;
+  p.stride_h = a->kv_stride_h;
+  p.batch = a->batch;
+  p.num_heads = a->num_kv_heads;
+  p.idx_len = a->idx_len;
+  if (a->kind == TKA_PROBE_STREAM) return launch_probe_stream(p, a->threads, a->rounds, a->nontemporal != 0, (hipStream_t)a->stream);
+  if (a->kind == TKA_PROBE_GATHER) {
+    if (!a->values || !a->idx || !aligned16(a->values) || a->idx_len < 1 || a->tokens_per_wg < 128 || a->tokens_per_wg % 128) return TKA_EINVAL;
+    return launch_probe_gather(p, a->tokens_per_wg, (hipStream_t)a->stream);
+  }
+  return TKA_EUNSUPPORTED;
 }
 
 // ---- per-kernel timing ------------------------------------------------------------------------

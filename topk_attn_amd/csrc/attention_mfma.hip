@@ -20,7 +20,12 @@ namespace {
 
 using namespace mfma_attn;
 
-template <int DT, int G, bool INDEXED>
+// STAGED (indexed form, splits of up to kStagedIds tokens): the split's ids go to LDS in one coalesced trip before the
+// first tile, so that a tile's row requests do not wait for a load of their ids first (a tile then costs one round trip
+// to memory instead of two: c4's gathered attention 20.4 -> 18.6 us).
+constexpr int kStagedIds = 2048;
+
+template <int DT, int G, bool INDEXED, bool STAGED>
 __global__ __launch_bounds__(kThreads) void attn_mfma_kernel(AttnParams p) {
   const int split = p.head_fastest ? blockIdx.y : blockIdx.x;
   const int h = p.head_fastest ? blockIdx.x : blockIdx.y;
@@ -36,15 +41,24 @@ __global__ __launch_bounds__(kThreads) void attn_mfma_kernel(AttnParams p) {
   int64_t end = begin + p.tokens_per_split;
   if (end > count) end = count;
   __shared__ AttendLds<G> sh;
-  attend<DT, G, INDEXED>(p, INDEXED ? p.kv_idx + seg * p.idx_len : nullptr, begin, end, b, h, split, sh);
+  if constexpr (INDEXED && STAGED) {
+    __shared__ int32_t sh_ids[kStagedIds];
+    const int32_t* idx = p.kv_idx + seg * p.idx_len + begin;
+    const int n = end > begin ? (int)(end - begin) : 0;
+    for (int i = threadIdx.x; i < n; i += kThreads) sh_ids[i] = idx[i];
+    __syncthreads();
+    attend<DT, G, true>(p, sh_ids, 0, n, b, h, split, sh);
+  } else {
+    attend<DT, G, INDEXED>(p, INDEXED ? p.kv_idx + seg * p.idx_len : nullptr, begin, end, b, h, split, sh);
+  }
 }
 
-template <int DT, bool INDEXED>
+template <int DT, bool INDEXED, bool STAGED>
 int launch_g(const AttnParams& p, dim3 grid, hipStream_t stream) {
   switch (p.group) {
-    case 2: attn_mfma_kernel<DT, 2, INDEXED><<<grid, kThreads, 0, stream>>>(p); break;
-    case 4: attn_mfma_kernel<DT, 4, INDEXED><<<grid, kThreads, 0, stream>>>(p); break;
-    case 8: attn_mfma_kernel<DT, 8, INDEXED><<<grid, kThreads, 0, stream>>>(p); break;
+    case 2: attn_mfma_kernel<DT, 2, INDEXED, STAGED><<<grid, kThreads, 0, stream>>>(p); break;
+    case 4: attn_mfma_kernel<DT, 4, INDEXED, STAGED><<<grid, kThreads, 0, stream>>>(p); break;
+    case 8: attn_mfma_kernel<DT, 8, INDEXED, STAGED><<<grid, kThreads, 0, stream>>>(p); break;
     default: return TKA_EUNSUPPORTED;
   }
   return hip_status(hipGetLastError());
@@ -64,8 +78,13 @@ int launch_attn_partial_mfma(const AttnParams& p0, int dtype, hipStream_t stream
   dim3 grid((unsigned)p.num_splits, (unsigned)p.num_kv_heads, (unsigned)p.batch);
   if (p.head_fastest) grid = dim3((unsigned)p.num_kv_heads, (unsigned)p.num_splits, (unsigned)p.batch);
   LaunchTimer timer(p.kv_idx ? "attn_mfma_indexed" : "attn_mfma_dense", stream);
-  if (dtype == TKA_F16) return p.kv_idx ? launch_g<TKA_F16, true>(p, grid, stream) : launch_g<TKA_F16, false>(p, grid, stream);
-  return p.kv_idx ? launch_g<TKA_BF16, true>(p, grid, stream) : launch_g<TKA_BF16, false>(p, grid, stream);
+  // (a split of one step has nothing to gain: each wave asks for its only tile's ids once either way)
+  const bool staged = p.kv_idx && p.tokens_per_split <= kStagedIds && p.tokens_per_split > kStep;
+  if (dtype == TKA_F16)
+    return !p.kv_idx ? launch_g<TKA_F16, false, false>(p, grid, stream)
+                     : (staged ? launch_g<TKA_F16, true, true>(p, grid, stream) : launch_g<TKA_F16, true, false>(p, grid, stream));
+  return !p.kv_idx ? launch_g<TKA_BF16, false, false>(p, grid, stream)
+                   : (staged ? launch_g<TKA_BF16, true, true>(p, grid, stream) : launch_g<TKA_BF16, true, false>(p, grid, stream));
 }
 
 }  // namespace tka

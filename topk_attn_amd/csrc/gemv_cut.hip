@@ -317,24 +317,19 @@ __device__ __forceinline__ void sample_segment(const GemvParams& p, const SegPos
   rank_samples<S, ANNOUNCED>(sh_skey, sh_rkey, sh_rank, sh_cut, seg, stride, p.split_ranks, p.cut_splits);
 }
 
-// One workgroup per segment, in a launch of its own.
-template <int DT>
-__global__ __launch_bounds__(kCutThreads) void cut_sample_kernel(GemvParams p) {
-  sample_segment<DT, false>(p, seg_position(p));
-}
-
 // One workgroup per 512 tokens (two slices of the ranking kernel's layout): scores, and the tokens at or above the
 // segment's cut in p.cut_splits, stored as in gemv_cut_kernel.
-// FRONT = false: the cuts are there (cut_sample_kernel ran before).  FRONT = true: the first workgroups of this launch, one
-// per segment, find them (sample_segment) while the others score their tokens; each publishes its cut and part ends and
+// The first workgroups of the launch, one per segment, find the cuts (sample_segment) while the others score their tokens;
+// each publishes its cut and part ends and
 // then the call's epoch in the segment's word of p.tau_words, for which the first thread of a scoring workgroup waits
 // before the compare - a bounded wait: a workgroup that never sees the word marks its slices (kCutGaveUp in the count),
 // and the ranking kernel redoes such a segment from the keys.  The sampling workgroups come first in the grid, so they
 // run before any workgroup that waits for them; nothing depends on that but the speed.  With p.samplers_score they are not
 // extra workgroups: having published their segment's cut they score the tokens that their place in the grid names, like
 // the others (the cut they then wait for is that of a sampling workgroup no later in the grid than themselves).
-template <int DT, bool FRONT, int L>
+template <int DT, int L>
 __global__ __launch_bounds__(kCutThreads, 8) void gemv_cut_slices_kernel(GemvParams p) {
+  constexpr bool FRONT = true;   // (the cuts come from the first workgroups of this launch)
   constexpr int kTokens = 2 * kCutTokensPerWg;
   __shared__ uint32_t sh_key[kTokens];
   __shared__ uint32_t sh_wcnt[kTokens / kWave];
@@ -400,7 +395,6 @@ __global__ __launch_bounds__(kCutThreads, 8) void gemv_cut_slices_kernel(GemvPar
     kv[u] = __builtin_nontemporal_load((const u32x4*)(kbase + (int64_t)(t_begin + (row < n_local ? row : n_local - 1)) * p.key_stride_n));
   }
   uint64_t cut = 0;
-  if (!FRONT) cut = p.cut_splits[(int64_t)seg * kCutParts + (kCutParts - 1)];   // (the same for all: a scalar load beside the rows)
   __builtin_amdgcn_sched_barrier(0);
   float qf[8];
   group_query_through_lds<DT>(p, qpiece, j, sh_q, qf);
@@ -423,6 +417,10 @@ __global__ __launch_bounds__(kCutThreads, 8) void gemv_cut_slices_kernel(GemvPar
         v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       const bool ok = (uint32_t)(v >> 32) == p.epoch;
+      // The cut was written, and had completed, before the word that announces it; it is asked for only behind the poll
+      // that has seen the word.  The hardware returns a wave's loads in the order they were issued; the fence keeps the
+      // compiler from issuing them in another.
+      __atomic_signal_fence(__ATOMIC_SEQ_CST);
       sh_cutc[1] = ok ? 1ull : 0ull;
       sh_cutc[0] = ok ? __hip_atomic_load(p.cut_splits + (int64_t)seg * kCutParts + (kCutParts - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : ~0ull;
     }
@@ -466,43 +464,23 @@ int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream) {
   return hip_status(hipGetLastError());
 }
 
-// The route in three launches (this one and the next, then launch_select_rank): same arguments and the same outputs
-// as launch_gemv_cut.
-int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream) {
-  const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
-  if (p.num_samples != kCutSamplesOnce || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
-      !p.cut_splits || segs > 0x7fffffffLL || !grid_ok(p))
-    return TKA_EINVAL;
-  const dim3 wgs(1u, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
-  LaunchTimer timer("cut_sample", stream);
-  if (dtype == TKA_F16)
-    cut_sample_kernel<TKA_F16><<<wgs, kCutThreads, 0, stream>>>(p);
-  else
-    cut_sample_kernel<TKA_BF16><<<wgs, kCutThreads, 0, stream>>>(p);
-  return hip_status(hipGetLastError());
-}
-
-// front_sampling: the cuts come from the first workgroups of this launch (p.tau_words, p.epoch, p.tau_spin_limit and the
-// sampling arguments of launch_cut_samples are then needed) instead of from a launch before it.
-int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream) {
+// The cuts come from the first workgroups of the launch (p.tau_words, p.epoch, p.tau_spin_limit, p.num_samples = kCutSamplesOnce,
+// p.sample_rank, p.split_ranks, p.cut_splits).
+int launch_gemv_cut_slices(const GemvParams& p, int dtype, hipStream_t stream) {
   const int64_t segs = (int64_t)p.batch * p.num_kv_heads * p.num_chunks;
   const int64_t wgs_per_seg = (p.chunk_len + 2 * kCutTokensPerWg - 1) / (2 * kCutTokensPerWg);
   if (!slices_ok(p) || segs * (wgs_per_seg + 1) > 0x7fffffffLL || !grid_ok(p)) return TKA_EINVAL;
-  const dim3 wgs = front_sampling ? dim3((unsigned)(segs * (wgs_per_seg + (p.samplers_score ? 0 : 1))))
-                                  : dim3((unsigned)wgs_per_seg, (unsigned)(p.num_kv_heads * p.num_chunks), (unsigned)p.batch);
-  if (front_sampling && (p.num_samples != kCutSamplesOnce || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
-                         !p.tau_words || p.epoch == 0 || p.tau_spin_limit < 1))
+  const dim3 wgs((unsigned)(segs * (wgs_per_seg + (p.samplers_score ? 0 : 1))));
+  if (p.num_samples != kCutSamplesOnce || p.chunk_len < p.num_samples || p.sample_rank < kCutParts || p.sample_rank > p.num_samples ||
+      !p.cut_splits || !p.tau_words || p.epoch == 0 || p.tau_spin_limit < 1)
     return TKA_EINVAL;
   LaunchTimer timer("gemv_cut_slices", stream);
   typedef void (*Kernel)(GemvParams);
   constexpr int kLong = kCutTokensPerWg, kShort = kCutTokensPerWg / 2;
-  static const Kernel kernels[2][2][2] = {   // [dtype][cuts from the first workgroups][slices of 128 tokens]
-      {{gemv_cut_slices_kernel<TKA_F16, false, kLong>, gemv_cut_slices_kernel<TKA_F16, false, kShort>},
-       {gemv_cut_slices_kernel<TKA_F16, true, kLong>, gemv_cut_slices_kernel<TKA_F16, true, kShort>}},
-      {{gemv_cut_slices_kernel<TKA_BF16, false, kLong>, gemv_cut_slices_kernel<TKA_BF16, false, kShort>},
-       {gemv_cut_slices_kernel<TKA_BF16, true, kLong>, gemv_cut_slices_kernel<TKA_BF16, true, kShort>}}};
-  hipLaunchKernelGGL(kernels[dtype == TKA_F16 ? 0 : 1][front_sampling ? 1 : 0][p.tokens_per_wg == kShort ? 1 : 0], wgs, dim3(kCutThreads), 0,
-                     stream, p);
+  static const Kernel kernels[2][2] = {   // [dtype][slices of 128 tokens]
+      {gemv_cut_slices_kernel<TKA_F16, kLong>, gemv_cut_slices_kernel<TKA_F16, kShort>},
+      {gemv_cut_slices_kernel<TKA_BF16, kLong>, gemv_cut_slices_kernel<TKA_BF16, kShort>}};
+  hipLaunchKernelGGL(kernels[dtype == TKA_F16 ? 0 : 1][p.tokens_per_wg == kShort ? 1 : 0], wgs, dim3(kCutThreads), 0, stream, p);
   return hip_status(hipGetLastError());
 }
 

@@ -612,6 +612,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
           v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         early_word = 0;
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);   // (the cut below is asked for behind the word that announces it: program order, which the compiler must keep)
         const uint32_t ep = (uint32_t)(v >> 32);
         sh_tau[0] = (uint32_t)v;
         sh_tau[1] = (ep & ~kTauHasCut) == p.epoch ? 1u : 0u;
@@ -746,6 +747,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(4,
       if (spin) __builtin_amdgcn_s_sleep(16);
       v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);   // (the cut below is asked for behind the word that announces it)
     const uint32_t ep = (uint32_t)(v >> 32);
     sh_tau[4 * tid] = (uint32_t)v;
     sh_tau[4 * tid + 1] = (ep & ~kTauHasCut) == p.epoch ? 1u : 0u;

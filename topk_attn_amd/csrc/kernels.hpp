@@ -62,11 +62,10 @@ int gemv_tokens_per_wg(int64_t total_rows, int64_t chunk_len);
 // (p.cand_head: the first kCutHead of a slice as composites, zeros behind; p.cand: the rest; p.cand_count; p.num_samples /
 // p.sample_rank and the slice length p.tokens_per_wg from gemv_cut_plan; p.wgs_per_chunk: the slices of a segment).
 int launch_gemv_cut(const GemvParams& p, int dtype, hipStream_t stream);
-// The same in two launches for calls that fill the GPU: one workgroup per segment finds the cut and the part ends, then the
-// GEMV workgroups (512 tokens each) score nothing twice.
-int launch_cut_samples(const GemvParams& p, int dtype, hipStream_t stream);
-int launch_gemv_cut_slices(const GemvParams& p, int dtype, bool front_sampling, hipStream_t stream);
-// sampled_once: the plan for launch_cut_samples / launch_gemv_cut_slices (kCutSamplesOnce samples) instead of launch_gemv_cut (256).
+// The same for calls that fill the GPU: the first workgroups of the launch, one per segment, find the cut and the part ends and
+// announce them; the GEMV workgroups (512 tokens each) score nothing twice.
+int launch_gemv_cut_slices(const GemvParams& p, int dtype, hipStream_t stream);
+// sampled_once: the plan for launch_gemv_cut_slices (kCutSamplesOnce samples) instead of launch_gemv_cut (256).
 void gemv_cut_plan(int64_t chunk_len, int k, bool sampled_once, int* num_samples, int* sample_rank, int* slice_len);
 uint64_t gemv_cut_split_ranks(int64_t chunk_len, int k, int num_samples, int sample_rank);
 
@@ -211,5 +210,17 @@ int launch_lse_combine(const CombineParams& p, hipStream_t stream);
 // g, s: the stage-1 parameters of the step (s.out_idx must be null: no rank order); a: q, values, strides, scale.
 int launch_lse_combine_redo(const CombineParams& c, const GemvParams& g, const SelectParams& s, const AttnParams& a, int dtype,
                             hipStream_t stream);
+
+// ---- read probes (probes.hip) ------------------------------------------------------------------
+struct ProbeParams {
+  const void* base;     // rows of 256 bytes: row (b, t, h) at base + 2 * (b * stride_b + t * stride_n + h * stride_h)
+  const void* base2;    // gather: the second cache (values)
+  const int32_t* idx;   // gather: [batch][num_heads][idx_len] token ids
+  uint32_t* sink;       // one word that no run writes (it keeps the loads alive)
+  int64_t seq_len, stride_b, stride_n, stride_h;
+  int batch, num_heads, idx_len;
+};
+int launch_probe_stream(const ProbeParams& p, int threads, int rounds, bool nontemporal, hipStream_t stream);
+int launch_probe_gather(const ProbeParams& p, int tokens_per_wg, hipStream_t stream);
 
 }  // namespace tka

@@ -1064,7 +1064,7 @@ __global__ __launch_bounds__(kSelThreads) void lse_combine_redo_kernel(CombinePa
   fallback_segment<DT>(g, p, seg, 0, nullptr, sh.hist, sh.off, sh.wtot, sh.res, sh.mm);
   __threadfence_block();
   __syncthreads();   // the list and its count, written by this workgroup, are read by it below
-  const int count = p.union_count[seg];
+  const int count = __hip_atomic_load(p.union_count + seg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   redo_attention<DT>(a, p.union_idx + (int64_t)seg * (p.k + p.sink + p.local), count, seg / g.num_kv_heads, seg % g.num_kv_heads,
                      c.out, c.out_stride_b, c.out_dtype, sh.acc, sh.ml);
 }

@@ -391,6 +391,34 @@ def set_test_hooks(force_segment_redo=0, tau_spin_limit=0, tau_withhold_mod=0, t
     L.check(L.lib().tka_set_test_hooks(C.byref(h)), "tka_set_test_hooks")
 
 
+class ReadProbe:
+    """A kernel that only reads a KV cache in the access pattern of the long-segment GEMV (`stream`) or of the gathered
+    attention (`gather`, over idx [B,H,L]): what the memory system gives to that pattern (tka_probe_read)."""
+
+    def __init__(self, keys, values=None, idx=None, threads=512, rounds=2, nontemporal=True, tokens_per_wg=256):
+        _need_cuda(keys)
+        B = keys.shape[0] if keys.dim() == 4 else 1
+        sb, sn, sh, N, H = _kv_strides(keys, B)
+        self.keep = (keys, values, idx)
+        self.sink = torch.zeros(1, dtype=torch.int32, device=keys.device)
+        a = L.ProbeArgs()
+        a.keys, a.sink = keys.data_ptr(), self.sink.data_ptr()
+        a.kind = L.TKA_PROBE_STREAM if idx is None else L.TKA_PROBE_GATHER
+        a.batch, a.num_kv_heads, a.seq_len = B, H, N
+        a.kv_stride_b, a.kv_stride_n, a.kv_stride_h = sb, sn, sh
+        a.threads, a.rounds, a.nontemporal, a.tokens_per_wg = threads, rounds, int(nontemporal), tokens_per_wg
+        if idx is not None:
+            if values is None or _kv_strides(values, B) != (sb, sn, sh, N, H) or idx.dtype != torch.int32 or not idx.is_contiguous():
+                raise ValueError("gather probe: values like keys, idx int32 [B,H,L] contiguous")
+            a.values, a.idx, a.idx_len = values.data_ptr(), idx.data_ptr(), idx.shape[-1]
+        self.args = a
+
+    def run(self):
+        self.args.stream = _stream()
+        L.check(L.lib().tka_probe_read(C.byref(self.args)), "tka_probe_read")
+        return self
+
+
 def profile_enable(on=True):
     L.lib().tka_profile_enable(int(on))
 
