@@ -112,6 +112,11 @@ class SparseDecode:
         self.desc = "%s: B=%d Hq=%d Hkv=%d D=128 N=%d %s k=%d sink=%d local=%d out=%s" % (
             name, B, H * G, H, N, dtype, k, sink, local, out_dtype)
         self.dominant = "gemv_scores"
+        self.hooks = {}            # testing hooks the workload runs under (kept when the worst case adds its own)
+        self.make_rank_plan = None
+        if want_union:             # the same step with the rank-ordered top-k output as well (a sort per KV head)
+            self.make_rank_plan = lambda: ops.SparseDecodePlan(self.q, self.K, self.V, k, sink, local, SCALE, G,
+                                                               out_dtype=getattr(torch, out_dtype), num_splits=num_splits, want_topk=True)
 
     def step(self):
         self.plan.step()
@@ -177,6 +182,7 @@ class GemvTopk:
         self.desc = "%s: B=%d Hkv=%d G=%d D=128 N=%d %s k=%d (GEMV + top-k only)%s" % (
             name, batch, hkv, group, seq_len, dtype, k, ", %d rotating key sets" % rotate if rotate > 1 else "")
         self.dominant = "gemv_scores"
+        self.hooks = {}
 
     def step(self):
         self.plans[self.turn % len(self.plans)].run()
@@ -338,7 +344,9 @@ def build_workload(name, torch, ops, dev, args):
         return SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-out", want_union=False)
     if name == "c4-one-launch":  # ... with selection and attention in one launch (the library takes that form from 256 segments on)
         ops.set_test_hooks(fused_tail=1)
-        return SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-one-launch", want_union=False)
+        w = SparseDecode(torch, ops, dev, num_splits=args.splits, name="c4-one-launch", want_union=False)
+        w.hooks = {"fused_tail": 1}
+        return w
     if name == "c4-small":
         return SparseDecode(torch, ops, dev, batch=2, seq_len=16384, name="c4-small")
     if name == "c4-b1-32k":     # one sequence of 32768 tokens on one GPU (all 8 KV heads), output only
@@ -486,12 +494,43 @@ def main():
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     traffic, traffic_source = recorded_traffic(args.workload, dominant) if not args.splits else (None, None)
 
+    def median_us(step, n):
+        """Median over n steps, each between its own pair of events (two untimed steps first)."""
+        step()
+        step()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for e0, e1 in ev:
+            e0.record()
+            step()
+            e1.record()
+        torch.cuda.synchronize()
+        return sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in ev)[n // 2]
+
+    # The step when EVERY segment is redone from its keys (the testing hook makes the selection refuse every candidate
+    # count): the bound on what a step can cost whatever the data does.
+    worst_us = worst_redone = None
+    if hasattr(w, "hooks") and hasattr(w, "redone_segments"):
+        ops.set_test_hooks(force_segment_redo=1, **w.hooks)
+        worst_us = median_us(w.step, min(args.steps, 10))
+        worst_redone = w.redone_segments()
+        ops.set_test_hooks(**w.hooks)
+        w.step()
+        torch.cuda.synchronize()
+        assert w.redone_segments() == 0 or redone, "segments still redone after the hook was cleared"
+    rank_us = None
+    if getattr(w, "make_rank_plan", None):
+        rank_plan = w.make_rank_plan()
+        rank_us = median_us(rank_plan.step, min(args.steps, 20))
+        del rank_plan
+
     out = {
         "metric": "us/decode-step + achieved HBM GB/s (% of peak), GEMV+top-k+sparse attn @128k",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "us_per_step": round(ms_per_step * 1e3, 2),
         "us_per_step_median": round(us_median, 2), "us_per_step_min": round(us_min, 2),
         "redone_segments": redone,
+        "worst_case_us_per_step": None if worst_us is None else round(worst_us, 2), "worst_case_redone_segments": worst_redone,
+        "us_per_step_with_rank_order": None if rank_us is None else round(rank_us, 2),
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (seeded torch generator on the GPU)",

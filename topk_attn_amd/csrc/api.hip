@@ -464,7 +464,14 @@ int run_gemv_topk(const tka_gemv_topk_args* a, int32_t* out_expand, int expand, 
   if (ft && !sc.out_idx && sc.union_idx && a->num_chunks == 1 && !cluster_ids && attn_select_fits(sc.parts, a->group) &&
       fused_tail_take(ft, gp, sc))
     return TKA_OK;
-  return launch_select_finalize_cand(gp, sc, a->dtype, stream);
+  // A segment that the selection cannot take from its candidates is flagged and redone by the launch behind it, whose
+  // workgroups share the work (they leave at once when no segment is flagged: 2 us per step).
+  // (Key rows more than half a megabyte apart, or more than 2048 segments: the selection launch redoes its flagged segment itself, as it does on the other routes.)
+  const bool shared_redo = redo_segments_fits(gp, sc.num_segments);
+  if (shared_redo) sc.redo_hist = sp.hist;
+  rc = launch_select_finalize_cand(gp, sc, a->dtype, stream);
+  if (rc != TKA_OK || !shared_redo) return rc;
+  return launch_redo_segments(gp, sc, a->dtype, stream);
 }
 
 int check_flash(const tka_flash_decode_args* a) {

@@ -80,6 +80,9 @@ struct SelectParams {
   uint32_t* sample_pool;  // [num_segments][kGemvMaxSamples] sampled keys (workspace)
   uint32_t* seg_flags;    // [num_segments] candidate mode: bit 0 = the segment was redone from the keys, bits 8.. = how many
                           // of its slices came from workgroups whose wait for the threshold had expired
+  uint32_t* redo_queue;   // candidate route: the chunk counter of launch_redo_segments
+  uint32_t* redo_hist;    // candidate route: [num_segments][kHistBins]; set = a flagged segment is left to launch_redo_segments
+  uint32_t* redo_arrive;  // [num_segments] chunks of a flagged segment that have been scored (cleared when the segment is flagged)
   int max_entries;        // candidate mode: a segment with more candidates than this is also redone from the keys
   int from_keys;          // candidate selection kernel: no slices, the workgroup scores its (short) segment itself
   int from_scores;        // candidate selection kernel: no slices, the entries are all scores of the segment (<= 16384)
@@ -120,6 +123,8 @@ int launch_select_filter(const SelectParams& p, hipStream_t stream);
 int launch_select_finalize(const SelectParams& p, hipStream_t stream);
 // Candidate slices -> outputs; a segment whose slices cannot be used is redone from the keys by its workgroup.
 int launch_select_finalize_cand(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
+bool redo_segments_fits(const GemvParams& g, int num_segments);   // chunks of key rows addressed with 32-bit offsets, flagged segments listed in LDS
+int launch_redo_segments(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream);
 int select_cand_max_parts();   // most candidate slices per segment
 // Common-cut route: ranks the candidates of a segment by counting and writes the top k in rank order (and the expansion);
 // p.list / p.list_stride / p.parts describe the slices written by launch_gemv_cut.

@@ -211,7 +211,10 @@ __device__ __forceinline__ void rank_sort_desc(uint64_t* sh_sort, uint64_t* sh_x
     sort_lds_desc(sh_sort, sh_xchg, kpad);
     return;
   }
-  const int tid = threadIdx.x;
+  int tid = threadIdx.x;
+  // (inlined into long kernels, some of them inside loops: the addresses below are computed here, from a thread number
+  // that the compiler cannot trace, instead of being kept in registers from the top of the kernel on)
+  asm volatile("" : "+v"(tid));
   const int lane = tid & 63, wave = tid >> 6;
   constexpr int kMaxPer = TKA_MAX_TOPK / kSelThreads;   // 8 composites per thread at most
   uint32_t* sh_big = (uint32_t*)(sh_mm + 2);
@@ -477,58 +480,80 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
 // ---- fallback of the candidate mode ---------------------------------------------------------------
 
 // A segment whose candidate slices cannot be used (fewer than k candidates, or more than fit) is redone from
-// the keys by its workgroup alone: scores in the canonical order (stored, and a histogram of the top key bits
-// kept in LDS), radix passes over the stored scores until the k-th largest key is fixed, then one walk in
-// index order that takes every key above the threshold bucket and the first `need` keys inside it.  Exact for
-// any data; slow (one CU streams the segment), which is acceptable for an event that the sampling makes rare.
+// the keys: scores in the canonical order (stored, and a histogram of the top key bits), radix passes over the stored
+// scores until the k-th largest key is fixed, then one walk in index order that takes every key above the threshold
+// bucket and the first `need` keys inside it.  Exact for any data.  Two forms: one workgroup does all of it for its
+// segment (fallback_segment: one CU streams the segment, about a millisecond per 131072 tokens; the short segments of
+// the common-cut route and the combine launch of the one-launch selection + attention), or the workgroups of a launch of
+// their own share the scoring of all flagged segments and the last of them to finish a segment selects from its scores
+// (redo_segments_kernel; the long segments of the candidate route).
+
+// Scores of tokens [t0, t1) of segment `seg` (all 1024 threads: 64 row groups of 16 lanes, 16 rows in flight each),
+// stored to the segment's place in g.scores, with the top key bits counted in sh_hist (LDS, 2048 bins; not cleared here).
+// kRows: rows in flight per lane (16 where one CU has to pull a whole segment; 8 where many workgroups share the work).
+template <int DT, int kRows = 16>
+__device__ __forceinline__ void fallback_score_range(const GemvParams& g, const SelectParams& p, int seg, int64_t t0, int64_t t1, uint32_t* sh_hist) {
+  const int tid = threadIdx.x;
+  float* sc = g.scores + (int64_t)seg * p.seg_stride;
+  const int j = tid & 15, rg = tid >> 4;
+  const int chunk = seg % g.num_chunks, bh = seg / g.num_chunks;
+  const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
+  const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
+  float qf[8];
+  load_group_query<DT>(g.q, g.q_stride_b, b, h, g.group, j, qf);
+  const uint16_t* kbase = (const uint16_t*)g.keys + (int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h +
+                          chunk_base * g.key_stride_n + 8 * j;
+  for (int64_t base = t0; base < t1; base += (kSelThreads / 16) * kRows) {
+    u32x4 kv[kRows];
+#pragma unroll
+    for (int u = 0; u < kRows; ++u) {
+      const int64_t t = base + rg * kRows + u;
+      kv[u] = *(const u32x4*)(kbase + (t < t1 ? t : t1 - 1) * g.key_stride_n);
+    }
+    __builtin_amdgcn_sched_barrier(0);   // all loads go out before the first score is computed
+    float mine = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kRows; ++u) {
+      const float s = row_score<DT>(qf, kv[u], g.scale);
+      if (j == u) mine = s;
+    }
+    const int64_t t = base + rg * kRows + j;
+    if (j < kRows && t < t1) {
+      sc[t] = mine;
+      atomicAdd(&sh_hist[score_key(mine) >> (32 - kHistBits)], 1u);
+    }
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void fallback_select_from_scores(const GemvParams& g, const SelectParams& p, int seg, int kpad, uint64_t* sh_sort,
+                                                            uint32_t* sh_hist, uint32_t* sh_off, uint32_t* sh_wtot, uint32_t* sh_res,
+                                                            uint64_t* sh_mm);
+
 // sh_sort: 2*kpad composites (rank mode only); sh_hist, sh_off: 2048 words each.  Every thread of the block must call it.
 template <int DT>
 __device__ __forceinline__ void fallback_segment(const GemvParams& g, const SelectParams& p, int seg, int kpad, uint64_t* sh_sort,
                                                  uint32_t* sh_hist, uint32_t* sh_off, uint32_t* sh_wtot, uint32_t* sh_res,
                                                  uint64_t* sh_mm) {
+  const int tid = threadIdx.x;
+  sh_hist[2 * tid] = 0;
+  sh_hist[2 * tid + 1] = 0;
+  __syncthreads();
+  fallback_score_range<DT>(g, p, seg, 0, p.seg_len, sh_hist);
+  __syncthreads();   // also orders this workgroup's score stores before its loads below
+  fallback_select_from_scores<DT>(g, p, seg, kpad, sh_sort, sh_hist, sh_off, sh_wtot, sh_res, sh_mm);
+}
+
+// The selection half: sh_hist holds the counts of the top key bits of the segment's stored scores.
+template <int DT>
+__device__ __forceinline__ void fallback_select_from_scores(const GemvParams& g, const SelectParams& p, int seg, int kpad, uint64_t* sh_sort,
+                                                            uint32_t* sh_hist, uint32_t* sh_off, uint32_t* sh_wtot, uint32_t* sh_res,
+                                                            uint64_t* sh_mm) {
   uint64_t* sh_xchg = sh_sort + kpad;
   const int tid = threadIdx.x;
   const uint32_t k = (uint32_t)p.k;
   const int64_t n = p.seg_len;
   float* sc = g.scores + (int64_t)seg * p.seg_stride;
-
-  sh_hist[2 * tid] = 0;
-  sh_hist[2 * tid + 1] = 0;
-  __syncthreads();
-
-  // scores of the whole segment: 64 row groups of 16 lanes, 8 rows in flight each
-  {
-    const int j = tid & 15, rg = tid >> 4;
-    const int chunk = seg % g.num_chunks, bh = seg / g.num_chunks;
-    const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
-    const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
-    float qf[8];
-    load_group_query<DT>(g.q, g.q_stride_b, b, h, g.group, j, qf);
-    const uint16_t* kbase = (const uint16_t*)g.keys + (int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h +
-                            chunk_base * g.key_stride_n + 8 * j;
-    constexpr int kRows = 16;   // rows in flight per lane: one CU has to pull the whole segment
-    for (int64_t base = 0; base < n; base += (kSelThreads / 16) * kRows) {
-      u32x4 kv[kRows];
-#pragma unroll
-      for (int u = 0; u < kRows; ++u) {
-        const int64_t t = base + rg * kRows + u;
-        kv[u] = *(const u32x4*)(kbase + (t < n ? t : n - 1) * g.key_stride_n);
-      }
-      __builtin_amdgcn_sched_barrier(0);   // all loads go out before the first score is computed
-      float mine = 0.0f;
-#pragma unroll
-      for (int u = 0; u < kRows; ++u) {
-        const float s = row_score<DT>(qf, kv[u], g.scale);
-        if (j == u) mine = s;
-      }
-      const int64_t t = base + rg * kRows + j;
-      if (j < kRows && t < n) {
-        sc[t] = mine;
-        atomicAdd(&sh_hist[score_key(mine) >> (32 - kHistBits)], 1u);
-      }
-    }
-  }
-  __syncthreads();   // also orders this workgroup's score stores before its loads below
 
   // radix passes: `prefix` = value of the top `fixed` key bits of the k-th largest key, `need` = how many
   // keys of that bucket belong to the top k
@@ -818,6 +843,16 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
     if (tid == 0) p.tau_words[2 * seg] = 0ull;
   }
   if (redo) {
+    if (p.redo_hist) {
+      // the launch behind this one redoes the segment (redo_segments_kernel): its histogram and arrival count start at zero
+      p.redo_hist[(int64_t)seg * kHistBins + 2 * tid] = 0u;
+      p.redo_hist[(int64_t)seg * kHistBins + 2 * tid + 1] = 0u;
+      if (tid == 0) {
+        p.redo_arrive[seg] = 0u;
+        *p.redo_queue = 0u;   // (the chunk counter of that launch: every flagged segment clears it)
+      }
+      return;
+    }
     __syncthreads();
     fallback_segment<DT>(g, p, seg, kpad, sh_ent, sh_hist, sh_pos, sh_wtot, sh_res, sh_mm);
     return;
@@ -962,6 +997,459 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
   __syncthreads();
   rank_sort_desc(sh_sort, sh_xchg, k, kpad, sh_hist, sh_pos, sh_wtot, sh_mm);   // (the slice positions are spent)
   write_rank_outputs(sh_sort, p, seg);
+}
+
+// ---- redo of flagged long segments, in a launch of its own --------------------------------------------------
+
+// Launched behind select_finalize_cand_kernel on the candidate route, one workgroup per CU.  Every workgroup reads the
+// segment flags; when none is set (all but always) it leaves at once.  Otherwise the flagged segments, in order, are cut
+// into chunks of kRedoChunk tokens and the workgroups draw chunk numbers from a counter in memory: scores stored, top key
+// bits counted in LDS and, when the workgroup's next chunk belongs to another segment, added to the segment's histogram in
+// memory.  Scores and counts go out as stores and adds performed at the point of coherence; the workgroup waits until its
+// own have completed and adds the number of its chunks to the segment's arrival count.  The workgroup that completes
+// the count selects from the stored scores (redo_select_from_scores) while the others go on scoring the next segments -
+// it draws no chunks meanwhile, so it does not fall behind and end up with every selection.  Nobody waits for anybody.
+// All 64 segments of 131072 tokens flagged: the step costs twice and a bit what it costs otherwise (the keys are read a
+// second time at the rate of the first), where one workgroup per segment took 14 times as long.
+constexpr int kRedoChunk = 4096;
+constexpr int kRedoMaxFlagged = 2048;   // segments of a call (the list of the flagged ones is kept in LDS)
+constexpr int kRedoBucketCap = 16384;   // composites of the threshold bucket held in LDS (128 KB) while the cut inside it is searched
+
+// U vectors of four stored keys per lane: vector u holds the keys of tokens base + u * stride + first .. + 3.  A block
+// that lies inside [.., end) whole is loaded without a branch per vector (all U loads are in flight together: a pass over
+// the stored keys is bound by their latency first); the last block of a range is guarded, key 0 and a clear bit in vm
+// for a token at or beyond `end`.
+template <int U>
+__device__ __forceinline__ void load_stored_keys(const uint32_t* sk, int64_t base, int first, int stride, int64_t end, bool vec_ok,
+                                                 uint32_t (&keys)[U][4], uint32_t (&vm)[U]) {
+  if (vec_ok && base + (int64_t)stride * U <= end) {   // (uniform)
+    u32x4 x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = *(const u32x4*)(sk + base + stride * u + first);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) keys[u][e] = x[u][e];
+      vm[u] = 0xfu;
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      vm[u] = 0u;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int64_t i = base + stride * u + first + e;
+        const bool ok = i < end;
+        keys[u][e] = ok ? sk[i] : 0u;
+        vm[u] |= (ok ? 1u : 0u) << e;
+      }
+    }
+  }
+}
+
+// How redo_wave_walk tells which of the ties (tokens whose top `fixed` key bits equal `prefix`) are selected.
+enum : int {
+  kTiesAll = 0,        // all of them
+  kTiesByComposite,    // those whose composite (key, ~index) is at least `cut`
+  kTiesByRank          // the first `need` of them in index order
+};
+
+// One walk of this wave over tokens [w0, w1) of the stored keys (w0 a multiple of 256; all 64 lanes).  The selected
+// tokens are those whose top `fixed` key bits exceed `prefix`, and of the ties those that `mode` says; run_tie = ties
+// in front of w0 (kTiesByRank).  Blocks of 256 tokens without a selected one (most, where k is small against the
+// segment) cost a compare per token and a few scalar instructions.
+//   WRITE = false: returns how many selected ties lie in [lo, hi) - for the one wave in whose range the cut among the
+//                  ties falls (kTiesByRank), whose count of them cannot be had from totals.
+//   WRITE = true:  writes the ids of the selected tokens in [lo, hi) to uo[run_mid ...] in index order, and (sort != 0)
+//                  the composites of all selected tokens to sort[run_sel ...].
+// U: vector loads in flight per lane.
+template <bool WRITE, int U>
+__device__ __forceinline__ uint32_t redo_wave_walk(const uint32_t* sk, bool vec_ok, int64_t w0, int64_t w1, uint32_t prefix, int fixed,
+                                                   int mode, uint64_t cut, uint32_t need, uint32_t lo, uint32_t hi, uint32_t run_tie,
+                                                   uint32_t run_mid, uint32_t run_sel, int32_t* uo, uint64_t* sort, uint32_t sort_cap) {
+  const int lane = threadIdx.x & 63;
+  const int shift = 32 - fixed;   // (0 .. 21)
+  uint32_t tie_mid_selected = 0;   // (uniform)
+  for (int64_t base = w0; base < w1; base += 256 * U) {
+    uint32_t keys[U][4], vm[U];
+    load_stored_keys<U>(sk, base, 4 * lane, 256, w1, vec_ok, keys, vm);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t first = (uint32_t)(base + 256 * u) + 4u * (uint32_t)lane;
+      uint32_t above = 0, tie = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t top = keys[u][e] >> shift;
+        const bool ok = vm[u] >> e & 1u;
+        above |= (ok && top > prefix ? 1u : 0u) << e;
+        tie |= (ok && top == prefix ? 1u : 0u) << e;
+      }
+      if (__ballot((above | tie) != 0u) == 0ull) continue;   // (uniform) nothing to select among these 256
+      uint32_t sel = above | tie;
+      if (mode == kTiesByComposite) {   // (uniform)
+        sel = above;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sel |= ((tie >> e & 1u) && composite(keys[u][e], first + e) >= cut ? 1u : 0u) << e;
+      } else if (mode == kTiesByRank) {
+        const uint32_t mine = (uint32_t)__builtin_popcount(tie);
+        const uint32_t inc = wave_inclusive_scan(mine);
+        uint32_t r = run_tie + inc - mine;
+        run_tie += (uint32_t)__builtin_amdgcn_readlane((int)inc, 63);
+        sel = above;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (tie >> e & 1u) {
+            sel |= (r < need ? 1u : 0u) << e;
+            ++r;
+          }
+      }
+      uint32_t mid = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) mid |= ((sel >> e & 1u) && first + e - lo < hi - lo ? 1u : 0u) << e;   // (lo <= hi)
+      if (!WRITE) {
+        tie_mid_selected += (uint32_t)__popcll(__ballot((mid & tie & 1u) != 0u)) + (uint32_t)__popcll(__ballot((mid & tie & 2u) != 0u)) +
+                            (uint32_t)__popcll(__ballot((mid & tie & 4u) != 0u)) + (uint32_t)__popcll(__ballot((mid & tie & 8u) != 0u));
+      } else {
+        const uint32_t packed = ((uint32_t)__builtin_popcount(sel) << 16) | (uint32_t)__builtin_popcount(mid);
+        const uint32_t inc = wave_inclusive_scan(packed);   // (at most 256 of either per wave and block)
+        const uint32_t ex = inc - packed;
+        uint32_t pos_sel = run_sel + (ex >> 16), pos_mid = run_mid + (ex & 0xffffu);
+        const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)inc, 63);
+        run_sel += tot >> 16;
+        run_mid += tot & 0xffffu;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (sort && (sel >> e & 1u)) {
+            if (pos_sel < sort_cap) sort[pos_sel] = composite(keys[u][e], first + e);
+            ++pos_sel;
+          }
+          if (uo && (mid >> e & 1u)) uo[pos_mid++] = (int32_t)(first + e);
+        }
+      }
+    }
+  }
+  return tie_mid_selected;
+}
+
+// Exact selection for segment `seg` from its stored keys (redo_segments_kernel stores the keys of the scores, not the
+// scores); sh_hist holds the counts of their top 11 bits.  Same result as fallback_select_from_scores, in two passes
+// over the keys and few barriers.  Every wave takes a contiguous sixteenth of the segment.  Pass one counts, per wave,
+// the tokens above the threshold bucket and its members (all, and those between the sink range and the local window),
+// and gathers the members' composites in LDS, where the cut inside the bucket is then searched (radix passes over the
+// composites: ties in the key fall to the smaller index, as everywhere); the waves' totals are summed once; pass two
+// writes every wave's part in index order.  A bucket with more members than the LDS holds is narrowed by counting
+// passes over the keys first; members that all carry one key (narrowing cannot help) are told apart by their rank
+// among themselves in pass two instead.  The counts are kept on the scalar side (a compare per token gives a lane mask,
+// its population is a scalar instruction): one CU has a million tokens to get through.
+// Every thread of the block must call it.  smem: max(kRedoBucketCap, 2 * kpad) composites.
+template <int DT, bool RANK>
+__device__ __forceinline__ void redo_select_from_scores(const GemvParams& g, const SelectParams& p, int seg, int kpad, unsigned char* smem,
+                                                        uint32_t* sh_hist, uint32_t* sh_off, uint32_t* sh_wtot, uint32_t* sh_res,
+                                                        uint64_t* sh_mm) {
+  uint64_t* sh_buck = (uint64_t*)smem;
+  uint64_t* sh_sort = (uint64_t*)smem;
+  uint64_t* sh_xchg = sh_sort + kpad;
+  int tid = threadIdx.x;
+  // (Called from inside the loop of a long kernel: what follows is computed here, each time, from a thread number that
+  // the compiler cannot trace - hoisted to the top of the kernel these values cost it more registers than it has.)
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63, wave = tid >> 6;
+  const uint32_t k = (uint32_t)p.k;
+  const int64_t n = p.seg_len;
+  const uint32_t* sk = (const uint32_t*)(g.scores + (int64_t)seg * p.seg_stride);
+  const bool vec_ok = (((uintptr_t)sk) & 15u) == 0;
+
+  // the k-th largest key: `prefix` = its top `fixed` bits, `need` = how many of the `cnt` keys with these bits belong
+  // to the top k
+  find_threshold_bin_1024(sh_hist, k, sh_wtot, sh_res);
+  uint32_t prefix = sh_res[0], need = k - sh_res[1], cnt = sh_res[2];
+  int fixed = kHistBits;
+  while (cnt != need && cnt > (uint32_t)kRedoBucketCap && fixed < 32) {   // (rare) narrow the bucket: count its members' next bits
+    const int bits = (32 - fixed) >= kHistBits ? kHistBits : (32 - fixed);
+    const int shift = 32 - fixed - bits;
+    __syncthreads();
+    sh_hist[2 * tid] = 0;
+    sh_hist[2 * tid + 1] = 0;
+    __syncthreads();
+    constexpr int U = 4;
+    for (int64_t base = 0; base < n; base += 4 * kSelThreads * U) {
+      uint32_t keys[U][4], vm[U];
+      load_stored_keys<U>(sk, base, 4 * tid, 4 * kSelThreads, n, vec_ok, keys, vm);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if ((vm[u] >> e & 1u) && (keys[u][e] >> (32 - fixed)) == prefix) atomicAdd(&sh_hist[(keys[u][e] >> shift) & ((1u << bits) - 1u)], 1u);
+    }
+    __syncthreads();
+    find_threshold_bin_1024(sh_hist, need, sh_wtot, sh_res);
+    need -= sh_res[1];
+    prefix = (prefix << bits) | sh_res[0];
+    cnt = sh_res[2];
+    fixed += bits;
+  }
+  const bool gather = cnt != need && cnt <= (uint32_t)kRedoBucketCap;
+  const int mode = cnt == need ? kTiesAll : (gather ? kTiesByComposite : kTiesByRank);
+
+  constexpr bool want_rank = RANK;   // (p.out_idx set)
+  const bool want_union = p.union_idx != nullptr;
+  const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
+  const uint32_t hi = (uint32_t)(n - p.local > lo ? n - p.local : lo);
+  int32_t* uo = want_union ? p.union_idx + (int64_t)seg * (p.k + p.sink + p.local) : nullptr;
+
+  // this wave's sixteenth (a multiple of 256 tokens: the vector loads stay aligned)
+  const int64_t per_wave = (n + 256 * kSelWaves - 1) / (256 * kSelWaves) * 256;
+  const int64_t w0 = (int64_t)wave * per_wave < n ? (int64_t)wave * per_wave : n;
+  const int64_t w1 = w0 + per_wave < n ? w0 + per_wave : n;
+
+  // pass one
+  if (tid == 0) sh_res[3] = 0u;   // members gathered so far
+  if (tid < 6 * kSelWaves + 1) sh_off[tid] = 0u;   // per wave: above, above in [lo, hi), ties, ties in [lo, hi), selected ties, selected ties in [lo, hi); then one word for the wave with the cut
+  __syncthreads();
+  uint32_t c_above = 0, c_above_mid = 0, c_tie = 0, c_tie_mid = 0;   // (uniform: totals of the wave)
+  {
+    const int shift = 32 - fixed;
+    constexpr int U = 4;   // (what the registers allow)
+    for (int64_t base = w0; base < w1; base += 256 * U) {
+      uint32_t keys[U][4], vm[U];
+      load_stored_keys<U>(sk, base, 4 * lane, 256, w1, vec_ok, keys, vm);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t block = (uint32_t)(base + 256 * u);
+        // the block against [lo, hi): inside whole (nearly always), outside whole, or cut by an end of it
+        const bool all_mid = block >= lo && block + 256u <= hi, some_mid = block < hi && block + 256u > lo;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t top = keys[u][e] >> shift;
+          const bool ok = vm[u] >> e & 1u;
+          const bool above = ok && top > prefix, tie = ok && top == prefix;
+          const unsigned long long ma = __ballot(above), mt = __ballot(tie);
+          c_above += (uint32_t)__popcll(ma);
+          c_tie += (uint32_t)__popcll(mt);
+          if (all_mid) {
+            c_above_mid += (uint32_t)__popcll(ma);
+            c_tie_mid += (uint32_t)__popcll(mt);
+          } else if (some_mid) {
+            const bool in_mid = block + 4u * (uint32_t)lane + e - lo < hi - lo;
+            c_above_mid += (uint32_t)__popcll(__ballot(above && in_mid));
+            c_tie_mid += (uint32_t)__popcll(__ballot(tie && in_mid));
+          }
+          if (gather && mt != 0ull) {   // (uniform) one reservation per wave
+            uint32_t first = 0;
+            if (lane == 0) first = atomicAdd(&sh_res[3], (uint32_t)__popcll(mt));
+            first = (uint32_t)__builtin_amdgcn_readfirstlane((int)first);
+            if (tie) sh_buck[first + (uint32_t)__popcll(mt & ((1ull << lane) - 1ull))] = composite(keys[u][e], block + 4u * (uint32_t)lane + e);
+          }
+        }
+      }
+    }
+  }
+  if (lane == 0) {
+    sh_off[6 * wave] = c_above;
+    sh_off[6 * wave + 1] = c_above_mid;
+    sh_off[6 * wave + 2] = c_tie;
+    sh_off[6 * wave + 3] = c_tie_mid;
+  }
+  __syncthreads();
+
+  // the cut inside the bucket: the need-th largest of the gathered composites
+  uint64_t cut = 0;
+  if (gather) {
+    uint64_t cprefix = prefix;   // top `cfixed` bits of the composite
+    int cfixed = fixed;
+    uint32_t left = need, among = cnt;
+    while (among != left && cfixed < 64) {
+      const int bits = (64 - cfixed) >= kHistBits ? kHistBits : (64 - cfixed);
+      const int shift = 64 - cfixed - bits;
+      sh_hist[2 * tid] = 0;
+      sh_hist[2 * tid + 1] = 0;
+      __syncthreads();
+      for (uint32_t i = tid; i < cnt; i += kSelThreads) {
+        const uint64_t c = sh_buck[i];
+        if ((c >> (64 - cfixed)) == cprefix) atomicAdd(&sh_hist[(uint32_t)(c >> shift) & ((1u << bits) - 1u)], 1u);
+      }
+      __syncthreads();
+      find_threshold_bin_1024(sh_hist, left, sh_wtot, sh_res);
+      left -= sh_res[1];
+      cprefix = (cprefix << bits) | sh_res[0];
+      among = sh_res[2];
+      cfixed += bits;
+    }
+    cut = cfixed == 64 ? cprefix : cprefix << (64 - cfixed);   // every composite with these leading bits is taken
+    // the selected members of every wave's range
+    for (uint32_t i = tid; i < cnt; i += kSelThreads) {
+      const uint64_t c = sh_buck[i];
+      if (c >= cut) {
+        const uint32_t idx = ~(uint32_t)c;
+        const uint32_t w = idx / (uint32_t)per_wave;
+        atomicAdd(&sh_off[6 * w + 4], 1u);
+        if (idx - lo < hi - lo) atomicAdd(&sh_off[6 * w + 5], 1u);
+      }
+    }
+    __syncthreads();
+  }
+  if (want_rank) {
+    for (int i = tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite (the bucket is spent)
+  }
+  // kTiesByRank: the wave in whose range the cut among the ties falls (at most one) counts its selected ties in [lo, hi) itself
+  uint32_t tie_before = 0;
+  for (int v = 0; v < wave; ++v) tie_before += sh_off[6 * v + 2];
+  if (mode == kTiesByRank) {
+    const uint32_t my_ties = sh_off[6 * wave + 2];
+    if (tie_before < need && tie_before + my_ties > need) {
+      const uint32_t c = redo_wave_walk<false, 2>(sk, vec_ok, w0, w1, prefix, fixed, mode, 0ull, need, lo, hi, tie_before, 0u, 0u, nullptr,
+                                                  nullptr, 0u);
+      if (lane == 0) sh_off[6 * kSelWaves] = c;
+    }
+  }
+  __syncthreads();
+  uint32_t mid_before = 0, sel_before = 0, mid_total = 0, run = 0;
+  for (int v = 0; v < kSelWaves; ++v) {
+    const uint32_t ties = sh_off[6 * v + 2];
+    uint32_t taken, taken_mid;
+    if (mode == kTiesAll) {
+      taken = ties;
+      taken_mid = sh_off[6 * v + 3];
+    } else if (mode == kTiesByComposite) {
+      taken = sh_off[6 * v + 4];
+      taken_mid = sh_off[6 * v + 5];
+    } else {
+      taken = run >= need ? 0u : (need - run < ties ? need - run : ties);
+      taken_mid = taken == ties ? sh_off[6 * v + 3] : (taken == 0u ? 0u : sh_off[6 * kSelWaves]);
+    }
+    run += ties;
+    const uint32_t m = sh_off[6 * v + 1] + taken_mid, s = sh_off[6 * v] + taken;
+    if (v < wave) {
+      mid_before += m;
+      sel_before += s;
+    }
+    mid_total += m;
+  }
+  // pass two
+  redo_wave_walk<true, RANK ? 2 : 4>(sk, vec_ok, w0, w1, prefix, fixed, mode, cut, need, lo, hi, tie_before, lo + mid_before, sel_before, uo,
+                                     want_rank ? sh_sort : nullptr, (uint32_t)kpad);
+  if (want_union) write_union_edges(uo, p, seg, lo, hi, mid_total);
+  if (!want_rank) return;
+  __syncthreads();
+  rank_sort_desc(sh_sort, sh_xchg, k, kpad, sh_hist, sh_off, sh_wtot, sh_mm);
+  write_rank_outputs(sh_sort, p, seg);
+}
+
+template <int DT, bool RANK>
+__global__ __launch_bounds__(kSelThreads) void redo_segments_kernel(GemvParams g, SelectParams p, int kpad) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // the bucket's composites, then (rank mode) 2 * kpad composites
+  __shared__ uint32_t sh_hist[kHistBins], sh_off[kHistBins];
+  __shared__ uint32_t sh_wtot[kSelWaves], sh_res[4];
+  __shared__ uint64_t sh_mm[3];
+  __shared__ uint16_t sh_flagged[kRedoMaxFlagged];
+  __shared__ uint32_t sh_item, sh_last;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  // the flagged segments, in order (every workgroup builds the same list)
+  uint32_t n_flagged = 0;
+  for (int s0 = 0; s0 < p.num_segments; s0 += kSelThreads) {
+    const int s = s0 + tid;
+    const bool flagged = s < p.num_segments && (p.seg_flags[s] & 1u) != 0u;
+    const unsigned long long m = __ballot(flagged);
+    if (lane == 0) sh_wtot[wave] = (uint32_t)__popcll(m);
+    __syncthreads();
+    uint32_t before = n_flagged, all = 0;
+    for (int w = 0; w < kSelWaves; ++w) {
+      const uint32_t c = sh_wtot[w];
+      before += w < wave ? c : 0u;
+      all += c;
+    }
+    if (flagged) sh_flagged[before + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = (uint16_t)s;
+    n_flagged += all;
+    __syncthreads();
+  }
+  if (n_flagged == 0u) return;   // the ordinary case
+
+  const uint32_t chunks_per_seg = (uint32_t)((p.seg_len + kRedoChunk - 1) / kRedoChunk);
+  const uint32_t n_items = n_flagged * chunks_per_seg;
+  int cur = -1;        // segment of the chunks counted in sh_hist
+  uint32_t done = 0;   // how many of them
+  while (true) {
+    if (tid == 0) sh_item = __hip_atomic_fetch_add(p.redo_queue, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const uint32_t item = sh_item;
+    const int seg = item < n_items ? (int)sh_flagged[item / chunks_per_seg] : -1;
+    if (seg != cur) {
+      if (cur >= 0) {
+        uint32_t* gh = p.redo_hist + (int64_t)cur * kHistBins;
+        for (int i = tid; i < kHistBins; i += kSelThreads)
+          if (sh_hist[i]) __hip_atomic_fetch_add(gh + i, sh_hist[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // Scores and counts were performed at the point of coherence; the arrival below must not overtake them: every
+        // wave waits until its own have completed (no write-back of the L2, which a release fence would ask for).
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+          const uint32_t old = __hip_atomic_fetch_add(p.redo_arrive + cur, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          sh_last = old + done == chunks_per_seg ? 1u : 0u;
+        }
+        __syncthreads();
+        if (sh_last != 0u) {   // (uniform over the workgroup)
+          // the other workgroups' scores, announced by their arrivals, are read from here on: drop what the caches hold
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+          sh_hist[2 * tid] = __hip_atomic_load(gh + 2 * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          sh_hist[2 * tid + 1] = __hip_atomic_load(gh + 2 * tid + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __syncthreads();
+          redo_select_from_scores<DT, RANK>(g, p, cur, kpad, smem, sh_hist, sh_off, sh_wtot, sh_res, sh_mm);
+        }
+      }
+      if (seg >= 0) {
+        __syncthreads();
+        sh_hist[2 * tid] = 0;
+        sh_hist[2 * tid + 1] = 0;
+      }
+      cur = seg;
+      done = 0;
+    }
+    if (seg < 0) break;   // no chunk left (a workgroup that never drew one leaves here as well)
+    __syncthreads();      // (sh_item is drawn again; the histogram is cleared)
+    {
+      // (as the streaming GEMV does it: a uniform base per chunk and one 32-bit lane offset serve all loads - the launcher
+      // has checked that a chunk's rows lie within 2 GB of its first)
+      const uint32_t c = item % chunks_per_seg;
+      const int j = tid & 15, rg = tid >> 4;
+      const int bh = seg / g.num_chunks, chunk = seg % g.num_chunks;
+      const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
+      const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
+      float qf[8];
+      load_group_query<DT, 1>(g.q, g.q_stride_b, b, h, g.group, j, qf);
+      const uint32_t row_bytes = (uint32_t)g.key_stride_n * 2u;
+      const int64_t t0 = (int64_t)c * kRedoChunk;
+      const unsigned char* cbase = (const unsigned char*)g.keys +
+                                   2 * ((int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h + (chunk_base + t0) * g.key_stride_n);   // uniform
+      uint32_t* sk = (uint32_t*)(g.scores + (int64_t)seg * p.seg_stride + t0);   // (keys, not scores: what the selection compares)
+      const int n_local = (int)(p.seg_len - t0 < kRedoChunk ? p.seg_len - t0 : kRedoChunk);
+      constexpr int kRows = 8;
+      for (int base = 0; base < n_local; base += (kSelThreads / 16) * kRows) {
+        u32x4 kv[kRows];
+#pragma unroll
+        for (int u = 0; u < kRows; ++u) {
+          int lt = base + rg * kRows + u;
+          lt = lt < n_local ? lt : n_local - 1;
+          kv[u] = __builtin_nontemporal_load((const u32x4*)(cbase + ((uint32_t)lt * row_bytes + 16u * (uint32_t)j)));
+        }
+        __builtin_amdgcn_sched_barrier(0);   // all loads go out before the first score is computed
+        float mine = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kRows; ++u) {
+          const float s = row_score<DT>(qf, kv[u], g.scale);
+          if (j == u) mine = s;
+        }
+        const int lt = base + rg * kRows + j;
+        if (j < kRows && lt < n_local) {
+          const uint32_t key = score_key(mine);
+          __hip_atomic_store(sk + lt, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          atomicAdd(&sh_hist[key >> (32 - kHistBits)], 1u);
+        }
+      }
+      ++done;
+    }
+    __syncthreads();   // (every wave has counted its scores before the histogram may be flushed)
+  }
 }
 
 // ---- combine launch of the fused selection + attention, with the redo of flagged segments ----------------
@@ -1740,7 +2228,7 @@ int kpad_for(int k) {
 //   list [S][slices*slice_len] u64      (slices: dense 4096/16384 scores, candidate mode one per GEMV workgroup)
 namespace {
 struct SelectLayout {
-  size_t hist, flags, tau, ctr, pool, head, list_cnt, list, total;
+  size_t hist, flags, tau, ctr, pool, head, list_cnt, list, arrive, total;
   int64_t list_stride;
 };
 SelectLayout select_layout(int num_segments, int64_t seg_len) {
@@ -1764,6 +2252,7 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   l.head = take(head_cand > head_cut ? head_cand : head_cut);
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
+  l.arrive = take((cand_segs + 1) * sizeof(uint32_t));   // arrival counts of the redo launch and its chunk counter (cleared by the selection when it flags a segment)
   l.total = off;
   return l;
 }
@@ -1784,6 +2273,8 @@ size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p
   p->list_cnt = (uint32_t*)(c + l.list_cnt);
   p->list = (uint64_t*)(c + l.list);
   p->list_stride = l.list_stride;
+  p->redo_arrive = (uint32_t*)(c + l.arrive);
+  p->redo_queue = p->redo_arrive + num_segments;   // (redo_hist: the histograms, on the route that does not use them otherwise; set by the caller)
   return (size_t)num_segments * kHistBins;  // the flags follow the histograms; candidate mode writes them itself
 }
 
@@ -1906,6 +2397,39 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
   if (p.segs_per_row < 1 || p.num_segments % p.segs_per_row || p.num_segments > (1 << 24)) return TKA_EINVAL;
   const dim3 wgs((unsigned)((p.num_segments + 7) / 8 * 8 * kCutParts));   // (see the kernel)
   hipLaunchKernelGGL(kernel, wgs, dim3(kSelThreads), lds, stream, g, p, kpad_for(p.k));
+  return hip_status(hipGetLastError());
+}
+
+// Behind launch_select_finalize_cand on the candidate route (p.redo_hist / p.redo_arrive set there too): redoes the segments
+// that the selection flagged, all workgroups of the launch sharing the work; leaves at once when there is none.
+bool redo_segments_fits(const GemvParams& g, int num_segments) {
+  return g.key_stride_n * 2 * (int64_t)kRedoChunk <= 0x7fffffffLL && num_segments <= kRedoMaxFlagged;
+}
+
+int launch_redo_segments(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
+  if (!p.redo_hist || !p.redo_arrive || !p.redo_queue || !p.seg_flags || !g.scores || !redo_segments_fits(g, p.num_segments))
+    return TKA_EINVAL;
+  const bool want_rank = p.out_idx != nullptr;
+  const int kpad = kpad_for(p.k);
+  const size_t bucket = (size_t)kRedoBucketCap * sizeof(uint64_t), sort = want_rank ? 2 * (size_t)kpad * sizeof(uint64_t) : 0;
+  const size_t lds = bucket > sort ? bucket : sort;
+  const int lds_max = 2 * kpad_for(TKA_MAX_TOPK) * (int)sizeof(uint64_t) > (int)bucket ? 2 * kpad_for(TKA_MAX_TOPK) * (int)sizeof(uint64_t) : (int)bucket;
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+    return n;
+  }();
+  const void* fn = dtype == TKA_F16 ? (want_rank ? (const void*)redo_segments_kernel<TKA_F16, true> : (const void*)redo_segments_kernel<TKA_F16, false>)
+                                    : (want_rank ? (const void*)redo_segments_kernel<TKA_BF16, true> : (const void*)redo_segments_kernel<TKA_BF16, false>);
+  if (allow_dynamic_lds(fn, lds_max) != TKA_OK) return TKA_EHIP;
+  LaunchTimer timer("redo_segments", stream);
+#define TKA_LAUNCH_REDO(DT, RANK) redo_segments_kernel<DT, RANK><<<(unsigned)cus, kSelThreads, lds, stream>>>(g, p, kpad)
+  if (dtype == TKA_F16) {
+    if (want_rank) TKA_LAUNCH_REDO(TKA_F16, true); else TKA_LAUNCH_REDO(TKA_F16, false);
+  } else {
+    if (want_rank) TKA_LAUNCH_REDO(TKA_BF16, true); else TKA_LAUNCH_REDO(TKA_BF16, false);
+  }
+#undef TKA_LAUNCH_REDO
   return hip_status(hipGetLastError());
 }
 
