@@ -80,9 +80,10 @@ struct SelectParams {
   uint32_t* sample_pool;  // [num_segments][kGemvMaxSamples] sampled keys (workspace)
   uint32_t* seg_flags;    // [num_segments] candidate mode: bit 0 = the segment was redone from the keys, bits 8.. = how many
                           // of its slices came from workgroups whose wait for the threshold had expired
-  uint32_t* redo_queue;   // candidate route: the chunk counter of launch_redo_segments
+  uint32_t* redo_queue;   // candidate route: the item counters of launch_redo_segments (drawn, done per phase)
+  uint32_t* redo_rec;     // ... its record per segment: 16 words, then four per chunk of 4096 tokens
+  int64_t redo_rec_stride;
   uint32_t* redo_hist;    // candidate route: [num_segments][kHistBins]; set = a flagged segment is left to launch_redo_segments
-  uint32_t* redo_arrive;  // [num_segments] chunks of a flagged segment that have been scored (cleared when the segment is flagged)
   int max_entries;        // candidate mode: a segment with more candidates than this is also redone from the keys
   int from_keys;          // candidate selection kernel: no slices, the workgroup scores its (short) segment itself
   int from_scores;        // candidate selection kernel: no slices, the entries are all scores of the segment (<= 16384)

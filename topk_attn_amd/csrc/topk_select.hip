@@ -161,7 +161,8 @@ __global__ __launch_bounds__(kSelThreads) void select_filter_kernel(SelectParams
 // Union list of one segment outside the selected middle part: the sink ids, the local window behind
 // `mid` selected ids, -1 padding, and the count.
 __device__ __forceinline__ void write_union_edges(int32_t* uo, const SelectParams& p, int seg, uint32_t lo, uint32_t hi, uint32_t mid) {
-  const int tid = threadIdx.x;
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));   // (inlined into long kernels, inside their loops: addresses are computed here, not kept from the top of the kernel on)
   const int64_t n = p.seg_len;
   const int cap = p.k + p.sink + p.local;
   for (uint32_t t = tid; t < lo; t += kSelThreads) uo[t] = (int32_t)t;
@@ -175,7 +176,8 @@ __device__ __forceinline__ void write_union_edges(int32_t* uo, const SelectParam
 // Rank-ordered outputs of one segment from the sorted composites in sh_sort[0 .. k).
 // (`chunk`: the segment's number inside its row, for a caller that has it without a division; -1: seg % p.segs_per_row)
 __device__ __forceinline__ void write_rank_outputs(const uint64_t* sh_sort, const SelectParams& p, int seg, int chunk = -1) {
-  const int tid = threadIdx.x;
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));   // (as in write_union_edges)
   const uint32_t k = (uint32_t)p.k;
   const uint32_t idx_base = p.seg_base_ids ? (uint32_t)(p.seg_base_ids[seg] * p.seg_len)
                                            : (uint32_t)((chunk >= 0 ? chunk : seg % p.segs_per_row) * p.seg_len);
@@ -640,6 +642,7 @@ __device__ __forceinline__ void fallback_select_from_scores(const GemvParams& g,
 
 // ---- finalize of the candidate mode -------------------------------------------------------------
 
+constexpr int kRedoPhasesMax = 8;   // item counters of the redo launch: two words per phase
 constexpr int kCandCap = 16384;    // candidates of one segment held in LDS (128 KB of composites)
 constexpr int kCandPerThread = kCandCap / kSelThreads;
 constexpr int kCandMaxParts = 4096;
@@ -847,10 +850,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
       // the launch behind this one redoes the segment (redo_segments_kernel): its histogram and arrival count start at zero
       p.redo_hist[(int64_t)seg * kHistBins + 2 * tid] = 0u;
       p.redo_hist[(int64_t)seg * kHistBins + 2 * tid + 1] = 0u;
-      if (tid == 0) {
-        p.redo_arrive[seg] = 0u;
-        *p.redo_queue = 0u;   // (the chunk counter of that launch: every flagged segment clears it)
-      }
+      if (tid < 2 * kRedoPhasesMax) p.redo_queue[tid] = 0u;   // (the item counters of that launch: every flagged segment clears them)
       return;
     }
     __syncthreads();
@@ -1001,16 +1001,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
 
 // ---- redo of flagged long segments, in a launch of its own --------------------------------------------------
 
-// Launched behind select_finalize_cand_kernel on the candidate route, one workgroup per CU.  Every workgroup reads the
-// segment flags; when none is set (all but always) it leaves at once.  Otherwise the flagged segments, in order, are cut
-// into chunks of kRedoChunk tokens and the workgroups draw chunk numbers from a counter in memory: scores stored, top key
-// bits counted in LDS and, when the workgroup's next chunk belongs to another segment, added to the segment's histogram in
-// memory.  Scores and counts go out as stores and adds performed at the point of coherence; the workgroup waits until its
-// own have completed and adds the number of its chunks to the segment's arrival count.  The workgroup that completes
-// the count selects from the stored scores (redo_select_from_scores) while the others go on scoring the next segments -
-// it draws no chunks meanwhile, so it does not fall behind and end up with every selection.  Nobody waits for anybody.
-// All 64 segments of 131072 tokens flagged: the step costs twice and a bit what it costs otherwise (the keys are read a
-// second time at the rate of the first), where one workgroup per segment took 14 times as long.
+// (redo_segments_kernel, below, says how the work is shared.)
 constexpr int kRedoChunk = 4096;
 constexpr int kRedoMaxFlagged = 2048;   // segments of a call (the list of the flagged ones is kept in LDS)
 constexpr int kRedoBucketCap = 16384;   // composites of the threshold bucket held in LDS (128 KB) while the cut inside it is searched
@@ -1061,13 +1052,14 @@ enum : int {
 //   WRITE = false: returns how many selected ties lie in [lo, hi) - for the one wave in whose range the cut among the
 //                  ties falls (kTiesByRank), whose count of them cannot be had from totals.
 //   WRITE = true:  writes the ids of the selected tokens in [lo, hi) to uo[run_mid ...] in index order, and (sort != 0)
-//                  the composites of all selected tokens to sort[run_sel ...].
+//                  the composites of all selected tokens to sort[run_sel ...] (memory that another workgroup reads).
 // U: vector loads in flight per lane.
 template <bool WRITE, int U>
 __device__ __forceinline__ uint32_t redo_wave_walk(const uint32_t* sk, bool vec_ok, int64_t w0, int64_t w1, uint32_t prefix, int fixed,
                                                    int mode, uint64_t cut, uint32_t need, uint32_t lo, uint32_t hi, uint32_t run_tie,
                                                    uint32_t run_mid, uint32_t run_sel, int32_t* uo, uint64_t* sort, uint32_t sort_cap) {
-  const int lane = threadIdx.x & 63;
+  int lane = threadIdx.x & 63;
+  asm volatile("" : "+v"(lane));   // (addresses computed here, at every call: see redo_segments_kernel)
   const int shift = 32 - fixed;   // (0 .. 21)
   uint32_t tie_mid_selected = 0;   // (uniform)
   for (int64_t base = w0; base < w1; base += 256 * U) {
@@ -1120,7 +1112,7 @@ __device__ __forceinline__ uint32_t redo_wave_walk(const uint32_t* sk, bool vec_
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           if (sort && (sel >> e & 1u)) {
-            if (pos_sel < sort_cap) sort[pos_sel] = composite(keys[u][e], first + e);
+            if (pos_sel < sort_cap) __hip_atomic_store(sort + pos_sel, composite(keys[u][e], first + e), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             ++pos_sel;
           }
           if (uo && (mid >> e & 1u)) uo[pos_mid++] = (int32_t)(first + e);
@@ -1139,16 +1131,16 @@ __device__ __forceinline__ uint32_t redo_wave_walk(const uint32_t* sk, bool vec_
 // composites: ties in the key fall to the smaller index, as everywhere); the waves' totals are summed once; pass two
 // writes every wave's part in index order.  A bucket with more members than the LDS holds is narrowed by counting
 // passes over the keys first; members that all carry one key (narrowing cannot help) are told apart by their rank
-// among themselves in pass two instead.  The counts are kept on the scalar side (a compare per token gives a lane mask,
+// among themselves in pass two instead.  Writes the ids of the selected tokens between the sink range and the local
+// window to their place in the union list and returns how many they are (the ends of the list are the caller's), and
+// (RANK) the composites of all selected tokens to `selection`, in memory, in index order.  The counts are kept on the scalar side (a compare per token gives a lane mask,
 // its population is a scalar instruction): one CU has a million tokens to get through.
-// Every thread of the block must call it.  smem: max(kRedoBucketCap, 2 * kpad) composites.
+// Every thread of the block must call it.  smem: kRedoBucketCap composites.
 template <int DT, bool RANK>
-__device__ __forceinline__ void redo_select_from_scores(const GemvParams& g, const SelectParams& p, int seg, int kpad, unsigned char* smem,
-                                                        uint32_t* sh_hist, uint32_t* sh_off, uint32_t* sh_wtot, uint32_t* sh_res,
-                                                        uint64_t* sh_mm) {
+__device__ __forceinline__ uint32_t redo_select_from_scores(const GemvParams& g, const SelectParams& p, int seg, uint64_t* selection,
+                                                            unsigned char* smem, uint32_t* sh_hist, uint32_t* sh_off, uint32_t* sh_wtot,
+                                                            uint32_t* sh_res) {
   uint64_t* sh_buck = (uint64_t*)smem;
-  uint64_t* sh_sort = (uint64_t*)smem;
-  uint64_t* sh_xchg = sh_sort + kpad;
   int tid = threadIdx.x;
   // (Called from inside the loop of a long kernel: what follows is computed here, each time, from a thread number that
   // the compiler cannot trace - hoisted to the top of the kernel these values cost it more registers than it has.)
@@ -1288,9 +1280,6 @@ __device__ __forceinline__ void redo_select_from_scores(const GemvParams& g, con
     }
     __syncthreads();
   }
-  if (want_rank) {
-    for (int i = tid; i < kpad; i += kSelThreads) sh_sort[i] = 0;  // pad: below every real composite (the bucket is spent)
-  }
   // kTiesByRank: the wave in whose range the cut among the ties falls (at most one) counts its selected ties in [lo, hi) itself
   uint32_t tie_before = 0;
   for (int v = 0; v < wave; ++v) tie_before += sh_off[6 * v + 2];
@@ -1326,15 +1315,103 @@ __device__ __forceinline__ void redo_select_from_scores(const GemvParams& g, con
     mid_total += m;
   }
   // pass two
-  redo_wave_walk<true, RANK ? 2 : 4>(sk, vec_ok, w0, w1, prefix, fixed, mode, cut, need, lo, hi, tie_before, lo + mid_before, sel_before, uo,
-                                     want_rank ? sh_sort : nullptr, (uint32_t)kpad);
-  if (want_union) write_union_edges(uo, p, seg, lo, hi, mid_total);
-  if (!want_rank) return;
-  __syncthreads();
-  rank_sort_desc(sh_sort, sh_xchg, k, kpad, sh_hist, sh_off, sh_wtot, sh_mm);
-  write_rank_outputs(sh_sort, p, seg);
+  redo_wave_walk<true, 4>(sk, vec_ok, w0, w1, prefix, fixed, mode, cut, need, lo, hi, tie_before, lo + mid_before, sel_before, uo,
+                          want_rank ? selection : nullptr, k);
+  return mid_total;
 }
 
+// The phases of redo_segments_kernel and the words of a segment's record in memory.
+enum : int {
+  kRedoScore = 0,   // per chunk of 4096 tokens: keys of the scores stored, top key bits counted
+  kRedoCount,       // per batch of 32768 tokens: tokens above the threshold bucket counted, the bucket's members gathered
+  kRedoCut,         // per segment: the cut inside the bucket, every batch's place in the outputs
+  kRedoWrite,       // per batch: the selected tokens written
+  kRedoFinish,      // per segment, rank-ordered output only: the rank order
+  kRedoPhases
+};
+enum : int { kRecPrefix = 0, kRecMode, kRecCutLo, kRecCutHi, kRecMidTotal, kRecWords = 16 };   // (the first four: one 16-byte load)
+enum : int {
+  kRedoTakeBucket = 0,   // the whole bucket belongs to the top k
+  kRedoCutBucket,        // the bucket's members are gathered and the cut among them searched
+  kRedoAlone             // (a bucket beyond the LDS, a segment of more than 2048 batches) one workgroup selects: redo_select_from_scores
+};
+constexpr int kRedoBatch = 32 * kSelThreads;   // tokens of a batch: 32 consecutive ones per thread
+constexpr int kRedoMaxBatches = kHistBins;     // batches of a segment whose counts one workgroup sums in LDS
+constexpr int kRedoWaitSpins = 1 << 22;        // about a second
+
+// The bucket of the k-th largest key from the segment's histogram in memory (all 1024 threads; sh_hist is overwritten):
+// *prefix = its 11 bits, *need = how many of its *cnt members belong to the top k; returns how the segment goes on.
+__device__ __forceinline__ int redo_threshold(const uint32_t* gh, uint32_t k, uint32_t batches_per_seg, uint32_t* sh_hist, uint32_t* sh_wtot,
+                                              uint32_t* sh_res, uint32_t* prefix, uint32_t* need, uint32_t* cnt) {
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));   // (addresses computed here, at every call: see redo_segments_kernel)
+  __syncthreads();
+  sh_hist[2 * tid] = __hip_atomic_load(gh + 2 * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  sh_hist[2 * tid + 1] = __hip_atomic_load(gh + 2 * tid + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  find_threshold_bin_1024(sh_hist, k, sh_wtot, sh_res);
+  *prefix = sh_res[0];
+  *need = k - sh_res[1];
+  *cnt = sh_res[2];
+  return *cnt == *need ? kRedoTakeBucket
+                       : (*cnt <= (uint32_t)kRedoBucketCap && batches_per_seg <= (uint32_t)kRedoMaxBatches ? kRedoCutBucket : kRedoAlone);
+}
+
+// This thread's 32 consecutive stored keys from token `first` on (a multiple of 32); key 0 at and beyond `n`.
+__device__ __forceinline__ void redo_load_run(const uint32_t* sk, uint32_t first, int64_t n, uint32_t (&keys)[32]) {
+  if ((((uintptr_t)sk) & 15u) == 0 && (int64_t)first + 32 <= n) {
+    u32x4 x[8];
+#pragma unroll
+    for (int v = 0; v < 8; ++v) x[v] = *(const u32x4*)(sk + first + 4 * v);
+#pragma unroll
+    for (int v = 0; v < 8; ++v)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) keys[4 * v + e] = x[v][e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < 32; ++e) keys[e] = (int64_t)first + e < n ? sk[first + e] : 0u;
+  }
+}
+
+// acc = 2 * acc + (a > b), and the same for a == b: two instructions per token build a mask of 32 tokens in the reverse
+// order of their bits.  (Written out: left to itself the compiler ors in one constant per bit position and keeps all of
+// them in registers across the kernel's loops, more registers than are left.)
+__device__ __forceinline__ void shift_in_gt(uint32_t& acc, uint32_t a, uint32_t b) {
+  asm("v_cmp_gt_u32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc" : "+v"(acc) : "v"(a), "v"(b) : "vcc");
+}
+__device__ __forceinline__ void shift_in_eq(uint32_t& acc, uint32_t a, uint32_t b) {
+  asm("v_cmp_eq_u32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc" : "+v"(acc) : "v"(a), "v"(b) : "vcc");
+}
+
+// Bits [a, b) of a 32-bit word, for 0 <= a, b <= 32 (none when b <= a).
+__device__ __forceinline__ uint32_t bit_range(uint32_t a, uint32_t b) {
+  const uint32_t below_b = b >= 32u ? ~0u : (1u << b) - 1u, below_a = a >= 32u ? ~0u : (1u << a) - 1u;
+  return b > a ? below_b & ~below_a : 0u;
+}
+
+// Launched behind select_finalize_cand_kernel on the candidate route, one workgroup per CU.  Every workgroup reads the
+// segment flags; when none is set (all but always) it leaves at once.  Otherwise the flagged segments are redone from
+// the keys, exactly, by all workgroups together, in phases.  The work of a phase is a list of items - a run of tokens,
+// or a segment - that the workgroups draw from a counter in memory; what an item leaves for a later phase goes out as
+// stores performed at the point of coherence, and when a workgroup finds the counter exhausted it waits until its
+// stores have completed and adds the number of its items to the phase's done count.  Then it waits until that count is
+// complete: every item it waits for has been drawn, so it is in the hands of a workgroup that is running - no
+// workgroup waits for one that has not started, and one workgroup alone would get through all phases by itself.  (The
+// wait is bounded all the same; a workgroup whose wait runs out leaves - it holds no item then, and the others finish
+// without it.)
+//   score   per chunk of 4096 tokens: the keys of the scores stored (canonical order), their top 11 bits counted into
+//           the segment's histogram in memory
+//   count   per batch of 32768 tokens, 32 consecutive ones per thread: the bucket of the k-th key from the histogram (a
+//           bucket that the top k take whole, or whose members fit the LDS, goes on here; any other segment is left to
+//           one workgroup in `cut`, redo_select_from_scores); tokens above the bucket counted (all / between the sink
+//           range and the local window), the members' composites written to the batch's part of the segment's list
+//   cut     per segment: the need-th largest of the members by radix passes in LDS (ties in the key fall to the
+//           smaller index, as everywhere), then every batch's first place in the union list and in the selection
+//   write   per batch: ids of the selected tokens to their place in the union list (the batch at the front of a segment
+//           also writes sink range, local window and count), composites to the selection
+//   finish  per segment, rank-ordered output only: the selection sorted and written
+// All 64 segments of 131072 tokens flagged: the step costs a bit over twice what it costs otherwise (the keys are read
+// a second time at the rate of the first, and little else), where one workgroup per segment took 14 times as long.
 template <int DT, bool RANK>
 __global__ __launch_bounds__(kSelThreads) void redo_segments_kernel(GemvParams g, SelectParams p, int kpad) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // the bucket's composites, then (rank mode) 2 * kpad composites
@@ -1342,113 +1419,347 @@ __global__ __launch_bounds__(kSelThreads) void redo_segments_kernel(GemvParams g
   __shared__ uint32_t sh_wtot[kSelWaves], sh_res[4];
   __shared__ uint64_t sh_mm[3];
   __shared__ uint16_t sh_flagged[kRedoMaxFlagged];
-  __shared__ uint32_t sh_item, sh_last;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-  // the flagged segments, in order (every workgroup builds the same list)
+  __shared__ uint32_t sh_item;
+  const int wave = threadIdx.x >> 6;
   uint32_t n_flagged = 0;
-  for (int s0 = 0; s0 < p.num_segments; s0 += kSelThreads) {
-    const int s = s0 + tid;
-    const bool flagged = s < p.num_segments && (p.seg_flags[s] & 1u) != 0u;
-    const unsigned long long m = __ballot(flagged);
-    if (lane == 0) sh_wtot[wave] = (uint32_t)__popcll(m);
-    __syncthreads();
-    uint32_t before = n_flagged, all = 0;
-    for (int w = 0; w < kSelWaves; ++w) {
-      const uint32_t c = sh_wtot[w];
-      before += w < wave ? c : 0u;
-      all += c;
+  {
+    // the flagged segments, in order (every workgroup builds the same list)
+    const int tid = threadIdx.x, lane = tid & 63;
+    for (int s0 = 0; s0 < p.num_segments; s0 += kSelThreads) {
+      const int s = s0 + tid;
+      const bool flagged = s < p.num_segments && (p.seg_flags[s] & 1u) != 0u;
+      const unsigned long long m = __ballot(flagged);
+      if (lane == 0) sh_wtot[wave] = (uint32_t)__popcll(m);
+      __syncthreads();
+      uint32_t before = n_flagged, all = 0;
+      for (int w = 0; w < kSelWaves; ++w) {
+        const uint32_t c = sh_wtot[w];
+        before += w < wave ? c : 0u;
+        all += c;
+      }
+      if (flagged) sh_flagged[before + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = (uint16_t)s;
+      n_flagged += all;
+      __syncthreads();
     }
-    if (flagged) sh_flagged[before + (uint32_t)__popcll(m & ((1ull << lane) - 1ull))] = (uint16_t)s;
-    n_flagged += all;
-    __syncthreads();
   }
   if (n_flagged == 0u) return;   // the ordinary case
 
-  const uint32_t chunks_per_seg = (uint32_t)((p.seg_len + kRedoChunk - 1) / kRedoChunk);
-  const uint32_t n_items = n_flagged * chunks_per_seg;
-  int cur = -1;        // segment of the chunks counted in sh_hist
-  uint32_t done = 0;   // how many of them
-  while (true) {
-    if (tid == 0) sh_item = __hip_atomic_fetch_add(p.redo_queue, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    const uint32_t item = sh_item;
-    const int seg = item < n_items ? (int)sh_flagged[item / chunks_per_seg] : -1;
-    if (seg != cur) {
-      if (cur >= 0) {
-        uint32_t* gh = p.redo_hist + (int64_t)cur * kHistBins;
-        for (int i = tid; i < kHistBins; i += kSelThreads)
-          if (sh_hist[i]) __hip_atomic_fetch_add(gh + i, sh_hist[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // Scores and counts were performed at the point of coherence; the arrival below must not overtake them: every
-        // wave waits until its own have completed (no write-back of the L2, which a release fence would ask for).
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (tid == 0) {
-          const uint32_t old = __hip_atomic_fetch_add(p.redo_arrive + cur, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          sh_last = old + done == chunks_per_seg ? 1u : 0u;
-        }
-        __syncthreads();
-        if (sh_last != 0u) {   // (uniform over the workgroup)
-          // the other workgroups' scores, announced by their arrivals, are read from here on: drop what the caches hold
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-          sh_hist[2 * tid] = __hip_atomic_load(gh + 2 * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          sh_hist[2 * tid + 1] = __hip_atomic_load(gh + 2 * tid + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          __syncthreads();
-          redo_select_from_scores<DT, RANK>(g, p, cur, kpad, smem, sh_hist, sh_off, sh_wtot, sh_res, sh_mm);
-        }
-      }
-      if (seg >= 0) {
-        __syncthreads();
+  const uint32_t k = (uint32_t)p.k;
+  const int64_t n = p.seg_len;
+  const uint32_t chunks_per_seg = (uint32_t)((n + kRedoChunk - 1) / kRedoChunk);
+  const uint32_t batches_per_seg = (uint32_t)((n + kRedoBatch - 1) / kRedoBatch);
+  const uint32_t lo = (uint32_t)(p.sink < n ? p.sink : n);
+  const uint32_t hi = (uint32_t)(n - p.local > lo ? n - p.local : lo);
+  const bool want_union = p.union_idx != nullptr;
+  constexpr int kTopShift = 32 - kHistBits;
+
+  for (int phase = 0; phase < (RANK ? kRedoPhases : kRedoFinish); ++phase) {
+    const uint32_t per_seg = phase == kRedoScore ? chunks_per_seg : (phase == kRedoCount || phase == kRedoWrite ? batches_per_seg : 1u);
+    const uint32_t n_items = n_flagged * per_seg;
+    uint32_t* drawn = p.redo_queue + 2 * phase;
+    uint32_t* finished = drawn + 1;
+    uint32_t done = 0, next = 0;
+    if (threadIdx.x == 0) next = __hip_atomic_fetch_add(drawn, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while (true) {
+      if (threadIdx.x == 0) sh_item = next;
+      __syncthreads();
+      const uint32_t item = sh_item;
+      __syncthreads();
+      if (item >= n_items) break;
+      ++done;
+      // (the next item is asked for now: the answer is back when this one is done)
+      if (threadIdx.x == 0) next = __hip_atomic_fetch_add(drawn, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // (What an item needs is computed at its start, from a thread number that the compiler cannot trace: kept in
+      // registers from the top of the kernel on, for all phases, these values cost more registers than there are.)
+      int tid = threadIdx.x;
+      asm volatile("" : "+v"(tid));
+      const int lane = tid & 63;
+      const int seg = (int)sh_flagged[item / per_seg];
+      const uint32_t part = item % per_seg;   // chunk or batch of the segment
+      uint32_t* rec = p.redo_rec + (int64_t)seg * p.redo_rec_stride;        // the segment's record, then four words per batch:
+      uint32_t* batch_words = rec + kRecWords + 4 * part;                    // above, above in [lo, hi), members (then: first place in the union list), first place in the selection
+      uint32_t* sk = (uint32_t*)(g.scores + (int64_t)seg * p.seg_stride);   // (keys, not scores: what the selection compares)
+      uint64_t* bucket = p.list + (int64_t)seg * p.list_stride;             // the bucket's members, every batch's at its own tokens' places
+      uint64_t* selection = bucket;                                         // (rank mode, from `write` on, when the members are spent) the selected composites
+      const uint32_t* gh = p.redo_hist + (int64_t)seg * kHistBins;
+      int32_t* uo = want_union ? p.union_idx + (int64_t)seg * (p.k + p.sink + p.local) : nullptr;
+
+      if (phase == kRedoScore) {
+        const int64_t t0 = (int64_t)part * kRedoChunk;
         sh_hist[2 * tid] = 0;
         sh_hist[2 * tid + 1] = 0;
-      }
-      cur = seg;
-      done = 0;
-    }
-    if (seg < 0) break;   // no chunk left (a workgroup that never drew one leaves here as well)
-    __syncthreads();      // (sh_item is drawn again; the histogram is cleared)
-    {
-      // (as the streaming GEMV does it: a uniform base per chunk and one 32-bit lane offset serve all loads - the launcher
-      // has checked that a chunk's rows lie within 2 GB of its first)
-      const uint32_t c = item % chunks_per_seg;
-      const int j = tid & 15, rg = tid >> 4;
-      const int bh = seg / g.num_chunks, chunk = seg % g.num_chunks;
-      const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
-      const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
-      float qf[8];
-      load_group_query<DT, 1>(g.q, g.q_stride_b, b, h, g.group, j, qf);
-      const uint32_t row_bytes = (uint32_t)g.key_stride_n * 2u;
-      const int64_t t0 = (int64_t)c * kRedoChunk;
-      const unsigned char* cbase = (const unsigned char*)g.keys +
-                                   2 * ((int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h + (chunk_base + t0) * g.key_stride_n);   // uniform
-      uint32_t* sk = (uint32_t*)(g.scores + (int64_t)seg * p.seg_stride + t0);   // (keys, not scores: what the selection compares)
-      const int n_local = (int)(p.seg_len - t0 < kRedoChunk ? p.seg_len - t0 : kRedoChunk);
-      constexpr int kRows = 8;
-      for (int base = 0; base < n_local; base += (kSelThreads / 16) * kRows) {
-        u32x4 kv[kRows];
+        __syncthreads();
+        {
+          // (as the streaming GEMV does it: a uniform base per chunk and one 32-bit lane offset serve all loads - the
+          // launcher has checked that a chunk's rows lie within 2 GB of its first)
+          const int j = tid & 15, rg = tid >> 4;
+          const int bh = seg / g.num_chunks, chunk = seg % g.num_chunks;
+          const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
+          const int64_t chunk_base = g.cluster_ids ? (int64_t)g.cluster_ids[seg] * g.chunk_len : (int64_t)chunk * g.chunk_len;
+          float qf[8];
+          load_group_query<DT, 1>(g.q, g.q_stride_b, b, h, g.group, j, qf);
+          const uint32_t row_bytes = (uint32_t)g.key_stride_n * 2u;
+          const unsigned char* cbase = (const unsigned char*)g.keys +
+                                       2 * ((int64_t)b * g.key_stride_b + (int64_t)h * g.key_stride_h + (chunk_base + t0) * g.key_stride_n);   // uniform
+          const int n_local = (int)(n - t0 < kRedoChunk ? n - t0 : kRedoChunk);
+          constexpr int kRows = 8;
+          for (int base = 0; base < n_local; base += (kSelThreads / 16) * kRows) {
+            u32x4 kv[kRows];
 #pragma unroll
-        for (int u = 0; u < kRows; ++u) {
-          int lt = base + rg * kRows + u;
-          lt = lt < n_local ? lt : n_local - 1;
-          kv[u] = __builtin_nontemporal_load((const u32x4*)(cbase + ((uint32_t)lt * row_bytes + 16u * (uint32_t)j)));
-        }
-        __builtin_amdgcn_sched_barrier(0);   // all loads go out before the first score is computed
-        float mine = 0.0f;
+            for (int u = 0; u < kRows; ++u) {
+              int lt = base + rg * kRows + u;
+              lt = lt < n_local ? lt : n_local - 1;
+              kv[u] = __builtin_nontemporal_load((const u32x4*)(cbase + ((uint32_t)lt * row_bytes + 16u * (uint32_t)j)));
+            }
+            __builtin_amdgcn_sched_barrier(0);   // all loads go out before the first score is computed
+            float mine = 0.0f;
 #pragma unroll
-        for (int u = 0; u < kRows; ++u) {
-          const float s = row_score<DT>(qf, kv[u], g.scale);
-          if (j == u) mine = s;
+            for (int u = 0; u < kRows; ++u) {
+              const float s = row_score<DT>(qf, kv[u], g.scale);
+              if (j == u) mine = s;
+            }
+            const int lt = base + rg * kRows + j;
+            if (j < kRows && lt < n_local) {
+              const uint32_t key = score_key(mine);
+              __hip_atomic_store(sk + t0 + lt, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              atomicAdd(&sh_hist[key >> kTopShift], 1u);
+            }
+          }
         }
-        const int lt = base + rg * kRows + j;
-        if (j < kRows && lt < n_local) {
-          const uint32_t key = score_key(mine);
-          __hip_atomic_store(sk + lt, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          atomicAdd(&sh_hist[key >> (32 - kHistBits)], 1u);
+        __syncthreads();
+        uint32_t* ghw = p.redo_hist + (int64_t)seg * kHistBins;
+        for (int i = tid; i < kHistBins; i += kSelThreads)
+          if (sh_hist[i]) __hip_atomic_fetch_add(ghw + i, sh_hist[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else if (phase == kRedoCount) {
+        // this thread's 32 tokens first: the loads do not depend on the threshold
+        const uint32_t first = part * (uint32_t)kRedoBatch + 32u * (uint32_t)tid;
+        uint32_t keys[32];
+        redo_load_run(sk, first, n, keys);
+        uint32_t prefix, need, cnt;
+        const int mode = redo_threshold(gh, k, batches_per_seg, sh_hist, sh_wtot, sh_res, &prefix, &need, &cnt);
+        if (mode != kRedoAlone) {   // (uniform)
+          if (tid == 0) {
+            sh_res[2] = 0u;
+            sh_res[3] = 0u;
+          }
+          __syncthreads();
+          const uint32_t valid = (int64_t)first < n ? bit_range(0u, (uint32_t)(n - first < 32 ? n - first : 32)) : 0u;
+          const uint32_t in_mid = bit_range(lo > first ? lo - first : 0u, hi > first ? hi - first : 0u);
+          uint32_t above = 0, tie = 0;
+#pragma unroll
+          for (int e = 0; e < 32; ++e) {
+            const uint32_t top = keys[e] >> kTopShift;
+            shift_in_gt(above, top, prefix);
+            shift_in_eq(tie, top, prefix);
+          }
+          above = __builtin_bitreverse32(above) & valid;
+          tie = __builtin_bitreverse32(tie) & valid;
+          if (mode == kRedoTakeBucket) {   // the members are taken like the tokens above them
+            above |= tie;
+            tie = 0;
+          }
+          const uint32_t packed = ((uint32_t)__builtin_popcount(above) << 16) | (uint32_t)__builtin_popcount(above & in_mid);
+          const uint32_t inc = wave_inclusive_scan(packed);   // (at most 2048 of either per wave)
+          if (lane == 63 && inc != 0u) atomicAdd(&sh_res[3], inc);
+          // the members: to the batch's own part of the segment's list (as many places as it has tokens), in any order
+          uint64_t* mine_at = bucket + (int64_t)part * kRedoBatch;
+          while (tie != 0u) {   // (few)
+            const uint32_t e = (uint32_t)__builtin_ctz(tie);
+            tie &= tie - 1u;
+            uint32_t key = 0;
+#pragma unroll
+            for (int q = 0; q < 32; ++q) key = (uint32_t)q == e ? keys[q] : key;   // (registers cannot be indexed)
+            __hip_atomic_store(mine_at + atomicAdd(&sh_res[2], 1u), composite(key, first + e), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          __syncthreads();
+          if (tid == 0) {
+            __hip_atomic_store(batch_words, sh_res[3] >> 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(batch_words + 1, sh_res[3] & 0xffffu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(batch_words + 2, sh_res[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
         }
+      } else if (phase == kRedoCut) {
+        uint32_t prefix, need, cnt;
+        const int mode = redo_threshold(gh, k, batches_per_seg, sh_hist, sh_wtot, sh_res, &prefix, &need, &cnt);
+        uint64_t cut = (uint64_t)prefix << (64 - kHistBits);   // kRedoTakeBucket: every member is taken
+        uint32_t mid_total;
+        if (mode == kRedoAlone) {
+          mid_total = redo_select_from_scores<DT, RANK>(g, p, seg, selection, smem, sh_hist, sh_off, sh_wtot, sh_res);
+        } else {
+          uint64_t* sh_buck = (uint64_t*)smem;
+          // (kRedoTakeBucket: the members were counted with the tokens above them, nothing was gathered and nothing is cut)
+          if (mode == kRedoCutBucket) {
+            // the members lie in their batches' parts of the list: first place of every batch's members among all of them
+            // (thread t: batches 2t, 2t+1), then every thread fetches members by their number
+            uint32_t held[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              const uint32_t b = 2u * (uint32_t)tid + e;
+              held[e] = b < batches_per_seg ? __hip_atomic_load(rec + kRecWords + 4 * b + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+            }
+            uint32_t total;
+            const uint32_t ex = block_exclusive_scan(held[0] + held[1], sh_wtot, &total);
+            sh_off[2 * tid] = ex;
+            sh_off[2 * tid + 1] = ex + held[0];
+            __syncthreads();
+            for (uint32_t i = tid; i < cnt; i += kSelThreads) {
+              uint32_t b = 0;   // the last batch whose first place is at or below i
+#pragma unroll
+              for (uint32_t step = kRedoMaxBatches / 2; step != 0u; step >>= 1)
+                if (b + step < batches_per_seg && sh_off[b + step] <= i) b += step;
+              sh_buck[i] = bucket[(int64_t)b * kRedoBatch + (i - sh_off[b])];
+            }
+            // the cut inside the bucket: the need-th largest of its members
+            uint64_t cprefix = prefix;   // top `cfixed` bits of the composite
+            int cfixed = kHistBits;
+            uint32_t left = need, among = cnt;
+            while (among != left && cfixed < 64) {
+              const int bits = (64 - cfixed) >= kHistBits ? kHistBits : (64 - cfixed);
+              const int shift = 64 - cfixed - bits;
+              __syncthreads();
+              sh_hist[2 * tid] = 0;
+              sh_hist[2 * tid + 1] = 0;
+              __syncthreads();
+              for (uint32_t i = tid; i < cnt; i += kSelThreads) {
+                const uint64_t cc = sh_buck[i];
+                if ((cc >> (64 - cfixed)) == cprefix) atomicAdd(&sh_hist[(uint32_t)(cc >> shift) & ((1u << bits) - 1u)], 1u);
+              }
+              __syncthreads();
+              find_threshold_bin_1024(sh_hist, left, sh_wtot, sh_res);
+              left -= sh_res[1];
+              cprefix = (cprefix << bits) | sh_res[0];
+              among = sh_res[2];
+              cfixed += bits;
+            }
+            cut = cfixed == 64 ? cprefix : cprefix << (64 - cfixed);   // every composite with these leading bits is taken
+          }
+          // the selected members of every batch (all / in [lo, hi))
+          __syncthreads();
+          sh_hist[2 * tid] = 0;
+          sh_hist[2 * tid + 1] = 0;
+          sh_off[2 * tid] = 0;
+          sh_off[2 * tid + 1] = 0;
+          __syncthreads();
+          for (uint32_t i = tid; i < (mode == kRedoCutBucket ? cnt : 0u); i += kSelThreads) {
+            const uint64_t cc = sh_buck[i];
+            if (cc >= cut) {
+              const uint32_t idx = ~(uint32_t)cc;
+              atomicAdd(&sh_hist[idx / (uint32_t)kRedoBatch], 1u);
+              if (idx - lo < hi - lo) atomicAdd(&sh_off[idx / (uint32_t)kRedoBatch], 1u);
+            }
+          }
+          __syncthreads();
+          // every batch's first place: thread t sums batches 2t, 2t+1 (selected << 16 | selected in [lo, hi): at most k each)
+          uint32_t mine[2];
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const uint32_t b = 2u * (uint32_t)tid + e;
+            mine[e] = 0u;
+            if (b < batches_per_seg) {
+              const uint32_t* bw = rec + kRecWords + 4 * b;
+              mine[e] = ((__hip_atomic_load(bw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + sh_hist[b]) << 16) |
+                        (__hip_atomic_load(bw + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + sh_off[b]);
+            }
+          }
+          uint32_t total;
+          const uint32_t ex = block_exclusive_scan(mine[0] + mine[1], sh_wtot, &total);
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const uint32_t b = 2u * (uint32_t)tid + e;
+            if (b < batches_per_seg) {
+              const uint32_t at = ex + (e ? mine[0] : 0u);
+              uint32_t* bw = rec + kRecWords + 4 * b;
+              __hip_atomic_store(bw + 2, at & 0xffffu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              __hip_atomic_store(bw + 3, at >> 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+          }
+          mid_total = total & 0xffffu;
+        }
+        if (tid == 0) {
+          __hip_atomic_store(rec + kRecPrefix, prefix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(rec + kRecMode, (uint32_t)mode, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(rec + kRecCutLo, (uint32_t)cut, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(rec + kRecCutHi, (uint32_t)(cut >> 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(rec + kRecMidTotal, mid_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      } else if (phase == kRedoWrite) {
+        // (the record and the batch's words were written by other workgroups in earlier phases, and what this CU's caches
+        // held was dropped at the end of the last one: plain loads, all of them in flight together)
+        const uint32_t first = part * (uint32_t)kRedoBatch + 32u * (uint32_t)tid;
+        uint32_t keys[32];
+        redo_load_run(sk, first, n, keys);
+        const u32x4 r = *(const u32x4*)rec;          // prefix, mode, cut
+        const u32x4 w = *(const u32x4*)batch_words;   // .., .., first place in the union list, in the selection
+        const uint32_t mid_total = rec[kRecMidTotal];
+        const int mode = (int)r[kRecMode];
+        if (mode != kRedoAlone) {   // (uniform)
+          // selected: the composite (key, ~index) is at least the cut
+          const uint32_t cut_key = r[kRecCutHi], cut_low = r[kRecCutLo];
+          const uint32_t valid = (int64_t)first < n ? bit_range(0u, (uint32_t)(n - first < 32 ? n - first : 32)) : 0u;
+          const uint32_t in_mid = bit_range(lo > first ? lo - first : 0u, hi > first ? hi - first : 0u);
+          uint32_t sel = 0, same = 0;
+#pragma unroll
+          for (int e = 0; e < 32; ++e) {
+            shift_in_gt(sel, keys[e], cut_key);
+            shift_in_eq(same, keys[e], cut_key);
+          }
+          sel = __builtin_bitreverse32(sel);
+          same = __builtin_bitreverse32(same);
+          while (same != 0u) {   // (few: tokens with the key of the cut fall to the smaller index)
+            const uint32_t e = (uint32_t)__builtin_ctz(same);
+            same &= same - 1u;
+            sel |= (~(first + e) >= cut_low ? 1u : 0u) << e;
+          }
+          sel &= valid;
+          const uint32_t mid = sel & in_mid;
+          uint32_t total;
+          const uint32_t ex = block_exclusive_scan(((uint32_t)__builtin_popcount(sel) << 16) | (uint32_t)__builtin_popcount(mid), sh_wtot, &total);
+          uint32_t pos_mid = lo + w[2] + (ex & 0xffffu), pos_sel = w[3] + (ex >> 16);
+          uint32_t rest = sel;
+          while (rest != 0u) {   // (few: k tokens out of the whole segment)
+            const uint32_t e = (uint32_t)__builtin_ctz(rest);
+            rest &= rest - 1u;
+            uint32_t key = 0;
+#pragma unroll
+            for (int q = 0; q < 32; ++q) key = (uint32_t)q == e ? keys[q] : key;   // (registers cannot be indexed)
+            if (RANK) {
+              if (pos_sel < k) __hip_atomic_store(selection + pos_sel, composite(key, first + e), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              ++pos_sel;
+            }
+            if (uo && (mid >> e & 1u)) uo[pos_mid++] = (int32_t)(first + e);
+          }
+        }
+        if (part == 0u && uo) write_union_edges(uo, p, seg, lo, hi, mid_total);
+      } else {   // kRedoFinish (RANK)
+        uint64_t* sh_sort = (uint64_t*)smem;
+        for (int i = tid; i < kpad; i += kSelThreads) sh_sort[i] = (uint32_t)i < k ? selection[i] : 0ull;  // pad: below every real composite
+        __syncthreads();
+        rank_sort_desc(sh_sort, sh_sort + kpad, k, kpad, sh_hist, sh_off, sh_wtot, sh_mm);
+        write_rank_outputs(sh_sort, p, seg);
       }
-      ++done;
     }
-    __syncthreads();   // (every wave has counted its scores before the histogram may be flushed)
+    if (phase == (RANK ? kRedoFinish : kRedoWrite)) break;
+    // what this workgroup's items leave for later phases has completed before they count as done
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    // ... and the items of this phase that other workgroups hold
+    if (threadIdx.x == 0) {
+      if (done != 0u) __hip_atomic_fetch_add(finished, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      int spins = 0;
+      while (__hip_atomic_load(finished, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < n_items && spins < kRedoWaitSpins) {
+        __builtin_amdgcn_s_sleep(8);
+        ++spins;
+      }
+      sh_item = spins < kRedoWaitSpins ? 1u : 0u;
+    }
+    __syncthreads();
+    const bool go_on = sh_item != 0u;
+    __syncthreads();
+    if (!go_on) return;   // (this workgroup holds no item: the others finish without it)
+    // what the other workgroups stored is read from here on: drop what the caches of this CU and its L2 hold (one wave
+    // does that for the workgroup; 4096 waves at it cost tens of microseconds per phase)
+    if (wave == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    __syncthreads();
   }
 }
 
@@ -2252,7 +2563,7 @@ SelectLayout select_layout(int num_segments, int64_t seg_len) {
   l.head = take(head_cand > head_cut ? head_cand : head_cut);
   l.list_cnt = take((size_t)num_segments * (size_t)max_parts * sizeof(uint32_t));
   l.list = take((size_t)num_segments * (size_t)l.list_stride * sizeof(uint64_t));
-  l.arrive = take((cand_segs + 1) * sizeof(uint32_t));   // arrival counts of the redo launch and its chunk counter (cleared by the selection when it flags a segment)
+  l.arrive = take(cand_segs ? 2 * kRedoPhasesMax * sizeof(uint32_t) : 0);   // item counters of the redo launch (cleared by the selection when it flags a segment)
   l.total = off;
   return l;
 }
@@ -2273,8 +2584,10 @@ size_t select_carve(void* ws, int num_segments, int64_t seg_len, SelectParams* p
   p->list_cnt = (uint32_t*)(c + l.list_cnt);
   p->list = (uint64_t*)(c + l.list);
   p->list_stride = l.list_stride;
-  p->redo_arrive = (uint32_t*)(c + l.arrive);
-  p->redo_queue = p->redo_arrive + num_segments;   // (redo_hist: the histograms, on the route that does not use them otherwise; set by the caller)
+  p->redo_queue = (uint32_t*)(c + l.arrive);
+  p->redo_rec = p->list_cnt;   // (the slice counts of the other routes: a record and four words per chunk of 4096 tokens fit)
+  p->redo_rec_stride = (seg_len / 128 + 2) & ~(int64_t)3;   // (whole 16-byte groups: the record is read with vector loads)
+  // (redo_hist: the histograms, on the route that does not use them otherwise; set by the caller)
   return (size_t)num_segments * kHistBins;  // the flags follow the histograms; candidate mode writes them itself
 }
 
@@ -2400,14 +2713,15 @@ int launch_select_rank(const GemvParams& g, const SelectParams& p, int dtype, hi
   return hip_status(hipGetLastError());
 }
 
-// Behind launch_select_finalize_cand on the candidate route (p.redo_hist / p.redo_arrive set there too): redoes the segments
+// Behind launch_select_finalize_cand on the candidate route (p.redo_hist / p.redo_queue set there too): redoes the segments
 // that the selection flagged, all workgroups of the launch sharing the work; leaves at once when there is none.
 bool redo_segments_fits(const GemvParams& g, int num_segments) {
   return g.key_stride_n * 2 * (int64_t)kRedoChunk <= 0x7fffffffLL && num_segments <= kRedoMaxFlagged;
 }
 
 int launch_redo_segments(const GemvParams& g, const SelectParams& p, int dtype, hipStream_t stream) {
-  if (!p.redo_hist || !p.redo_arrive || !p.redo_queue || !p.seg_flags || !g.scores || !redo_segments_fits(g, p.num_segments))
+  if (!p.redo_hist || !p.redo_queue || !p.redo_rec || !p.list || !p.seg_flags || !g.scores || !redo_segments_fits(g, p.num_segments) ||
+      p.list_stride < p.seg_len || p.redo_rec_stride < kRecWords + 4 * ((p.seg_len + kRedoBatch - 1) / kRedoBatch))
     return TKA_EINVAL;
   const bool want_rank = p.out_idx != nullptr;
   const int kpad = kpad_for(p.k);
