@@ -609,6 +609,16 @@ def test_sparse_decode_step_forced_redo(hooks):
     test_sparse_decode_step_union_only(oracle.BF16, 1, 2, 4, 66001, 1500, 32, 100, "levels")
 
 
+@pytest.mark.parametrize("kind,N,k,sink,local", [("equal", 70000, 1500, 32, 100), ("levels", 140000, 2048, 64, 512),
+                                                 ("heavy", 80000, 2048, 30000, 60000), ("heavy", 70001, 1000, 0, 0)])
+def test_sparse_decode_step_redo_launch_union(hooks, kind, N, k, sink, local):
+    """Union mode of the launch that redoes flagged long segments: one score for all tokens (a bucket beyond the LDS, cut
+    by rank in index order), 16-level keys (ties inside the bucket), a sink range and a local window that overlap (nothing
+    between them), and neither of the two."""
+    hooks(force_segment_redo=1)
+    test_sparse_decode_step_union_only(oracle.F16, 1, 2, 4, N, k, sink, local, kind)
+
+
 def test_sparse_decode_step_list_behind_forced_redo(hooks):
     """A caller that asks for the ascending list on segments that the common-cut route takes (the list for the attention stays
     in the workspace, the caller's list is made from the rank-ordered ids by one more launch), with every segment redone from

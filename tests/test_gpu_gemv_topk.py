@@ -466,6 +466,46 @@ def test_long_segment_forced_redo(hooks):
     _check_long(K, randn_bits(rng, (1, 8, 128), oracle.F16), oracle.F16, 4, 3000, redone=2)
 
 
+def _redo_keys(rng, N, H, dtype, kind):
+    """Keys for the three ways the launch that redoes flagged segments can go on after the bucket of the k-th key is
+    known (the query of these cases is the same in all 128 dimensions, so a key row's score is a multiple of its sum)."""
+    if kind == "two_values":   # scores +c and -c: with k = number of the larger ones the bucket is taken whole
+        rows = np.where(rng.random((1, N, H, 1)) < 0.03, 0.5, -0.5) * np.ones((1, 1, 1, 128))
+    elif kind == "equal":      # one score for all tokens: a bucket beyond the LDS whose members only their index tells apart
+        rows = np.full((1, N, H, 128), 0.25)
+    elif kind == "narrow":     # all scores inside one bucket of the 11 leading key bits, many of them different
+        rows = 0.25 + rng.integers(0, 64, (1, N, H, 128)) / 4096.0
+    else:                      # "heavy": ordinary data, a few rows four times as long
+        rows = rng.standard_normal((1, N, H, 128))
+        rows[0, rng.permutation(N)[:N // 100]] *= 4.0
+    return oracle.to_bits(rows, dtype)
+
+
+@pytest.mark.parametrize("kind,N,k", [("heavy", 70001, 3000), ("two_values", 80000, 0), ("equal", 66000, 2000), ("narrow", 131072, 2048),
+                                      ("heavy", 300000, 4096)])
+def test_long_segment_redo_launch(hooks, kind, N, k):
+    """Every segment flagged (force_segment_redo) on the route of the long segments: the launch behind the selection
+    redoes them, all workgroups sharing the work, and goes on - by the bucket of the k-th key - with the whole bucket taken,
+    with its members gathered and cut, or with one workgroup selecting (a bucket beyond the LDS: narrowed by counting
+    passes, or, where all its members carry one key, cut by their rank in index order).  Rank-ordered output."""
+    from topk_attn_amd import ops
+    announce("gemv_topk long segments, all redone by the launch behind the selection: %s N=%d k=%d" % (kind, N, k))
+    hooks(force_segment_redo=1)
+    rng = np.random.default_rng(91)
+    dtype, H, G = oracle.F16, 2, 2
+    K = _redo_keys(rng, N, H, dtype, kind)
+    q = randn_bits(rng, (1, H * G, 128), dtype) if kind == "heavy" else oracle.to_bits(np.full((1, H * G, 128), 0.125), dtype)
+    if kind == "two_values":   # (head 0's count of the larger score; head 1 then cuts inside its bucket or takes less than it)
+        ref = oracle.scores_canonical(K[0, :, 0, :], dtype, oracle.group_query(q[0, 0:G], dtype, G), SCALE)
+        k = int((ref > 0).sum())
+    ops.profile_reset()
+    ops.profile_enable(True)
+    _check_long(K, q, dtype, G, k, redone=H)
+    ran = ops.profile_read()
+    ops.profile_enable(False)
+    assert "redo_segments" in ran and "select_finalize_cand" in ran, sorted(ran)
+
+
 def test_long_segments_sixteen_heads():
     """Sixteen KV heads: the rows of one head lie 4 KB apart, and the streaming workgroups take their slices in units
     that go round the segments instead of segment by segment (137 slices per segment: the last unit of each is short)."""
