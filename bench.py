@@ -384,10 +384,10 @@ def build_workload(name, torch, ops, dev, args):
 # the counter run and the digest of the kernel's source at the time of that run: a figure is only reported
 # while the source still has that digest.
 RECORDED_TRAFFIC = {
-    ("c4", "gemv_candidates"): {"bytes": 2186875801,   # 2 x 1066323.2 KiB + 2974.5 KiB
+    ("c4", "gemv_candidates"): {"bytes": 2189277696,   # 2 x 1066292.4 KiB + 5381.7 KiB
                                 "source": "profiles/gemv_candidates_c4.md",
                                 "kernel_source": "topk_attn_amd/csrc/gemv_scores.hip",
-                                "kernel_source_sha16": "17a93e35519f2916"},
+                                "kernel_source_sha16": "74ccf271f9b5266a"},
 }
 
 
@@ -424,6 +424,9 @@ def main():
                     help="c1, c2, c2-ref, ra: number of key sets taken in turn (working set beyond the Infinity Cache)")
     ap.add_argument("--probe-threads", type=int, default=512, choices=[256, 512], help="probe-stream: threads per workgroup")
     ap.add_argument("--probe-rounds", type=int, default=2, help="probe-stream: rounds of eight loads per lane (512 x 2 = the GEMV's shape)")
+    ap.add_argument("--force-redo", action="store_true",
+                    help="every step with every long segment redone from the keys (the library's testing hook): the worst case of the "
+                         "step, for a kernel trace of it; the line says so in config.forced_redo")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-runs", type=int, default=5)
     args = ap.parse_args()
@@ -441,6 +444,12 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = build_workload(args.workload, torch, ops, dev, args)
+    if args.force_redo:
+        if not hasattr(w, "hooks"):
+            print("bench.py: --force-redo applies to the workloads that select (c1, c4*, c5*)", file=sys.stderr)
+            return 2
+        w.hooks = dict(w.hooks, force_segment_redo=1)
+        ops.set_test_hooks(**w.hooks)
 
     for _ in range(args.warmup):
         w.step()
@@ -509,7 +518,7 @@ def main():
     # The step when EVERY segment is redone from its keys (the testing hook makes the selection refuse every candidate
     # count): the bound on what a step can cost whatever the data does.
     worst_us = worst_redone = None
-    if hasattr(w, "hooks") and hasattr(w, "redone_segments"):
+    if hasattr(w, "hooks") and hasattr(w, "redone_segments") and not args.force_redo:
         ops.set_test_hooks(force_segment_redo=1, **w.hooks)
         worst_us = median_us(w.step, min(args.steps, 10))
         worst_redone = w.redone_segments()
@@ -534,7 +543,7 @@ def main():
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (seeded torch generator on the GPU)",
-        "config": dict({"workload": w.desc, "algorithmic_bytes_per_step": step_bytes}, **extra),
+        "config": dict({"workload": w.desc, "algorithmic_bytes_per_step": step_bytes}, **dict(extra, **({"forced_redo": True} if args.force_redo else {}))),
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_us, 2)},
