@@ -426,6 +426,13 @@ def test_two_level_long_clusters(CSZ, CLEN):
         assert np.array_equal(out[h], want)
 
 
+def test_two_level_long_clusters_redone(hooks):
+    """The same with every token-stage segment flagged: the launch that redoes them scores the clusters that the centre
+    stage picked (the segments' places come from the cluster ids) and writes global token ids."""
+    hooks(force_segment_redo=1)
+    test_two_level_long_clusters(3, 131072)
+
+
 def test_long_segment_plan_reuse():
     """One plan (one workspace) run three times with a new query each time: thresholds of an earlier run must
     never be taken for the current one."""

@@ -486,17 +486,17 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_kernel(SelectPara
 // scores until the k-th largest key is fixed, then one walk in index order that takes every key above the threshold
 // bucket and the first `need` keys inside it.  Exact for any data.  Two forms: one workgroup does all of it for its
 // segment (fallback_segment: one CU streams the segment, about a millisecond per 131072 tokens; the short segments of
-// the common-cut route and the combine launch of the one-launch selection + attention), or the workgroups of a launch of
-// their own share the scoring of all flagged segments and the last of them to finish a segment selects from its scores
-// (redo_segments_kernel; the long segments of the candidate route).
+// the common-cut route and the combine launch of the one-launch selection + attention), or all workgroups of a launch of
+// their own share the work on all flagged segments, phase by phase (redo_segments_kernel; the long segments of the
+// candidate route).
 
 // Scores of tokens [t0, t1) of segment `seg` (all 1024 threads: 64 row groups of 16 lanes, 16 rows in flight each),
 // stored to the segment's place in g.scores, with the top key bits counted in sh_hist (LDS, 2048 bins; not cleared here).
-// kRows: rows in flight per lane (16 where one CU has to pull a whole segment; 8 where many workgroups share the work).
-template <int DT, int kRows = 16>
+template <int DT>
 __device__ __forceinline__ void fallback_score_range(const GemvParams& g, const SelectParams& p, int seg, int64_t t0, int64_t t1, uint32_t* sh_hist) {
   const int tid = threadIdx.x;
   float* sc = g.scores + (int64_t)seg * p.seg_stride;
+  constexpr int kRows = 16;
   const int j = tid & 15, rg = tid >> 4;
   const int chunk = seg % g.num_chunks, bh = seg / g.num_chunks;
   const int h = bh % g.num_kv_heads, b = bh / g.num_kv_heads;
@@ -1002,7 +1002,7 @@ __global__ __launch_bounds__(kSelThreads) void select_finalize_cand_kernel(GemvP
 // ---- redo of flagged long segments, in a launch of its own --------------------------------------------------
 
 // (redo_segments_kernel, below, says how the work is shared.)
-constexpr int kRedoChunk = 4096;
+constexpr int kRedoChunk = 4096;        // tokens of an item of the scoring phase
 constexpr int kRedoMaxFlagged = 2048;   // segments of a call (the list of the flagged ones is kept in LDS)
 constexpr int kRedoBucketCap = 16384;   // composites of the threshold bucket held in LDS (128 KB) while the cut inside it is searched
 
