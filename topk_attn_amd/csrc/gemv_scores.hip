@@ -669,7 +669,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(8,
 // (entry, head), exactly as the one-entry kernel leaves them: the selection behind it does not know the difference.
 // The kernel is bound by the vector units, not by memory (B x 128 multiply-adds per row and their 16-lane sums, with
 // the packed two-per-instruction form of the fp32 multiply-add not used here): batch 8 over 8 heads x 131072 tokens
-// takes 108 us where the one-entry kernel takes 314 for the same scores.
+// takes 84 us where the one-entry kernel takes 311 for the same scores.
 // One slice per workgroup, slices numbered (head, batch tile)-major (workgroups that take several slices each at the
 // front of the grid, as the one-entry kernel has them, cost 3 us here).  Sampling workgroups: sample_role, one
 // segment each.
@@ -680,6 +680,7 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(4,
   // streaming: keys of the slice for BQ entries, then wave counts and thresholds; sampling: histogram
   constexpr int kWords = BQ * kCandThreads + BQ * kCandWaves + 4 * BQ;
   __shared__ uint32_t sh[kWords > kHistBins + 16 ? kWords : kHistBins + 16];
+  __shared__ __attribute__((aligned(16))) float sh_q[BQ * kHeadDim];   // group queries of the tile's entries
   const int tid = threadIdx.x;
   if ((int)blockIdx.x < p.sample_wgs) {
     __builtin_amdgcn_s_setprio(3);   // everyone else waits for these few waves
@@ -702,36 +703,80 @@ __global__ __launch_bounds__(kCandThreads) __attribute__((amdgpu_waves_per_eu(4,
   const uint32_t row_bytes = (uint32_t)p.key_stride_n * 2u;
   const int my_q = j / LPQ, my_row0 = (j % LPQ) * RPL;
 
-  // ---- scores of the slice for the BQ entries of the tile, as keys into LDS
+  // ---- the rows of the first round are asked for before anything else: they travel beside the queries
+  const unsigned char* sbase = (const unsigned char*)p.keys + 2 * ((int64_t)h * p.key_stride_h + t_begin * p.key_stride_n);
+  u32x4 kv[kGemvUnroll];
+  auto ask = [&](int it, int first) {   // four rows of round `it`
+#pragma unroll
+    for (int u = first; u < first + 4; ++u) {
+      int lt = it * kCandRowsPerIter + rg * kGemvUnroll + u;
+      lt = lt < n_local ? lt : n_local - 1;
+      kv[u] = __builtin_nontemporal_load((const u32x4*)(sbase + ((uint32_t)lt * row_bytes + 16u * (uint32_t)j)));
+    }
+  };
+  ask(0, 0);
+  ask(0, 4);
+
+  // ---- the group queries of the tile's entries, summed once for the workgroup: every one of its 32 row groups needs all
+  // of them, and each lane summing its own (BQ entries x G heads: 32 loads, 256 widenings and 192 adds at G = 4) was a
+  // fifth of the kernel's instructions.  Thread x: two dims of one entry, heads added in ascending order in fp32
+  // (sum_group_query's order).
+  for (int x = tid; x < BQ * (kHeadDim / 2); x += kCandThreads) {
+    const int e = x / (kHeadDim / 2), d = x % (kHeadDim / 2) * 2;
+    const int b = b0 + e < p.batch ? b0 + e : p.batch - 1;
+    const uint16_t* qb = (const uint16_t*)p.q + (int64_t)b * p.q_stride_b + (int64_t)h * p.group * kHeadDim + d;
+    uint32_t w[8];
+#pragma unroll
+    for (int g = 0; g < 8; ++g) w[g] = g < p.group ? *(const uint32_t*)(qb + g * kHeadDim) : 0u;
+    float s0 = Elem<DT>::widen((uint16_t)w[0]), s1 = Elem<DT>::widen((uint16_t)(w[0] >> 16));
+#pragma unroll
+    for (int g = 1; g < 8; ++g)
+      if (g < p.group) {
+        s0 = s0 + Elem<DT>::widen((uint16_t)w[g]);
+        s1 = s1 + Elem<DT>::widen((uint16_t)(w[g] >> 16));
+      }
+    sh_q[e * kHeadDim + d] = s0;
+    sh_q[e * kHeadDim + d + 1] = s1;
+  }
+  __syncthreads();
+
+  // ---- scores of the slice for the BQ entries of the tile, as keys into LDS.  Four rows are computed while the next four
+  // are on their way (the kernel is bound by the vector units; with all eight rows of a round asked for and then awaited
+  // together its four waves per SIMD did not cover the wait).
   {
     float qf[BQ][8];
 #pragma unroll
-    for (int q = 0; q < BQ; ++q) load_group_query<DT, 1>(p.q, p.q_stride_b, b0 + q < p.batch ? b0 + q : p.batch - 1, h, p.group, j, qf[q]);
-    const unsigned char* sbase = (const unsigned char*)p.keys + 2 * ((int64_t)h * p.key_stride_h + t_begin * p.key_stride_n);
-    for (int it = 0; it < kCandThreads / kCandRowsPerIter; ++it) {
-      u32x4 kv[kGemvUnroll];
+    for (int q = 0; q < BQ; ++q) {
+      const f32x4 lo = *(const f32x4*)(sh_q + q * kHeadDim + 8 * j), hi = *(const f32x4*)(sh_q + q * kHeadDim + 8 * j + 4);
 #pragma unroll
-      for (int u = 0; u < kGemvUnroll; ++u) {
-        int lt = it * kCandRowsPerIter + rg * kGemvUnroll + u;
-        lt = lt < n_local ? lt : n_local - 1;
-        kv[u] = __builtin_nontemporal_load((const u32x4*)(sbase + ((uint32_t)lt * row_bytes + 16u * (uint32_t)j)));
+      for (int i = 0; i < 4; ++i) {
+        qf[q][i] = lo[i];
+        qf[q][4 + i] = hi[i];
       }
-      __builtin_amdgcn_sched_barrier(0);   // all eight loads go out before the first score is computed
+    }
+    constexpr int kRounds = kCandThreads / kCandRowsPerIter;
+#pragma unroll
+    for (int it = 0; it < kRounds; ++it) {
       float mine[RPL];
 #pragma unroll
       for (int i = 0; i < RPL; ++i) mine[i] = 0.0f;
 #pragma unroll
-      for (int u = 0; u < kGemvUnroll; ++u) {
-        float acc[BQ];
+      for (int half = 0; half < 2; ++half) {
 #pragma unroll
-        for (int q = 0; q < BQ; ++q) {
-          acc[q] = 0.0f;
+        for (int u = 4 * half; u < 4 * half + 4; ++u) {
+          float acc[BQ];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) acc[q] = __builtin_fmaf(qf[q][i], Elem<DT>::get(kv[u], i), acc[q]);
+          for (int q = 0; q < BQ; ++q) {
+            acc[q] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[q] = __builtin_fmaf(qf[q][i], Elem<DT>::get(kv[u], i), acc[q]);
+          }
+          const float sc = row16_reduce_scatter<BQ>(acc, j) * p.scale;
+          if (u / RPL * RPL == my_row0) mine[u % RPL] = sc;
+          __builtin_amdgcn_sched_barrier(0);   // one row at a time (see gemv_scores_shared_kernel)
         }
-        const float sc = row16_reduce_scatter<BQ>(acc, j) * p.scale;
-        if (u / RPL * RPL == my_row0) mine[u % RPL] = sc;
-        __builtin_amdgcn_sched_barrier(0);   // one row at a time (see gemv_scores_shared_kernel)
+        if (it + 1 < kRounds) ask(it + 1, 4 * half);   // (their registers are free now)
+        __builtin_amdgcn_sched_barrier(0);
       }
       uint32_t* dst = sh_key + my_q * kCandThreads + it * kCandRowsPerIter + rg * kGemvUnroll + my_row0;
 #pragma unroll
