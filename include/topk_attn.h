@@ -122,7 +122,9 @@ int tka_gemv_scores(const tka_gemv_topk_args* args);
  * how many of its segments were redone from the keys by the selection kernel.  Long segments are selected from
  * candidates above a threshold sampled inside the GEMV launch; a segment whose candidates turn out fewer than k,
  * or more than fit, or one of whose streaming workgroups ran out of its bounded wait for the threshold, is
- * redone - exact, but about a millisecond per 131072 tokens.  0 for calls that do not take that path.
+ * redone - exact; all CUs share that work in a launch behind the selection, and a call with EVERY segment redone
+ * costs about 2.3 times the ordinary one (one workgroup redoes a segment on the routes of the shorter segments:
+ * a quarter of a millisecond per 32768 tokens).  0 for calls that do not take that path.
  * Waits for the stream. */
 int tka_gemv_topk_redone_segments(const tka_gemv_topk_args* args, int32_t* count);
 /* Same protocol: *count = candidate slices of that call (512 tokens each; 256 on calls that announce the cut of a
