@@ -619,6 +619,16 @@ def test_sparse_decode_step_redo_launch_union(hooks, kind, N, k, sink, local):
     test_sparse_decode_step_union_only(oracle.F16, 1, 2, 4, N, k, sink, local, kind)
 
 
+@pytest.mark.parametrize("N,k", [(70001, 1500), (140000, 4096)])
+def test_sparse_decode_step_redo_launch_all_outputs(hooks, N, k):
+    """The step that returns everything - rank-ordered top-k, ascending union list, attention output - on long segments
+    with every segment redone by the launch behind the selection (its form that sorts the selection at the end); and
+    without the hook, from the candidates."""
+    for forced in (1, 0):
+        hooks(force_segment_redo=forced)
+        test_sparse_decode_step(oracle.F16, torch.float16, 1, 2, 4, N, k, 64, 512)
+
+
 def test_sparse_decode_step_list_behind_forced_redo(hooks):
     """A caller that asks for the ascending list on segments that the common-cut route takes (the list for the attention stays
     in the workspace, the caller's list is made from the rank-ordered ids by one more launch), with every segment redone from
