@@ -132,6 +132,43 @@ def test_c4_end_to_end_full_size():
     print("c4 full size: worst attention error %.2e (bf16 output), %.2e (fp16 output, strict 2e-3)" % (worst, worst16), flush=True)
 
 
+def test_c4_shared_cache_full_size():
+    """c4's shapes over ONE cache that the batch shares (kv_stride_b = 0), where one pass over the keys scores the eight
+    batch entries: the step must give, bit for bit in its lists and its output, what it gives when every batch entry
+    holds its own copy of that cache (the per-entry kernels, pinned above) - and one (batch entry, KV head) pair goes through
+    the CPU oracle as well."""
+    from topk_attn_amd import ops
+    announce("c4 over a shared cache: B=8 Hq=32 Hkv=8 N=131072 fp16 k=2048, against per-entry copies of the cache")
+    B, H, G, N, k, sink, local = 8, 8, 4, 131072, 2048, 64, 512
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(404)
+    dt = torch.float16
+    q = torch.randn((B, H * G, 128), generator=gen, device="cuda").to(dt)
+    K1 = _randn16((1, N, H, 128), dt, gen)
+    V1 = _randn16((1, N, H, 128), dt, gen)
+    for h in range(H):
+        hh = torch.randperm(N, generator=gen, device="cuda")[:N // 100]
+        K1[0, hh, h] = (K1[0, hh, h].float() * 4.0).to(dt)
+    shared = ops.SparseDecodePlan(q, K1[0], V1[0], k, sink, local, SCALE, G, out_dtype=torch.float16)
+    ops.profile_reset()
+    ops.profile_enable(True)
+    shared.step()
+    torch.cuda.synchronize()
+    ran = ops.profile_read()
+    ops.profile_enable(False)
+    assert "gemv_candidates_shared" in ran, sorted(ran)
+    assert shared.redone_segments() == 0
+    Kb, Vb = K1.expand(B, N, H, 128).contiguous(), V1.expand(B, N, H, 128).contiguous()
+    own = ops.SparseDecodePlan(q, Kb, Vb, k, sink, local, SCALE, G, out_dtype=torch.float16)
+    own.step()
+    torch.cuda.synchronize()
+    assert torch.equal(shared.topk_idx, own.topk_idx) and torch.equal(shared.topk_val.view(torch.int32), own.topk_val.view(torch.int32))
+    assert torch.equal(shared.union_count, own.union_count) and torch.equal(shared.union_idx, own.union_idx)
+    assert torch.equal(shared.out, own.out), "outputs differ: %g" % (shared.out.float() - own.out.float()).abs().max().item()
+    _check_against_oracle([(B - 1, 3)], q, Kb, Vb, G, oracle.F16, k, sink, local, shared.topk_idx, shared.topk_val, shared.union_idx,
+                          shared.union_count, [(shared.out, lambda ro: 2e-3)])
+
+
 def _levels16(shape, dt, gen):
     levels = torch.linspace(-2, 2, 16, device="cuda")
     out = torch.empty(shape, dtype=dt, device="cuda")
