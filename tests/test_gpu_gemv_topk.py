@@ -695,6 +695,29 @@ def test_common_cut_route_chunked():
             assert np.array_equal(val[0, h, c * k:(c + 1) * k].view(np.uint32), ev.view(np.uint32))
 
 
+@pytest.mark.parametrize("forced", [0, 1])
+def test_long_chunks_route_chunked(hooks, forced):
+    """Two chunks of 70 000 tokens per head on the route of the long segments (a chunk is a segment; indices count over the
+    whole sequence), from the candidates and with every chunk redone by the launch behind the selection."""
+    announce("gemv_topk long segments, 2 chunks x 70000, forced redo %d" % forced)
+    from topk_attn_amd import ops
+    hooks(force_segment_redo=forced)
+    rng = np.random.default_rng(57)
+    dtype, C, k, G = oracle.BF16, 70000, 1500, 2
+    K = randn_bits(rng, (1, 2 * C, 2, 128), dtype)
+    q = randn_bits(rng, (1, 2 * G, 128), dtype)
+    plan = ops.GemvTopkPlan(to_dev(q, dtype), to_dev(K, dtype), k, group=G, scale=SCALE, num_chunks=2).run()
+    torch.cuda.synchronize()
+    assert plan.redone_segments() == (4 if forced else 0)
+    idx, val = plan.idx.cpu().numpy(), plan.val.cpu().numpy()
+    for h in range(2):
+        ref = oracle.scores_canonical(K[0, :, h, :], dtype, oracle.group_query(q[0, h * G:(h + 1) * G], dtype, G), SCALE)
+        for c in range(2):
+            ei, ev = oracle.topk_stable(ref[c * C:(c + 1) * C], k)
+            assert np.array_equal(idx[0, h, c * k:(c + 1) * k], ei + c * C), "indices differ (h=%d chunk %d)" % (h, c)
+            assert np.array_equal(val[0, h, c * k:(c + 1) * k].view(np.uint32), ev.view(np.uint32))
+
+
 # ---- key caches that are views: padded head dimension, head-major storage ----
 
 @pytest.mark.parametrize("layout", ["padded_heads", "head_major"])
